@@ -1,0 +1,219 @@
+/*
+ * poptransformer_hip.h — C ABI of libpoptransformer_hip.so (gfx950 / MI355X).
+ *
+ * This library replaces PopTransformer's `custom_ops.so` (PopART custom ops whose bodies
+ * are Poplar programs and IPU codelets) for the per-token decode path.  The reference
+ * library exports no C symbols: its ops self-register with PopART when it is dlopen'ed at
+ * poptransformer/ops/customized.py:17-18.  Here each op is one extern "C" function over raw
+ * device pointers, called from the Python `ops` layer with ctypes.
+ *
+ * Rules common to every entry point
+ *   - all pointers are DEVICE pointers unless the parameter name starts with `host_`;
+ *   - fp16 tensors are passed as `pta_half*` (IEEE binary16 bit patterns);
+ *   - `stream` is a hipStream_t (NULL = the default stream);
+ *   - nothing is allocated, freed or synchronised: work is only enqueued on `stream`, so a
+ *     call may be recorded into a HIP graph;
+ *   - return value: PTA_OK (0) or a negative PTA_E* code; the message of the most recent
+ *     failure on the calling thread is returned by pta_last_error().  Nothing throws.
+ *     Shape/dtype predicates mirror the reference's setup()/grow() guards so that an
+ *     invalid call fails where the reference would have refused to build its graph.
+ */
+#ifndef POPTRANSFORMER_HIP_H
+#define POPTRANSFORMER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t pta_half;
+typedef void* pta_stream_t;
+
+enum {
+  PTA_OK = 0,
+  PTA_EINVAL = -1,       /* bad shape / dtype / alignment / null pointer            */
+  PTA_EUNSUPPORTED = -2, /* valid in the reference but not implemented here         */
+  PTA_EHIP = -3          /* the HIP runtime reported an error (see pta_last_error)  */
+};
+
+/* Library version (major*10000 + minor*100 + patch).  Stands in for the SDK-version
+ * check custom_ops/compile_time_version.h:33-43 performs in a dlopen constructor. */
+int pta_version(void);
+const char* pta_last_error(void);
+
+/* ------------------------------------------------------------------------------------
+ * INT4 weights
+ * ---------------------------------------------------------------------------------- */
+
+/* Int4ToHalf (ops/customized.py:115-125; custom_ops/int4_to_half_custom_op.cpp:65-108,
+ * 168-278, 280-380; codelets custom_ops/int4_to_half_codelets.cpp:18-74).
+ * packed int8 [n, m]; every byte holds two signed 4-bit values, hi = b >> 4 (arithmetic),
+ * lo = (int8)(b << 4) >> 4.
+ *   axis == 1: scale fp16 [n]; out fp16 [2m, n]; out[2j,r] = hi(P[r,j])*scale[r],
+ *              out[2j+1,r] = lo(P[r,j])*scale[r]
+ *   axis == 0: scale fp16 [m]; out fp16 [2n, m]; out[2i,c] = hi(P[i,c])*scale[c],
+ *              out[2i+1,c] = lo(P[i,c])*scale[c]
+ * The product is one fp16 multiply (round to nearest even).  Bit-exact. */
+int pta_int4_to_half(const int8_t* packed, const pta_half* scale, pta_half* out, int n, int m,
+                     int axis, pta_stream_t stream);
+
+/* Re-tiling of a packed INT4 weight for the fused GEMV/GEMM below.  The reference does the
+ * same kind of load-time re-layout when it copies the unpacked matrix into the matmul-RHS
+ * layout (custom_ops/int4_to_half_custom_op.cpp:366-378).  `packed` is the checkpoint layout
+ * int8 [N, K/2] (N output channels, K input features); `tiled` receives
+ * pta_w4_tiled_bytes(N, K) bytes.  K must be even. */
+size_t pta_w4_tiled_bytes(int N, int K);
+int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t stream);
+
+/* Epilogue applied to the fp16-rounded product Y0 = fp16(X @ W) of the fused GEMMs.
+ * Each step is one fp16 operation, in the order the reference graphs apply them
+ * (layers/linear.py:42-46 bias add; models' residual `ops.add`). */
+typedef struct pta_epilogue {
+  const pta_half* bias;     /* [N] or NULL:      Y = Y0 + bias                                  */
+  const pta_half* residual; /* [M, N] or NULL:   Y = Y + residual                               */
+  int act;                  /* PTA_ACT_*: applied after bias, before residual                   */
+} pta_epilogue;
+
+enum { PTA_ACT_NONE = 0, PTA_ACT_GELU_TANH = 1, PTA_ACT_RELU_SQUARE = 2, PTA_ACT_SIGMOID = 3 };
+
+/* Fused Int4ToHalf(axis=1) + MatMul (utils/param_handler/precision_strategy.py:56-60,74-75):
+ * Y[M,N] = fp16( X[M,K] @ W ), W[k,n] = fp16(nibble(k,n) * scale[n]) exactly as
+ * pta_int4_to_half(axis=1) would produce, fp32 accumulation, never materialised.
+ * `tiled` comes from pta_w4_tile.  1 <= M <= 64.  `epi` may be NULL. */
+int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
+                   int M, int K, int N, const pta_epilogue* epi, pta_stream_t stream);
+
+/* Up to 4 weights sharing the same X and K in one launch (q/k/v projections of
+ * models/llama2/attention.py:65-67).  host_* arrays have `count` entries. */
+int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
+                         const pta_half* const* host_scale, pta_half* const* host_Y,
+                         const int* host_N, int M, int K, pta_stream_t stream);
+
+/* SwiGLU pair (models/llama2/mlp.py:20-28, models/chatglm2/mlp.py:51-59):
+ * Y[M,F] = fp16( fp16(X@Wup) * fp16(swish(fp16(X@Wgate))) ), swish(g) = g*sigmoid(g). */
+int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
+                          const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M,
+                          int K, int F, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * FP16 weights (embedding-tied heads, lm_head, GPT-2 linears): ops.matmul of
+ * ops/popart.py:55-67 with an initializer on the right-hand side.
+ * ---------------------------------------------------------------------------------- */
+
+/* `w` is fp16 [N, K] (the [out, in] orientation of the state dict, layers/linear.py:30-33). */
+size_t pta_f16_tiled_bytes(int N, int K);
+int pta_f16_tile(const pta_half* w, void* tiled, int N, int K, pta_stream_t stream);
+/* Y[M,N] = fp16(X[M,K] @ w^T), fp32 accumulation. 1 <= M <= 64. */
+int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
+                 const pta_epilogue* epi, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Normalisation
+ * ---------------------------------------------------------------------------------- */
+
+/* RMSNorm as composed by layers/rms_layer_norm.py:26-36: v = mean(fp32(x)^2) + eps;
+ * r = fp16(1/sqrt(v)); y = fp16(fp16(x*r) * weight).  x, y fp16 [rows, cols]. cols % 8 == 0. */
+int pta_rmsnorm(const pta_half* x, const pta_half* weight, pta_half* y, int rows, int cols, float eps,
+                pta_stream_t stream);
+
+/* NormCE LayerNorm (ops/customized.py:69-102; custom_ops/NormCE.cpp:534-610).  fp16 in/out,
+ * fp32 statistics.  rows == 1 follows calSmallBatchNorm + GetInPlaceNorm (NormCE.cpp:122-200,
+ * NormCECodelets.cpp:65-112): var = E[x^2] - mean^2 + eps with the fp32 mean, no clamp.
+ * rows > 1 follows normInfKernel (NormCE.S:243-423, NormCECodelets.cpp:181-211): the mean is
+ * rounded to fp16 before it is squared and the variance is clamped at 0.  In both,
+ * y = fp16(fp16(fp16(fp16(x - mean16) * rstd16) * gamma) + beta).  cols % 8 == 0, cols < 8192. */
+int pta_layer_norm_ce(const pta_half* x, const pta_half* gamma, const pta_half* beta, pta_half* y, int rows,
+                      int cols, float eps, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Softmax
+ * ---------------------------------------------------------------------------------- */
+enum { PTA_F16 = 0, PTA_F32 = 1 };
+
+/* SoftmaxV3 over the last axis (ops/customized.py:57-65; custom_ops/softmax.cpp:41-83).
+ * x, y are [rows, n] of `dtype`; stable_mode != 0 subtracts the row maximum first. */
+int pta_softmax_ce(const void* x, void* y, int rows, int n, int dtype, int stable_mode, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * KV cache.  Shapes are [outer, seq, inner] (inner contiguous); with the models' layout
+ * [2, B, H, seq, D] and sequence_axis = 3, outer = 2*B*H and inner = D.  `step` is a device
+ * int32 scalar, as it is a graph tensor in the reference.
+ * ---------------------------------------------------------------------------------- */
+
+/* KVCache, literal (ops/customized.py:21-35; custom_ops/kv_cache.cpp:94-187):
+ *   clone = (*step != 0) ? cache : 0;  cache = concat(updater, clone[:, 0 : max_len-step_len]).
+ * cache and clone are [outer, max_len, inner]; updater is [outer, step_len, inner].  The
+ * result (the op's output) is `cache` itself. */
+int pta_kv_cache_update(void* cache, void* clone, const void* updater, const int32_t* step, int outer,
+                        int max_len, int step_len, int inner, int elem_bytes, pta_stream_t stream);
+
+/* The same cache kept as a ring in arrival order: one row written per call, nothing shifted.
+ * cache is [max_bps, outer, max_len, inner]; the call at step s writes updater [outer, inner]
+ * to row (s / max_bps) % max_len of register s % max_bps.  max_bps == 1 is KVCache; larger
+ * values are KVCachePipeline (custom_ops/kv_cache_pipeline.cpp:374-451,
+ * custom_ops/kv_cache_codelet.cpp:18-131) with step_len == 1 and the sequence axis at
+ * rank - 2.  Calls must come with step = 0, 1, 2, ... as the generation loop issues them. */
+int pta_kv_cache_append(void* cache, const void* updater, const int32_t* step, int outer, int max_len, int inner,
+                        int elem_bytes, int max_bps, pta_stream_t stream);
+
+/* Materialises the reference op's output from the ring after the append of the same step:
+ * out [outer, max_len, inner], out[:, i] = i-th newest row of register step % max_bps, zero for
+ * rows the shift register would not have received since step 0. */
+int pta_kv_cache_read(const void* cache, void* out, const int32_t* step, int outer, int max_len, int inner,
+                      int elem_bytes, int max_bps, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Attention for one new position per sequence
+ * ---------------------------------------------------------------------------------- */
+enum { PTA_ROPE_NONE = 0, PTA_ROPE_LLAMA = 1, PTA_ROPE_GLM2 = 2 };
+
+/* Rotary embedding of q and k at position *step and append of (k, v) to the ring cache
+ * (models/llama2/attention.py:28-94; models/chatglm2/attention.py:77-232;
+ * models/gpt2/attention.py:50-66 with PTA_ROPE_NONE).
+ * q/k/v point at the projection outputs, row b at q + b*q_stride etc.: heads are contiguous,
+ * [Hq*D] for q and [Hkv*D] for k and v.  q_out is [B, Hq, D].  kv_ring is the cache of
+ * pta_kv_cache_append with max_bps = 1, outer = 2*B*Hkv, inner = D: keys first, then values.
+ * inv_freq: PTA_ROPE_LLAMA fp16 [D/2] (the graph constant of llama2/attention.py:29-31);
+ *           PTA_ROPE_GLM2 fp32 [D/4] (chatglm2/attention.py:80-83). */
+int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                        int v_stride, pta_half* q_out, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                        int B, int Hq, int Hkv, int D, int max_len, int rope, pta_stream_t stream);
+
+/* softmax(q K^T [* fp16(1/sqrt(D))] + mask) V over the rows received so far, heads merged:
+ * out [B, Hq*D] (forward_attention + forward_output up to the output projection,
+ * models/llama2/attention.py:97-113, models/gpt2/attention.py:68-90,
+ * models/chatglm2/attention.py:277-302).  The mask of models/base_model.py:258-262,321-325 is
+ * implied by *step: rows 0..step are open.  Hq % Hkv == 0 (multi-query groups share a cache
+ * head).  D is 64 or 128.  workspace: pta_decode_attention_workspace_bytes(...) bytes. */
+size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int max_len);
+int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                         pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
+                         pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Token selection and loop bookkeeping
+ * ---------------------------------------------------------------------------------- */
+
+/* ops.topk(k=1) over the last axis (layers/lm_head.py:55; ops/popart.py:135-137): ids[r] = index
+ * of the largest logit of row r, the lowest index among equals; values (optional) receives it. */
+int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, pta_stream_t stream);
+
+/* Embedding rows (layers/embedding.py:34-36); with pos_table also GPT-2's wte[id] + wpe[*pos]
+ * (models/gpt2/embedding.py:31-36).  out [rows, cols]. */
+int pta_embedding(const pta_half* table, const int32_t* ids, const pta_half* pos_table, const int32_t* pos,
+                  pta_half* out, int rows, int cols, int vocab, pta_stream_t stream);
+
+/* step_containers + step_loop_cond of models/base_model.py:313-355 for one iteration; all
+ * arrays on the device.  container int32 [B, max_len]; mask fp16 [B, max_len] or NULL;
+ * stop_mask int32 [B]; step int32 scalar (advanced by one); next_ids int32 [B];
+ * ids_out (optional) int32 [B] receives the ids written; keep_going (optional) int32 scalar. */
+int pta_step_update(int32_t* container, pta_half* mask, int32_t* stop_mask, int32_t* step, const int32_t* next_ids,
+                    int32_t* ids_out, int32_t* keep_going, int B, int max_len, int pad_id, int eos_id,
+                    int early_stop, pta_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* POPTRANSFORMER_HIP_H */

@@ -1,0 +1,90 @@
+"""ctypes binding of libpoptransformer_hip.so.
+
+The reference loads its native ops with ``ctypes.cdll.LoadLibrary('../../custom_ops.so')`` at
+import of ``poptransformer/ops/customized.py`` (lines 14-18); this module is the counterpart.
+The library must have been built (``python -m poptransformer_amd.build`` or
+``__graft_entry__.build()``): a missing library is an error, there is no fallback.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_size_t, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libpoptransformer_hip.so")
+
+PTA_OK, PTA_EINVAL, PTA_EUNSUPPORTED, PTA_EHIP = 0, -1, -2, -3
+ACT_NONE, ACT_GELU_TANH, ACT_RELU_SQUARE, ACT_SIGMOID = 0, 1, 2, 3
+F16, F32 = 0, 1
+ROPE_NONE, ROPE_LLAMA, ROPE_GLM2 = 0, 1, 2
+
+
+class Epilogue(ctypes.Structure):
+    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int)]
+
+
+# name -> (restype, argtypes); the order follows include/poptransformer_hip.h
+SIGNATURES = {
+    "pta_version": (c_int, []),
+    "pta_last_error": (c_char_p, []),
+    "pta_int4_to_half": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_w4_tiled_bytes": (c_size_t, [c_int, c_int]),
+    "pta_w4_tile": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "pta_w4a16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Epilogue), c_void_p]),
+    "pta_w4a16_gemm_multi": (c_int, [c_void_p, c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                     POINTER(c_int), c_int, c_int, c_void_p]),
+    "pta_w4a16_gemm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_f16_tiled_bytes": (c_size_t, [c_int, c_int]),
+    "pta_f16_tile": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "pta_f16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Epilogue), c_void_p]),
+    "pta_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "pta_layer_norm_ce": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "pta_softmax_ce": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "pta_kv_cache_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "pta_kv_cache_append": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "pta_kv_cache_read": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "pta_qkv_rope_append": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                    c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "pta_decode_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "pta_decode_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                     c_int, c_int, c_void_p]),
+    "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "pta_embedding": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                c_int, c_int, c_int, c_void_p]),
+}
+
+_lib = None
+
+
+class PtaError(RuntimeError):
+    pass
+
+
+def load():
+    """Load the shared library and declare every prototype. Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise PtaError(
+            f"{LIB_PATH} is missing: build it with `python -m poptransformer_amd.build` "
+            "(there is no CPU fallback for the HIP kernels)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    _lib = lib
+    return lib
+
+
+def check(rc, what=""):
+    """Translate a status code into the exception the reference would have raised: invalid
+    shapes/attributes are graph-build errors (ValueError), runtime failures RuntimeError."""
+    if rc == PTA_OK:
+        return
+    msg = load().pta_last_error().decode()
+    if rc == PTA_EINVAL:
+        raise ValueError(msg or what)
+    if rc == PTA_EUNSUPPORTED:
+        raise NotImplementedError(msg or what)
+    raise PtaError(msg or what)

@@ -1,0 +1,248 @@
+// Decode attention (one query position per sequence) over the ring KV cache, and the
+// query/key preparation that precedes it.
+//
+// Reference graphs: models/gpt2/attention.py:50-90, models/llama2/attention.py:28-114,
+// models/chatglm2/attention.py:77-302.  They compute q.K^T over all max_len cache rows, add a
+// mask of 0 / -10000, apply the non-stable SoftmaxV3 and multiply by V.  A masked row
+// contributes exp(-10000 + s) = 0 exactly (in fp16 and in fp32), so attending to the valid rows
+// only gives the same sums; subtracting the running maximum before exp is the same function
+// without the overflow.  Roundings that the reference performs on the scores (fp16 MatMul
+// output, fp16 multiply by 1/sqrt(D)) are reproduced; probabilities stay fp32 up to the final
+// fp16 rounding of the context vector.
+#include "common.h"
+
+// ------------------------------------------------------------------------------------------
+// q/k rotary embedding + KV ring append.
+// ------------------------------------------------------------------------------------------
+struct QkvArgs {
+  const f16* q; const f16* k; const f16* v;   // rows of the projection outputs
+  int q_stride, k_stride, v_stride;           // elements between batch rows
+  f16* q_out;                                 // [B, Hq, D]
+  f16* kring; f16* vring;                     // [B*Hkv, max_len, D] each
+  const int32_t* step;
+  const void* inv_freq;                       // fp16 [D/2] (PTA_ROPE_LLAMA) or fp32 [D/4] (PTA_ROPE_GLM2)
+  int B, Hq, Hkv, D, max_len, rope;
+};
+
+// Llama: angle = fp16(fp16(step) * inv_freq16) (an fp16 MatMul of a 1x1 by a 1xD/2 matrix,
+// llama2/attention.py:28-38), sin/cos rounded to fp16, rotate-half over the whole head
+// (llama2/attention.py:40-56): y = fp16(fp16(x*cos) + fp16(rot(x)*sin)).
+__device__ __forceinline__ void rope_llama(const f16* x, f16* y, int d, int D, int step, const f16* inv_freq) {
+  const int half = D >> 1;
+  const int i = d < half ? d : d - half;
+  const f16 ang = (f16)((float)(f16)(float)step * (float)inv_freq[i]);
+  const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
+  const f16 rot = d < half ? -x[d + half] : x[d - half];
+  y[d] = x[d] * c + rot * s;
+}
+
+// ChatGLM2: only the first D/2 features of a head rotate, as interleaved pairs (2j, 2j+1) with
+// angle fp16(fp32(step) * inv_freq32[j]) (chatglm2/attention.py:77-164).
+__device__ __forceinline__ void rope_glm2(const f16* x, f16* y, int d, int D, int step, const float* inv_freq) {
+  const int rot_dim = D >> 1;
+  if (d >= rot_dim) { y[d] = x[d]; return; }
+  const int j = d >> 1;
+  const f16 ang = (f16)((float)step * inv_freq[j]);
+  const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
+  const f16 rot = (d & 1) ? x[d - 1] : -x[d + 1];
+  y[d] = x[d] * c + rot * s;
+}
+
+__global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
+  const int D = a.D;
+  const int per_b = (a.Hq + 2 * a.Hkv) * D;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= a.B * per_b) return;
+  const int b = idx / per_b;
+  int r = idx % per_b;
+  const int step = *a.step;
+  const int pos = step % a.max_len;
+  if (r < a.Hq * D) {
+    const int h = r / D, d = r % D;
+    const f16* x = a.q + (size_t)b * a.q_stride + h * D;
+    f16* y = a.q_out + ((size_t)b * a.Hq + h) * D;
+    if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
+    else if (a.rope == PTA_ROPE_GLM2) rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
+    else y[d] = x[d];
+    return;
+  }
+  r -= a.Hq * D;
+  if (r < a.Hkv * D) {
+    const int h = r / D, d = r % D;
+    const f16* x = a.k + (size_t)b * a.k_stride + h * D;
+    f16* y = a.kring + (((size_t)b * a.Hkv + h) * a.max_len + pos) * D;
+    if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
+    else if (a.rope == PTA_ROPE_GLM2) rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
+    else y[d] = x[d];
+    return;
+  }
+  r -= a.Hkv * D;
+  const int h = r / D, d = r % D;
+  a.vring[(((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d] = a.v[(size_t)b * a.v_stride + h * D + d];
+}
+
+extern "C" int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
+                                   int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring,
+                                   const int32_t* step, const void* inv_freq, int B, int Hq, int Hkv, int D,
+                                   int max_len, int rope, pta_stream_t stream) {
+  PTA_REQUIRE(q && k && v && q_out && kv_ring && step, "pta_qkv_rope_append: null pointer");
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_qkv_rope_append: bad head counts %d/%d", Hq, Hkv);
+  PTA_REQUIRE(D > 0 && D % 4 == 0 && max_len > 0, "pta_qkv_rope_append: bad head size %d or max_len %d", D, max_len);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "pta_qkv_rope_append: unknown rope mode %d", rope);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "pta_qkv_rope_append: inv_freq is required for rotary modes");
+  QkvArgs a{(const f16*)q, (const f16*)k, (const f16*)v, q_stride, k_stride, v_stride, (f16*)q_out,
+            (f16*)kv_ring, (f16*)kv_ring + (size_t)B * Hkv * max_len * D, step, inv_freq, B, Hq, Hkv, D, max_len, rope};
+  const int total = B * (Hq + 2 * Hkv) * D;
+  hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream, a);
+  PTA_CHECK_LAUNCH("pta_qkv_rope_append");
+  return PTA_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// Split-K decode attention with online softmax.
+// ------------------------------------------------------------------------------------------
+constexpr int ATT_THREADS = 256;
+constexpr int ATT_WAVES = ATT_THREADS / 64;
+
+struct AttnArgs {
+  const f16* q;       // [B, Hq, D]
+  const f16* kring;   // [B*Hkv, max_len, D]
+  const f16* vring;
+  const int32_t* step;
+  float* part;        // [B*Hq, nsplit, D + 2]: running max, denominator, numerator
+  f16* out;           // [B, Hq*D]
+  int B, Hq, Hkv, max_len, chunk, nsplit;
+  int use_scale;
+  f16 scale;
+};
+
+// Partial attention of one (sequence, query head) over one chunk of cache rows.
+// LPP = D/8 lanes share a cache row (16 bytes each); a wave covers 64/LPP rows per load.
+template <int D>
+__global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
+  constexpr int LPP = D / 8;
+  constexpr int PPW = 64 / LPP;
+  constexpr int NG = ATT_WAVES * PPW;
+  __shared__ float sm_m[NG], sm_l[NG];
+  __shared__ float sm_acc[NG][D];
+  const int split = blockIdx.x, bh = blockIdx.y;
+  const int step = *a.step;
+  const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
+  const int c0 = split * a.chunk;
+  if (c0 >= valid) return;
+  const int c1 = c0 + a.chunk < valid ? c0 + a.chunk : valid;
+  const int b = bh / a.Hq, h = bh % a.Hq;
+  const int hk = h / (a.Hq / a.Hkv);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = lane / LPP, sub = lane % LPP;
+  const int d0 = sub * 8;
+
+  float qf[8];
+  {
+    const f16x8 q8 = *reinterpret_cast<const f16x8*>(a.q + (size_t)bh * D + d0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[e] = (float)q8[e];
+  }
+  const f16* kb = a.kring + ((size_t)b * a.Hkv + hk) * a.max_len * D + d0;
+  const f16* vb = a.vring + ((size_t)b * a.Hkv + hk) * a.max_len * D + d0;
+
+  float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+
+  for (int p0 = c0 + wave * PPW; p0 < c1; p0 += ATT_WAVES * PPW) {
+    const int p = p0 + grp;
+    const bool on = p < c1;
+    const int pc = on ? p : c1 - 1;
+    const f16x8 k8 = *reinterpret_cast<const f16x8*>(kb + (size_t)pc * D);
+    const f16x8 v8 = *reinterpret_cast<const f16x8*>(vb + (size_t)pc * D);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
+#pragma unroll
+    for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    f16 s16 = (f16)s;                       // fp16 output of the q.K^T MatMul
+    if (a.use_scale) s16 = s16 * a.scale;   // fp16 multiply by fp16(1/sqrt(D))
+    const float x = on ? (float)s16 : -INFINITY;
+    const float mn = fmaxf(m, x);
+    const float corr = m == -INFINITY ? 0.f : __expf(m - mn);  // nothing accumulated yet
+    const float pe = on ? __expf(x - mn) : 0.f;
+    l = l * corr + pe;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
+    m = mn;
+  }
+
+  const int g = wave * PPW + grp;
+  if (sub == 0) { sm_m[g] = m; sm_l[g] = l; }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) sm_acc[g][d0 + e] = acc[e];
+  __syncthreads();
+  float* out = a.part + ((size_t)bh * a.nsplit + split) * (D + 2);
+  for (int d = threadIdx.x; d < D; d += ATT_THREADS) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NG; ++i) M = fmaxf(M, sm_m[i]);
+    float L = 0.f, A = 0.f;
+#pragma unroll
+    for (int i = 0; i < NG; ++i) {
+      const float w = sm_m[i] == -INFINITY ? 0.f : __expf(sm_m[i] - M);
+      L = __builtin_fmaf(sm_l[i], w, L);
+      A = __builtin_fmaf(sm_acc[i][d], w, A);
+    }
+    out[2 + d] = A;
+    if (d == 0) { out[0] = M; out[1] = L; }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
+  const int bh = blockIdx.x, d = threadIdx.x;
+  const int step = *a.step;
+  const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
+  const int nact = (valid + a.chunk - 1) / a.chunk;
+  const float* p = a.part + (size_t)bh * a.nsplit * (D + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < nact; ++s) M = fmaxf(M, p[(size_t)s * (D + 2)]);
+  float L = 0.f, A = 0.f;
+  for (int s = 0; s < nact; ++s) {
+    const float* ps = p + (size_t)s * (D + 2);
+    const float w = __expf(ps[0] - M);
+    L = __builtin_fmaf(ps[1], w, L);
+    A = __builtin_fmaf(ps[2 + d], w, A);
+  }
+  a.out[(size_t)bh * D + d] = (f16)(A / L);
+}
+
+extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int max_len) {
+  if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
+  const int chunk = 64;
+  const int nsplit = (max_len + chunk - 1) / chunk;
+  return (size_t)B * Hq * nsplit * (D + 2) * sizeof(float);
+}
+
+extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                                    pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
+                                    pta_stream_t stream) {
+  PTA_REQUIRE(q && kv_ring && step && workspace && out, "pta_decode_attention: null pointer");
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_decode_attention: bad head counts %d/%d", Hq, Hkv);
+  PTA_REQUIRE(D == 64 || D == 128, "pta_decode_attention: head size must be 64 or 128, got %d", D);
+  PTA_REQUIRE(max_len > 0, "pta_decode_attention: max_len = %d", max_len);
+  PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "pta_decode_attention: q and kv_ring must be 16-byte aligned");
+  AttnArgs a{};
+  a.q = (const f16*)q; a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
+  a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.chunk = 64; a.nsplit = (max_len + 63) / 64;
+  a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(a.nsplit, B * Hq);
+  if (D == 128) {
+    hipLaunchKernelGGL(attn_partial_kernel<128>, grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * Hq), dim3(128), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(attn_partial_kernel<64>, grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * Hq), dim3(64), 0, s, a);
+  }
+  PTA_CHECK_LAUNCH("pta_decode_attention");
+  return PTA_OK;
+}

@@ -1,0 +1,227 @@
+// Epilogue shared by the fused GEMV/GEMM kernels (INT4, FP16 and FP8 weights).
+//
+// The reference builds these as separate fp16 graph ops after the MatMul: the bias `ops.add`
+// of poptransformer/layers/linear.py:42-46, the activation of layers/mlp.py:34-41 /
+// models/rwkv/ffn.py:47-59, and the residual `ops.add` of the transformer blocks
+// (e.g. models/llama2/model.py:38-46).  Each step therefore rounds to fp16.
+#pragma once
+#include "common.h"
+
+struct GemmEpilogue {
+  const f16* bias;
+  const f16* residual;
+  int act;
+};
+
+__device__ __forceinline__ f16 sigmoid_f16(f16 x) {
+  return (f16)(1.0f / (1.0f + __expf(-(float)x)));
+}
+
+// x * sigmoid(x), evaluated in fp32 from the fp16 input and rounded once.
+__device__ __forceinline__ f16 swish_f16(f16 x) {
+  const float v = (float)x;
+  return (f16)(v / (1.0f + __expf(-v)));
+}
+
+// tanh-form GELU, evaluated in fp32 from the fp16 input and rounded once.
+__device__ __forceinline__ f16 gelu_tanh_f16(f16 x) {
+  const float v = (float)x;
+  const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+  return (f16)(0.5f * v * (1.0f + tanhf(u)));
+}
+
+__device__ __forceinline__ f16 apply_act(int act, f16 y) {
+  switch (act) {
+    case PTA_ACT_GELU_TANH: return gelu_tanh_f16(y);
+    case PTA_ACT_RELU_SQUARE: { f16 r = y > (f16)0.0f ? y : (f16)0.0f; return r * r; }
+    case PTA_ACT_SIGMOID: return sigmoid_f16(y);
+    default: return y;
+  }
+}
+
+__device__ __forceinline__ f16 apply_epilogue(const GemmEpilogue& e, f16 y, int m, int n, int N) {
+  if (e.bias) y = y + e.bias[n];
+  y = apply_act(e.act, y);
+  if (e.residual) y = y + e.residual[(size_t)m * N + n];
+  return y;
+}
+
+static inline int make_epilogue(const pta_epilogue* in, GemmEpilogue* out, const char* name) {
+  out->bias = nullptr; out->residual = nullptr; out->act = PTA_ACT_NONE;
+  if (!in) return PTA_OK;
+  PTA_REQUIRE(in->act >= PTA_ACT_NONE && in->act <= PTA_ACT_SIGMOID, "%s: unknown activation %d", name, in->act);
+  out->bias = (const f16*)in->bias; out->residual = (const f16*)in->residual; out->act = in->act;
+  return PTA_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// Small-M GEMM core: Y[M,N] = fp16(X[M,K] @ W^T) for M <= 64, weights streamed once.
+//
+// Weights are stored tiled (see the *_tile entry points): a tile is 16 output channels x 128
+// input features, made of Fmt::kVec vectors of 1 KiB; in each vector lane l owns the 16 bytes
+// at offset 16*l.  The tiles of one 16-channel block are contiguous over the feature axis.
+// One workgroup owns one 16-channel block; its NW waves take feature tiles round-robin, each
+// wave feeding the 16x16x32 fp16 MFMA with A = 16 channels x 32 features of weights (decoded
+// in registers) and B = 32 features x 16 activation rows read straight from X, and the
+// partial sums meet in LDS.  HBM traffic is the weight bytes, once; X comes from L2.
+// ------------------------------------------------------------------------------------------
+struct GemmMat {
+  const void* tiled;
+  const void* scale;
+  f16* Y;
+  int N;
+  int nb_begin;  // first 16-channel block of this matrix in the launch grid
+};
+
+struct GemmArgs {
+  GemmMat mat[4];
+  int count;
+  const f16* X;
+  int M, K, KT;
+  GemmEpilogue epi;
+  // PAIR mode (SwiGLU): mat[0] is the gate weight, mat[1] the up weight, output in mat[0].Y.
+};
+
+template <class Fmt, int MT, int NW, bool PAIR>
+__global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int KV = Fmt::kVec;
+  __shared__ float red[NW * NACC * MT * 256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int mi = 0;
+  if (!PAIR) {
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (i < a.count && (int)blockIdx.x >= a.mat[i].nb_begin) mi = i;
+  }
+  const int nb = blockIdx.x - a.mat[mi].nb_begin;
+  const int N = a.mat[mi].N;
+  const int row = nb * 16 + (lane & 15);
+  const int K = a.K, KT = a.KT;
+
+  typename Fmt::Scale sc[NACC];
+  const u32x4* wp[NACC];
+#pragma unroll
+  for (int g = 0; g < NACC; ++g) {
+    const GemmMat& m = a.mat[PAIR ? g : mi];
+    sc[g] = Fmt::load_scale(m.scale, row, N);
+    wp[g] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb * KT * (64 * KV) + lane;
+  }
+  // B operand source: row (mt*16 + lane%16) of X, clamped into range; lanes of padding rows
+  // compute values that are never stored.
+  const f16* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = mt * 16 + (lane & 15);
+    m = m < a.M ? m : a.M - 1;
+    xrow[mt] = a.X + (size_t)m * K + (lane >> 4) * 8;
+  }
+
+  f32x4 acc[NACC][MT];
+#pragma unroll
+  for (int g = 0; g < NACC; ++g)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 2
+  for (int kt = wave; kt < KT; kt += NW) {
+    u32x4 w[NACC][KV];
+#pragma unroll
+    for (int g = 0; g < NACC; ++g)
+#pragma unroll
+      for (int v = 0; v < KV; ++v)
+        w[g][v] = __builtin_nontemporal_load(wp[g] + ((size_t)kt * KV + v) * 64);
+    f16x8 xb[4][MT];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kt * 128 + j * 32;
+      const bool in = k + (lane >> 4) * 8 < K;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        xb[j][mt] = in ? *reinterpret_cast<const f16x8*>(xrow[mt] + k) : z;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int g = 0; g < NACC; ++g) {
+        const f16x8 av = Fmt::a_operand(w[g], j, sc[g]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[j][mt], acc[g][mt], 0, 0, 0);
+      }
+    }
+  }
+
+  // Cross-wave reduction through LDS, then the epilogue.  The accumulator of lane l holds
+  // channels (l/16)*4 + r, r = 0..3, for activation row l%16.
+#pragma unroll
+  for (int g = 0; g < NACC; ++g)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        red[(((wave * NACC + g) * MT + mt) * 4 + r) * 64 + lane] = acc[g][mt][r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < MT * 256; idx += NW * 64) {
+    const int nn = idx & 15;  // channel inside the block
+    const int m = idx >> 4;   // activation row
+    const int n = nb * 16 + nn;
+    if (m >= a.M || n >= N) continue;
+    const int mt = m >> 4, r = nn & 3, ln = (nn >> 2) * 16 + (m & 15);
+    float sum[NACC];
+#pragma unroll
+    for (int g = 0; g < NACC; ++g) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) t += red[(((w * NACC + g) * MT + mt) * 4 + r) * 64 + ln];
+      sum[g] = Fmt::finish(t, sc[g]);
+    }
+    if (PAIR) {
+      const f16 gate = (f16)sum[0];
+      const f16 up = (f16)sum[1];
+      a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
+    } else {
+      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, (f16)sum[0], m, n, N);
+    }
+  }
+}
+
+template <class Fmt, int MT, bool PAIR>
+static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
+  // Waves per block: enough to split K finely when there are few channel blocks, fewer when
+  // the grid alone already fills the machine.  The LDS reduction buffer caps the wide cases.
+  if constexpr (MT == 4 && PAIR) {
+    hipLaunchKernelGGL((gemv_mfma_kernel<Fmt, MT, 4, PAIR>), dim3(total_nb), dim3(4 * 64), 0, s, a);
+  } else if constexpr (MT == 4 || PAIR) {
+    hipLaunchKernelGGL((gemv_mfma_kernel<Fmt, MT, 8, PAIR>), dim3(total_nb), dim3(8 * 64), 0, s, a);
+  } else {
+    if (a.KT >= 16 && total_nb <= 1024)
+      hipLaunchKernelGGL((gemv_mfma_kernel<Fmt, MT, 16, PAIR>), dim3(total_nb), dim3(16 * 64), 0, s, a);
+    else
+      hipLaunchKernelGGL((gemv_mfma_kernel<Fmt, MT, 8, PAIR>), dim3(total_nb), dim3(8 * 64), 0, s, a);
+  }
+}
+
+template <class Fmt, bool PAIR>
+static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  if (a.M <= 16) launch_gemv<Fmt, 1, PAIR>(a, total_nb, s);
+  else if (a.M <= 32) launch_gemv<Fmt, 2, PAIR>(a, total_nb, s);
+  else launch_gemv<Fmt, 4, PAIR>(a, total_nb, s);
+  PTA_CHECK_LAUNCH(name);
+  return PTA_OK;
+}
+
+static inline int check_gemv_common(const char* name, const void* X, int M, int K) {
+  PTA_REQUIRE(X, "%s: null X", name);
+  PTA_REQUIRE(M >= 1 && M <= 64, "%s: M must be in [1, 64], got %d", name, M);
+  PTA_REQUIRE(K > 0 && (K % 8) == 0, "%s: K must be a positive multiple of 8, got %d", name, K);
+  PTA_REQUIRE(pta_aligned(X, 16), "%s: X must be 16-byte aligned", name);
+  return PTA_OK;
+}
+
+static inline size_t gemv_tiled_bytes(int N, int K, int kvec) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)((N + 15) / 16) * (size_t)((K + 127) / 128) * 1024 * kvec;
+}

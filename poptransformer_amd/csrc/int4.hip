@@ -1,0 +1,222 @@
+// INT4 weight path: exact Int4ToHalf, load-time tiling, and the fused
+// dequantise-in-register W4A16 GEMV/GEMM built on the gfx950 16x16x32 fp16 MFMA.
+//
+// Reference semantics: custom_ops/int4_to_half_codelets.cpp:18-74 (nibble extraction),
+// custom_ops/int4_to_half_custom_op.cpp:139-149 (the 256x2 truth table), :362-378 (layout of
+// the axis=1 result and the fp16 multiply by the per-channel scale),
+// poptransformer/utils/param_handler/precision_strategy.py:56-60,74-75 (unpack then MatMul).
+#include "common.h"
+#include "gemm_core.h"
+
+// ------------------------------------------------------------------------------------------
+// Int4ToHalf, standalone and bit-exact.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ int nib_hi(int8_t b) { return ((int)b) >> 4; }
+__device__ __forceinline__ int nib_lo(int8_t b) { return ((int)(int8_t)((uint8_t)b << 4)) >> 4; }
+
+// axis == 1: out[2j + h, r] = nib_h(P[r, j]) * scale[r]; out is [2m, n].
+// A 64x64-byte tile of P goes through LDS so that both the reads of P (along j) and the
+// writes of out (along r) are coalesced.
+__global__ __launch_bounds__(256) void int4_to_half_axis1_kernel(const int8_t* __restrict__ P,
+                                                                 const f16* __restrict__ scale,
+                                                                 f16* __restrict__ out, int n, int m) {
+  __shared__ int8_t tile[64][65];
+  const int r0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int rr = ty; rr < 64; rr += 4) {
+    int r = r0 + rr, j = j0 + tx;
+    tile[rr][tx] = (r < n && j < m) ? P[(size_t)r * m + j] : (int8_t)0;
+  }
+  __syncthreads();
+  const int r = r0 + tx;
+  if (r >= n) return;
+  const f16 s = scale[r];
+  for (int jj = ty; jj < 64; jj += 4) {
+    int j = j0 + jj;
+    if (j >= m) break;
+    int8_t b = tile[tx][jj];
+    out[(size_t)(2 * j) * n + r] = (f16)nib_hi(b) * s;
+    out[(size_t)(2 * j + 1) * n + r] = (f16)nib_lo(b) * s;
+  }
+}
+
+// axis == 0: out[2i + h, c] = nib_h(P[i, c]) * scale[c]; out is [2n, m].
+__global__ __launch_bounds__(256) void int4_to_half_axis0_kernel(const int8_t* __restrict__ P,
+                                                                 const f16* __restrict__ scale,
+                                                                 f16* __restrict__ out, int n, int m) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)n * m) return;
+  const int i = (int)(idx / m), c = (int)(idx % m);
+  const int8_t b = P[idx];
+  const f16 s = scale[c];
+  out[(size_t)(2 * i) * m + c] = (f16)nib_hi(b) * s;
+  out[(size_t)(2 * i + 1) * m + c] = (f16)nib_lo(b) * s;
+}
+
+extern "C" int pta_int4_to_half(const int8_t* packed, const pta_half* scale, pta_half* out, int n,
+                                int m, int axis, pta_stream_t stream) {
+  // Guards of Int4ToHalfOp::setup (int4_to_half_custom_op.cpp:65-98): rank/shape agreement is
+  // the caller's to state through n and m; the axis must be 0 or 1.
+  PTA_REQUIRE(axis == 0 || axis == 1, "[Int4ToHalf] 'axis' should be 0 or 1. But now it is %d.", axis);
+  PTA_REQUIRE(packed && scale && out, "[Int4ToHalf] null pointer");
+  PTA_REQUIRE(n > 0 && m > 0, "[Int4ToHalf] empty input [%d,%d]", n, m);
+  hipStream_t s = (hipStream_t)stream;
+  if (axis == 1) {
+    dim3 grid((m + 63) / 64, (n + 63) / 64);
+    hipLaunchKernelGGL(int4_to_half_axis1_kernel, grid, dim3(256), 0, s, packed, (const f16*)scale,
+                       (f16*)out, n, m);
+  } else {
+    size_t total = (size_t)n * m;
+    hipLaunchKernelGGL(int4_to_half_axis0_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       packed, (const f16*)scale, (f16*)out, n, m);
+  }
+  PTA_CHECK_LAUNCH("pta_int4_to_half");
+  return PTA_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// Load-time tiling.
+//
+// A tile covers 16 output channels x 128 input features and is 1 KiB, stored so that lane l
+// of a wave finds its 16 bytes at byte offset 16*l: dword j (0..3) of that lane holds the 8
+// weights of channel (l % 16) for features  kt*128 + j*32 + (l/16)*8 + 0..7, i.e. exactly the
+// A operand of one 16x16x32 MFMA.  Tiles of one 16-channel block are contiguous over kt, so a
+// block streams one contiguous range.  Inside a dword weight i sits in nibble slot
+// (i & 1) * 4 + (i >> 1) and is stored offset-binary (q + 8): with that order two AND/OR
+// operations per shifted dword yield fp16 pairs of consecutive features.
+// Padding rows / features hold the code of zero.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void w4_tile_kernel(const int8_t* __restrict__ P,
+                                                      uint32_t* __restrict__ tiled, int N, int K,
+                                                      int KT, size_t total_dwords) {
+  const size_t d = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (d >= total_dwords) return;
+  const int j = (int)(d & 3);
+  const int lane = (int)((d >> 2) & 63);
+  const size_t tile = d >> 8;
+  const int kt = (int)(tile % KT);
+  const int nb = (int)(tile / KT);
+  const int row = nb * 16 + (lane & 15);
+  const int k0 = kt * 128 + j * 32 + (lane >> 4) * 8;
+  uint32_t w = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int k = k0 + i;
+    uint32_t u = 8;  // q = 0
+    if (row < N && k < K) {
+      const int8_t b = P[(size_t)row * (K / 2) + (k >> 1)];
+      const int q = (k & 1) ? nib_lo(b) : nib_hi(b);
+      u = (uint32_t)(q + 8);
+    }
+    const int slot = (i & 1) * 4 + (i >> 1);
+    w |= u << (4 * slot);
+  }
+  tiled[d] = w;
+}
+
+extern "C" size_t pta_w4_tiled_bytes(int N, int K) {
+  if (N <= 0 || K <= 0) return 0;
+  return (size_t)((N + 15) / 16) * (size_t)((K + 127) / 128) * 1024;
+}
+
+extern "C" int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t stream) {
+  PTA_REQUIRE(packed && tiled, "pta_w4_tile: null pointer");
+  PTA_REQUIRE(N > 0 && K > 0 && (K % 2) == 0, "pta_w4_tile: need N > 0 and even K > 0, got N=%d K=%d", N, K);
+  PTA_REQUIRE(pta_aligned(tiled, 16), "pta_w4_tile: tiled buffer must be 16-byte aligned");
+  const int KT = (K + 127) / 128;
+  const size_t total = pta_w4_tiled_bytes(N, K) / 4;
+  hipLaunchKernelGGL(w4_tile_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, packed, (uint32_t*)tiled, N, K, KT, total);
+  PTA_CHECK_LAUNCH("pta_w4_tile");
+  return PTA_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// Fused W4A16 GEMV/GEMM.
+// ------------------------------------------------------------------------------------------
+
+// One tiled dword -> 8 fp16 weights, each fp16(q * s) with a single rounding (the product of
+// an integer in [-8, 7] held exactly in fp16 and the fp16 scale), which is what the
+// reference's `half(nibble) * scale` computes.
+__device__ __forceinline__ f16x8 dequant8(uint32_t w, f16x2 s2) {
+  const uint32_t MAGIC = 0x64006400u;  // fp16 1024.0 in both halves
+  const f16x2 c1032 = {(f16)1032.0f, (f16)1032.0f};
+  const f16x2 c16th = {(f16)0.0625f, (f16)0.0625f};
+  const f16x2 c72 = {(f16)-72.0f, (f16)-72.0f};
+  const uint32_t w8 = w >> 8;
+  f16x2 p0 = bitcast<f16x2>((w & 0x000f000fu) | MAGIC);   // 1024 + u      (features 0,1)
+  f16x2 p1 = bitcast<f16x2>((w & 0x00f000f0u) | MAGIC);   // 1024 + 16 u   (features 2,3)
+  f16x2 p2 = bitcast<f16x2>((w8 & 0x000f000fu) | MAGIC);  // features 4,5
+  f16x2 p3 = bitcast<f16x2>((w8 & 0x00f000f0u) | MAGIC);  // features 6,7
+  p0 = (p0 - c1032) * s2;                                  // exact integer, then one rounding
+  p2 = (p2 - c1032) * s2;
+  p1 = __builtin_elementwise_fma(p1, c16th, c72) * s2;     // (1024 + 16u)/16 - 72 = u - 8, exact
+  p3 = __builtin_elementwise_fma(p3, c16th, c72) * s2;
+  f16x8 r;
+  r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
+  r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+  return r;
+}
+
+
+struct FmtW4 {
+  static constexpr int kVec = 1;
+  typedef f16x2 Scale;
+  static __device__ __forceinline__ Scale load_scale(const void* scale, int row, int N) {
+    const f16 s = row < N ? reinterpret_cast<const f16*>(scale)[row] : (f16)0.0f;
+    return f16x2{s, s};
+  }
+  static __device__ __forceinline__ f16x8 a_operand(const u32x4 (&raw)[1], int j, Scale s) {
+    return dequant8(raw[0][j], s);
+  }
+  static __device__ __forceinline__ float finish(float acc, Scale) { return acc; }
+};
+
+extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
+                                    const pta_half* const* host_scale, pta_half* const* host_Y,
+                                    const int* host_N, int M, int K, pta_stream_t stream) {
+  int rc = check_gemv_common("pta_w4a16_gemm_multi", X, M, K);
+  if (rc) return rc;
+  PTA_REQUIRE(count >= 1 && count <= 4, "pta_w4a16_gemm_multi: count must be in [1, 4], got %d", count);
+  GemmArgs a{};
+  a.count = count; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
+  int nb = 0;
+  for (int i = 0; i < count; ++i) {
+    PTA_REQUIRE(host_tiled[i] && host_scale[i] && host_Y[i], "pta_w4a16_gemm_multi: null pointer in entry %d", i);
+    PTA_REQUIRE(host_N[i] > 0, "pta_w4a16_gemm_multi: N[%d] = %d", i, host_N[i]);
+    PTA_REQUIRE(pta_aligned(host_tiled[i], 16), "pta_w4a16_gemm_multi: tiled[%d] must be 16-byte aligned", i);
+    a.mat[i] = GemmMat{(const void*)host_tiled[i], (const void*)host_scale[i], (f16*)host_Y[i], host_N[i], nb};
+    nb += (host_N[i] + 15) / 16;
+  }
+  return dispatch_gemv<FmtW4, false>(a, nb, (hipStream_t)stream, "pta_w4a16_gemm_multi");
+}
+
+extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
+                              int M, int K, int N, const pta_epilogue* epi, pta_stream_t stream) {
+  int rc = check_gemv_common("pta_w4a16_gemm", X, M, K);
+  if (rc) return rc;
+  PTA_REQUIRE(tiled && scale && Y, "pta_w4a16_gemm: null pointer");
+  PTA_REQUIRE(N > 0, "pta_w4a16_gemm: N = %d", N);
+  PTA_REQUIRE(pta_aligned(tiled, 16), "pta_w4a16_gemm: tiled must be 16-byte aligned");
+  GemmArgs a{};
+  a.count = 1; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
+  a.mat[0] = GemmMat{(const void*)tiled, (const void*)scale, (f16*)Y, N, 0};
+  rc = make_epilogue(epi, &a.epi, "pta_w4a16_gemm");
+  if (rc) return rc;
+  return dispatch_gemv<FmtW4, false>(a, (N + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm");
+}
+
+extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
+                                     const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M,
+                                     int K, int F, pta_stream_t stream) {
+  int rc = check_gemv_common("pta_w4a16_gemm_swiglu", X, M, K);
+  if (rc) return rc;
+  PTA_REQUIRE(tiled_gate && scale_gate && tiled_up && scale_up && Y, "pta_w4a16_gemm_swiglu: null pointer");
+  PTA_REQUIRE(F > 0, "pta_w4a16_gemm_swiglu: F = %d", F);
+  PTA_REQUIRE(pta_aligned(tiled_gate, 16) && pta_aligned(tiled_up, 16), "pta_w4a16_gemm_swiglu: tiled buffers must be 16-byte aligned");
+  GemmArgs a{};
+  a.count = 2; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
+  a.mat[0] = GemmMat{(const void*)tiled_gate, (const void*)scale_gate, (f16*)Y, F, 0};
+  a.mat[1] = GemmMat{(const void*)tiled_up, (const void*)scale_up, (f16*)Y, F, 0};
+  return dispatch_gemv<FmtW4, true>(a, (F + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm_swiglu");
+}

@@ -1,0 +1,122 @@
+// Row normalisations of the decode step: RMSNorm and the NormCE LayerNorm.
+//
+// RMSNorm follows poptransformer/layers/rms_layer_norm.py:26-36 (fp32 statistics, the inverse
+// RMS rounded to fp16, then two fp16 multiplies).  LayerNorm follows the NormCE custom op:
+// custom_ops/NormCE.cpp:122-200 + NormCECodelets.cpp:65-112 when there is a single row, and
+// the assembly kernel custom_ops/NormCE.S:243-423 (C form NormCECodelets.cpp:181-211) when
+// there are several.  One workgroup normalises one row in a single pass over registers.
+#include "common.h"
+
+constexpr int NORM_THREADS = 256;
+constexpr int NORM_MAX_VEC = 4;  // 8-element vectors per thread: rows up to 8192 columns
+
+__device__ __forceinline__ float block_sum(float v, float* sh) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) sh[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < NORM_THREADS / 64; ++w) t += sh[w];
+  return t;
+}
+
+// mode 0: RMSNorm.  mode 1: NormCE with one row.  mode 2: NormCE with several rows.
+template <int MODE>
+__global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restrict__ x, const f16* __restrict__ gamma,
+                                                            const f16* __restrict__ beta, f16* __restrict__ y,
+                                                            int cols, float eps) {
+  __shared__ float sh[NORM_THREADS / 64];
+  const size_t base = (size_t)blockIdx.x * cols;
+  const int nvec = cols >> 3;
+  f16x8 v[NORM_MAX_VEC];
+  float s = 0.f, sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NORM_MAX_VEC; ++i) {
+    const int c = threadIdx.x + i * NORM_THREADS;
+    if (c < nvec) {
+      v[i] = *reinterpret_cast<const f16x8*>(x + base + (size_t)c * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float f = (float)v[i][e];
+        s += f;
+        sq = __builtin_fmaf(f, f, sq);
+      }
+    }
+  }
+  const float inv_n = 1.0f / (float)cols;
+  f16 mean16 = (f16)0.0f, r16;
+  if (MODE == 0) {
+    const float ms = block_sum(sq, sh) * inv_n;
+    r16 = (f16)(1.0f / sqrtf(ms + eps));
+  } else {
+    const float sum = block_sum(s, sh);
+    const float sqs = block_sum(sq, sh);
+    const float mean = sum * inv_n;
+    mean16 = (f16)mean;
+    float var;
+    if (MODE == 1) {
+      var = sqs * inv_n - mean * mean + eps;  // fp32 mean, no clamp
+    } else {
+      const float m = (float)mean16;          // the rounded mean is what gets squared
+      var = fmaxf(sqs * inv_n - m * m, 0.0f) + eps;
+    }
+    r16 = (f16)(1.0f / sqrtf(var));
+  }
+#pragma unroll
+  for (int i = 0; i < NORM_MAX_VEC; ++i) {
+    const int c = threadIdx.x + i * NORM_THREADS;
+    if (c < nvec) {
+      const f16x8 g = *reinterpret_cast<const f16x8*>(gamma + (size_t)c * 8);
+      f16x8 o;
+      if (MODE == 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (v[i][e] * r16) * g[e];
+      } else {
+        const f16x8 b = *reinterpret_cast<const f16x8*>(beta + (size_t)c * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = ((v[i][e] - mean16) * r16) * g[e] + b[e];
+      }
+      *reinterpret_cast<f16x8*>(y + base + (size_t)c * 8) = o;
+    }
+  }
+}
+
+static int check_norm(const char* name, const void* x, const void* g, const void* y, int rows, int cols) {
+  PTA_REQUIRE(x && g && y, "%s: null pointer", name);
+  PTA_REQUIRE(rows > 0, "%s: rows = %d", name, rows);
+  PTA_REQUIRE(cols > 0 && (cols % 8) == 0 && cols <= 8 * NORM_THREADS * NORM_MAX_VEC,
+              "%s: the normalised size must be a multiple of 8 and at most %d, got %d", name,
+              8 * NORM_THREADS * NORM_MAX_VEC, cols);
+  PTA_REQUIRE(pta_aligned(x, 16) && pta_aligned(g, 16) && pta_aligned(y, 16), "%s: pointers must be 16-byte aligned", name);
+  return PTA_OK;
+}
+
+extern "C" int pta_rmsnorm(const pta_half* x, const pta_half* weight, pta_half* y, int rows, int cols,
+                           float eps, pta_stream_t stream) {
+  int rc = check_norm("pta_rmsnorm", x, weight, y, rows, cols);
+  if (rc) return rc;
+  hipLaunchKernelGGL(norm_kernel<0>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                     (const f16*)weight, (const f16*)nullptr, (f16*)y, cols, eps);
+  PTA_CHECK_LAUNCH("pta_rmsnorm");
+  return PTA_OK;
+}
+
+extern "C" int pta_layer_norm_ce(const pta_half* x, const pta_half* gamma, const pta_half* beta, pta_half* y,
+                                 int rows, int cols, float eps, pta_stream_t stream) {
+  int rc = check_norm("pta_layer_norm_ce", x, gamma, y, rows, cols);
+  if (rc) return rc;
+  // Guards of NormCEOutplaceOpx::grow (custom_ops/NormCE.cpp:541-577) and of the Python wrapper
+  // (poptransformer/ops/customized.py:81-82): fp16 only, size < 8192.
+  PTA_REQUIRE(beta && pta_aligned(beta, 16), "pta_layer_norm_ce: beta must be a 16-byte aligned pointer");
+  PTA_REQUIRE(cols < 8192, "pta_layer_norm_ce: the normalised size must be below 8192, got %d", cols);
+  if (rows == 1)
+    hipLaunchKernelGGL(norm_kernel<1>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps);
+  else
+    hipLaunchKernelGGL(norm_kernel<2>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps);
+  PTA_CHECK_LAUNCH("pta_layer_norm_ce");
+  return PTA_OK;
+}

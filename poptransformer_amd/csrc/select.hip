@@ -1,0 +1,117 @@
+// Next-token selection and the per-step loop bookkeeping.
+//
+// Greedy selection: layers/lm_head.py:47-57 -> ops.topk(k=1, axis=2) (ops/popart.py:135-137)
+// over fp16 logits; equal maxima resolve to the lowest index (ONNX TopK).
+// Loop bookkeeping: models/base_model.py:313-355 (step_containers, step_loop_cond).
+// Embedding rows: layers/embedding.py:34-36, models/gpt2/embedding.py:31-36.
+#include "common.h"
+
+constexpr int AM_THREADS = 1024;
+
+__global__ __launch_bounds__(AM_THREADS) void argmax_kernel(const f16* __restrict__ x, int32_t* __restrict__ idx,
+                                                            f16* __restrict__ val, int n) {
+  __shared__ float sv[AM_THREADS / 64];
+  __shared__ int si[AM_THREADS / 64];
+  const f16* xr = x + (size_t)blockIdx.x * n;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += AM_THREADS) {
+    const float v = (float)xr[i];
+    if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { sv[wave] = best; si[wave] = bi; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < AM_THREADS / 64; ++w)
+      if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
+    // A row without any finite-comparable value (all NaN) selects index 0.
+    idx[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    if (val) val[blockIdx.x] = (f16)best;
+  }
+}
+
+extern "C" int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, pta_stream_t stream) {
+  PTA_REQUIRE(logits && ids, "pta_argmax: null pointer");
+  PTA_REQUIRE(rows > 0 && n > 0, "pta_argmax: empty input [%d,%d]", rows, n);
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(AM_THREADS), 0, (hipStream_t)stream, (const f16*)logits, ids,
+                     (f16*)values, n);
+  PTA_CHECK_LAUNCH("pta_argmax");
+  return PTA_OK;
+}
+
+// out[b, :] = table[ids[b], :] (+ pos_table[*pos, :] in fp16 when pos_table is given).
+__global__ __launch_bounds__(256) void gather_rows_kernel(const f16* __restrict__ table, const int32_t* __restrict__ ids,
+                                                          const f16* __restrict__ pos_table, const int32_t* __restrict__ pos,
+                                                          f16* __restrict__ out, int cols, int vocab) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  int id = ids[b];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  f16 v = table[(size_t)id * cols + c];
+  if (pos_table) v = v + pos_table[(size_t)(*pos) * cols + c];
+  out[(size_t)b * cols + c] = v;
+}
+
+extern "C" int pta_embedding(const pta_half* table, const int32_t* ids, const pta_half* pos_table, const int32_t* pos,
+                             pta_half* out, int rows, int cols, int vocab, pta_stream_t stream) {
+  PTA_REQUIRE(table && ids && out, "pta_embedding: null pointer");
+  PTA_REQUIRE(!pos_table || pos, "pta_embedding: a position table needs a position");
+  PTA_REQUIRE(rows > 0 && cols > 0 && vocab > 0, "pta_embedding: empty shape");
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((cols + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream,
+                     (const f16*)table, ids, (const f16*)pos_table, pos, (f16*)out, cols, vocab);
+  PTA_CHECK_LAUNCH("pta_embedding");
+  return PTA_OK;
+}
+
+// One loop iteration of the generation bookkeeping, for all sequences:
+//   next_step = step + 1; mask[:, next_step] = 0;
+//   slot = container[:, next_step]; id = (slot == pad_id) ? next_ids : slot;
+//   container[:, next_step] = id; stop_mask |= (id == eos_id);
+//   keep_going = early_stop ? sum(stop_mask before this update) < B : true.
+// Writes at index max_len fall outside the containers and are dropped.  ids_out receives
+// container[:, next_step] (the input of the next iteration); *step is advanced last.
+__global__ void step_update_kernel(int32_t* container, f16* mask, int32_t* stop_mask, int32_t* step,
+                                   const int32_t* next_ids, int32_t* ids_out, int32_t* keep_going, int B,
+                                   int max_len, int pad_id, int eos_id, int early_stop) {
+  __shared__ int stopped_before;
+  if (threadIdx.x == 0) stopped_before = 0;
+  __syncthreads();
+  const int st = *step;
+  const int ns = st + 1;
+  for (int b = threadIdx.x; b < B; b += blockDim.x) {
+    if (stop_mask[b]) atomicAdd(&stopped_before, 1);
+    int id = next_ids[b];
+    if (ns < max_len) {
+      if (mask) mask[(size_t)b * max_len + ns] = (f16)0.0f;
+      const int slot = container[(size_t)b * max_len + ns];
+      id = slot == pad_id ? id : slot;
+      container[(size_t)b * max_len + ns] = id;
+    }
+    stop_mask[b] |= (id == eos_id) ? 1 : 0;
+    if (ids_out) ids_out[b] = id;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    if (keep_going) *keep_going = early_stop ? (stopped_before < B ? 1 : 0) : 1;
+    *step = ns;
+  }
+}
+
+extern "C" int pta_step_update(int32_t* container, pta_half* mask, int32_t* stop_mask, int32_t* step,
+                               const int32_t* next_ids, int32_t* ids_out, int32_t* keep_going, int B, int max_len,
+                               int pad_id, int eos_id, int early_stop, pta_stream_t stream) {
+  PTA_REQUIRE(container && stop_mask && step && next_ids, "pta_step_update: null pointer");
+  PTA_REQUIRE(B > 0 && max_len > 0, "pta_step_update: empty shape");
+  hipLaunchKernelGGL(step_update_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, container, (f16*)mask, stop_mask,
+                     step, next_ids, ids_out, keep_going, B, max_len, pad_id, eos_id, early_stop);
+  PTA_CHECK_LAUNCH("pta_step_update");
+  return PTA_OK;
+}

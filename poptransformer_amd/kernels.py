@@ -1,0 +1,269 @@
+"""Thin torch-tensor front end of the C ABI (include/poptransformer_hip.h).
+
+PyTorch is used for device memory and streams only: every function checks its operands on the
+host, passes raw pointers to libpoptransformer_hip.so on torch's current stream and returns
+torch tensors.  Nothing here computes on the CPU and nothing falls back to torch kernels.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import Epilogue, check
+
+_i32 = torch.int32
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _need(t, dtype, name, dims=None):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if dims is not None and t.dim() != dims:
+        raise ValueError(f"The rank of {name} should be {dims}. But now it is {t.dim()}.")
+
+
+def _epilogue(bias, residual, act):
+    if bias is None and residual is None and act == _lib.ACT_NONE:
+        return None
+    e = Epilogue(_p(bias) if bias is not None else None, _p(residual) if residual is not None else None, act)
+    return ctypes.byref(e)
+
+
+# ------------------------------------------------------------------ INT4 -----------------
+def int4_to_half(packed, scale, axis=1):
+    """ops.int4_to_half (reference: poptransformer/ops/customized.py:115-125)."""
+    _need(packed, torch.int8, "input", 2)
+    _need(scale, torch.float16, "scale", 1)
+    n, m = packed.shape
+    if axis == 1 and scale.shape[0] != n:
+        raise ValueError(f"[Int4ToHalfOp] input.shape[0]({n}) should be equal to  scale.shape[0]({scale.shape[0]})")
+    if axis == 0 and scale.shape[0] != m:
+        raise ValueError(f"[Int4ToHalfOp] input.shape[1]({m}) should be equal to  scale.shape[0]({scale.shape[0]})")
+    shape = (2 * m, n) if axis == 1 else (2 * n, m)
+    out = torch.empty(shape if axis in (0, 1) else (1,), dtype=torch.float16, device=packed.device)
+    check(_lib.load().pta_int4_to_half(_p(packed), _p(scale), _p(out), n, m, axis, _stream()))
+    return out
+
+
+class W4Weight:
+    """A packed INT4 Linear weight re-tiled for the fused kernels, with its fp16 scales."""
+
+    def __init__(self, packed, scale):
+        _need(packed, torch.int8, "packed weight", 2)
+        _need(scale, torch.float16, "scale", 1)
+        self.N, half_k = packed.shape
+        self.K = 2 * half_k
+        if scale.shape[0] != self.N:
+            raise ValueError(f"[Int4ToHalfOp] input.shape[0]({self.N}) should be equal to  scale.shape[0]({scale.shape[0]})")
+        lib = _lib.load()
+        nbytes = lib.pta_w4_tiled_bytes(self.N, self.K)
+        self.tiled = torch.empty(nbytes, dtype=torch.uint8, device=packed.device)
+        self.scale = scale
+        check(lib.pta_w4_tile(_p(packed), _p(self.tiled), self.N, self.K, _stream()))
+
+    @property
+    def nbytes(self):
+        return self.N * self.K // 2 + self.N * 2
+
+
+def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None):
+    _need(x, torch.float16, "x", 2)
+    M, K = x.shape
+    if K != w.K:
+        raise ValueError(f"matmul: contracting dimensions differ ({K} vs {w.K})")
+    if out is None:
+        out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
+    check(_lib.load().pta_w4a16_gemm(_p(x), _p(w.tiled), _p(w.scale), _p(out), M, K, w.N,
+                                     _epilogue(bias, residual, act), _stream()))
+    return out
+
+
+def w4a16_gemm_multi(x, weights, outs=None):
+    _need(x, torch.float16, "x", 2)
+    M, K = x.shape
+    n = len(weights)
+    if outs is None:
+        outs = [torch.empty((M, w.N), dtype=torch.float16, device=x.device) for w in weights]
+    for w in weights:
+        if w.K != K:
+            raise ValueError(f"matmul: contracting dimensions differ ({K} vs {w.K})")
+    VP = ctypes.c_void_p * n
+    tiled = VP(*[w.tiled.data_ptr() for w in weights])
+    scale = VP(*[w.scale.data_ptr() for w in weights])
+    ys = VP(*[o.data_ptr() for o in outs])
+    ns = (ctypes.c_int * n)(*[w.N for w in weights])
+    check(_lib.load().pta_w4a16_gemm_multi(_p(x), n, tiled, scale, ys, ns, M, K, _stream()))
+    return outs
+
+
+def w4a16_gemm_swiglu(x, w_gate, w_up, out=None):
+    _need(x, torch.float16, "x", 2)
+    M, K = x.shape
+    if w_gate.K != K or w_up.K != K or w_gate.N != w_up.N:
+        raise ValueError("swiglu: gate/up weights must share their shape and match x")
+    if out is None:
+        out = torch.empty((M, w_gate.N), dtype=torch.float16, device=x.device)
+    check(_lib.load().pta_w4a16_gemm_swiglu(_p(x), _p(w_gate.tiled), _p(w_gate.scale), _p(w_up.tiled),
+                                            _p(w_up.scale), _p(out), M, K, w_gate.N, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ FP16 -----------------
+class F16Weight:
+    """An fp16 Linear weight [N, K] (state-dict orientation) re-tiled for the fused kernel."""
+
+    def __init__(self, w):
+        _need(w, torch.float16, "weight", 2)
+        self.N, self.K = w.shape
+        lib = _lib.load()
+        self.tiled = torch.empty(lib.pta_f16_tiled_bytes(self.N, self.K), dtype=torch.uint8, device=w.device)
+        check(lib.pta_f16_tile(_p(w), _p(self.tiled), self.N, self.K, _stream()))
+
+    @property
+    def nbytes(self):
+        return self.N * self.K * 2
+
+
+def f16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None):
+    _need(x, torch.float16, "x", 2)
+    M, K = x.shape
+    if K != w.K:
+        raise ValueError(f"matmul: contracting dimensions differ ({K} vs {w.K})")
+    if out is None:
+        out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
+    check(_lib.load().pta_f16_gemm(_p(x), _p(w.tiled), _p(out), M, K, w.N, _epilogue(bias, residual, act), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ norms ----------------
+def rmsnorm(x, weight, eps, out=None):
+    _need(x, torch.float16, "x")
+    _need(weight, torch.float16, "weight", 1)
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if out is None:
+        out = torch.empty_like(x)
+    check(_lib.load().pta_rmsnorm(_p(x), _p(weight), _p(out), rows, cols, float(eps), _stream()))
+    return out
+
+
+def layer_norm_ce(x, gamma, beta, eps, out=None):
+    if x.dtype != torch.float16:
+        raise ValueError("[NormCE] only float16 is supported")
+    _need(x, torch.float16, "x")
+    _need(gamma, torch.float16, "gamma", 1)
+    _need(beta, torch.float16, "beta", 1)
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if out is None:
+        out = torch.empty_like(x)
+    check(_lib.load().pta_layer_norm_ce(_p(x), _p(gamma), _p(beta), _p(out), rows, cols, float(eps), _stream()))
+    return out
+
+
+def softmax_ce(x, stable_mode=True):
+    if x.dim() < 2:
+        raise ValueError("[Softmax] rank of input should be >= 2")
+    if x.dtype not in (torch.float16, torch.float32):
+        raise ValueError("[Softmax] input type must be FLOAT16 or FLOAT")
+    _need(x, x.dtype, "x")
+    n = x.shape[-1]
+    out = torch.empty_like(x)
+    dt = _lib.F16 if x.dtype == torch.float16 else _lib.F32
+    check(_lib.load().pta_softmax_ce(_p(x), _p(out), x.numel() // n, n, dt, 1 if stable_mode else 0, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ KV cache -------------
+def _kv_dims(t, axis):
+    outer = 1
+    for s in t.shape[:axis]:
+        outer *= s
+    inner = 1
+    for s in t.shape[axis + 1:]:
+        inner *= s
+    return outer, inner
+
+
+def kv_cache_update(cache, clone, updater, step, sequence_axis):
+    """Literal KVCache op on [.., max_len, ..] tensors; `cache` is updated in place and returned."""
+    outer, inner = _kv_dims(cache, sequence_axis)
+    _need(step, _i32, "step")
+    check(_lib.load().pta_kv_cache_update(_p(cache), _p(clone), _p(updater), _p(step), outer,
+                                          cache.shape[sequence_axis], updater.shape[sequence_axis], inner,
+                                          cache.element_size(), _stream()))
+    return cache
+
+
+def kv_cache_append(ring, updater, step, outer, max_len, inner, max_bps=1):
+    _need(step, _i32, "step")
+    check(_lib.load().pta_kv_cache_append(_p(ring), _p(updater), _p(step), outer, max_len, inner,
+                                          ring.element_size(), max_bps, _stream()))
+
+
+def kv_cache_read(ring, out, step, outer, max_len, inner, max_bps=1):
+    _need(step, _i32, "step")
+    check(_lib.load().pta_kv_cache_read(_p(ring), _p(out), _p(step), outer, max_len, inner, ring.element_size(),
+                                        max_bps, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ attention ------------
+def qkv_rope_append(q, k, v, q_out, kv_ring, step, inv_freq, B, Hq, Hkv, D, max_len, rope,
+                    q_stride=None, k_stride=None, v_stride=None):
+    q_stride = Hq * D if q_stride is None else q_stride
+    k_stride = Hkv * D if k_stride is None else k_stride
+    v_stride = Hkv * D if v_stride is None else v_stride
+    check(_lib.load().pta_qkv_rope_append(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(q_out), _p(kv_ring),
+                                          _p(step), _p(inv_freq), B, Hq, Hkv, D, max_len, rope, _stream()))
+
+
+def decode_attention_workspace(B, Hq, D, max_len, device):
+    n = _lib.load().pta_decode_attention_workspace_bytes(B, Hq, D, max_len)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def decode_attention(q, kv_ring, step, workspace, out, B, Hq, Hkv, D, max_len, use_scale):
+    check(_lib.load().pta_decode_attention(_p(q), _p(kv_ring), _p(step), _p(workspace), _p(out), B, Hq, Hkv, D,
+                                           max_len, 1 if use_scale else 0, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ selection ------------
+def argmax(logits, ids=None, values=None):
+    _need(logits, torch.float16, "logits")
+    n = logits.shape[-1]
+    rows = logits.numel() // n
+    if ids is None:
+        ids = torch.empty(rows, dtype=_i32, device=logits.device)
+    check(_lib.load().pta_argmax(_p(logits), _p(ids), _p(values), rows, n, _stream()))
+    return ids
+
+
+def embedding(table, ids, out=None, pos_table=None, pos=None):
+    _need(table, torch.float16, "table", 2)
+    _need(ids, _i32, "ids")
+    rows = ids.numel()
+    vocab, cols = table.shape
+    if out is None:
+        out = torch.empty((rows, cols), dtype=torch.float16, device=table.device)
+    check(_lib.load().pta_embedding(_p(table), _p(ids), _p(pos_table), _p(pos), _p(out), rows, cols, vocab, _stream()))
+    return out
+
+
+def step_update(container, mask, stop_mask, step, next_ids, ids_out, keep_going, pad_id, eos_id, early_stop):
+    B, max_len = container.shape
+    check(_lib.load().pta_step_update(_p(container), _p(mask), _p(stop_mask), _p(step), _p(next_ids), _p(ids_out),
+                                      _p(keep_going), B, max_len, int(pad_id), int(eos_id), 1 if early_stop else 0,
+                                      _stream()))

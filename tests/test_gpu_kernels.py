@@ -1,0 +1,404 @@
+"""Parity of each HIP kernel, called through the C ABI, against the numpy oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    from poptransformer_amd import kernels
+    return kernels
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rel_err(got, ref):
+    got = got.astype(np.float64)
+    ref = ref.astype(np.float64)
+    return np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30)
+
+
+# ---------------------------------------------------------------- Int4ToHalf (bit-exact)
+@pytest.mark.parametrize("n,m", [(3, 2), (16, 64), (130, 70), (11008, 64)])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_int4_to_half_bit_exact(K, n, m, axis):
+    rng = np.random.default_rng(n * 131 + m + axis)
+    packed = rng.integers(-128, 128, size=(n, m), dtype=np.int8)
+    scale = rng.uniform(0.005, 0.02, size=(n if axis == 1 else m,)).astype(np.float16)
+    got = host(K.int4_to_half(dev(packed), dev(scale), axis))
+    ref = O.int4_to_half(packed, scale, axis)
+    assert got.shape == ref.shape
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+def test_int4_to_half_all_bytes(K):
+    packed = np.arange(256, dtype=np.uint8).view(np.int8).reshape(256, 1)
+    scale = np.ones(256, np.float16)
+    got = host(K.int4_to_half(dev(packed), dev(scale), 1))        # [2, 256]
+    tab = O.int4_table()
+    assert np.array_equal(got.T.astype(np.float32), tab)
+
+
+def test_int4_to_half_guards(K):
+    p = dev(np.zeros((4, 4), np.int8))
+    s = dev(np.ones(4, np.float16))
+    with pytest.raises(ValueError):
+        K.int4_to_half(p, s, axis=2)
+    with pytest.raises(ValueError):
+        K.int4_to_half(p, dev(np.ones(5, np.float16)), axis=1)
+    with pytest.raises(ValueError):
+        K.int4_to_half(dev(np.zeros((4,), np.int8)), s, axis=1)
+
+
+# ---------------------------------------------------------------- W4A16 GEMM
+def _w4_case(seed, M, Kdim, N):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    packed = rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8)
+    scale = rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)
+    return x, packed, scale
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 17, 33, 64])
+@pytest.mark.parametrize("Kdim,N", [(128, 16), (256, 48), (1024, 100), (4096, 512), (11008, 64), (136, 24)])
+def test_w4a16_gemm(K, M, Kdim, N):
+    x, packed, scale = _w4_case(M * 7 + Kdim + N, M, Kdim, N)
+    w = K.W4Weight(dev(packed), dev(scale))
+    got = host(K.w4a16_gemm(dev(x), w))
+    ref64 = x.astype(np.float64) @ O.int4_to_half(packed, scale, 1).astype(np.float64)
+    ref = O.w4a16_matmul(x, packed, scale)
+    assert got.shape == ref.shape
+    # north-star tolerance: max rel err <= 1e-2 on fp16 outputs
+    assert rel_err(got, ref) <= 1e-2
+    # against exact arithmetic the kernel must be as good as fp16 rounding allows
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
+
+
+def test_w4a16_gemm_exact_integers(K):
+    """Integers small enough that every product and sum is exact: the result must be exact,
+    which catches any wrong nibble order, sign or feature permutation."""
+    rng = np.random.default_rng(5)
+    M, Kdim, N = 5, 256, 40
+    x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
+    q = rng.integers(-8, 8, size=(N, Kdim))
+    packed = O.pack_int4(q)
+    scale = np.ones(N, np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    got = host(K.w4a16_gemm(dev(x), w)).astype(np.int64)
+    ref = x.astype(np.int64) @ q.T.astype(np.int64)
+    assert np.array_equal(got, ref)
+
+
+def test_w4a16_gemm_epilogue(K):
+    x, packed, scale = _w4_case(11, 3, 512, 96)
+    rng = np.random.default_rng(12)
+    bias = rng.standard_normal(96).astype(np.float16)
+    res = rng.standard_normal((3, 96)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    got = host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res)))
+    y = O.w4a16_matmul(x, packed, scale)
+    ref = ((y + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+
+
+def test_w4a16_gemm_multi_and_swiglu(K):
+    rng = np.random.default_rng(3)
+    M, Kdim = 2, 1024
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    mats = []
+    for N in (256, 64, 80):
+        packed = rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8)
+        scale = rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)
+        mats.append((packed, scale))
+    ws = [K.W4Weight(dev(p), dev(s)) for p, s in mats]
+    outs = K.w4a16_gemm_multi(dev(x), ws)
+    for (p, s), o in zip(mats, outs):
+        assert rel_err(host(o), O.w4a16_matmul(x, p, s)) <= 1e-2
+    (pg, sg), (pu, su) = (mats[1], (rng.integers(-128, 128, size=(64, Kdim // 2), dtype=np.int8),
+                                    rng.uniform(0.005, 0.02, size=(64,)).astype(np.float16)))
+    got = host(K.w4a16_gemm_swiglu(dev(x), K.W4Weight(dev(pg), dev(sg)), K.W4Weight(dev(pu), dev(su))))
+    gate = O.swish(O.w4a16_matmul(x, pg, sg))
+    ref = (O.w4a16_matmul(x, pu, su) * gate).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+
+
+def test_w4a16_guards(K):
+    x, packed, scale = _w4_case(1, 1, 128, 16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    with pytest.raises(ValueError):
+        K.w4a16_gemm(dev(np.zeros((1, 64), np.float16)), w)
+    with pytest.raises(ValueError):
+        K.w4a16_gemm(dev(np.zeros((65, 128), np.float16)), w)
+
+
+# ---------------------------------------------------------------- FP16 GEMM
+@pytest.mark.parametrize("M,Kdim,N", [(1, 768, 50257), (4, 4096, 1000), (16, 128, 16), (64, 3072, 768), (1, 136, 20)])
+def test_f16_gemm(K, M, Kdim, N):
+    rng = np.random.default_rng(M + Kdim + N)
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    w = (rng.standard_normal((N, Kdim)) * 0.02).astype(np.float16)
+    got = host(K.f16_gemm(dev(x), K.F16Weight(dev(w))))
+    ref = O.matmul(x, w.T)
+    assert rel_err(got, ref) <= 1e-2
+    ref64 = x.astype(np.float64) @ w.T.astype(np.float64)
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-4
+
+
+def test_f16_gemm_gelu_bias(K):
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((2, 256)).astype(np.float16)
+    w = (rng.standard_normal((64, 256)) * 0.05).astype(np.float16)
+    b = rng.standard_normal(64).astype(np.float16)
+    from poptransformer_amd import _lib
+    got = host(K.f16_gemm(dev(x), K.F16Weight(dev(w)), bias=dev(b), act=_lib.ACT_GELU_TANH))
+    ref = O.gelu((O.matmul(x, w.T) + b).astype(np.float16))
+    assert rel_err(got, ref) <= 1e-2
+
+
+# ---------------------------------------------------------------- norms
+@pytest.mark.parametrize("rows,cols", [(1, 4096), (16, 4096), (3, 768), (2, 8)])
+def test_rmsnorm(K, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, cols).astype(np.float16)
+    got = host(K.rmsnorm(dev(x), dev(g), 1e-5))
+    ref = O.rms_norm(x, g, 1e-5)
+    # identical up to the rounding of the inverse RMS (summation order): 2 fp16 ulp
+    assert np.abs(got.astype(np.float32) - ref.astype(np.float32)).max() <= 2 * 2.0 ** -10 * np.abs(ref).max()
+    assert (got.view(np.uint16) == ref.view(np.uint16)).mean() > 0.5
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 768), (1, 4096), (32, 4096), (5, 1024)])
+def test_layer_norm_ce(K, rows, cols):
+    rng = np.random.default_rng(rows * 3 + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.3).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, cols).astype(np.float16)
+    b = rng.standard_normal(cols).astype(np.float16)
+    got = host(K.layer_norm_ce(dev(x), dev(g), dev(b), 1e-5))
+    ref = O.layer_norm_ce(x, g, b, 1e-5, rows, 1, cols)
+    assert np.abs(got.astype(np.float32) - ref.astype(np.float32)).max() <= 4 * 2.0 ** -10 * np.abs(ref).max()
+
+
+def test_layer_norm_ce_guards(K):
+    x = dev(np.zeros((1, 8192), np.float16))
+    g = dev(np.ones(8192, np.float16))
+    with pytest.raises(ValueError):
+        K.layer_norm_ce(x, g, g, 1e-5)
+    with pytest.raises(ValueError):
+        K.layer_norm_ce(dev(np.zeros((1, 64), np.float32)), g, g, 1e-5)
+
+
+# ---------------------------------------------------------------- softmax
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("stable", [False, True])
+@pytest.mark.parametrize("rows,n", [(1, 128), (32, 2048), (7, 33)])
+def test_softmax_ce(K, dtype, stable, rows, n):
+    rng = np.random.default_rng(rows + n)
+    x = (rng.standard_normal((rows, n)) * 2).astype(dtype)
+    x[:, n // 2:] -= 10000          # the attention mask value
+    got = host(K.softmax_ce(dev(x), stable))
+    ref = O.softmax_ce(x, -1, stable)
+    tol = 3e-3 if dtype == np.float16 else 1e-5
+    assert np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() <= tol
+    assert np.all(got[:, n // 2:] == 0)
+
+
+# ---------------------------------------------------------------- KV cache (bit-exact)
+@pytest.mark.parametrize("shape,axis,max_len,dtype", [((2, 1, 3, 1, 8), 3, 5, np.float16), ((2, 2, 4, 1, 128), 3, 7, np.float16),
+                                                      ((3, 1, 5), 1, 4, np.float32), ((2, 1, 2, 1, 3), 3, 6, np.float16)])
+def test_kv_cache_ring_matches_shift_register(K, shape, axis, max_len, dtype):
+    rng = np.random.default_rng(17)
+    ref_op = O.KVCache(max_len, axis, 1)
+    outer = int(np.prod(shape[:axis]))
+    inner = int(np.prod(shape[axis + 1:]))
+    out_shape = list(shape)
+    out_shape[axis] = max_len
+    ring = torch.empty((outer, max_len, inner), dtype=torch.from_numpy(np.zeros(1, dtype)).dtype, device="cuda")
+    ring.fill_(7)                                            # stale contents must never show
+    cache_lit = torch.full(out_shape, 7, dtype=ring.dtype, device="cuda")
+    clone = torch.empty_like(cache_lit)
+    view = torch.empty(out_shape, dtype=ring.dtype, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in range(max_len + 3):
+        upd = rng.standard_normal(shape).astype(dtype)
+        ref = ref_op(it, upd)
+        step.fill_(it)
+        u = dev(upd)
+        K.kv_cache_append(ring, u, step, outer, max_len, inner)
+        K.kv_cache_read(ring, view, step, outer, max_len, inner)
+        K.kv_cache_update(cache_lit, clone, u, step, axis)
+        assert np.array_equal(host(view), ref), f"ring view differs at step {it}"
+        assert np.array_equal(host(cache_lit), ref), f"literal cache differs at step {it}"
+    # step 0 again zeroes the history
+    upd = rng.standard_normal(shape).astype(dtype)
+    ref = ref_op(0, upd)
+    step.fill_(0)
+    K.kv_cache_append(ring, dev(upd), step, outer, max_len, inner)
+    K.kv_cache_read(ring, view, step, outer, max_len, inner)
+    assert np.array_equal(host(view), ref)
+
+
+def test_kv_cache_pipeline(K):
+    rng = np.random.default_rng(23)
+    max_len, max_bps, shape = 4, 3, (2, 2, 1, 16)
+    ref_op = O.KVCachePipeline(max_len, max_bps)
+    outer, inner = 4, 16
+    ring = torch.full((max_bps, outer, max_len, inner), 5, dtype=torch.float16, device="cuda")
+    view = torch.empty((2, 2, max_len, 16), dtype=torch.float16, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in range(max_bps * (max_len + 2)):
+        upd = rng.standard_normal(shape).astype(np.float16)
+        ref = ref_op(it, upd)
+        step.fill_(it)
+        K.kv_cache_append(ring, dev(upd), step, outer, max_len, inner, max_bps)
+        K.kv_cache_read(ring, view, step, outer, max_len, inner, max_bps)
+        assert np.array_equal(host(view), ref), f"pipeline cache differs at step {it}"
+
+
+# ---------------------------------------------------------------- attention
+def _attention_reference(family, qs, ks, vs, max_len, D):
+    """Runs the oracle chain step by step; returns the context vectors per step."""
+    B, Hq = qs[0].shape[0], qs[0].shape[1]
+    Hkv = ks[0].shape[1]
+    cache = O.KVCache(max_len, 3, 1)
+    mask = np.full((B, max_len), -10000, np.float16)
+    mask[:, 0] = 0
+    outs = []
+    for step, (q, k, v) in enumerate(zip(qs, ks, vs)):
+        q4 = q.reshape(B, Hq, 1, D)
+        k4 = k.reshape(B, Hkv, 1, D)
+        v4 = v.reshape(B, Hkv, 1, D)
+        if family == "llama":
+            sin, cos = O.llama_sincos(step, D)
+            q4, k4 = O.llama_rope(q4, sin, cos), O.llama_rope(k4, sin, cos)
+        elif family == "glm2":
+            cos, sin = O.glm2_sincos(step, D)
+            q4 = np.swapaxes(O.glm2_rope(np.swapaxes(q4, 1, 2), cos, sin), 1, 2)
+            k4 = np.swapaxes(O.glm2_rope(np.swapaxes(k4, 1, 2), cos, sin), 1, 2)
+        past = cache(step, np.stack([k4, v4]))
+        kk, vv = past[0], past[1]
+        if Hkv != Hq:
+            kk = np.repeat(kk, Hq // Hkv, axis=1)
+            vv = np.repeat(vv, Hq // Hkv, axis=1)
+        scale = None if family == "gpt2" else 1 / np.sqrt(D)
+        sdt = np.float32 if family == "llama" else np.float16
+        ctx = O.attention_scores_to_context(q4, np.swapaxes(kk, 2, 3), vv, mask[:, None, None, :], scale, sdt)
+        outs.append(np.swapaxes(ctx, 1, 2).reshape(B, Hq * D))
+        if step + 1 < max_len:
+            mask[:, step + 1] = 0
+    return outs
+
+
+@pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 70), ("gpt2", 1, 12, 12, 64, 40, 40),
+                                                             ("glm2", 2, 8, 2, 128, 150, 80), ("llama", 1, 2, 2, 128, 16, 20)])
+def test_rope_append_attention(K, family, B, Hq, Hkv, D, max_len, steps):
+    from poptransformer_amd import _lib
+    rng = np.random.default_rng(B + Hq + D)
+    qs = [(rng.standard_normal((B, Hq, D)) * (0.3 if family == "gpt2" else 1.0)).astype(np.float16) for _ in range(steps)]
+    ks = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(steps)]
+    vs = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(steps)]
+    refs = _attention_reference(family, qs, ks, vs, max_len, D)   # steps > max_len drops the oldest rows
+    rope = {"llama": _lib.ROPE_LLAMA, "glm2": _lib.ROPE_GLM2, "gpt2": _lib.ROPE_NONE}[family]
+    inv = None
+    if family == "llama":
+        inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    elif family == "glm2":
+        inv = dev(np.array([1.0 / (10000 ** (i / (D // 2))) for i in range(0, D // 2, 2)]).astype(np.float32))
+    ring = torch.full((2 * B * Hkv, max_len, D), float("nan"), dtype=torch.float16, device="cuda")
+    ws = K.decode_attention_workspace(B, Hq, D, max_len, "cuda")
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float16, device="cuda")
+    out = torch.empty((B, Hq * D), dtype=torch.float16, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in range(steps):
+        step.fill_(it)
+        K.qkv_rope_append(dev(qs[it]), dev(ks[it]), dev(vs[it]), q_rot, ring, step, inv, B, Hq, Hkv, D, max_len, rope)
+        K.decode_attention(q_rot, ring, step, ws, out, B, Hq, Hkv, D, max_len, family != "gpt2")
+        got = host(out)
+        assert np.isfinite(got).all(), f"non-finite output at step {it}"
+        assert rel_err(got, refs[it]) <= 1e-2, f"step {it}"
+
+
+def test_rope_bit_exact(K):
+    """q after rotary embedding and the appended key row are pure fp16 elementwise work: bit-exact."""
+    from poptransformer_amd import _lib
+    rng = np.random.default_rng(2)
+    B, H, D, max_len = 2, 3, 128, 64
+    inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    ring = torch.zeros((2 * B * H, max_len, D), dtype=torch.float16, device="cuda")
+    q_rot = torch.empty((B, H, D), dtype=torch.float16, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in (0, 1, 5, 37, 63):
+        q = rng.standard_normal((B, H, D)).astype(np.float16)
+        k = rng.standard_normal((B, H, D)).astype(np.float16)
+        v = rng.standard_normal((B, H, D)).astype(np.float16)
+        step.fill_(it)
+        K.qkv_rope_append(dev(q), dev(k), dev(v), q_rot, ring, step, inv, B, H, H, D, max_len, _lib.ROPE_LLAMA)
+        sin, cos = O.llama_sincos(it, D)
+        qr = O.llama_rope(q.reshape(B, H, 1, D), sin, cos).reshape(B, H, D)
+        kr = O.llama_rope(k.reshape(B, H, 1, D), sin, cos).reshape(B, H, D)
+        r = host(ring).reshape(2, B, H, max_len, D)
+        # sin/cos of the same fp16 angle may differ by one fp16 ulp between libm and the device
+        assert np.abs(host(q_rot).astype(np.float32) - qr.astype(np.float32)).max() <= 2 ** -9 * 4
+        assert np.abs(r[0, :, :, it].astype(np.float32) - kr.astype(np.float32)).max() <= 2 ** -9 * 4
+        assert np.array_equal(r[1, :, :, it], v)
+
+
+# ---------------------------------------------------------------- selection & loop
+@pytest.mark.parametrize("rows,n", [(1, 32000), (16, 50257), (3, 65536), (2, 5)])
+def test_argmax(K, rows, n):
+    rng = np.random.default_rng(rows + n)
+    x = rng.standard_normal((rows, n)).astype(np.float16)
+    x[0, [n // 3, n // 2]] = 9.0                       # a tie: the lower index wins
+    got = host(K.argmax(dev(x)))
+    _, ref = O.topk1(x, -1)
+    assert np.array_equal(got, ref[:, 0])
+
+
+def test_embedding(K):
+    rng = np.random.default_rng(4)
+    table = rng.standard_normal((100, 64)).astype(np.float16)
+    pos = rng.standard_normal((10, 64)).astype(np.float16)
+    ids = np.array([3, 99, 0], np.int32)
+    assert np.array_equal(host(K.embedding(dev(table), dev(ids))), table[ids])
+    p = torch.tensor(7, dtype=torch.int32, device="cuda")
+    got = host(K.embedding(dev(table), dev(ids), pos_table=dev(pos), pos=p))
+    assert np.array_equal(got, (table[ids] + pos[7]).astype(np.float16))
+
+
+@pytest.mark.parametrize("early_stop", [False, True])
+def test_step_update_matches_loop_simulator(K, early_stop):
+    rng = np.random.default_rng(8)
+    B, L, pad, eos = 3, 12, 0, 2
+    ids = np.full((B, L), pad, np.int32)
+    ids[0, :4] = [5, 6, 7, 8]
+    ids[1, :2] = [9, 3]
+    ids[2, :6] = [4, 4, 2, 4, 4, 4]
+    state = O.initial_loop_state(ids, L)
+    container = dev(ids.copy())
+    mask = dev(state["mask"].copy())
+    stop = torch.zeros(B, dtype=torch.int32, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    keep = torch.ones((), dtype=torch.int32, device="cuda")
+    ids_out = torch.zeros(B, dtype=torch.int32, device="cuda")
+    for it in range(L):
+        nxt = rng.integers(1, 6, size=B).astype(np.int32)
+        upd = O.step_containers(state, nxt, pad)
+        keep_ref = O.step_loop_cond(state, upd, eos, early_stop, B)
+        K.step_update(container, mask, stop, step, dev(nxt), ids_out, keep, pad, eos, early_stop)
+        assert np.array_equal(host(container), state["container"])
+        assert np.array_equal(host(mask), state["mask"])
+        assert np.array_equal(host(stop), state["stop_mask"])
+        assert int(host(step)) == state["step"]
+        assert bool(host(keep)) == keep_ref
+        assert np.array_equal(host(ids_out), upd)
