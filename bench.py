@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Decode benchmark: Llama2-7B-shape INT4 greedy decode on one MI355X.
+
+A "step" is one iteration of the decode loop (one new token per sequence): embedding, 32
+transformer blocks (RMSNorm, INT4 q/k/v/o and SwiGLU projections, rotary embedding, KV append,
+attention over the cache, residuals), final norm, fp16 lm_head, greedy selection and the loop
+bookkeeping.  The default run follows the headline configuration: batch 1, a 128-token prompt
+consumed token by token (the untimed warm-up), then 256 timed new tokens, KV cache length 2048.
+
+Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel (the fused INT4
+gate/up projection) measured with events on its own stream, and a CPU baseline (the numpy
+restatement of the same graph on the host cores, on a reduced number of layers).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+LLAMA2_7B = dict(vocab_size=32000, hidden_size=4096, rms_norm_eps=1e-5, num_attention_heads=32,
+                 intermediate_size=11008, num_hidden_layers=32)
+MAX_LEN = 2048
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_step_bytes(cfg, B, t):
+    """Bytes one decode step must move at context t: every weight once (INT4 + scales, norm
+    weights, fp16 lm_head), the KV rows written and read, the embedding rows."""
+    d, f, v, n = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
+    per_layer = (4 * d * d + 3 * d * f) // 2 + 2 * (4 * d + 2 * f + d)
+    weights = n * per_layer + 2 * (2 * n + 1) * d + 2 * v * d
+    kv = B * 2 * n * d * 2 * (t + 1)
+    return weights + kv + B * d * 2
+
+
+def cpu_baseline(seconds_budget=20.0):
+    """The numpy oracle of the same graph on the host: 2 full-width layers + head, scaled to 32."""
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from oracle import models as OM
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    layers = 2
+    cfg = dict(LLAMA2_7B, num_hidden_layers=layers)
+    sd = OM.make_llama2_state_dict(cfg, seed=0, int4=True)
+    L = 64
+    model = OM.Llama2Oracle(sd, cfg, L, 1)
+    ids = np.zeros((1, L), np.int32)
+    ids[0, :8] = np.arange(5, 13)
+    from oracle import ops as O
+    state = O.initial_loop_state(ids, L)
+    model.step(state["container"][:, 0].reshape(1, 1), 0, state["mask"])       # warm-up
+    n, t0 = 0, time.perf_counter()
+    t_layers = t_head = 0.0
+    while time.perf_counter() - t0 < seconds_budget and n < 12:
+        step = n + 1
+        a = time.perf_counter()
+        x = model.embed[state["container"][:, step].reshape(1, 1)]
+        mask4 = state["mask"][:, None, None, :]
+        for lay in model.layers:
+            t = O.rms_norm(x, lay["ln1"], model.eps)
+            t = model._attention(lay, t, step, mask4)
+            x = (x + t).astype(np.float16)
+            t = O.rms_norm(x, lay["ln2"], model.eps).reshape(-1, model.d)
+            u = (lay["up"](t) * O.swish(lay["gate"](t))).astype(np.float16)
+            x = (x + lay["down"](u).reshape(1, -1, model.d)).astype(np.float16)
+        b = time.perf_counter()
+        O.topk1(model.head(O.rms_norm(x, model.norm, model.eps)), axis=2)
+        c = time.perf_counter()
+        t_layers += b - a
+        t_head += c - b
+        state["mask"][:, step + 1] = 0
+        n += 1
+    per_token = (t_layers / n) * (LLAMA2_7B["num_hidden_layers"] / layers) + t_head / n
+    return {"value": 1.0 / per_token, "unit": "tokens/s", "cores": int(threads), "kind": "port",
+            "sample": f"numpy oracle, {layers} full-width layers + lm_head, {n} tokens at batch 1, "
+                      f"layer time scaled x{LLAMA2_7B['num_hidden_layers'] // layers}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if args.warmup + args.steps + 1 > MAX_LEN:
+        print(f"warmup + steps must stay below the KV cache length {MAX_LEN}", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from poptransformer_amd import kernels as K
+    from poptransformer_amd.engine import fused, loader, synthetic
+
+    if not torch.cuda.is_available():
+        print("no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    B, cfg = args.batch, LLAMA2_7B
+    weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
+    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
+    dec.capture()
+
+    rng = np.random.Generator(np.random.PCG64(1234))
+    prompt = 128
+    ids = np.zeros((B, MAX_LEN), np.int32)                       # pad id 0 after the prompt
+    ids[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B, prompt))
+    dec.reset(ids)
+
+    dec.run_steps(args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.run_steps(args.steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    tokens_per_s = B * args.steps / dt
+    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(args.warmup, args.warmup + args.steps)])
+    step_frac = mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9)
+
+    # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
+    # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
+    # (1.4 GB in total, so no launch finds its weights in a cache).
+    d, f = cfg["hidden_size"], cfg["intermediate_size"]
+    stream = torch.cuda.Stream()
+    reps = 10
+    with torch.cuda.stream(stream):
+        for blk in weights.blocks:
+            K.w4a16_gemm_swiglu(dec.h, blk.mlp_in[0].w, blk.mlp_in[1].w, dec.act)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        g = torch.cuda.CUDAGraph()
+        stream.synchronize()
+        with torch.cuda.graph(g, stream=stream):
+            for blk in weights.blocks:
+                K.w4a16_gemm_swiglu(dec.h, blk.mlp_in[0].w, blk.mlp_in[1].w, dec.act)
+        g.replay()
+        e0.record(stream)
+        for _ in range(reps):
+            g.replay()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    launches = reps * len(weights.blocks)
+    kernel_s = e0.elapsed_time(e1) * 1e-3 / launches
+    kernel_bytes = 2 * (d * f // 2 + 2 * f) + B * d * 2 + B * f * 2
+    achieved = kernel_bytes / kernel_s / 1e9
+
+    out = {
+        "metric": "decode tokens/s at Llama2-7B INT4 bs=1/16 + % of HBM roofline",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
+        "config": {"workload": f"Llama2-7B-shape INT4 greedy decode, batch {B}, prompt {prompt} consumed token by token, "
+                               f"context {args.warmup}..{args.warmup + args.steps - 1}, fp16 KV cache length {MAX_LEN}",
+                   "batch": B, "kv_cache_len": MAX_LEN},
+        "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
+        "roofline": {"bound": "hbm", "kernel": "gemv_mfma_kernel<FmtW4, 1, 8, true> (INT4 gate/up + SwiGLU)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": None, "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

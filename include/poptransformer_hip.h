@@ -201,9 +201,13 @@ int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32
 int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, pta_stream_t stream);
 
 /* Embedding rows (layers/embedding.py:34-36); with pos_table also GPT-2's wte[id] + wpe[*pos]
- * (models/gpt2/embedding.py:31-36).  out [rows, cols]. */
-int pta_embedding(const pta_half* table, const int32_t* ids, const pta_half* pos_table, const int32_t* pos,
-                  pta_half* out, int rows, int cols, int vocab, pta_stream_t stream);
+ * (models/gpt2/embedding.py:31-36).  out [rows, cols].  Row b uses
+ * id = ids[b*ids_stride + (ids_index ? *ids_index : 0)], so the `dynamic_slice(container, step)`
+ * of the model graphs (e.g. models/llama2/model.py:168) needs no copy: pass the container,
+ * ids_stride = max_length and ids_index = step.  For a plain id vector: ids_stride 1, NULL. */
+int pta_embedding(const pta_half* table, const int32_t* ids, int ids_stride, const int32_t* ids_index,
+                  const pta_half* pos_table, const int32_t* pos, pta_half* out, int rows, int cols, int vocab,
+                  pta_stream_t stream);
 
 /* step_containers + step_loop_cond of models/base_model.py:313-355 for one iteration; all
  * arrays on the device.  container int32 [B, max_len]; mask fp16 [B, max_len] or NULL;

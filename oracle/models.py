@@ -1,0 +1,255 @@
+"""CPU restatement (numpy) of the PopTransformer decode loop for whole models.
+
+TEST INFRASTRUCTURE ONLY (see oracle/ops.py): imported by tests/, by __graft_entry__.smoke()
+and by the cpu_baseline leg of bench.py.  Each model walks the reference graph op by op with the
+operator restatements of oracle/ops.py; state-dict keys and shapes are the reference's.
+"""
+import numpy as np
+
+from . import ops as O
+
+f16, f32 = np.float16, np.float32
+
+
+# --------------------------------------------------------------------------------------
+# synthetic checkpoints
+# --------------------------------------------------------------------------------------
+def quantize_int4(w):
+    """Symmetric per-output-channel INT4 quantisation of w [out, in]: scale = max|w| / 7 (fp16),
+    q = clip(round(w / scale), -8, 7), packed two per byte with feature 2j in the high nibble.
+    The reference has no quantiser (it loads ChatGLM-int4 style checkpoints:
+    `weight int8[out, in/2]`, `weight_scale fp16[out]`,
+    poptransformer/utils/param_handler/precision_strategy.py:24-42); this only produces
+    checkpoints of that layout for the synthetic configurations."""
+    w = np.asarray(w, f32)
+    scale = (np.abs(w).max(axis=1) / 7.0).astype(f16)
+    scale = np.maximum(scale, np.finfo(f16).tiny).astype(f16)
+    q = np.clip(np.rint(w / scale.astype(f32)[:, None]), -8, 7).astype(np.int8)
+    return O.pack_int4(q), scale
+
+
+def _normal(rng, shape, std=0.02):
+    return (rng.standard_normal(shape, dtype=f32) * std).astype(f16)
+
+
+def make_llama2_state_dict(cfg, seed=0, int4=True):
+    """Random-init Llama-2-shaped checkpoint: weights N(0, 0.02), RMSNorm weights 1, Linear
+    weights quantised to packed INT4 when `int4`, embeddings and lm_head fp16.  Keys and shapes:
+    poptransformer/models/llama2/model.py:31-36,64-85,119-132, attention.py:58-62, mlp.py:15-18."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, f, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    sd = {"model.embed_tokens.weight": _normal(rng, (v, d))}
+
+    def linear(key, out_f, in_f):
+        w = _normal(rng, (out_f, in_f))
+        if int4:
+            sd[key + ".weight"], sd[key + ".weight_scale"] = quantize_int4(w)
+        else:
+            sd[key + ".weight"] = w
+
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        sd[p + "input_layernorm.weight"] = np.ones(d, f16)
+        for n in ("q_proj", "k_proj", "v_proj", "o_proj"):
+            linear(p + "self_attn." + n, d, d)
+        sd[p + "post_attention_layernorm.weight"] = np.ones(d, f16)
+        linear(p + "mlp.gate_proj", f, d)
+        linear(p + "mlp.up_proj", f, d)
+        linear(p + "mlp.down_proj", d, f)
+    sd["model.norm.weight"] = np.ones(d, f16)
+    sd["lm_head.weight"] = _normal(rng, (v, d))
+    return sd
+
+
+def make_gpt2_state_dict(cfg, seed=0):
+    """Random-init GPT-2-shaped checkpoint as the reference holds it AFTER
+    GPT2DecModel.process_hf_model_state_dict (poptransformer/models/gpt2/model.py:154-166): Linear
+    weights in [out, in] orientation and the query third of c_attn pre-multiplied by
+    1/sqrt(head_dim).  N(0, 0.02) weights, zero biases, LayerNorm gamma 1 / beta 0.
+    Keys: models/gpt2/model.py:32-37,64-84, attention.py:33-35, embedding.py:27-29, layers/mlp.py:30-32."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, v, npos = cfg["n_embd"], cfg["vocab_size"], cfg["n_positions"]
+    hd = d // cfg["n_head"]
+    sd = {"transformer.wte.weight": _normal(rng, (v, d)), "transformer.wpe.weight": _normal(rng, (npos, d))}
+    for i in range(cfg["n_layer"]):
+        p = f"transformer.h.{i}."
+        for ln in ("ln_1", "ln_2"):
+            sd[p + ln + ".weight"] = np.ones(d, f16)
+            sd[p + ln + ".bias"] = np.zeros(d, f16)
+        w = (rng.standard_normal((3 * d, d), dtype=f32) * 0.02)
+        w[:d] *= np.float32(1 / hd ** 0.5)
+        sd[p + "attn.c_attn.weight"] = w.astype(f16)
+        sd[p + "attn.c_attn.bias"] = np.zeros(3 * d, f16)
+        sd[p + "attn.c_proj.weight"] = _normal(rng, (d, d))
+        sd[p + "attn.c_proj.bias"] = np.zeros(d, f16)
+        sd[p + "mlp.c_fc.weight"] = _normal(rng, (4 * d, d))
+        sd[p + "mlp.c_fc.bias"] = np.zeros(4 * d, f16)
+        sd[p + "mlp.c_proj.weight"] = _normal(rng, (d, 4 * d))
+        sd[p + "mlp.c_proj.bias"] = np.zeros(d, f16)
+    sd["transformer.ln_f.weight"] = np.ones(d, f16)
+    sd["transformer.ln_f.bias"] = np.zeros(d, f16)
+    return sd
+
+
+# --------------------------------------------------------------------------------------
+# shared pieces
+# --------------------------------------------------------------------------------------
+class _Linear:
+    """BaseLinear (poptransformer/layers/linear.py:19-46) + ParamHandler.matmul
+    (utils/param_handler/param_handler.py:57-61): `<ctx>.weight` is [out, in], stored transposed;
+    an int8 weight is a packed INT4 matrix [out, in/2] with `<ctx>.weight_scale`
+    (utils/param_handler/precision_strategy.py:24-42,56-60)."""
+
+    def __init__(self, sd, ctx, use_bias):
+        w = sd[ctx + ".weight"]
+        if w.dtype == np.int8:
+            self.w = O.int4_to_half(w, sd[ctx + ".weight_scale"], axis=1)   # [in, out] fp16
+        else:
+            self.w = np.ascontiguousarray(w.T)
+        self.b = sd[ctx + ".bias"] if use_bias else None
+
+    def __call__(self, x):
+        y = O.matmul(x, self.w)
+        return (y + self.b).astype(f16) if self.b is not None else y
+
+
+def run_decode_loop(model, input_ids, max_length, max_loop, pad_id, eos_id, early_stop=False, trace=None):
+    """HFDecBaseModel.build_graph / build_post_model_graph (poptransformer/models/base_model.py:271-311):
+    a Loop of max_loop iterations over {container, step, mask, stop_mask}; returns the container
+    and the final step like the anchors 'Loop:0' and 'Loop:1'."""
+    state = O.initial_loop_state(input_ids, max_length)
+    b = state["container"].shape[0]
+    for _ in range(max_loop):
+        step = state["step"]
+        ids = state["container"][:, min(step, max_length - 1)].reshape(b, 1)
+        next_ids, logits = model.step(ids, step, state["mask"])
+        if trace is not None:
+            trace.append((next_ids.copy(), logits.copy()))
+        upd = O.step_containers(state, next_ids, pad_id)
+        if not O.step_loop_cond(state, upd, eos_id, early_stop, b):
+            break
+    return state["container"], state["step"]
+
+
+# --------------------------------------------------------------------------------------
+# Llama 2
+# --------------------------------------------------------------------------------------
+class Llama2Oracle:
+    """LLAMA2DecModel.build_model_graph (poptransformer/models/llama2/model.py:162-197) for
+    sequence_length == 1: embedding gather, per block RMSNorm -> attention -> add -> RMSNorm ->
+    SwiGLU MLP -> add (model.py:38-46), final RMSNorm, LMHead top-1 (layers/lm_head.py:47-57)."""
+
+    def __init__(self, sd, cfg, max_length, batch_size):
+        self.cfg, self.L, self.B = cfg, max_length, batch_size
+        self.d, self.H = cfg["hidden_size"], cfg["num_attention_heads"]
+        self.D = self.d // self.H
+        self.eps = cfg["rms_norm_eps"]
+        self.embed = sd["model.embed_tokens.weight"]
+        self.layers = []
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            self.layers.append({
+                "ln1": sd[p + "input_layernorm.weight"], "ln2": sd[p + "post_attention_layernorm.weight"],
+                "q": _Linear(sd, p + "self_attn.q_proj", False), "k": _Linear(sd, p + "self_attn.k_proj", False),
+                "v": _Linear(sd, p + "self_attn.v_proj", False), "o": _Linear(sd, p + "self_attn.o_proj", False),
+                "gate": _Linear(sd, p + "mlp.gate_proj", False), "up": _Linear(sd, p + "mlp.up_proj", False),
+                "down": _Linear(sd, p + "mlp.down_proj", False),
+                "cache": O.KVCache(max_length, 3, 1),
+            })
+        self.norm = sd["model.norm.weight"]
+        self.head = _Linear(sd, "lm_head", False)
+
+    def _attention(self, lay, x, step, mask4):
+        """Attention.forward_qkv / forward_attention / forward_output
+        (poptransformer/models/llama2/attention.py:64-114)."""
+        B, H, D = self.B, self.H, self.D
+        q, k, v = lay["q"](x), lay["k"](x), lay["v"](x)
+        q = q.reshape(B, 1, H, D).transpose(0, 2, 1, 3)
+        k = k.reshape(B, 1, H, D).transpose(0, 2, 1, 3)
+        v = v.reshape(B, 1, H, D).transpose(0, 2, 1, 3)
+        sin, cos = O.llama_sincos(step, D)
+        q, k = O.llama_rope(q, sin, cos), O.llama_rope(k, sin, cos)
+        kv = np.concatenate([k, v], axis=0).reshape(2, B, H, 1, D)
+        past = lay["cache"](step, kv)
+        kt = past[0].transpose(0, 1, 3, 2)
+        a = O.attention_scores_to_context(q, kt, past[1], mask4, 1 / np.sqrt(D), f32, stable_mode=False)
+        a = a.transpose(0, 2, 1, 3).reshape(B, 1, H * D)
+        return lay["o"](a)
+
+    def step(self, ids, step, mask):
+        B = self.B
+        x = self.embed[ids.reshape(B, 1)]                        # [B, 1, d] gather
+        mask4 = mask[:, None, None, :]
+        for lay in self.layers:
+            t = O.rms_norm(x, lay["ln1"], self.eps)
+            t = self._attention(lay, t, step, mask4)
+            x = (x + t).astype(f16)
+            t = O.rms_norm(x, lay["ln2"], self.eps)
+            t2 = t.reshape(-1, self.d)                          # ShardMLP (models/llama2/mlp.py:20-28)
+            g = O.swish(lay["gate"](t2))
+            u = (lay["up"](t2) * g).astype(f16)
+            t = lay["down"](u).reshape(B, -1, self.d)
+            x = (x + t).astype(f16)
+        x = O.rms_norm(x, self.norm, self.eps)
+        logits = self.head(x)                                    # [B, 1, V]
+        _, idx = O.topk1(logits, axis=2)
+        return idx.reshape(B), logits.reshape(B, -1)
+
+
+# --------------------------------------------------------------------------------------
+# GPT-2
+# --------------------------------------------------------------------------------------
+class GPT2Oracle:
+    """GPT2DecModel.build_model_graph (poptransformer/models/gpt2/model.py:168-201), blocks
+    (model.py:39-46), embedding wte[id] + wpe[step] (models/gpt2/embedding.py:31-36), LayerNorm via
+    NormCE, head tied to wte (model.py:144-151, layers/lm_head.py:47-57)."""
+
+    def __init__(self, sd, cfg, max_length, batch_size):
+        self.cfg, self.L, self.B = cfg, max_length, batch_size
+        self.d, self.H = cfg["n_embd"], cfg["n_head"]
+        self.D = self.d // self.H
+        self.eps = cfg["layer_norm_epsilon"]
+        self.wte, self.wpe = sd["transformer.wte.weight"], sd["transformer.wpe.weight"]
+        self.layers = []
+        for i in range(cfg["n_layer"]):
+            p = f"transformer.h.{i}."
+            self.layers.append({
+                "ln1": (sd[p + "ln_1.weight"], sd[p + "ln_1.bias"]), "ln2": (sd[p + "ln_2.weight"], sd[p + "ln_2.bias"]),
+                "c_attn": _Linear(sd, p + "attn.c_attn", True), "c_proj": _Linear(sd, p + "attn.c_proj", True),
+                "c_fc": _Linear(sd, p + "mlp.c_fc", True), "mlp_proj": _Linear(sd, p + "mlp.c_proj", True),
+                "cache": O.KVCache(max_length, 3, 1),
+            })
+        self.ln_f = (sd["transformer.ln_f.weight"], sd["transformer.ln_f.bias"])
+        self.head_w = np.ascontiguousarray(self.wte.T)            # ops.transpose(wte, [1, 0])
+
+    def _ln(self, x, wb):
+        return O.layer_norm_ce(x, wb[0], wb[1], self.eps, self.B, 1, self.d)
+
+    def _attention(self, lay, x, step, mask4):
+        """BaseAttention (poptransformer/models/gpt2/attention.py:37-90)."""
+        B, H, D, d = self.B, self.H, self.D, self.d
+        qkv = lay["c_attn"](x)                                     # [B, 1, 3d]
+        q, kv = qkv[..., :d], qkv[..., d:]
+        q = q.reshape(B, 1, H, D).transpose(0, 2, 1, 3)
+        kv = kv.reshape(B, 1, 2, H, D).transpose(2, 0, 3, 1, 4)    # [2, B, H, 1, D]
+        past = lay["cache"](step, kv)
+        a = O.attention_scores_to_context(q, past[0].transpose(0, 1, 3, 2), past[1], mask4, None, f16, False)
+        a = a.transpose(0, 2, 1, 3).reshape(B, 1, d)
+        return lay["c_proj"](a)
+
+    def step(self, ids, step, mask):
+        B = self.B
+        x = (self.wte[ids.reshape(B, 1)] + self.wpe[np.full((B, 1), step)]).astype(f16)
+        mask4 = mask[:, None, None, :]
+        for lay in self.layers:
+            t = self._ln(x, lay["ln1"])
+            t = self._attention(lay, t, step, mask4)
+            x = (x + t).astype(f16)
+            t = self._ln(x, lay["ln2"])
+            t = t.reshape(-1, self.d)                              # BaseMLP (layers/mlp.py:34-41)
+            t = lay["mlp_proj"](O.gelu(lay["c_fc"](t))).reshape(B, -1, self.d)
+            x = (x + t).astype(f16)
+        x = self._ln(x, self.ln_f)
+        logits = O.matmul(x, self.head_w)
+        _, idx = O.topk1(logits, axis=2)
+        return idx.reshape(B), logits.reshape(B, -1)

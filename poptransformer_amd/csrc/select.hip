@@ -46,27 +46,33 @@ extern "C" int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values
   return PTA_OK;
 }
 
-// out[b, :] = table[ids[b], :] (+ pos_table[*pos, :] in fp16 when pos_table is given).
+// out[b, :] = table[id_b, :] (+ pos_table[*pos, :] in fp16 when pos_table is given), with
+// id_b = ids[b * ids_stride + (ids_index ? *ids_index : 0)]: the column `step` of the id container
+// (dynamic_slice of models/llama2/model.py:168) is read in place.
 __global__ __launch_bounds__(256) void gather_rows_kernel(const f16* __restrict__ table, const int32_t* __restrict__ ids,
+                                                          int ids_stride, const int32_t* __restrict__ ids_index,
                                                           const f16* __restrict__ pos_table, const int32_t* __restrict__ pos,
                                                           f16* __restrict__ out, int cols, int vocab) {
   const int b = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= cols) return;
-  int id = ids[b];
+  int col = ids_index ? *ids_index : 0;
+  col = col < 0 ? 0 : (col >= ids_stride ? ids_stride - 1 : col);
+  int id = ids[(size_t)b * ids_stride + col];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   f16 v = table[(size_t)id * cols + c];
   if (pos_table) v = v + pos_table[(size_t)(*pos) * cols + c];
   out[(size_t)b * cols + c] = v;
 }
 
-extern "C" int pta_embedding(const pta_half* table, const int32_t* ids, const pta_half* pos_table, const int32_t* pos,
-                             pta_half* out, int rows, int cols, int vocab, pta_stream_t stream) {
+extern "C" int pta_embedding(const pta_half* table, const int32_t* ids, int ids_stride, const int32_t* ids_index,
+                             const pta_half* pos_table, const int32_t* pos, pta_half* out, int rows, int cols,
+                             int vocab, pta_stream_t stream) {
   PTA_REQUIRE(table && ids && out, "pta_embedding: null pointer");
   PTA_REQUIRE(!pos_table || pos, "pta_embedding: a position table needs a position");
-  PTA_REQUIRE(rows > 0 && cols > 0 && vocab > 0, "pta_embedding: empty shape");
+  PTA_REQUIRE(rows > 0 && cols > 0 && vocab > 0 && ids_stride > 0, "pta_embedding: empty shape");
   hipLaunchKernelGGL(gather_rows_kernel, dim3((cols + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream,
-                     (const f16*)table, ids, (const f16*)pos_table, pos, (f16*)out, cols, vocab);
+                     (const f16*)table, ids, ids_stride, ids_index, (const f16*)pos_table, pos, (f16*)out, cols, vocab);
   PTA_CHECK_LAUNCH("pta_embedding");
   return PTA_OK;
 }
@@ -82,6 +88,9 @@ __global__ void step_update_kernel(int32_t* container, f16* mask, int32_t* stop_
                                    const int32_t* next_ids, int32_t* ids_out, int32_t* keep_going, int B,
                                    int max_len, int pad_id, int eos_id, int early_stop) {
   __shared__ int stopped_before;
+  // Once the loop condition has gone false the reference's Loop stops iterating: a further
+  // call must leave every container as it is.
+  if (keep_going && *keep_going == 0) return;
   if (threadIdx.x == 0) stopped_before = 0;
   __syncthreads();
   const int st = *step;

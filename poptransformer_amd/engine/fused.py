@@ -1,0 +1,246 @@
+"""Fused executor of the decode loop for decoder-only transformers.
+
+The reference runs one PopART `Loop` whose body is the model graph followed by the container /
+stop-mask bookkeeping (poptransformer/models/base_model.py:271-355), everything on the device.
+Here the same loop body is a fixed sequence of HIP kernel launches over persistent device
+buffers, recorded once into a HIP graph and replayed per token; `step`, the id container and
+the stop mask live in device memory exactly as they are graph tensors in the reference, so a
+replay needs no host data.
+
+The executor is parameterised by a `DecoderSpec` (what a transformer block looks like) and by
+prepared weights; sessions.py builds both from a recorded model graph.  Supported block
+shapes: GPT-2 (models/gpt2), Llama 2 (models/llama2), ChatGLM2 (models/chatglm2).
+"""
+from dataclasses import dataclass, field
+from typing import List, Optional
+
+import numpy as np
+import torch
+
+from .. import _lib
+from .. import kernels as K
+
+
+@dataclass
+class DecoderSpec:
+    family: str                      # 'gpt2' | 'llama2' | 'chatglm2'
+    n_layer: int
+    d_model: int
+    n_head: int
+    n_kv_head: int
+    head_dim: int
+    vocab: int
+    max_len: int
+    batch: int
+    eps: float
+    pad_id: int = 0
+    eos_id: int = -1
+    early_stop: bool = False
+
+    @property
+    def norm(self):
+        return "ln" if self.family == "gpt2" else "rms"
+
+    @property
+    def rope(self):
+        return {"gpt2": _lib.ROPE_NONE, "llama2": _lib.ROPE_LLAMA, "chatglm2": _lib.ROPE_GLM2}[self.family]
+
+    @property
+    def scale_scores(self):
+        # GPT-2 folds 1/sqrt(D) into the query weights at load (models/gpt2/model.py:154-166)
+        return self.family != "gpt2"
+
+
+class LinearWeights:
+    """One Linear: a tiled weight (INT4 or FP16) and an optional fp16 bias."""
+
+    def __init__(self, weight, bias=None):
+        self.w, self.bias = weight, bias
+        self.N, self.K = weight.N, weight.K
+
+    @property
+    def is_int4(self):
+        return isinstance(self.w, K.W4Weight)
+
+    def __call__(self, x, out, residual=None, act=_lib.ACT_NONE):
+        if self.is_int4:
+            return K.w4a16_gemm(x, self.w, self.bias, residual, act, out)
+        return K.f16_gemm(x, self.w, self.bias, residual, act, out)
+
+    @property
+    def nbytes(self):
+        return self.w.nbytes + (self.bias.numel() * 2 if self.bias is not None else 0)
+
+
+@dataclass
+class BlockWeights:
+    norm1: tuple                      # (gamma, beta or None)
+    norm2: tuple
+    qkv: List[LinearWeights]          # [q, k, v] or [fused qkv] or [q, kv]
+    out: LinearWeights
+    mlp_in: List[LinearWeights]       # [gate, up] (SwiGLU) or [fc] (GELU)
+    mlp_out: LinearWeights
+
+
+@dataclass
+class ModelWeights:
+    embed: torch.Tensor               # [V, d] fp16
+    pos_embed: Optional[torch.Tensor]
+    blocks: List[BlockWeights]
+    final_norm: tuple
+    head: LinearWeights
+    inv_freq: Optional[torch.Tensor] = None
+
+    def nbytes(self):
+        n = self.head.nbytes
+        for b in self.blocks:
+            for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]:
+                n += lw.nbytes
+            for g in (b.norm1, b.norm2):
+                n += sum(t.numel() * 2 for t in g if t is not None)
+        n += sum(t.numel() * 2 for t in self.final_norm if t is not None)
+        return n
+
+
+class FusedDecoder:
+    def __init__(self, spec: DecoderSpec, weights: ModelWeights, device="cuda"):
+        self.spec, self.w, self.dev = spec, weights, device
+        s = spec
+        B, d = s.batch, s.d_model
+        f16, i32 = torch.float16, torch.int32
+
+        def buf(*shape, dtype=f16):
+            return torch.zeros(shape, dtype=dtype, device=device)
+
+        self.x, self.h, self.ctx = buf(B, d), buf(B, d), buf(B, d)
+        qkv_n = sum(lw.N for lw in weights.blocks[0].qkv)
+        self.qkv = buf(B, qkv_n)
+        self.q_rot = buf(B, s.n_head, s.head_dim)
+        ffn = weights.blocks[0].mlp_out.K
+        self.act = buf(B, ffn)
+        self.logits = buf(B, s.vocab)
+        self.next_ids = buf(B, dtype=i32)
+        self.container = buf(B, s.max_len, dtype=i32)
+        self.mask = buf(B, s.max_len)
+        self.stop_mask = buf(B, dtype=i32)
+        self.step = torch.zeros((), dtype=i32, device=device)
+        self.keep_going = torch.ones((), dtype=i32, device=device)
+        # one ring per layer: keys then values, [2*B*Hkv, max_len, D]
+        self.rings = [buf(2 * B * s.n_kv_head, s.max_len, s.head_dim) for _ in range(s.n_layer)]
+        self.attn_ws = K.decode_attention_workspace(B, s.n_head, s.head_dim, s.max_len, device)
+        self.graph = None
+        self._stream = torch.cuda.Stream()
+
+    # ------------------------------------------------------------------ one loop iteration
+    def _norm(self, x, gb, out):
+        if self.spec.norm == "rms":
+            return K.rmsnorm(x, gb[0], self.spec.eps, out)
+        return K.layer_norm_ce(x, gb[0], gb[1], self.spec.eps, out)
+
+    def step_fn(self):
+        s, w = self.spec, self.w
+        B = s.batch
+        K.embedding(w.embed, self.container, self.x, pos_table=w.pos_embed,
+                    pos=self.step if w.pos_embed is not None else None, ids_index=self.step)
+        for li, blk in enumerate(w.blocks):
+            self._norm(self.x, blk.norm1, self.h)
+            self._project_qkv(blk)
+            qp, kp, vp, qs, ks, vs = self._qkv_views
+            K.qkv_rope_append(qp, kp, vp, self.q_rot, self.rings[li], self.step, w.inv_freq, B, s.n_head,
+                              s.n_kv_head, s.head_dim, s.max_len, s.rope, qs, ks, vs)
+            K.decode_attention(self.q_rot, self.rings[li], self.step, self.attn_ws, self.ctx, B, s.n_head,
+                               s.n_kv_head, s.head_dim, s.max_len, s.scale_scores)
+            blk.out(self.ctx, self.x, residual=self.x)
+            self._norm(self.x, blk.norm2, self.h)
+            if len(blk.mlp_in) == 2:
+                g, u = blk.mlp_in
+                if g.is_int4 and u.is_int4:
+                    K.w4a16_gemm_swiglu(self.h, g.w, u.w, self.act)
+                else:
+                    raise NotImplementedError("SwiGLU needs INT4 gate/up weights in the fused executor")
+            else:
+                blk.mlp_in[0](self.h, self.act, act=_lib.ACT_GELU_TANH)
+            blk.mlp_out(self.act, self.x, residual=self.x)
+        self._norm(self.x, w.final_norm, self.h)
+        w.head(self.h, self.logits)
+        K.argmax(self.logits, self.next_ids)
+        K.step_update(self.container, self.mask, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
+                      s.pad_id, s.eos_id, s.early_stop)
+
+    def _project_qkv(self, blk):
+        if not hasattr(self, "_qkv_views"):
+            self._prepare_qkv_views(blk)
+        if len(blk.qkv) == 1:
+            blk.qkv[0](self.h, self.qkv)
+        elif all(lw.is_int4 and lw.bias is None for lw in blk.qkv):
+            K.w4a16_gemm_multi(self.h, [lw.w for lw in blk.qkv], self._qkv_bufs)
+        else:
+            for lw, o in zip(blk.qkv, self._qkv_bufs):
+                lw(self.h, o)
+
+    def _prepare_qkv_views(self, blk):
+        """Output buffers of the projections and the (pointer, row stride) views of q, k, v."""
+        s = self.spec
+        B, Hq, Hkv, D = s.batch, s.n_head, s.n_kv_head, s.head_dim
+        f16 = torch.float16
+        if len(blk.qkv) == 1:           # GPT-2: one row holds q | k | v
+            row = (Hq + 2 * Hkv) * D
+            self._qkv_bufs = [self.qkv]
+            self._qkv_views = (self.qkv, self.qkv[:, Hq * D:], self.qkv[:, (Hq + Hkv) * D:], row, row, row)
+        elif len(blk.qkv) == 3:         # Llama 2: separate q, k, v
+            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
+            q, k, v = self._qkv_bufs
+            self._qkv_views = (q, k, v, Hq * D, Hkv * D, Hkv * D)
+        else:                           # ChatGLM2: query, and key_value holding k | v
+            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
+            q, kv = self._qkv_bufs
+            self._qkv_views = (q, kv, kv[:, Hkv * D:], Hq * D, 2 * Hkv * D, 2 * Hkv * D)
+
+    # ------------------------------------------------------------------ loop
+    def reset(self, input_ids):
+        """Initial loop state of build_model_graph_inputs (models/base_model.py:255-269)."""
+        s = self.spec
+        ids = torch.as_tensor(np.asarray(input_ids, np.int32))
+        if tuple(ids.shape) != (s.batch, s.max_len):
+            raise ValueError(f"input_ids must be [{s.batch}, {s.max_len}], got {tuple(ids.shape)}")
+        self.container.copy_(ids)
+        self.mask.fill_(-10000.0)
+        self.mask[:, 0] = 0
+        self.stop_mask.zero_()
+        self.step.zero_()
+        self.keep_going.fill_(1)
+
+    def capture(self):
+        """Record one loop iteration into a HIP graph (after an eager iteration has warmed up
+        every code path).  The iteration depends on device state only, so it can be replayed."""
+        self.reset(np.zeros((self.spec.batch, self.spec.max_len), np.int32))
+        with torch.cuda.stream(self._stream):
+            self.step_fn()
+            torch.cuda.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph, stream=self._stream):
+                self.step_fn()
+        torch.cuda.synchronize()
+        return self.graph
+
+    def run_steps(self, n):
+        if self.graph is None:
+            for _ in range(n):
+                self.step_fn()
+        else:
+            for _ in range(n):
+                self.graph.replay()
+
+    def run(self, input_ids, max_loop, check_every=16):
+        """The whole generation (one `session.run` of the reference, poptransformer/sessions.py:47-49).
+        Returns (container, step) like the anchors 'Loop:0' and 'Loop:1'."""
+        self.reset(input_ids)
+        done = 0
+        while done < max_loop:
+            n = min(check_every, max_loop - done) if self.spec.early_stop else max_loop - done
+            self.run_steps(n)
+            done += n
+            if self.spec.early_stop and int(self.keep_going.item()) == 0:
+                break
+        torch.cuda.synchronize()
+        return self.container.cpu().numpy(), int(self.step.item())

@@ -1,0 +1,78 @@
+"""State dict (numpy, reference key names) -> device weights of the fused executor.
+
+Mirrors what the reference layers do when they bind their weights
+(poptransformer/layers/linear.py:28-40 with utils/param_handler/precision_strategy.py:24-51):
+an int8 `<ctx>.weight` is a packed INT4 matrix [out, in/2] with `<ctx>.weight_scale`; other
+Linear weights are fp16 [out, in].  Weights are re-tiled on the device once, here.
+"""
+import numpy as np
+import torch
+
+from .. import kernels as K
+from .fused import BlockWeights, DecoderSpec, LinearWeights, ModelWeights
+
+
+def _dev(a, device):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def linear_from_state_dict(sd, ctx, use_bias, device="cuda"):
+    w = sd[ctx + ".weight"]
+    w = w if isinstance(w, np.ndarray) else np.asarray(w)
+    if w.dtype == np.int8:
+        scale = sd.get(ctx + ".weight_scale")
+        if scale is None:
+            raise KeyError(f"{ctx}.weight is packed INT4 but {ctx}.weight_scale is missing")
+        tw = K.W4Weight(_dev(w, device), _dev(np.asarray(scale, np.float16), device))
+    else:
+        tw = K.F16Weight(_dev(w.astype(np.float16), device))
+    bias = _dev(np.asarray(sd[ctx + ".bias"], np.float16), device) if use_bias else None
+    return LinearWeights(tw, bias)
+
+
+def llama2_weights(sd, cfg, device="cuda"):
+    d = cfg["hidden_size"]
+    hd = d // cfg["num_attention_heads"]
+    blocks = []
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        blocks.append(BlockWeights(
+            norm1=(_dev(sd[p + "input_layernorm.weight"], device), None),
+            norm2=(_dev(sd[p + "post_attention_layernorm.weight"], device), None),
+            qkv=[linear_from_state_dict(sd, p + "self_attn." + n, False, device) for n in ("q_proj", "k_proj", "v_proj")],
+            out=linear_from_state_dict(sd, p + "self_attn.o_proj", False, device),
+            mlp_in=[linear_from_state_dict(sd, p + "mlp." + n, False, device) for n in ("gate_proj", "up_proj")],
+            mlp_out=linear_from_state_dict(sd, p + "mlp.down_proj", False, device)))
+    inv_freq = np.array([1.0 / (10000 ** (i / hd)) for i in range(0, hd, 2)]).astype(np.float16)
+    return ModelWeights(embed=_dev(sd["model.embed_tokens.weight"], device), pos_embed=None, blocks=blocks,
+                        final_norm=(_dev(sd["model.norm.weight"], device), None),
+                        head=linear_from_state_dict(sd, "lm_head", False, device), inv_freq=_dev(inv_freq, device))
+
+
+def llama2_spec(cfg, max_len, batch, pad_id=0, eos_id=2, early_stop=False):
+    d, h = cfg["hidden_size"], cfg["num_attention_heads"]
+    return DecoderSpec("llama2", cfg["num_hidden_layers"], d, h, h, d // h, cfg["vocab_size"], max_len, batch,
+                       cfg["rms_norm_eps"], pad_id, eos_id, early_stop)
+
+
+def gpt2_weights(sd, cfg, device="cuda"):
+    blocks = []
+    for i in range(cfg["n_layer"]):
+        p = f"transformer.h.{i}."
+        blocks.append(BlockWeights(
+            norm1=(_dev(sd[p + "ln_1.weight"], device), _dev(sd[p + "ln_1.bias"], device)),
+            norm2=(_dev(sd[p + "ln_2.weight"], device), _dev(sd[p + "ln_2.bias"], device)),
+            qkv=[linear_from_state_dict(sd, p + "attn.c_attn", True, device)],
+            out=linear_from_state_dict(sd, p + "attn.c_proj", True, device),
+            mlp_in=[linear_from_state_dict(sd, p + "mlp.c_fc", True, device)],
+            mlp_out=linear_from_state_dict(sd, p + "mlp.c_proj", True, device)))
+    wte = _dev(sd["transformer.wte.weight"], device)
+    return ModelWeights(embed=wte, pos_embed=_dev(sd["transformer.wpe.weight"], device), blocks=blocks,
+                        final_norm=(_dev(sd["transformer.ln_f.weight"], device), _dev(sd["transformer.ln_f.bias"], device)),
+                        head=LinearWeights(K.F16Weight(wte)), inv_freq=None)
+
+
+def gpt2_spec(cfg, max_len, batch, pad_id=50257, eos_id=50256, early_stop=False):
+    d, h = cfg["n_embd"], cfg["n_head"]
+    return DecoderSpec("gpt2", cfg["n_layer"], d, h, h, d // h, cfg["vocab_size"], max_len, batch,
+                       cfg["layer_norm_epsilon"], pad_id, eos_id, early_stop)

@@ -251,14 +251,20 @@ def argmax(logits, ids=None, values=None):
     return ids
 
 
-def embedding(table, ids, out=None, pos_table=None, pos=None):
+def embedding(table, ids, out=None, pos_table=None, pos=None, ids_index=None):
+    """Rows of `table`.  ids int32 [rows] or, with ids_index (device int32 scalar), a container
+    [rows, L] of which column *ids_index is used."""
     _need(table, torch.float16, "table", 2)
     _need(ids, _i32, "ids")
-    rows = ids.numel()
+    if ids_index is None:
+        rows, stride = ids.numel(), 1
+    else:
+        rows, stride = ids.shape
     vocab, cols = table.shape
     if out is None:
         out = torch.empty((rows, cols), dtype=torch.float16, device=table.device)
-    check(_lib.load().pta_embedding(_p(table), _p(ids), _p(pos_table), _p(pos), _p(out), rows, cols, vocab, _stream()))
+    check(_lib.load().pta_embedding(_p(table), _p(ids), stride, _p(ids_index), _p(pos_table), _p(pos), _p(out), rows,
+                                    cols, vocab, _stream()))
     return out
 
 
