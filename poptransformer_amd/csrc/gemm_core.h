@@ -188,6 +188,130 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
   }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// Variant for very small M (M <= 4): the activation rows are staged once per workgroup in LDS
+// (M*K*2 bytes) and the B operand comes from LDS reads, which are broadcasts when M == 1.
+// The first weight tile is requested before the staging so that HBM latency overlaps it.
+// ------------------------------------------------------------------------------------------
+template <class Fmt, int NW, bool PAIR>
+__global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int KV = Fmt::kVec;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int mi = 0;
+  if (!PAIR) {
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (i < a.count && (int)blockIdx.x >= a.mat[i].nb_begin) mi = i;
+  }
+  const int nb = blockIdx.x - a.mat[mi].nb_begin;
+  const int N = a.mat[mi].N;
+  const int row = nb * 16 + (lane & 15);
+  const int K = a.K, KT = a.KT, M = a.M;
+  const int xstride = KT * 128 + 8;                 // +8 halves: rows land in different banks
+  f16* xs = reinterpret_cast<f16*>(smem);
+  float* red = reinterpret_cast<float*>(smem + (((size_t)M * xstride * 2 + 15) & ~(size_t)15));
+
+  typename Fmt::Scale sc[NACC];
+  const u32x4* wp[NACC];
+#pragma unroll
+  for (int g = 0; g < NACC; ++g) {
+    const GemmMat& m = a.mat[PAIR ? g : mi];
+    sc[g] = Fmt::load_scale(m.scale, row, N);
+    wp[g] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb * KT * (64 * KV) + lane;
+  }
+  // first tile of this wave: requested before anything else
+  u32x4 wcur[NACC][KV];
+  int kt = wave;
+  if (kt < KT) {
+#pragma unroll
+    for (int g = 0; g < NACC; ++g)
+#pragma unroll
+      for (int v = 0; v < KV; ++v) wcur[g][v] = __builtin_nontemporal_load(wp[g] + ((size_t)kt * KV + v) * 64);
+  }
+  // stage X (zero beyond K)
+  {
+    const int vec_per_row = KT * 16;               // 8-half vectors per padded row
+    for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
+      const int m = i / vec_per_row, c = i % vec_per_row;
+      f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (c * 8 < K) v = *reinterpret_cast<const f16x8*>(a.X + (size_t)m * K + c * 8);
+      *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+    }
+  }
+  __syncthreads();
+  int mrow = lane & 15;
+  mrow = mrow < M ? mrow : M - 1;
+  const f16* xl = xs + (size_t)mrow * xstride + (lane >> 4) * 8;
+
+  f32x4 acc[NACC];
+#pragma unroll
+  for (int g = 0; g < NACC; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  while (kt < KT) {
+    const int ktn = kt + NW;
+    u32x4 wnext[NACC][KV];
+    if (ktn < KT) {
+#pragma unroll
+      for (int g = 0; g < NACC; ++g)
+#pragma unroll
+        for (int v = 0; v < KV; ++v) wnext[g][v] = __builtin_nontemporal_load(wp[g] + ((size_t)ktn * KV + v) * 64);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
+#pragma unroll
+      for (int g = 0; g < NACC; ++g) {
+        const f16x8 av = Fmt::a_operand(wcur[g], j, sc[g]);
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb, acc[g], 0, 0, 0);
+      }
+    }
+    if (ktn < KT) {
+#pragma unroll
+      for (int g = 0; g < NACC; ++g)
+#pragma unroll
+        for (int v = 0; v < KV; ++v) wcur[g][v] = wnext[g][v];
+    }
+    kt = ktn;
+  }
+
+#pragma unroll
+  for (int g = 0; g < NACC; ++g)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[((wave * NACC + g) * 4 + r) * 64 + lane] = acc[g][r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 256; idx += NW * 64) {
+    const int nn = idx & 15, m = idx >> 4;
+    const int n = nb * 16 + nn;
+    if (m >= M || n >= N) continue;
+    const int r = nn & 3, ln = (nn >> 2) * 16 + m;
+    float sum[NACC];
+#pragma unroll
+    for (int g = 0; g < NACC; ++g) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) t += red[((w * NACC + g) * 4 + r) * 64 + ln];
+      sum[g] = Fmt::finish(t, sc[g]);
+    }
+    if (PAIR) {
+      const f16 gate = (f16)sum[0];
+      const f16 up = (f16)sum[1];
+      a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
+    } else {
+      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, (f16)sum[0], m, n, N);
+    }
+  }
+}
+
+template <class Fmt, int NW, bool PAIR>
+static void launch_gemv_lds(const GemmArgs& a, int total_nb, hipStream_t s) {
+  const size_t xbytes = (((size_t)a.M * (a.KT * 128 + 8) * 2) + 15) & ~(size_t)15;
+  const size_t smem = xbytes + (size_t)NW * (PAIR ? 2 : 1) * 256 * sizeof(float);
+  hipLaunchKernelGGL((gemv_lds_kernel<Fmt, NW, PAIR>), dim3(total_nb), dim3(NW * 64), smem, s, a);
+}
+
 template <class Fmt, int MT, bool PAIR>
 static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
   // Waves per block: enough to split K finely when there are few channel blocks, fewer when
@@ -206,7 +330,11 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 
 template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
-  if (a.M <= 16) launch_gemv<Fmt, 1, PAIR>(a, total_nb, s);
+  const size_t xbytes = (size_t)a.M * (a.KT * 128 + 8) * 2;
+  if (a.M <= 4 && xbytes <= 40 * 1024) {
+    if (a.KT >= 16 && total_nb <= 1024 && !PAIR) launch_gemv_lds<Fmt, 16, PAIR>(a, total_nb, s);
+    else launch_gemv_lds<Fmt, 8, PAIR>(a, total_nb, s);
+  } else if (a.M <= 16) launch_gemv<Fmt, 1, PAIR>(a, total_nb, s);
   else if (a.M <= 32) launch_gemv<Fmt, 2, PAIR>(a, total_nb, s);
   else launch_gemv<Fmt, 4, PAIR>(a, total_nb, s);
   PTA_CHECK_LAUNCH(name);

@@ -138,16 +138,24 @@ extern "C" int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_
 // One tiled dword -> 8 fp16 weights, each fp16(q * s) with a single rounding (the product of
 // an integer in [-8, 7] held exactly in fp16 and the fp16 scale), which is what the
 // reference's `half(nibble) * scale` computes.
+// (a & mask) | orv in one VALU instruction.  The mask travels in an SGPR and the OR value in a
+// VGPR: a VOP3 encoding on this target takes no literal and at most one scalar operand.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(orv));
+  return r;
+}
+
 __device__ __forceinline__ f16x8 dequant8(uint32_t w, f16x2 s2) {
   const uint32_t MAGIC = 0x64006400u;  // fp16 1024.0 in both halves
   const f16x2 c1032 = {(f16)1032.0f, (f16)1032.0f};
   const f16x2 c16th = {(f16)0.0625f, (f16)0.0625f};
   const f16x2 c72 = {(f16)-72.0f, (f16)-72.0f};
   const uint32_t w8 = w >> 8;
-  f16x2 p0 = bitcast<f16x2>((w & 0x000f000fu) | MAGIC);   // 1024 + u      (features 0,1)
-  f16x2 p1 = bitcast<f16x2>((w & 0x00f000f0u) | MAGIC);   // 1024 + 16 u   (features 2,3)
-  f16x2 p2 = bitcast<f16x2>((w8 & 0x000f000fu) | MAGIC);  // features 4,5
-  f16x2 p3 = bitcast<f16x2>((w8 & 0x00f000f0u) | MAGIC);  // features 6,7
+  f16x2 p0 = bitcast<f16x2>(and_or(w, 0x000f000fu, MAGIC));   // 1024 + u      (features 0,1)
+  f16x2 p1 = bitcast<f16x2>(and_or(w, 0x00f000f0u, MAGIC));   // 1024 + 16 u   (features 2,3)
+  f16x2 p2 = bitcast<f16x2>(and_or(w8, 0x000f000fu, MAGIC));  // features 4,5
+  f16x2 p3 = bitcast<f16x2>(and_or(w8, 0x00f000f0u, MAGIC));  // features 6,7
   p0 = (p0 - c1032) * s2;                                  // exact integer, then one rounding
   p2 = (p2 - c1032) * s2;
   p1 = __builtin_elementwise_fma(p1, c16th, c72) * s2;     // (1024 + 16u)/16 - 72 = u - 8, exact
