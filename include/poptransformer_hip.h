@@ -67,35 +67,48 @@ int pta_int4_to_half(const int8_t* packed, const pta_half* scale, pta_half* out,
 size_t pta_w4_tiled_bytes(int N, int K);
 int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t stream);
 
-/* Epilogue applied to the fp16-rounded product Y0 = fp16(X @ W) of the fused GEMMs.
- * Each step is one fp16 operation, in the order the reference graphs apply them
- * (layers/linear.py:42-46 bias add; models' residual `ops.add`). */
-typedef struct pta_epilogue {
-  const pta_half* bias;     /* [N] or NULL:      Y = Y0 + bias                                  */
-  const pta_half* residual; /* [M, N] or NULL:   Y = Y + residual                               */
-  int act;                  /* PTA_ACT_*: applied after bias, before residual                   */
-} pta_epilogue;
+/* Operations fused around the product Y0 = fp16(X' @ W) of the GEMM entry points.  Each one is
+ * a separate fp16 graph op in the reference and keeps its own fp16 rounding here.
+ * Before: X' = norm(X) over the K features of every row -
+ *   PTA_NORM_RMS:   pta_rmsnorm(X, norm_weight, norm_eps)               (layers/rms_layer_norm.py:26-36)
+ *   PTA_NORM_LAYER: pta_layer_norm_ce(X, norm_weight, norm_bias, eps)   (ops/customized.py:69-102)
+ *   The fused norm needs M <= 4 and K <= 20480 / M; otherwise the call returns PTA_EUNSUPPORTED and the
+ *   caller runs the norm entry point first.
+ * After, in this order: Y = Y0 + bias (layers/linear.py:42-46); Y = act(Y); Y = Y + residual (the
+ * blocks' residual `ops.add`, e.g. models/llama2/model.py:38-46). */
+typedef struct pta_fusion {
+  const pta_half* bias;        /* [N] or NULL                                   */
+  const pta_half* residual;    /* [M, N] or NULL; may alias Y                   */
+  int act;                     /* PTA_ACT_*                                     */
+  int norm;                    /* PTA_NORM_*                                    */
+  const pta_half* norm_weight; /* [K]                                           */
+  const pta_half* norm_bias;   /* [K], PTA_NORM_LAYER only                      */
+  float norm_eps;
+} pta_fusion;
 
+enum { PTA_NORM_NONE = 0, PTA_NORM_RMS = 1, PTA_NORM_LAYER = 2 };
 enum { PTA_ACT_NONE = 0, PTA_ACT_GELU_TANH = 1, PTA_ACT_RELU_SQUARE = 2, PTA_ACT_SIGMOID = 3 };
 
 /* Fused Int4ToHalf(axis=1) + MatMul (utils/param_handler/precision_strategy.py:56-60,74-75):
  * Y[M,N] = fp16( X[M,K] @ W ), W[k,n] = fp16(nibble(k,n) * scale[n]) exactly as
  * pta_int4_to_half(axis=1) would produce, fp32 accumulation, never materialised.
- * `tiled` comes from pta_w4_tile.  1 <= M <= 64.  `epi` may be NULL. */
+ * `tiled` comes from pta_w4_tile.  1 <= M <= 64.  `fuse` may be NULL. */
 int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
-                   int M, int K, int N, const pta_epilogue* epi, pta_stream_t stream);
+                   int M, int K, int N, const pta_fusion* fuse, pta_stream_t stream);
 
 /* Up to 4 weights sharing the same X and K in one launch (q/k/v projections of
- * models/llama2/attention.py:65-67).  host_* arrays have `count` entries. */
+ * models/llama2/attention.py:65-67).  host_* arrays have `count` entries.  Of `fuse` only the
+ * norm fields are used. */
 int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
                          const pta_half* const* host_scale, pta_half* const* host_Y,
-                         const int* host_N, int M, int K, pta_stream_t stream);
+                         const int* host_N, int M, int K, const pta_fusion* fuse, pta_stream_t stream);
 
 /* SwiGLU pair (models/llama2/mlp.py:20-28, models/chatglm2/mlp.py:51-59):
- * Y[M,F] = fp16( fp16(X@Wup) * fp16(swish(fp16(X@Wgate))) ), swish(g) = g*sigmoid(g). */
+ * Y[M,F] = fp16( fp16(X@Wup) * fp16(swish(fp16(X@Wgate))) ), swish(g) = g*sigmoid(g).
+ * Of `fuse` only the norm fields are used. */
 int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
                           const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M,
-                          int K, int F, pta_stream_t stream);
+                          int K, int F, const pta_fusion* fuse, pta_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * FP16 weights (embedding-tied heads, lm_head, GPT-2 linears): ops.matmul of
@@ -107,7 +120,7 @@ size_t pta_f16_tiled_bytes(int N, int K);
 int pta_f16_tile(const pta_half* w, void* tiled, int N, int K, pta_stream_t stream);
 /* Y[M,N] = fp16(X[M,K] @ w^T), fp32 accumulation. 1 <= M <= 64. */
 int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
-                 const pta_epilogue* epi, pta_stream_t stream);
+                 const pta_fusion* fuse, pta_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * Normalisation

@@ -18,8 +18,12 @@ F16, F32 = 0, 1
 ROPE_NONE, ROPE_LLAMA, ROPE_GLM2 = 0, 1, 2
 
 
-class Epilogue(ctypes.Structure):
-    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int)]
+NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
+
+
+class Fusion(ctypes.Structure):
+    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("norm", c_int),
+                ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float)]
 
 
 # name -> (restype, argtypes); the order follows include/poptransformer_hip.h
@@ -29,13 +33,14 @@ SIGNATURES = {
     "pta_int4_to_half": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "pta_w4_tiled_bytes": (c_size_t, [c_int, c_int]),
     "pta_w4_tile": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
-    "pta_w4a16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Epilogue), c_void_p]),
+    "pta_w4a16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Fusion), c_void_p]),
     "pta_w4a16_gemm_multi": (c_int, [c_void_p, c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
-                                     POINTER(c_int), c_int, c_int, c_void_p]),
-    "pta_w4a16_gemm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+                                     POINTER(c_int), c_int, c_int, POINTER(Fusion), c_void_p]),
+    "pta_w4a16_gemm_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                      POINTER(Fusion), c_void_p]),
     "pta_f16_tiled_bytes": (c_size_t, [c_int, c_int]),
     "pta_f16_tile": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
-    "pta_f16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Epilogue), c_void_p]),
+    "pta_f16_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, POINTER(Fusion), c_void_p]),
     "pta_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "pta_layer_norm_ce": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "pta_softmax_ce": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),

@@ -50,7 +50,7 @@ extern "C" int pta_f16_tile(const pta_half* w, void* tiled, int N, int K, pta_st
 }
 
 extern "C" int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
-                            const pta_epilogue* epi, pta_stream_t stream) {
+                            const pta_fusion* fuse, pta_stream_t stream) {
   int rc = check_gemv_common("pta_f16_gemm", X, M, K);
   if (rc) return rc;
   PTA_REQUIRE(tiled && Y, "pta_f16_gemm: null pointer");
@@ -59,7 +59,7 @@ extern "C" int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, i
   GemmArgs a{};
   a.count = 1; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
   a.mat[0] = GemmMat{tiled, nullptr, (f16*)Y, N, 0};
-  rc = make_epilogue(epi, &a.epi, "pta_f16_gemm");
+  rc = make_epilogue(fuse, &a.epi, "pta_f16_gemm");
   if (rc) return rc;
   return dispatch_gemv<FmtF16, false>(a, (N + 15) / 16, (hipStream_t)stream, "pta_f16_gemm");
 }

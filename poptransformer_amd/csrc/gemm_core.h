@@ -11,6 +11,10 @@ struct GemmEpilogue {
   const f16* bias;
   const f16* residual;
   int act;
+  int norm;                 // PTA_NORM_*, applied to the rows of X before the product
+  const f16* norm_weight;
+  const f16* norm_bias;
+  float norm_eps;
 };
 
 __device__ __forceinline__ f16 sigmoid_f16(f16 x) {
@@ -46,11 +50,16 @@ __device__ __forceinline__ f16 apply_epilogue(const GemmEpilogue& e, f16 y, int 
   return y;
 }
 
-static inline int make_epilogue(const pta_epilogue* in, GemmEpilogue* out, const char* name) {
-  out->bias = nullptr; out->residual = nullptr; out->act = PTA_ACT_NONE;
+static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const char* name) {
+  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, PTA_NORM_NONE, nullptr, nullptr, 0.f};
   if (!in) return PTA_OK;
   PTA_REQUIRE(in->act >= PTA_ACT_NONE && in->act <= PTA_ACT_SIGMOID, "%s: unknown activation %d", name, in->act);
+  PTA_REQUIRE(in->norm >= PTA_NORM_NONE && in->norm <= PTA_NORM_LAYER, "%s: unknown norm %d", name, in->norm);
+  PTA_REQUIRE(in->norm == PTA_NORM_NONE || in->norm_weight, "%s: fused norm needs norm_weight", name);
+  PTA_REQUIRE(in->norm != PTA_NORM_LAYER || in->norm_bias, "%s: fused LayerNorm needs norm_bias", name);
   out->bias = (const f16*)in->bias; out->residual = (const f16*)in->residual; out->act = in->act;
+  out->norm = in->norm; out->norm_weight = (const f16*)in->norm_weight; out->norm_bias = (const f16*)in->norm_bias;
+  out->norm_eps = in->norm_eps;
   return PTA_OK;
 }
 
@@ -231,14 +240,58 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 #pragma unroll
       for (int v = 0; v < KV; ++v) wcur[g][v] = __builtin_nontemporal_load(wp[g] + ((size_t)kt * KV + v) * 64);
   }
-  // stage X (zero beyond K)
+  // stage X (zero beyond K), normalising its rows on the way when a norm is fused
   {
     const int vec_per_row = KT * 16;               // 8-half vectors per padded row
+    float ps[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
     for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
       const int m = i / vec_per_row, c = i % vec_per_row;
       f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (c * 8 < K) v = *reinterpret_cast<const f16x8*>(a.X + (size_t)m * K + c * 8);
       *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+      if (a.epi.norm != PTA_NORM_NONE) {
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s1 += f; s2 = __builtin_fmaf(f, f, s2); }
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) if (mm == m) { ps[mm] += s1; pq[mm] += s2; }
+      }
+    }
+    if (a.epi.norm != PTA_NORM_NONE) {
+      // per-row sums over the workgroup: wave shuffle, then LDS (the reduction buffer is free here)
+#pragma unroll
+      for (int mm = 0; mm < 4; ++mm) { ps[mm] = wave_sum(ps[mm]); pq[mm] = wave_sum(pq[mm]); }
+      if (lane == 0) {
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) { red[(wave * 4 + mm) * 2] = ps[mm]; red[(wave * 4 + mm) * 2 + 1] = pq[mm]; }
+      }
+      __syncthreads();
+      const float inv_n = 1.0f / (float)K;
+      for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
+        const int m = i / vec_per_row, c = i % vec_per_row;
+        if (c * 8 >= K) continue;
+        float sum = 0.f, sq = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) { sum += red[(w * 4 + m) * 2]; sq += red[(w * 4 + m) * 2 + 1]; }
+        f16x8 v = *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8);
+        const f16x8 gm = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
+        if (a.epi.norm == PTA_NORM_RMS) {
+          const f16 r16 = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = (v[e] * r16) * gm[e];
+        } else {
+          const f16x8 bt = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
+          const float mean = sum * inv_n;
+          const f16 mean16 = (f16)mean;
+          float var;
+          if (M == 1) var = sq * inv_n - mean * mean + a.epi.norm_eps;          // single-row NormCE
+          else { const float mf = (float)mean16; var = fmaxf(sq * inv_n - mf * mf, 0.0f) + a.epi.norm_eps; }
+          const f16 r16 = (f16)(1.0f / sqrtf(var));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = ((v[e] - mean16) * r16) * gm[e] + bt[e];
+        }
+        *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+      }
     }
   }
   __syncthreads();
@@ -331,6 +384,10 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   const size_t xbytes = (size_t)a.M * (a.KT * 128 + 8) * 2;
+  if (a.epi.norm != PTA_NORM_NONE && !(a.M <= 4 && xbytes <= 40 * 1024)) {
+    pta_set_error("%s: the fused norm needs M <= 4 and M*K <= 20480 (got M=%d K=%d)", name, a.M, a.K);
+    return PTA_EUNSUPPORTED;
+  }
   if (a.M <= 4 && xbytes <= 40 * 1024) {
     if (a.KT >= 16 && total_nb <= 1024 && !PAIR) launch_gemv_lds<Fmt, 16, PAIR>(a, total_nb, s);
     else launch_gemv_lds<Fmt, 8, PAIR>(a, total_nb, s);

@@ -182,7 +182,7 @@ struct FmtW4 {
 
 extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
                                     const pta_half* const* host_scale, pta_half* const* host_Y,
-                                    const int* host_N, int M, int K, pta_stream_t stream) {
+                                    const int* host_N, int M, int K, const pta_fusion* fuse, pta_stream_t stream) {
   int rc = check_gemv_common("pta_w4a16_gemm_multi", X, M, K);
   if (rc) return rc;
   PTA_REQUIRE(count >= 1 && count <= 4, "pta_w4a16_gemm_multi: count must be in [1, 4], got %d", count);
@@ -196,11 +196,14 @@ extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* co
     a.mat[i] = GemmMat{(const void*)host_tiled[i], (const void*)host_scale[i], (f16*)host_Y[i], host_N[i], nb};
     nb += (host_N[i] + 15) / 16;
   }
+  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm_multi");
+  if (rc) return rc;
+  PTA_REQUIRE(!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE, "pta_w4a16_gemm_multi: only the norm fields of `fuse` are supported");
   return dispatch_gemv<FmtW4, false>(a, nb, (hipStream_t)stream, "pta_w4a16_gemm_multi");
 }
 
 extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
-                              int M, int K, int N, const pta_epilogue* epi, pta_stream_t stream) {
+                              int M, int K, int N, const pta_fusion* fuse, pta_stream_t stream) {
   int rc = check_gemv_common("pta_w4a16_gemm", X, M, K);
   if (rc) return rc;
   PTA_REQUIRE(tiled && scale && Y, "pta_w4a16_gemm: null pointer");
@@ -209,14 +212,14 @@ extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_ha
   GemmArgs a{};
   a.count = 1; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
   a.mat[0] = GemmMat{(const void*)tiled, (const void*)scale, (f16*)Y, N, 0};
-  rc = make_epilogue(epi, &a.epi, "pta_w4a16_gemm");
+  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm");
   if (rc) return rc;
   return dispatch_gemv<FmtW4, false>(a, (N + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm");
 }
 
 extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
                                      const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M,
-                                     int K, int F, pta_stream_t stream) {
+                                     int K, int F, const pta_fusion* fuse, pta_stream_t stream) {
   int rc = check_gemv_common("pta_w4a16_gemm_swiglu", X, M, K);
   if (rc) return rc;
   PTA_REQUIRE(tiled_gate && scale_gate && tiled_up && scale_up && Y, "pta_w4a16_gemm_swiglu: null pointer");
@@ -226,5 +229,8 @@ extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, 
   a.count = 2; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
   a.mat[0] = GemmMat{(const void*)tiled_gate, (const void*)scale_gate, (f16*)Y, F, 0};
   a.mat[1] = GemmMat{(const void*)tiled_up, (const void*)scale_up, (f16*)Y, F, 0};
+  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm_swiglu");
+  if (rc) return rc;
+  PTA_REQUIRE(!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE, "pta_w4a16_gemm_swiglu: only the norm fields of `fuse` are supported");
   return dispatch_gemv<FmtW4, true>(a, (F + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm_swiglu");
 }

@@ -9,7 +9,7 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import Epilogue, check
+from ._lib import Fusion, check
 
 _i32 = torch.int32
 
@@ -33,10 +33,27 @@ def _need(t, dtype, name, dims=None):
         raise ValueError(f"The rank of {name} should be {dims}. But now it is {t.dim()}.")
 
 
-def _epilogue(bias, residual, act):
-    if bias is None and residual is None and act == _lib.ACT_NONE:
+class Norm:
+    """A row normalisation to fuse in front of a GEMM: RMSNorm (bias None) or NormCE LayerNorm."""
+
+    def __init__(self, weight, bias, eps):
+        self.weight, self.bias, self.eps = weight, bias, float(eps)
+
+    @property
+    def kind(self):
+        return _lib.NORM_RMS if self.bias is None else _lib.NORM_LAYER
+
+
+def norm_fusable(M, K):
+    """Whether the GEMM entry points can apply a fused norm for this shape."""
+    return M <= 4 and M * (((K + 127) // 128) * 128 + 8) * 2 <= 40 * 1024
+
+
+def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None):
+    if bias is None and residual is None and act == _lib.ACT_NONE and norm is None:
         return None
-    e = Epilogue(_p(bias) if bias is not None else None, _p(residual) if residual is not None else None, act)
+    e = Fusion(_p(bias), _p(residual), act, norm.kind if norm else _lib.NORM_NONE,
+               _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0)
     return ctypes.byref(e)
 
 
@@ -77,7 +94,7 @@ class W4Weight:
         return self.N * self.K // 2 + self.N * 2
 
 
-def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None):
+def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm=None):
     _need(x, torch.float16, "x", 2)
     M, K = x.shape
     if K != w.K:
@@ -85,11 +102,11 @@ def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None):
     if out is None:
         out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
     check(_lib.load().pta_w4a16_gemm(_p(x), _p(w.tiled), _p(w.scale), _p(out), M, K, w.N,
-                                     _epilogue(bias, residual, act), _stream()))
+                                     _fusion(bias, residual, act, norm), _stream()))
     return out
 
 
-def w4a16_gemm_multi(x, weights, outs=None):
+def w4a16_gemm_multi(x, weights, outs=None, norm=None):
     _need(x, torch.float16, "x", 2)
     M, K = x.shape
     n = len(weights)
@@ -103,11 +120,11 @@ def w4a16_gemm_multi(x, weights, outs=None):
     scale = VP(*[w.scale.data_ptr() for w in weights])
     ys = VP(*[o.data_ptr() for o in outs])
     ns = (ctypes.c_int * n)(*[w.N for w in weights])
-    check(_lib.load().pta_w4a16_gemm_multi(_p(x), n, tiled, scale, ys, ns, M, K, _stream()))
+    check(_lib.load().pta_w4a16_gemm_multi(_p(x), n, tiled, scale, ys, ns, M, K, _fusion(norm=norm), _stream()))
     return outs
 
 
-def w4a16_gemm_swiglu(x, w_gate, w_up, out=None):
+def w4a16_gemm_swiglu(x, w_gate, w_up, out=None, norm=None):
     _need(x, torch.float16, "x", 2)
     M, K = x.shape
     if w_gate.K != K or w_up.K != K or w_gate.N != w_up.N:
@@ -115,7 +132,7 @@ def w4a16_gemm_swiglu(x, w_gate, w_up, out=None):
     if out is None:
         out = torch.empty((M, w_gate.N), dtype=torch.float16, device=x.device)
     check(_lib.load().pta_w4a16_gemm_swiglu(_p(x), _p(w_gate.tiled), _p(w_gate.scale), _p(w_up.tiled),
-                                            _p(w_up.scale), _p(out), M, K, w_gate.N, _stream()))
+                                            _p(w_up.scale), _p(out), M, K, w_gate.N, _fusion(norm=norm), _stream()))
     return out
 
 
@@ -135,14 +152,14 @@ class F16Weight:
         return self.N * self.K * 2
 
 
-def f16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None):
+def f16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm=None):
     _need(x, torch.float16, "x", 2)
     M, K = x.shape
     if K != w.K:
         raise ValueError(f"matmul: contracting dimensions differ ({K} vs {w.K})")
     if out is None:
         out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
-    check(_lib.load().pta_f16_gemm(_p(x), _p(w.tiled), _p(out), M, K, w.N, _epilogue(bias, residual, act), _stream()))
+    check(_lib.load().pta_f16_gemm(_p(x), _p(w.tiled), _p(out), M, K, w.N, _fusion(bias, residual, act, norm), _stream()))
     return out
 
 

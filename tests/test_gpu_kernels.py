@@ -133,6 +133,29 @@ def test_w4a16_gemm_multi_and_swiglu(K):
     assert rel_err(got, ref) <= 1e-2
 
 
+@pytest.mark.parametrize("M", [1, 3])
+def test_gemm_fused_norms(K, M):
+    """RMSNorm / NormCE applied inside the GEMM must equal the norm entry point followed by the GEMM."""
+    x, packed, scale = _w4_case(21, M, 768, 96)
+    rng = np.random.default_rng(22)
+    g = rng.uniform(0.5, 1.5, 768).astype(np.float16)
+    b = rng.standard_normal(768).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    xd, gd, bd = dev(x), dev(g), dev(b)
+    two = host(K.w4a16_gemm(K.rmsnorm(xd, gd, 1e-5), w))
+    one = host(K.w4a16_gemm(xd, w, norm=K.Norm(gd, None, 1e-5)))
+    assert rel_err(one, two) <= 2e-3
+    assert rel_err(one, O.w4a16_matmul(O.rms_norm(x, g, 1e-5), packed, scale)) <= 1e-2
+    w16 = (rng.standard_normal((64, 768)) * 0.05).astype(np.float16)
+    fw = K.F16Weight(dev(w16))
+    two = host(K.f16_gemm(K.layer_norm_ce(xd, gd, bd, 1e-5), fw))
+    one = host(K.f16_gemm(xd, fw, norm=K.Norm(gd, bd, 1e-5)))
+    assert rel_err(one, two) <= 2e-3
+    assert rel_err(one, O.matmul(O.layer_norm_ce(x, g, b, 1e-5, M, 1, 768), w16.T)) <= 1e-2
+    with pytest.raises(NotImplementedError):
+        K.w4a16_gemm(dev(np.zeros((16, 768), np.float16)), w, norm=K.Norm(gd, None, 1e-5))
+
+
 def test_w4a16_guards(K):
     x, packed, scale = _w4_case(1, 1, 128, 16)
     w = K.W4Weight(dev(packed), dev(scale))
