@@ -230,6 +230,34 @@ int pta_step_update(int32_t* container, pta_half* mask, int32_t* stop_mask, int3
                     int32_t* ids_out, int32_t* keep_going, int B, int max_len, int pad_id, int eos_id,
                     int early_stop, pta_stream_t stream);
 
+/* ------------------------------------------------------------------------------------
+ * FP8 (Graphcore F143 / F152 bytes, value = decode(byte) * 2^scale).  Scales are device int32
+ * tensors of which element 0 is read, as in custom_ops/matmul_fp8.cpp:890-891.
+ * ---------------------------------------------------------------------------------- */
+enum { PTA_F143 = 0, PTA_F152 = 1 };
+
+/* CastToUint8 (ops/customized.py:127-135; custom_ops/cast_to_uint8.cpp:107-127): fp16 -> byte,
+ * round to nearest even, saturating, NaN -> 0x80.  out has the shape of x (n elements). */
+int pta_half_to_fp8(const pta_half* x, uint8_t* out, const int32_t* scale, size_t n, int format,
+                    pta_stream_t stream);
+/* The cast back (custom_ops/matmul_fp8.cpp:925-930, custom_ops/kv_cache.cpp:56-74). */
+int pta_fp8_to_half(const uint8_t* in, pta_half* out, const int32_t* scale, size_t n, int format,
+                    pta_stream_t stream);
+
+/* Re-tiling of an FP8 weight.  `w` is uint8 [N, K] (w_is_kn == 0, state-dict orientation) or
+ * [K, N] (w_is_kn != 0, the orientation the reference graph holds after layers/linear.py:32). */
+size_t pta_fp8_tiled_bytes(int N, int K);
+int pta_fp8_tile(const uint8_t* w, void* tiled, int N, int K, int w_is_kn, pta_stream_t stream);
+
+/* FP8MatMul (ops/customized.py:137-148; custom_ops/matmul_fp8.cpp:177-250, 885-1003).
+ * lhs is fp16 [M, K] (lhs_is_fp8 == 0: the weight is cast to fp16, then an fp16 MatMul) or uint8
+ * [M, K] (both operands FP8).  Y fp16 [M, N], fp32 accumulation.  1 <= M <= 64.
+ * workspace: pta_fp8_gemm_workspace_bytes(M, K) bytes, 16-byte aligned.  `fuse` may be NULL. */
+size_t pta_fp8_gemm_workspace_bytes(int M, int K);
+int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_rhs, pta_half* Y, int M, int K, int N,
+                 int format_lhs, int format_rhs, const int32_t* scale_lhs, const int32_t* scale_rhs,
+                 void* workspace, const pta_fusion* fuse, pta_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -407,3 +407,86 @@ def attention_scores_to_context(q, k_t, v, mask, scale, softmax_dtype, stable_mo
     else:
         w = softmax_ce(w, -1, stable_mode)
     return matmul(w, v)
+
+
+# --------------------------------------------------------------------------------------
+# A4/A5/A6  FP8 (Graphcore F143 / F152).  PARITY UNPINNED: the encode/decode routines live in
+# poprt (`convert_float_to_uint8`, requirements.txt:7) and in the Poplar SDK (`popops::cast` to
+# QUARTER), neither of which is part of the reference tree.  The formats implemented here are
+# the published ones ("8-bit Numerical Formats for Deep Neural Networks", Graphcore 2022):
+#   F143: 1 sign, 4 exponent, 3 mantissa bits, bias 8, subnormals, no infinities, NaN = 0x80,
+#         largest magnitude 240;  F152: 1-5-2, bias 16, NaN = 0x80, largest magnitude 57344
+# (the `float8_e4m3fnuz` / `float8_e5m2fnuz` encodings).  A QuarterMetadata scale s means
+# real value = decode(byte) * 2**s.  Encoding rounds to nearest even and saturates.
+# --------------------------------------------------------------------------------------
+_F8 = {"F143": (4, 3, 8), "F152": (5, 2, 16)}
+
+
+def f8_table(fmt):
+    """All 256 decoded values of a format as float32 (NaN at 0x80)."""
+    if fmt not in _F8:
+        raise ValueError(f"Unsupport fp8 meata data {fmt}, it must be F143 or F152")
+    eb, mb, bias = _F8[fmt]
+    out = np.zeros(256, np.float64)
+    for code in range(256):
+        s = -1.0 if code & 0x80 else 1.0
+        e = (code >> mb) & ((1 << eb) - 1)
+        m = code & ((1 << mb) - 1)
+        if code == 0x80:
+            out[code] = np.nan
+        elif e == 0:
+            out[code] = s * 2.0 ** (1 - bias) * (m / (1 << mb))
+        else:
+            out[code] = s * 2.0 ** (e - bias) * (1 + m / (1 << mb))
+    return out.astype(f32)
+
+
+def f8_decode(codes, fmt="F143", scale=0, dtype=f16):
+    """popops::cast QUARTER -> HALF with QuarterMetadata(fmt, scale)
+    (custom_ops/matmul_fp8.cpp:904-930, custom_ops/kv_cache.cpp:56-74)."""
+    t = f8_table(fmt).astype(np.float64) * 2.0 ** int(scale)
+    with np.errstate(over="ignore"):
+        return t[np.asarray(codes, np.uint8)].astype(dtype)
+
+
+def f8_encode(x, fmt="F143", scale=0):
+    """CastToUint8 (poptransformer/ops/customized.py:127-135, custom_ops/cast_to_uint8.cpp:107-127)
+    and the host-side `convert_float_to_uint8(w, fmt, scale)` of
+    utils/param_handler/precision_strategy.py:44-51: byte whose decoded value * 2**scale is
+    nearest to x (ties to the even mantissa), saturating at the largest magnitude; NaN -> 0x80."""
+    if fmt not in _F8:
+        raise ValueError(f"Unsupport fp8 meata data {fmt}, it must be F143 or F152")
+    x = np.asarray(x)
+    v = x.astype(np.float64) * 2.0 ** (-int(scale))
+    pos = f8_table(fmt)[:128].astype(np.float64)            # codes 0x00..0x7F ascend with the value
+    mag = np.abs(v)
+    hi = np.searchsorted(pos, mag, side="left").clip(1, 127)
+    lo = hi - 1
+    d_lo, d_hi = mag - pos[lo], pos[hi] - mag
+    pick_hi = (d_hi < d_lo) | ((d_hi == d_lo) & (hi % 2 == 0))
+    code = np.where(pick_hi, hi, lo)
+    code = np.where(mag >= pos[127], 127, code)              # saturate
+    code = np.where(mag <= 0, 0, code).astype(np.uint8)
+    out = np.where((v < 0) & (code != 0), code | 0x80, code).astype(np.uint8)   # no negative zero
+    return np.where(np.isnan(v), np.uint8(0x80), out).astype(np.uint8)
+
+
+def fp8_matmul(lhs, rhs, scale_lhs, scale_rhs, fmt_lhs="F143", fmt_rhs="F143"):
+    """FP8MatMul (poptransformer/ops/customized.py:137-148; custom_ops/matmul_fp8.cpp:177-250, 885-1003).
+    rhs must be uint8; lhs is uint8 (both operands QUARTER, fp32 partials, HALF output) or
+    float16 (rhs cast to HALF first, then an fp16 MatMul).  Scales are int32 tensors of which
+    element 0 is read (:890-891)."""
+    lhs, rhs = np.asarray(lhs), np.asarray(rhs)
+    if lhs.dtype not in (f16, np.uint8):
+        raise ValueError(f"Invalid input data type of {lhs.dtype}, it must be FLOAT16 or UINT8")
+    if rhs.dtype != np.uint8:
+        raise ValueError(f"Invalid weight data type of {rhs.dtype}, it must be UINT8")
+    sl, sr = int(np.asarray(scale_lhs).reshape(-1)[0]), int(np.asarray(scale_rhs).reshape(-1)[0])
+    if lhs.shape[-1] != rhs.shape[-2]:
+        raise ValueError("contracting dimensions differ")
+    if lhs.dtype == np.uint8:
+        a = f8_decode(lhs, fmt_lhs, sl, np.float64)
+        b = f8_decode(rhs, fmt_rhs, sr, np.float64)
+        with np.errstate(over="ignore"):
+            return np.matmul(a, b).astype(f32).astype(f16)
+    return matmul(lhs, f8_decode(rhs, fmt_rhs, sr, f16))

@@ -16,6 +16,8 @@ PTA_OK, PTA_EINVAL, PTA_EUNSUPPORTED, PTA_EHIP = 0, -1, -2, -3
 ACT_NONE, ACT_GELU_TANH, ACT_RELU_SQUARE, ACT_SIGMOID = 0, 1, 2, 3
 F16, F32 = 0, 1
 ROPE_NONE, ROPE_LLAMA, ROPE_GLM2 = 0, 1, 2
+F143, F152 = 0, 1
+FP8_FORMATS = {"F143": F143, "F152": F152}
 
 
 NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
@@ -54,6 +56,13 @@ SIGNATURES = {
                                      c_int, c_int, c_void_p]),
     "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "pta_embedding": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_half_to_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "pta_fp8_to_half": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "pta_fp8_tiled_bytes": (c_size_t, [c_int, c_int]),
+    "pta_fp8_tile": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_fp8_gemm_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "pta_fp8_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+                             c_void_p, POINTER(Fusion), c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
 }

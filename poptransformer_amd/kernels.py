@@ -163,6 +163,75 @@ def f16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm=N
     return out
 
 
+# ------------------------------------------------------------------ FP8 ------------------
+def _fmt(name):
+    if name not in _lib.FP8_FORMATS:
+        raise ValueError(f"Unsupport fp8 meata data {name}, it must be F143 or F152")
+    return _lib.FP8_FORMATS[name]
+
+
+def half_to_fp8(x, scale, fp8_format="F143"):
+    """ops.half_to_uint8 (reference: poptransformer/ops/customized.py:127-135)."""
+    fmt = _fmt(fp8_format)
+    _need(x, torch.float16, "x")
+    _need(scale, _i32, "fp8_scale")
+    out = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    check(_lib.load().pta_half_to_fp8(_p(x), _p(out), _p(scale), x.numel(), fmt, _stream()))
+    return out
+
+
+def fp8_to_half(codes, scale, fp8_format="F143"):
+    fmt = _fmt(fp8_format)
+    _need(codes, torch.uint8, "codes")
+    _need(scale, _i32, "fp8_scale")
+    out = torch.empty(codes.shape, dtype=torch.float16, device=codes.device)
+    check(_lib.load().pta_fp8_to_half(_p(codes), _p(out), _p(scale), codes.numel(), fmt, _stream()))
+    return out
+
+
+class F8Weight:
+    """An FP8 Linear weight re-tiled for the fused kernel.  `w` is uint8 [N, K], or [K, N] with
+    kn=True (the orientation the reference graph holds)."""
+
+    def __init__(self, w, scale, fp8_format="F143", kn=False):
+        _need(w, torch.uint8, "weight", 2)
+        _need(scale, _i32, "weight scale")
+        self.format = _fmt(fp8_format)
+        self.N, self.K = (w.shape[1], w.shape[0]) if kn else w.shape
+        self.scale = scale
+        lib = _lib.load()
+        self.tiled = torch.empty(lib.pta_fp8_tiled_bytes(self.N, self.K), dtype=torch.uint8, device=w.device)
+        check(lib.pta_fp8_tile(_p(w), _p(self.tiled), self.N, self.K, 1 if kn else 0, _stream()))
+
+    @property
+    def nbytes(self):
+        return self.N * self.K
+
+
+def fp8_gemm_workspace(M, K, device):
+    return torch.empty(_lib.load().pta_fp8_gemm_workspace_bytes(M, K), dtype=torch.uint8, device=device)
+
+
+def fp8_gemm(x, w, workspace, x_scale=None, x_format="F143", bias=None, residual=None, act=_lib.ACT_NONE, out=None,
+             norm=None):
+    """ops.fp8_matmul (reference: poptransformer/ops/customized.py:137-148): x fp16 or uint8 [M, K]."""
+    if x.dtype not in (torch.float16, torch.uint8):
+        raise ValueError(f"Invalid input data type of {x.dtype}, it must be FLOAT16 or UINT8")
+    _need(x, x.dtype, "x", 2)
+    M, K = x.shape
+    if K != w.K:
+        raise ValueError(f"matmul: contracting dimensions differ ({K} vs {w.K})")
+    is8 = x.dtype == torch.uint8
+    if is8 and x_scale is None:
+        raise ValueError("an fp8 left-hand side needs its scale")
+    if out is None:
+        out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
+    check(_lib.load().pta_fp8_gemm(_p(x), 1 if is8 else 0, _p(w.tiled), _p(out), M, K, w.N, _fmt(x_format) if is8 else 0,
+                                   w.format, _p(x_scale), _p(w.scale), _p(workspace),
+                                   _fusion(bias, residual, act, norm), _stream()))
+    return out
+
+
 # ------------------------------------------------------------------ norms ----------------
 def rmsnorm(x, weight, eps, out=None):
     _need(x, torch.float16, "x")

@@ -189,6 +189,69 @@ def test_f16_gemm_gelu_bias(K):
     assert rel_err(got, ref) <= 1e-2
 
 
+# ---------------------------------------------------------------- FP8 (bit-exact codecs)
+@pytest.mark.parametrize("fmt", ["F143", "F152"])
+@pytest.mark.parametrize("scale", [0, -1, 3])
+def test_fp8_codecs_bit_exact(K, fmt, scale):
+    codes = np.arange(256, dtype=np.uint8)
+    s = dev(np.array([scale], np.int32))
+    got = host(K.fp8_to_half(dev(codes), s, fmt))
+    ref = O.f8_decode(codes, fmt, scale, np.float16)
+    ok = codes != 0x80
+    assert np.array_equal(got[ok].view(np.uint16), ref[ok].view(np.uint16)) and np.isnan(got[0x80])
+    rng = np.random.default_rng(31)
+    mx = 240.0 if fmt == "F143" else 57344.0
+    x = np.concatenate([rng.standard_normal(20000) * 0.05, rng.uniform(-mx, mx, 20000) * 2.0 ** scale,
+                        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504, -65504, 6e-8, -6e-8])]).astype(np.float16)
+    # every fp16 value near the grid boundaries: all midpoints between adjacent codes
+    tab = O.f8_table(fmt)[:128].astype(np.float64) * 2.0 ** scale
+    mids = ((tab[:-1] + tab[1:]) / 2)
+    x = np.concatenate([x, mids.astype(np.float16), -mids.astype(np.float16), np.nextafter(mids.astype(np.float16), np.float16(np.inf))])
+    got = host(K.half_to_fp8(dev(x), s, fmt))
+    ref = O.f8_encode(x, fmt, scale)
+    assert np.array_equal(got, ref)
+    with pytest.raises(ValueError):
+        K.half_to_fp8(dev(x), s, "F999")
+
+
+@pytest.mark.parametrize("M,Kdim,N", [(1, 4096, 512), (8, 512, 4096), (3, 136, 40), (64, 1024, 64)])
+@pytest.mark.parametrize("fmt", ["F143", "F152"])
+def test_fp8_gemm_both_modes(K, M, Kdim, N, fmt):
+    rng = np.random.default_rng(M + Kdim + N)
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    w = (rng.standard_normal((Kdim, N)) * 0.02).astype(np.float32)          # [K, N] as the graph holds it
+    scale = -1
+    w8 = O.f8_encode(w, fmt, scale)
+    w8[0, 0] = 0x7F if fmt == "F143" else 0x5F                              # the saturation code (+max) / a large finite code
+    w8[1, 0] = 0x01                                                          # the smallest subnormal
+    sd = dev(np.array([scale], np.int32))
+    fw = K.F8Weight(dev(w8), sd, fmt, kn=True)
+    ws = K.fp8_gemm_workspace(M, Kdim, "cuda")
+    got16 = host(K.fp8_gemm(dev(x), fw, ws))
+    ref16 = O.fp8_matmul(x, w8, [scale], [scale], fmt, fmt)
+    assert rel_err(got16, ref16) <= 1e-2
+    x8 = O.f8_encode(x, "F143", scale)
+    got8 = host(K.fp8_gemm(dev(x8), fw, ws, x_scale=sd, x_format="F143"))
+    ref8 = O.fp8_matmul(x8, w8, [scale], [scale], "F143", fmt)
+    assert rel_err(got8, ref8) <= 1e-2
+    # same weights given in [N, K] orientation tile identically
+    fw2 = K.F8Weight(dev(np.ascontiguousarray(w8.T)), sd, fmt, kn=False)
+    assert torch.equal(fw.tiled, fw2.tiled)
+
+
+def test_fp8_gemm_exact_on_representable_values(K):
+    """Small integers and powers of two are exact in F143, in fp16 and in the fp32 sums."""
+    rng = np.random.default_rng(32)
+    M, Kdim, N = 4, 256, 32
+    x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
+    w = rng.choice([-4.0, -1.5, -0.25, 0.0, 0.5, 1.0, 3.0], size=(N, Kdim)).astype(np.float32)
+    w8 = O.f8_encode(w, "F143", 0)
+    assert np.array_equal(O.f8_decode(w8, "F143", 0, np.float32), w)
+    s0 = dev(np.array([0], np.int32))
+    got = host(K.fp8_gemm(dev(x), K.F8Weight(dev(w8), s0, "F143"), K.fp8_gemm_workspace(M, Kdim, "cuda")))
+    assert np.array_equal(got.astype(np.float64), x.astype(np.float64) @ w.T.astype(np.float64))
+
+
 # ---------------------------------------------------------------- norms
 @pytest.mark.parametrize("rows,cols", [(1, 4096), (16, 4096), (3, 768), (2, 8)])
 def test_rmsnorm(K, rows, cols):

@@ -338,3 +338,51 @@ def test_activations():
     x = np.linspace(-6, 6, 101).astype(f16)
     assert np.abs(O.gelu(x).astype(f32) - torch.nn.functional.gelu(torch.from_numpy(x.astype(f32)), approximate="tanh").numpy()).max() < 3e-3
     assert np.abs(O.swish(x).astype(f32) - torch.nn.functional.silu(torch.from_numpy(x.astype(f32))).numpy()).max() < 3e-3
+
+
+# ---------------------------------------------------------------- FP8 (format assumption, see oracle/ops.py)
+@pytest.mark.parametrize("fmt,tdt", [("F143", torch.float8_e4m3fnuz), ("F152", torch.float8_e5m2fnuz)])
+def test_f8_tables_match_fnuz_formats(fmt, tdt):
+    codes = torch.arange(256, dtype=torch.uint8)
+    ref = codes.view(tdt).to(torch.float32).numpy()
+    tab = O.f8_table(fmt)
+    assert np.isnan(tab[0x80]) and np.isnan(ref[0x80])
+    ok = np.arange(256) != 0x80
+    assert np.array_equal(tab[ok], ref[ok])
+    assert np.nanmax(tab) == (240.0 if fmt == "F143" else 57344.0)
+
+
+@pytest.mark.parametrize("fmt,tdt", [("F143", torch.float8_e4m3fnuz), ("F152", torch.float8_e5m2fnuz)])
+def test_f8_encode_matches_fnuz_cast_and_roundtrips(fmt, tdt):
+    rng = np.random.default_rng(12)
+    mx = 240.0 if fmt == "F143" else 57344.0
+    x = np.concatenate([rng.standard_normal(4000) * 0.05, rng.uniform(-mx, mx, 4000), [0.0, -0.0, mx, -mx]]).astype(f16)
+    got = O.f8_encode(x, fmt, 0)
+    ref = torch.from_numpy(x.astype(f32)).to(tdt).view(torch.uint8).numpy()
+    assert np.array_equal(got, ref)
+    # every representable value encodes to its own code; values beyond the range saturate
+    codes = np.array([c for c in range(256) if c not in (0x80,)], np.uint8)
+    assert np.array_equal(O.f8_encode(O.f8_decode(codes, fmt, 0, np.float32), fmt, 0), codes)
+    assert O.f8_encode(np.array([1e9, -1e9], f32), fmt, 0).tolist() == [0x7F, 0xFF]
+    # scale: encode(x, s) stores x * 2^-s
+    assert np.array_equal(O.f8_encode(x, fmt, -1), O.f8_encode((x.astype(f32) * 2), fmt, 0))
+
+
+def test_fp8_matmul_modes():
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((3, 32)).astype(f16)
+    w = (rng.standard_normal((32, 8)) * 0.05).astype(f32)
+    w8 = O.f8_encode(w, "F143", -1)
+    s = np.array([-1], np.int32)
+    wd = O.f8_decode(w8, "F143", -1, np.float64)
+    assert np.abs(wd - w).max() <= 2.0 ** -11 + np.abs(w).max() * 2.0 ** -4   # 3 mantissa bits
+    y16 = O.fp8_matmul(x, w8, s, s)
+    assert np.abs(y16.astype(np.float64) - x.astype(np.float64) @ wd).max() <= 2e-3
+    x8 = O.f8_encode(x, "F143", -1)
+    y8 = O.fp8_matmul(x8, w8, s, s)
+    xd = O.f8_decode(x8, "F143", -1, np.float64)
+    assert np.abs(y8.astype(np.float64) - xd @ wd).max() <= 2e-3
+    with pytest.raises(ValueError):
+        O.fp8_matmul(x.astype(f32), w8, s, s)
+    with pytest.raises(ValueError):
+        O.f8_encode(x, "F999", 0)
