@@ -258,6 +258,33 @@ int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_rhs, pta_hal
                  int format_lhs, int format_rhs, const int32_t* scale_lhs, const int32_t* scale_rhs,
                  void* workspace, const pta_fusion* fuse, pta_stream_t stream);
 
+/* fp16 values on the FP8 grid: out = decode(encode(x * 2^-scale)) WITHOUT the scale, i.e. what an
+ * FP8 operand contributes to a product before the power of two is applied.  Lets
+ * half_to_uint8 + fp8_matmul (precision_strategy.py:62-66,77-81) run as one rounding pass plus
+ * pta_linear with x_scale. */
+int pta_half_to_fp8_grid(const pta_half* x, pta_half* out, const int32_t* scale, size_t n, int format,
+                         pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Linear layers, general form (layers/linear.py:19-46 + precision_strategy.py:56-81)
+ * ---------------------------------------------------------------------------------- */
+enum { PTA_W_INT4 = 0, PTA_W_F16 = 1, PTA_W_F143 = 2, PTA_W_F152 = 3 };
+
+typedef struct pta_weight {
+  int kind;            /* PTA_W_*                                                              */
+  const void* tiled;   /* from pta_w4_tile / pta_f16_tile / pta_fp8_tile                      */
+  const void* scale;   /* INT4: fp16 [N]; FP8: device int32 exponent; FP16: NULL              */
+  int N, K;
+} pta_weight;
+
+/* Y_i[M, N_i] = fp16(X' @ W_i) + bias_i for `count` (1..4) weights of one kind and one K in one
+ * launch; with swiglu != 0 (count == 2: gate, up) Y_0 = fp16(up * swish(gate)).  x_scale (FP8
+ * weights only, may be NULL): X holds unscaled FP8-grid values whose device int32 exponent it is.
+ * host_bias may be NULL.  With count == 1 all of `fuse` applies, otherwise its norm fields. */
+int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_weight* host_w,
+               const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
+               const pta_fusion* fuse, pta_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

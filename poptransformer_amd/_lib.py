@@ -23,6 +23,13 @@ FP8_FORMATS = {"F143": F143, "F152": F152}
 NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
 
 
+class Weight(ctypes.Structure):
+    _fields_ = [("kind", c_int), ("tiled", c_void_p), ("scale", c_void_p), ("N", c_int), ("K", c_int)]
+
+
+W_INT4, W_F16, W_F143, W_F152 = 0, 1, 2, 3
+
+
 class Fusion(ctypes.Structure):
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("norm", c_int),
                 ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float)]
@@ -63,6 +70,9 @@ SIGNATURES = {
     "pta_fp8_gemm_workspace_bytes": (c_size_t, [c_int, c_int]),
     "pta_fp8_gemm": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                              c_void_p, POINTER(Fusion), c_void_p]),
+    "pta_half_to_fp8_grid": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
+    "pta_linear": (c_int, [c_void_p, c_void_p, c_int, POINTER(Weight), POINTER(c_void_p), POINTER(c_void_p), c_int, c_int,
+                           POINTER(Fusion), c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
 }

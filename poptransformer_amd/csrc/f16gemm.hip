@@ -3,20 +3,7 @@
 // and every Linear of an fp16 model (layers/linear.py:42-46).  fp16 in, fp32 accumulate
 // (the reference's default partials type), fp16 out.
 #include "common.h"
-#include "gemm_core.h"
-
-// Tile = 16 output channels x 128 input features = 4 vectors of 1 KiB; in vector j lane l holds
-// the 8 consecutive features  kt*128 + j*32 + (l/16)*8 + 0..7  of channel l%16, which is the
-// A operand of one 16x16x32 MFMA as it stands.
-struct FmtF16 {
-  static constexpr int kVec = 4;
-  struct Scale {};
-  static __device__ __forceinline__ Scale load_scale(const void*, int, int) { return Scale{}; }
-  static __device__ __forceinline__ f16x8 a_operand(const u32x4 (&raw)[4], int j, Scale) {
-    return bitcast<f16x8>(raw[j]);
-  }
-  static __device__ __forceinline__ float finish(float acc, Scale) { return acc; }
-};
+#include "formats.h"
 
 __global__ __launch_bounds__(256) void f16_tile_kernel(const f16* __restrict__ w, u32x4* __restrict__ tiled,
                                                        int N, int K, int KT, size_t total_vec) {
@@ -49,17 +36,3 @@ extern "C" int pta_f16_tile(const pta_half* w, void* tiled, int N, int K, pta_st
   return PTA_OK;
 }
 
-extern "C" int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
-                            const pta_fusion* fuse, pta_stream_t stream) {
-  int rc = check_gemv_common("pta_f16_gemm", X, M, K);
-  if (rc) return rc;
-  PTA_REQUIRE(tiled && Y, "pta_f16_gemm: null pointer");
-  PTA_REQUIRE(N > 0, "pta_f16_gemm: N = %d", N);
-  PTA_REQUIRE(pta_aligned(tiled, 16), "pta_f16_gemm: tiled must be 16-byte aligned");
-  GemmArgs a{};
-  a.count = 1; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
-  a.mat[0] = GemmMat{tiled, nullptr, (f16*)Y, N, 0};
-  rc = make_epilogue(fuse, &a.epi, "pta_f16_gemm");
-  if (rc) return rc;
-  return dispatch_gemv<FmtF16, false>(a, (N + 15) / 16, (hipStream_t)stream, "pta_f16_gemm");
-}

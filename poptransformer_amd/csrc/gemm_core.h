@@ -76,16 +76,18 @@ static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const c
 // ------------------------------------------------------------------------------------------
 struct GemmMat {
   const void* tiled;
-  const void* scale;
+  const void* scale;   // fp16 [N] (INT4), device int32 exponent (FP8), unused (FP16)
+  const f16* bias;     // [N] or null; used when the launch holds several matrices
   f16* Y;
   int N;
-  int nb_begin;  // first 16-channel block of this matrix in the launch grid
+  int nb_begin;        // first 16-channel block of this matrix in the launch grid
 };
 
 struct GemmArgs {
   GemmMat mat[4];
   int count;
   const f16* X;
+  const int32_t* x_scale;  // device exponent of X when X holds unscaled FP8 grid values, else null
   int M, K, KT;
   GemmEpilogue epi;
   // PAIR mode (SwiGLU): mat[0] is the gate weight, mat[1] the up weight, output in mat[0].Y.
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
 #pragma unroll
   for (int g = 0; g < NACC; ++g) {
     const GemmMat& m = a.mat[PAIR ? g : mi];
-    sc[g] = Fmt::load_scale(m.scale, row, N);
+    sc[g] = Fmt::load_scale(m.scale, a.x_scale, row, N);
     wp[g] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb * KT * (64 * KV) + lane;
   }
   // B operand source: row (mt*16 + lane%16) of X, clamped into range; lanes of padding rows
@@ -192,7 +194,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
       const f16 up = (f16)sum[1];
       a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
     } else {
-      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, (f16)sum[0], m, n, N);
+      f16 y0 = (f16)sum[0];
+      if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
+      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
     }
   }
 }
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 #pragma unroll
   for (int g = 0; g < NACC; ++g) {
     const GemmMat& m = a.mat[PAIR ? g : mi];
-    sc[g] = Fmt::load_scale(m.scale, row, N);
+    sc[g] = Fmt::load_scale(m.scale, a.x_scale, row, N);
     wp[g] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb * KT * (64 * KV) + lane;
   }
   // first tile of this wave: requested before anything else
@@ -353,7 +357,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
       const f16 up = (f16)sum[1];
       a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
     } else {
-      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, (f16)sum[0], m, n, N);
+      f16 y0 = (f16)sum[0];
+      if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
+      a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
     }
   }
 }

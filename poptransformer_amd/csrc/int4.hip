@@ -6,7 +6,7 @@
 // the axis=1 result and the fp16 multiply by the per-channel scale),
 // poptransformer/utils/param_handler/precision_strategy.py:56-60,74-75 (unpack then MatMul).
 #include "common.h"
-#include "gemm_core.h"
+#include "formats.h"
 
 // ------------------------------------------------------------------------------------------
 // Int4ToHalf, standalone and bit-exact.
@@ -131,106 +131,3 @@ extern "C" int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_
   return PTA_OK;
 }
 
-// ------------------------------------------------------------------------------------------
-// Fused W4A16 GEMV/GEMM.
-// ------------------------------------------------------------------------------------------
-
-// One tiled dword -> 8 fp16 weights, each fp16(q * s) with a single rounding (the product of
-// an integer in [-8, 7] held exactly in fp16 and the fp16 scale), which is what the
-// reference's `half(nibble) * scale` computes.
-// (a & mask) | orv in one VALU instruction.  The mask travels in an SGPR and the OR value in a
-// VGPR: a VOP3 encoding on this target takes no literal and at most one scalar operand.
-__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(orv));
-  return r;
-}
-
-__device__ __forceinline__ f16x8 dequant8(uint32_t w, f16x2 s2) {
-  const uint32_t MAGIC = 0x64006400u;  // fp16 1024.0 in both halves
-  const f16x2 c1032 = {(f16)1032.0f, (f16)1032.0f};
-  const f16x2 c16th = {(f16)0.0625f, (f16)0.0625f};
-  const f16x2 c72 = {(f16)-72.0f, (f16)-72.0f};
-  const uint32_t w8 = w >> 8;
-  f16x2 p0 = bitcast<f16x2>(and_or(w, 0x000f000fu, MAGIC));   // 1024 + u      (features 0,1)
-  f16x2 p1 = bitcast<f16x2>(and_or(w, 0x00f000f0u, MAGIC));   // 1024 + 16 u   (features 2,3)
-  f16x2 p2 = bitcast<f16x2>(and_or(w8, 0x000f000fu, MAGIC));  // features 4,5
-  f16x2 p3 = bitcast<f16x2>(and_or(w8, 0x00f000f0u, MAGIC));  // features 6,7
-  p0 = (p0 - c1032) * s2;                                  // exact integer, then one rounding
-  p2 = (p2 - c1032) * s2;
-  p1 = __builtin_elementwise_fma(p1, c16th, c72) * s2;     // (1024 + 16u)/16 - 72 = u - 8, exact
-  p3 = __builtin_elementwise_fma(p3, c16th, c72) * s2;
-  f16x8 r;
-  r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
-  r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
-  return r;
-}
-
-
-struct FmtW4 {
-  static constexpr int kVec = 1;
-  typedef f16x2 Scale;
-  static __device__ __forceinline__ Scale load_scale(const void* scale, int row, int N) {
-    const f16 s = row < N ? reinterpret_cast<const f16*>(scale)[row] : (f16)0.0f;
-    return f16x2{s, s};
-  }
-  static __device__ __forceinline__ f16x8 a_operand(const u32x4 (&raw)[1], int j, Scale s) {
-    return dequant8(raw[0][j], s);
-  }
-  static __device__ __forceinline__ float finish(float acc, Scale) { return acc; }
-};
-
-extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
-                                    const pta_half* const* host_scale, pta_half* const* host_Y,
-                                    const int* host_N, int M, int K, const pta_fusion* fuse, pta_stream_t stream) {
-  int rc = check_gemv_common("pta_w4a16_gemm_multi", X, M, K);
-  if (rc) return rc;
-  PTA_REQUIRE(count >= 1 && count <= 4, "pta_w4a16_gemm_multi: count must be in [1, 4], got %d", count);
-  GemmArgs a{};
-  a.count = count; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
-  int nb = 0;
-  for (int i = 0; i < count; ++i) {
-    PTA_REQUIRE(host_tiled[i] && host_scale[i] && host_Y[i], "pta_w4a16_gemm_multi: null pointer in entry %d", i);
-    PTA_REQUIRE(host_N[i] > 0, "pta_w4a16_gemm_multi: N[%d] = %d", i, host_N[i]);
-    PTA_REQUIRE(pta_aligned(host_tiled[i], 16), "pta_w4a16_gemm_multi: tiled[%d] must be 16-byte aligned", i);
-    a.mat[i] = GemmMat{(const void*)host_tiled[i], (const void*)host_scale[i], (f16*)host_Y[i], host_N[i], nb};
-    nb += (host_N[i] + 15) / 16;
-  }
-  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm_multi");
-  if (rc) return rc;
-  PTA_REQUIRE(!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE, "pta_w4a16_gemm_multi: only the norm fields of `fuse` are supported");
-  return dispatch_gemv<FmtW4, false>(a, nb, (hipStream_t)stream, "pta_w4a16_gemm_multi");
-}
-
-extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
-                              int M, int K, int N, const pta_fusion* fuse, pta_stream_t stream) {
-  int rc = check_gemv_common("pta_w4a16_gemm", X, M, K);
-  if (rc) return rc;
-  PTA_REQUIRE(tiled && scale && Y, "pta_w4a16_gemm: null pointer");
-  PTA_REQUIRE(N > 0, "pta_w4a16_gemm: N = %d", N);
-  PTA_REQUIRE(pta_aligned(tiled, 16), "pta_w4a16_gemm: tiled must be 16-byte aligned");
-  GemmArgs a{};
-  a.count = 1; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
-  a.mat[0] = GemmMat{(const void*)tiled, (const void*)scale, (f16*)Y, N, 0};
-  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm");
-  if (rc) return rc;
-  return dispatch_gemv<FmtW4, false>(a, (N + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm");
-}
-
-extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
-                                     const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M,
-                                     int K, int F, const pta_fusion* fuse, pta_stream_t stream) {
-  int rc = check_gemv_common("pta_w4a16_gemm_swiglu", X, M, K);
-  if (rc) return rc;
-  PTA_REQUIRE(tiled_gate && scale_gate && tiled_up && scale_up && Y, "pta_w4a16_gemm_swiglu: null pointer");
-  PTA_REQUIRE(F > 0, "pta_w4a16_gemm_swiglu: F = %d", F);
-  PTA_REQUIRE(pta_aligned(tiled_gate, 16) && pta_aligned(tiled_up, 16), "pta_w4a16_gemm_swiglu: tiled buffers must be 16-byte aligned");
-  GemmArgs a{};
-  a.count = 2; a.X = (const f16*)X; a.M = M; a.K = K; a.KT = (K + 127) / 128;
-  a.mat[0] = GemmMat{(const void*)tiled_gate, (const void*)scale_gate, (f16*)Y, F, 0};
-  a.mat[1] = GemmMat{(const void*)tiled_up, (const void*)scale_up, (f16*)Y, F, 0};
-  rc = make_epilogue(fuse, &a.epi, "pta_w4a16_gemm_swiglu");
-  if (rc) return rc;
-  PTA_REQUIRE(!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE, "pta_w4a16_gemm_swiglu: only the norm fields of `fuse` are supported");
-  return dispatch_gemv<FmtW4, true>(a, (F + 15) / 16, (hipStream_t)stream, "pta_w4a16_gemm_swiglu");
-}

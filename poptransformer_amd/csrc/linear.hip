@@ -1,0 +1,116 @@
+// Linear layers of the decode step: Y = [act](X' @ W + bias) [+ residual] for INT4, FP16 and FP8
+// weights, one or several weights per launch, optionally as a SwiGLU pair.
+//
+// Reference: poptransformer/layers/linear.py:19-46 with the precision hooks of
+// poptransformer/utils/param_handler/precision_strategy.py:56-81 (int4: Int4ToHalf + MatMul;
+// fp8: CastToUint8 + FP8MatMul; fp8_weight: FP8MatMul on fp16 activations; fp16: MatMul).
+#include "common.h"
+#include "formats.h"
+
+int f8_decode_unscaled_launch(const uint8_t* in, f16* out, size_t n, int format, hipStream_t s);
+
+template <class Fmt>
+static int run_linear(GemmArgs& a, int total_nb, int swiglu, hipStream_t s, const char* name) {
+  if (swiglu) return dispatch_gemv<Fmt, true>(a, total_nb, s, name);
+  return dispatch_gemv<Fmt, false>(a, total_nb, s, name);
+}
+
+extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_weight* host_w,
+                          const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
+                          const pta_fusion* fuse, pta_stream_t stream) {
+  PTA_REQUIRE(host_w && host_Y, "pta_linear: null pointer");
+  PTA_REQUIRE(count >= 1 && count <= 4, "pta_linear: count must be in [1, 4], got %d", count);
+  PTA_REQUIRE(!swiglu || count == 2, "pta_linear: a SwiGLU pair is exactly two weights (gate, up)");
+  const int kind = host_w[0].kind, K = host_w[0].K;
+  int rc = check_gemv_common("pta_linear", X, M, K);
+  if (rc) return rc;
+  PTA_REQUIRE(kind >= PTA_W_INT4 && kind <= PTA_W_F152, "pta_linear: unknown weight kind %d", kind);
+  GemmArgs a{};
+  a.count = count; a.X = (const f16*)X; a.x_scale = x_scale; a.M = M; a.K = K; a.KT = (K + 127) / 128;
+  PTA_REQUIRE(!x_scale || kind == PTA_W_F143 || kind == PTA_W_F152, "pta_linear: x_scale is only meaningful with FP8 weights");
+  int nb = 0;
+  for (int i = 0; i < count; ++i) {
+    const pta_weight& w = host_w[i];
+    PTA_REQUIRE(w.kind == kind && w.K == K, "pta_linear: weights of one call must share their kind and K");
+    PTA_REQUIRE(w.tiled && host_Y[i] && w.N > 0, "pta_linear: entry %d is incomplete", i);
+    PTA_REQUIRE(kind == PTA_W_F16 || w.scale, "pta_linear: entry %d needs its scale", i);
+    PTA_REQUIRE(pta_aligned(w.tiled, 16), "pta_linear: tiled[%d] must be 16-byte aligned", i);
+    PTA_REQUIRE(!swiglu || w.N == host_w[0].N, "pta_linear: the SwiGLU weights must have the same shape");
+    a.mat[i] = GemmMat{w.tiled, w.scale, host_bias ? (const f16*)host_bias[i] : nullptr, (f16*)host_Y[i], w.N,
+                       swiglu ? 0 : nb};
+    nb += (w.N + 15) / 16;
+  }
+  if (swiglu) {
+    nb = (host_w[0].N + 15) / 16;
+    PTA_REQUIRE(!a.mat[0].bias && !a.mat[1].bias, "pta_linear: the SwiGLU pair takes no bias");
+  }
+  rc = make_epilogue(fuse, &a.epi, "pta_linear");
+  if (rc) return rc;
+  PTA_REQUIRE(count == 1 || (!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE),
+              "pta_linear: with several weights only the norm fields of `fuse` apply (use host_bias for biases)");
+  hipStream_t s = (hipStream_t)stream;
+  switch (kind) {
+    case PTA_W_INT4: return run_linear<FmtW4>(a, nb, swiglu, s, "pta_linear");
+    case PTA_W_F16: return run_linear<FmtF16>(a, nb, swiglu, s, "pta_linear");
+    case PTA_W_F143: return run_linear<FmtF8<0>>(a, nb, swiglu, s, "pta_linear");
+    default: return run_linear<FmtF8<1>>(a, nb, swiglu, s, "pta_linear");
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Operator-shaped entry points over pta_linear.
+// ------------------------------------------------------------------------------------------
+extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y, int M, int K,
+                              int N, const pta_fusion* fuse, pta_stream_t stream) {
+  pta_weight w{PTA_W_INT4, tiled, scale, N, K};
+  return pta_linear(X, nullptr, 1, &w, nullptr, &Y, M, 0, fuse, stream);
+}
+
+extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* const* host_tiled,
+                                    const pta_half* const* host_scale, pta_half* const* host_Y, const int* host_N,
+                                    int M, int K, const pta_fusion* fuse, pta_stream_t stream) {
+  PTA_REQUIRE(count >= 1 && count <= 4 && host_tiled && host_scale && host_N, "pta_w4a16_gemm_multi: bad arguments");
+  pta_weight w[4];
+  for (int i = 0; i < count; ++i) w[i] = pta_weight{PTA_W_INT4, host_tiled[i], host_scale[i], host_N[i], K};
+  return pta_linear(X, nullptr, count, w, nullptr, host_Y, M, 0, fuse, stream);
+}
+
+extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
+                                     const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M, int K, int F,
+                                     const pta_fusion* fuse, pta_stream_t stream) {
+  pta_weight w[2] = {{PTA_W_INT4, tiled_gate, scale_gate, F, K}, {PTA_W_INT4, tiled_up, scale_up, F, K}};
+  pta_half* ys[2] = {Y, Y};
+  return pta_linear(X, nullptr, 2, w, nullptr, ys, M, 1, fuse, stream);
+}
+
+extern "C" int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
+                            const pta_fusion* fuse, pta_stream_t stream) {
+  pta_weight w{PTA_W_F16, tiled, nullptr, N, K};
+  return pta_linear(X, nullptr, 1, &w, nullptr, &Y, M, 0, fuse, stream);
+}
+
+extern "C" size_t pta_fp8_gemm_workspace_bytes(int M, int K) {
+  if (M <= 0 || K <= 0) return 0;
+  return (size_t)M * K * 2;     // the left-hand side decoded to fp16
+}
+
+extern "C" int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_rhs, pta_half* Y, int M, int K, int N,
+                            int format_lhs, int format_rhs, const int32_t* scale_lhs, const int32_t* scale_rhs,
+                            void* workspace, const pta_fusion* fuse, pta_stream_t stream) {
+  // dtype guards of FP8MatMulOp::setup (custom_ops/matmul_fp8.cpp:237-245) are the caller's to state
+  // through lhs_is_fp8; formats must be F143 or F152 (:324-351).
+  PTA_REQUIRE(format_rhs == PTA_F143 || format_rhs == PTA_F152, "pta_fp8_gemm: unsupported fp8 format %d, it must be F143 or F152", format_rhs);
+  PTA_REQUIRE(lhs && scale_rhs, "pta_fp8_gemm: null pointer");
+  const f16* X = (const f16*)lhs;
+  const int32_t* xs = nullptr;
+  if (lhs_is_fp8) {
+    PTA_REQUIRE(format_lhs == PTA_F143 || format_lhs == PTA_F152, "pta_fp8_gemm: unsupported fp8 format %d, it must be F143 or F152", format_lhs);
+    PTA_REQUIRE(scale_lhs && workspace && pta_aligned(workspace, 16), "pta_fp8_gemm: an fp8 left-hand side needs its scale and a 16-byte aligned workspace");
+    PTA_REQUIRE(M >= 1 && K >= 1, "pta_fp8_gemm: empty left-hand side");
+    f8_decode_unscaled_launch((const uint8_t*)lhs, (f16*)workspace, (size_t)M * K, format_lhs, (hipStream_t)stream);
+    X = (const f16*)workspace;
+    xs = scale_lhs;
+  }
+  pta_weight w{format_rhs == PTA_F143 ? PTA_W_F143 : PTA_W_F152, tiled_rhs, scale_rhs, N, K};
+  return pta_linear((const pta_half*)X, xs, 1, &w, nullptr, &Y, M, 0, fuse, stream);
+}

@@ -232,6 +232,50 @@ def fp8_gemm(x, w, workspace, x_scale=None, x_format="F143", bias=None, residual
     return out
 
 
+def half_to_fp8_grid(x, scale, fp8_format="F143", out=None):
+    """x rounded to the FP8 grid, returned as fp16 WITHOUT the scale (see pta_half_to_fp8_grid)."""
+    fmt = _fmt(fp8_format)
+    _need(x, torch.float16, "x")
+    _need(scale, _i32, "fp8_scale")
+    if out is None:
+        out = torch.empty_like(x)
+    check(_lib.load().pta_half_to_fp8_grid(_p(x), _p(out), _p(scale), x.numel(), fmt, _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ general Linear -------
+def _desc(w):
+    if isinstance(w, W4Weight):
+        return _lib.Weight(_lib.W_INT4, w.tiled.data_ptr(), w.scale.data_ptr(), w.N, w.K)
+    if isinstance(w, F16Weight):
+        return _lib.Weight(_lib.W_F16, w.tiled.data_ptr(), None, w.N, w.K)
+    if isinstance(w, F8Weight):
+        return _lib.Weight(_lib.W_F143 if w.format == _lib.F143 else _lib.W_F152, w.tiled.data_ptr(), w.scale.data_ptr(),
+                           w.N, w.K)
+    raise TypeError(f"not a tiled weight: {type(w)}")
+
+
+def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None, residual=None, act=_lib.ACT_NONE,
+           norm=None):
+    """pta_linear: up to four weights of one kind sharing x.  `biases` is a per-weight list (or None);
+    bias/residual/act apply to the single-weight form only."""
+    _need(x, torch.float16, "x", 2)
+    M = x.shape[0]
+    n = len(weights)
+    descs = (_lib.Weight * n)(*[_desc(w) for w in weights])
+    VP = ctypes.c_void_p * n
+    ys = VP(*[o.data_ptr() for o in outs])
+    bs = None
+    if biases is not None and any(b is not None for b in biases):
+        bs = VP(*[(b.data_ptr() if b is not None else None) for b in biases])
+    for w in weights:
+        if w.K != x.shape[1]:
+            raise ValueError(f"matmul: contracting dimensions differ ({x.shape[1]} vs {w.K})")
+    check(_lib.load().pta_linear(_p(x), _p(x_scale), n, descs, bs, ys, M, 1 if swiglu else 0,
+                                 _fusion(bias, residual, act, norm), _stream()))
+    return outs
+
+
 # ------------------------------------------------------------------ norms ----------------
 def rmsnorm(x, weight, eps, out=None):
     _need(x, torch.float16, "x")
