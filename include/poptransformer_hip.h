@@ -285,6 +285,10 @@ int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_w
                const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
                const pta_fusion* fuse, pta_stream_t stream);
 
+/* out = up * swish(gate), two fp16 ops (models/llama2/mlp.py:22-26): the unfused form of the
+ * SwiGLU pair, for gate/up weights that cannot share a launch. */
+int pta_swiglu(const pta_half* gate, const pta_half* up, pta_half* out, size_t n, pta_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -253,3 +253,131 @@ class GPT2Oracle:
         logits = O.matmul(x, self.head_w)
         _, idx = O.topk1(logits, axis=2)
         return idx.reshape(B), logits.reshape(B, -1)
+
+
+# --------------------------------------------------------------------------------------
+# ChatGLM2
+# --------------------------------------------------------------------------------------
+def make_chatglm2_state_dict(cfg, seed=0):
+    """Random-init ChatGLM2-shaped checkpoint in the form the reference holds it after
+    ChatGLM2DecModel.prepare_state_dict (poptransformer/models/chatglm2/model.py:256-274):
+    `query_key_value` split into `query` / `key_value`, `dense_h_to_4h` into `_1` (gate) / `_2` (up).
+    fp16 throughout: FP8 conversion happens when the Linear layers bind their weights
+    (utils/param_handler/precision_strategy.py:44-51)."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, f, v = cfg["hidden_size"], cfg["ffn_hidden_size"], cfg["padded_vocab_size"]
+    kv = 2 * cfg["multi_query_group_num"] * cfg["kv_channels"]
+    sd = {"transformer.embedding.word_embeddings.weight": _normal(rng, (v, d))}
+    for i in range(cfg["num_layers"]):
+        p = f"transformer.encoder.layers.{i}."
+        sd[p + "input_layernorm.weight"] = np.ones(d, f16)
+        sd[p + "self_attention.query.weight"] = _normal(rng, (d, d))
+        sd[p + "self_attention.query.bias"] = _normal(rng, (d,))
+        sd[p + "self_attention.key_value.weight"] = _normal(rng, (kv, d))
+        sd[p + "self_attention.key_value.bias"] = _normal(rng, (kv,))
+        sd[p + "self_attention.dense.weight"] = _normal(rng, (d, d))
+        sd[p + "post_attention_layernorm.weight"] = np.ones(d, f16)
+        sd[p + "mlp.dense_h_to_4h_1.weight"] = _normal(rng, (f, d))
+        sd[p + "mlp.dense_h_to_4h_2.weight"] = _normal(rng, (f, d))
+        sd[p + "mlp.dense_4h_to_h.weight"] = _normal(rng, (d, f))
+    sd["transformer.encoder.final_layernorm.weight"] = np.ones(d, f16)
+    sd["transformer.output_layer.weight"] = _normal(rng, (v, d))
+    return sd
+
+
+def fp8_weight_scale(w, fmt="F143"):
+    """Power-of-two exponent s such that max|w| * 2^-s lands in (max/2, max] of the format: the
+    "per-tensor scale bias chosen so max|w| maps near format max" of the FP8 benchmark
+    configuration.  (The reference itself always uses -1, precision_strategy.py:46.)"""
+    mx = 240.0 if fmt == "F143" else 57344.0
+    m = float(np.abs(np.asarray(w, f32)).max())
+    return int(np.ceil(np.log2(m / mx))) if m > 0 else 0
+
+
+class _LinearFP8:
+    """Linear under precision 'fp8' / 'fp8_weight' (utils/param_handler/precision_strategy.py:44-51,
+    62-69,77-81): the [in, out] weight is converted to F143 bytes with exponent `scale`; with 'fp8'
+    the activations are cast with the same scale tensor before the FP8 MatMul."""
+
+    def __init__(self, sd, ctx, use_bias, precision, scale=-1):
+        w = np.asarray(sd[ctx + ".weight"], f32).T               # [in, out]
+        self.scale = np.array([scale], np.int32)
+        self.w8 = O.f8_encode(w, "F143", scale)
+        self.b = sd[ctx + ".bias"] if use_bias else None
+        self.act_fp8 = precision == "fp8"
+
+    def __call__(self, x):
+        if self.act_fp8:
+            x = O.f8_encode(x, "F143", int(self.scale[0]))
+        y = O.fp8_matmul(x, self.w8, self.scale, self.scale, "F143", "F143")
+        return (y + self.b).astype(f16) if self.b is not None else y
+
+
+class ChatGLM2Oracle:
+    """ChatGLM2DecModel.build_model_graph (poptransformer/models/chatglm2/model.py:296-341): embedding,
+    blocks RMSNorm -> multi-query attention -> add -> RMSNorm -> SwiGLU MLP -> add (model.py:95-117),
+    final RMSNorm, LMHead top-1.  precision: 'fp16', 'fp8' or 'fp8_weight'; `scales` maps a Linear
+    context to its FP8 exponent (default -1 as in the reference)."""
+
+    def __init__(self, sd, cfg, max_length, batch_size, precision="fp16", scales=None):
+        self.cfg, self.L, self.B = cfg, max_length, batch_size
+        self.d, self.H, self.G = cfg["hidden_size"], cfg["num_attention_heads"], cfg["multi_query_group_num"]
+        self.D = self.d // self.H
+        self.eps = cfg["layernorm_epsilon"]
+        scales = scales or {}
+
+        def lin(ctx, bias):
+            if precision in ("fp8", "fp8_weight"):
+                return _LinearFP8(sd, ctx, bias, precision, scales.get(ctx, -1))
+            return _Linear(sd, ctx, bias)
+
+        self.embed = sd["transformer.embedding.word_embeddings.weight"]
+        self.layers = []
+        for i in range(cfg["num_layers"]):
+            p = f"transformer.encoder.layers.{i}."
+            self.layers.append({
+                "ln1": sd[p + "input_layernorm.weight"], "ln2": sd[p + "post_attention_layernorm.weight"],
+                "query": lin(p + "self_attention.query", True), "key_value": lin(p + "self_attention.key_value", True),
+                "dense": lin(p + "self_attention.dense", False),
+                "gate": lin(p + "mlp.dense_h_to_4h_1", False), "up": lin(p + "mlp.dense_h_to_4h_2", False),
+                "down": lin(p + "mlp.dense_4h_to_h", False), "cache": O.KVCache(max_length, 3, 1)})
+        self.norm = sd["transformer.encoder.final_layernorm.weight"]
+        self.head = lin("transformer.output_layer", False)
+
+    def _attention(self, lay, x, step, mask4):
+        """MultiQueryAttention.forward_qkv / forward_attention / forward_output
+        (poptransformer/models/chatglm2/attention.py:166-302)."""
+        B, H, G, D = self.B, self.H, self.G, self.D
+        q = lay["query"](x)
+        mixed = lay["key_value"](x)
+        k, v = mixed[..., : G * D], mixed[..., G * D:]
+        q = q.reshape(B, 1, H, D)
+        k = k.reshape(B, 1, G, D)
+        v = v.reshape(B, 1, G, D)
+        cos, sin = O.glm2_sincos(step, D)
+        q, k = O.glm2_rope(q, cos, sin), O.glm2_rope(k, cos, sin)
+        q = q.transpose(0, 2, 1, 3)
+        kv = np.concatenate([k, v], axis=0).reshape(2, B, 1, G, D).transpose(0, 1, 3, 2, 4)
+        past = lay["cache"](step, kv)
+        kk = np.repeat(past[0][:, :, None], H // G, axis=2).reshape(B, H, self.L, D)
+        vv = np.repeat(past[1][:, :, None], H // G, axis=2).reshape(B, H, self.L, D)
+        a = O.attention_scores_to_context(q, kk.transpose(0, 1, 3, 2), vv, mask4, 1 / np.sqrt(D), f16, False)
+        a = a.transpose(0, 2, 1, 3).reshape(B, 1, H * D)
+        return lay["dense"](a)
+
+    def step(self, ids, step, mask):
+        B = self.B
+        x = self.embed[ids.reshape(B, 1)]
+        mask4 = mask[:, None, None, :]
+        for lay in self.layers:
+            t = O.rms_norm(x, lay["ln1"], self.eps)
+            t = self._attention(lay, t, step, mask4)
+            x = (x + t).astype(f16)
+            t = O.rms_norm(x, lay["ln2"], self.eps).reshape(-1, self.d)      # BaseMLP (models/chatglm2/mlp.py:51-59)
+            g = O.swish(lay["gate"](t))
+            u = (lay["up"](t) * g).astype(f16)
+            x = (x + lay["down"](u).reshape(B, -1, self.d)).astype(f16)
+        x = O.rms_norm(x, self.norm, self.eps)
+        logits = self.head(x)
+        _, idx = O.topk1(logits, axis=2)
+        return idx.reshape(B), logits.reshape(B, -1)

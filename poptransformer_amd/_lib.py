@@ -73,6 +73,7 @@ SIGNATURES = {
     "pta_half_to_fp8_grid": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "pta_linear": (c_int, [c_void_p, c_void_p, c_int, POINTER(Weight), POINTER(c_void_p), POINTER(c_void_p), c_int, c_int,
                            POINTER(Fusion), c_void_p]),
+    "pta_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
 }

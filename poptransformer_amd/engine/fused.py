@@ -52,20 +52,28 @@ class DecoderSpec:
 
 
 class LinearWeights:
-    """One Linear: a tiled weight (INT4 or FP16) and an optional fp16 bias."""
+    """One Linear: a tiled weight (INT4, FP16 or FP8), an optional fp16 bias and, for FP8 weights,
+    whether the activations are cast to FP8 first (precision 'fp8') or stay fp16 ('fp8_weight')."""
 
-    def __init__(self, weight, bias=None):
-        self.w, self.bias = weight, bias
+    def __init__(self, weight, bias=None, act_fp8=False, scale_value=None):
+        self.w, self.bias, self.act_fp8 = weight, bias, act_fp8
         self.N, self.K = weight.N, weight.K
+        self.scale_value = scale_value            # host copy of the FP8 exponent (for grouping)
 
     @property
     def is_int4(self):
         return isinstance(self.w, K.W4Weight)
 
-    def __call__(self, x, out, residual=None, act=_lib.ACT_NONE, norm=None):
-        if self.is_int4:
-            return K.w4a16_gemm(x, self.w, self.bias, residual, act, out, norm)
-        return K.f16_gemm(x, self.w, self.bias, residual, act, out, norm)
+    @property
+    def is_fp8(self):
+        return isinstance(self.w, K.F8Weight)
+
+    def group_key(self):
+        """Linears with equal keys can share one launch (same weight kind; for FP8 also the same
+        format, activation handling and exponent, since they share the cast activations)."""
+        if self.is_fp8:
+            return ("fp8", self.w.format, self.act_fp8, self.scale_value if self.act_fp8 else None)
+        return ("int4",) if self.is_int4 else ("f16",)
 
     @property
     def nbytes(self):
@@ -133,6 +141,9 @@ class FusedDecoder:
         # Measured on MI355X at d = 4096: the norm inside the GEMM costs every workgroup a pass over X
         # and two barriers (+5 us per launch), the stand-alone norm kernel 2.4 us, so it stays separate.
         self.fuse_norm = False
+        # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
+        self._fp8_buf = {k: buf(B, k) for k in {d, ffn}}
+        self._gate, self._up = buf(B, ffn), buf(B, ffn)
 
     # ------------------------------------------------------------------ one loop iteration
     def _norm(self, x, gb, out):
@@ -148,46 +159,64 @@ class FusedDecoder:
         self._norm(x, gb, self.h)
         return self.h, None
 
+    def _lhs(self, x, lw, norm):
+        """Left-hand side for a Linear: FP8 activations are rounded to the FP8 grid first
+        (half_to_uint8 of precision_strategy.py:62-66), everything else passes through."""
+        if not (lw.is_fp8 and lw.act_fp8):
+            return x, None, norm
+        if norm is not None:                      # the cast needs the normalised values
+            raise NotImplementedError("fused norm is not combined with FP8 activations")
+        buf = self._fp8_buf[x.shape[1]]
+        K.half_to_fp8_grid(x, lw.w.scale, "F143", out=buf)
+        return buf, lw.w.scale, None
+
+    def _linear(self, x, lw, out, residual=None, act=_lib.ACT_NONE, norm=None):
+        xin, xs, norm = self._lhs(x, lw, norm)
+        K.linear(xin, [lw.w], [out], x_scale=xs, bias=lw.bias, residual=residual, act=act, norm=norm)
+        return out
+
+    def _linear_group(self, x, lws, outs, norm=None, swiglu=False):
+        """Several Linears on the same input: one launch when they are alike, else one each."""
+        keys = {lw.group_key() for lw in lws}
+        if len(keys) == 1 and (not swiglu or all(lw.bias is None for lw in lws)):
+            xin, xs, norm = self._lhs(x, lws[0], norm)
+            K.linear(xin, [lw.w for lw in lws], outs, biases=[lw.bias for lw in lws], x_scale=xs, swiglu=swiglu, norm=norm)
+            return
+        if swiglu:                                 # unlike weights: two launches and the elementwise form
+            self._linear(x, lws[0], self._gate, norm=norm)
+            self._linear(x, lws[1], self._up, norm=norm)
+            K.swiglu(self._gate, self._up, outs[0])
+            return
+        for lw, o in zip(lws, outs):
+            self._linear(x, lw, o, norm=norm)
+
     def step_fn(self):
         s, w = self.spec, self.w
         B = s.batch
         K.embedding(w.embed, self.container, self.x, pos_table=w.pos_embed,
                     pos=self.step if w.pos_embed is not None else None, ids_index=self.step)
         for li, blk in enumerate(w.blocks):
-            self._project_qkv(blk)
+            if not hasattr(self, "_qkv_views"):
+                self._prepare_qkv_views(blk)
+            h, nrm = self._normed(self.x, blk.norm1)
+            self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
             K.qkv_rope_append(qp, kp, vp, self.q_rot, self.rings[li], self.step, w.inv_freq, B, s.n_head,
                               s.n_kv_head, s.head_dim, s.max_len, s.rope, qs, ks, vs)
             K.decode_attention(self.q_rot, self.rings[li], self.step, self.attn_ws, self.ctx, B, s.n_head,
                                s.n_kv_head, s.head_dim, s.max_len, s.scale_scores)
-            blk.out(self.ctx, self.x, residual=self.x)
+            self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2)
             if len(blk.mlp_in) == 2:
-                g, u = blk.mlp_in
-                if g.is_int4 and u.is_int4:
-                    K.w4a16_gemm_swiglu(h, g.w, u.w, self.act, nrm)
-                else:
-                    raise NotImplementedError("SwiGLU needs INT4 gate/up weights in the fused executor")
+                self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True)
             else:
-                blk.mlp_in[0](h, self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
-            blk.mlp_out(self.act, self.x, residual=self.x)
+                self._linear(h, blk.mlp_in[0], self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
+            self._linear(self.act, blk.mlp_out, self.x, residual=self.x)
         h, nrm = self._normed(self.x, w.final_norm)
-        w.head(h, self.logits, norm=nrm)
+        self._linear(h, w.head, self.logits, norm=nrm)
         K.argmax(self.logits, self.next_ids)
         K.step_update(self.container, self.mask, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
                       s.pad_id, s.eos_id, s.early_stop)
-
-    def _project_qkv(self, blk):
-        if not hasattr(self, "_qkv_views"):
-            self._prepare_qkv_views(blk)
-        h, nrm = self._normed(self.x, blk.norm1)
-        if len(blk.qkv) == 1:
-            blk.qkv[0](h, self.qkv, norm=nrm)
-        elif all(lw.is_int4 and lw.bias is None for lw in blk.qkv):
-            K.w4a16_gemm_multi(h, [lw.w for lw in blk.qkv], self._qkv_bufs, nrm)
-        else:
-            for lw, o in zip(blk.qkv, self._qkv_bufs):
-                lw(h, o, norm=nrm)
 
     def _prepare_qkv_views(self, blk):
         """Output buffers of the projections and the (pointer, row stride) views of q, k, v."""

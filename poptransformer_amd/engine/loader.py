@@ -16,9 +16,20 @@ def _dev(a, device):
     return torch.from_numpy(np.ascontiguousarray(a)).to(device)
 
 
-def linear_from_state_dict(sd, ctx, use_bias, device="cuda"):
+def f143_encode_device(w, scale):
+    """fp32/fp16 device tensor -> F143 bytes with exponent `scale` (the bind-time conversion of
+    utils/param_handler/precision_strategy.py:44-51), through the library's own encoder."""
+    sc = torch.tensor([scale], dtype=torch.int32, device=w.device)
+    return K.half_to_fp8(w.half().contiguous(), sc, "F143"), sc
+
+
+def linear_from_state_dict(sd, ctx, use_bias, device="cuda", precision="fp16", fp8_scale=-1):
     w = sd[ctx + ".weight"]
     w = w if isinstance(w, np.ndarray) else np.asarray(w)
+    bias = _dev(np.asarray(sd[ctx + ".bias"], np.float16), device) if use_bias else None
+    if precision in ("fp8", "fp8_weight"):
+        w8, sc = f143_encode_device(_dev(w.astype(np.float16), device), fp8_scale)
+        return LinearWeights(K.F8Weight(w8, sc, "F143"), bias, act_fp8=precision == "fp8", scale_value=fp8_scale)
     if w.dtype == np.int8:
         scale = sd.get(ctx + ".weight_scale")
         if scale is None:
@@ -26,7 +37,6 @@ def linear_from_state_dict(sd, ctx, use_bias, device="cuda"):
         tw = K.W4Weight(_dev(w, device), _dev(np.asarray(scale, np.float16), device))
     else:
         tw = K.F16Weight(_dev(w.astype(np.float16), device))
-    bias = _dev(np.asarray(sd[ctx + ".bias"], np.float16), device) if use_bias else None
     return LinearWeights(tw, bias)
 
 
@@ -76,3 +86,33 @@ def gpt2_spec(cfg, max_len, batch, pad_id=50257, eos_id=50256, early_stop=False)
     d, h = cfg["n_embd"], cfg["n_head"]
     return DecoderSpec("gpt2", cfg["n_layer"], d, h, h, d // h, cfg["vocab_size"], max_len, batch,
                        cfg["layer_norm_epsilon"], pad_id, eos_id, early_stop)
+
+
+def chatglm2_weights(sd, cfg, precision="fp16", scales=None, device="cuda"):
+    scales = scales or {}
+    hd = cfg["hidden_size"] // cfg["num_attention_heads"]
+
+    def lin(ctx, bias):
+        return linear_from_state_dict(sd, ctx, bias, device, precision, scales.get(ctx, -1))
+
+    blocks = []
+    for i in range(cfg["num_layers"]):
+        p = f"transformer.encoder.layers.{i}."
+        blocks.append(BlockWeights(
+            norm1=(_dev(sd[p + "input_layernorm.weight"], device), None),
+            norm2=(_dev(sd[p + "post_attention_layernorm.weight"], device), None),
+            qkv=[lin(p + "self_attention.query", True), lin(p + "self_attention.key_value", True)],
+            out=lin(p + "self_attention.dense", False),
+            mlp_in=[lin(p + "mlp.dense_h_to_4h_1", False), lin(p + "mlp.dense_h_to_4h_2", False)],
+            mlp_out=lin(p + "mlp.dense_4h_to_h", False)))
+    rot = hd // 2
+    inv_freq = np.array([1.0 / (10000 ** (i / rot)) for i in range(0, rot, 2)]).astype(np.float32)
+    return ModelWeights(embed=_dev(sd["transformer.embedding.word_embeddings.weight"], device), pos_embed=None,
+                        blocks=blocks, final_norm=(_dev(sd["transformer.encoder.final_layernorm.weight"], device), None),
+                        head=lin("transformer.output_layer", False), inv_freq=_dev(inv_freq, device))
+
+
+def chatglm2_spec(cfg, max_len, batch, pad_id=0, eos_id=2, early_stop=False):
+    d, h = cfg["hidden_size"], cfg["num_attention_heads"]
+    return DecoderSpec("chatglm2", cfg["num_layers"], d, h, cfg["multi_query_group_num"], d // h,
+                       cfg["padded_vocab_size"], max_len, batch, cfg["layernorm_epsilon"], pad_id, eos_id, early_stop)

@@ -28,6 +28,7 @@ def _linear_int4(gen, out_f, in_f, device):
     return LinearWeights(K.W4Weight(packed, scale))
 
 
+
 def llama2_synthetic_weights(cfg, seed=0, device="cuda"):
     gen = torch.Generator(device=device)
     gen.manual_seed(seed)

@@ -276,6 +276,15 @@ def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None,
     return outs
 
 
+def swiglu(gate, up, out=None):
+    _need(gate, torch.float16, "gate")
+    _need(up, torch.float16, "up")
+    if out is None:
+        out = torch.empty_like(up)
+    check(_lib.load().pta_swiglu(_p(gate), _p(up), _p(out), up.numel(), _stream()))
+    return out
+
+
 # ------------------------------------------------------------------ norms ----------------
 def rmsnorm(x, weight, eps, out=None):
     _need(x, torch.float16, "x")

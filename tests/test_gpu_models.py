@@ -21,7 +21,7 @@ def _prompt(rng, B, L, plen, vocab, pad):
     return ids
 
 
-def _compare(dec, oracle, ids, L, steps, pad, eos):
+def _compare(dec, oracle, ids, L, steps, pad, eos, tol=1e-2):
     trace = []
     ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos, trace=trace)
     dec.reset(ids)
@@ -33,7 +33,7 @@ def _compare(dec, oracle, ids, L, steps, pad, eos):
         ref = trace[it][1].astype(np.float64)
         worst = max(worst, np.abs(got - ref).max() / np.abs(ref).max())
         assert np.array_equal(dec.next_ids.cpu().numpy(), trace[it][0]), f"token ids differ at step {it}"
-    assert worst <= 1e-2, f"logits max rel err {worst}"
+    assert worst <= tol, f"logits max rel err {worst}"
     assert np.array_equal(dec.container.cpu().numpy(), ref_container)
     assert int(dec.step.item()) == ref_step
     return worst
@@ -59,6 +59,28 @@ def test_gpt2_fp16_decode_matches_oracle(B):
     dec = fused.FusedDecoder(loader.gpt2_spec(GPT2_TINY, L, B, pad, eos), loader.gpt2_weights(sd, GPT2_TINY))
     ids = _prompt(np.random.default_rng(8), B, L, 6, 900, pad)
     _compare(dec, oracle, ids, L, steps, pad, eos)
+
+
+GLM2_TINY = dict(padded_vocab_size=384, hidden_size=256, layernorm_epsilon=1e-5, multi_query_group_num=2,
+                 num_attention_heads=4, ffn_hidden_size=352, num_layers=2, kv_channels=64)
+
+
+@pytest.mark.parametrize("precision", ["fp16", "fp8_weight", "fp8"])
+def test_chatglm2_decode_matches_oracle(precision):
+    from poptransformer_amd.engine import fused, loader
+    B, L, steps, pad, eos = 2, 48, 32, 0, 2
+    sd = OM.make_chatglm2_state_dict(GLM2_TINY, seed=4)
+    # exponents near the format maximum for half of the Linears, the reference's -1 for the rest
+    scales = {k[:-7]: OM.fp8_weight_scale(v) for k, v in sd.items() if k.endswith("dense.weight") or "h_to_4h_1" in k}
+    oracle = OM.ChatGLM2Oracle(sd, GLM2_TINY, L, B, precision, scales)
+    dec = fused.FusedDecoder(loader.chatglm2_spec(GLM2_TINY, L, B, pad, eos),
+                             loader.chatglm2_weights(sd, GLM2_TINY, precision, scales))
+    ids = _prompt(np.random.default_rng(10), B, L, 7, GLM2_TINY["padded_vocab_size"], pad)
+    # With FP8 activations (3 mantissa bits) a one-ulp fp16 difference in an activation - which two
+    # correct fp32-accumulating MatMuls already produce - can flip its FP8 rounding, a 6 % step in that
+    # element: whole-model logits agree to a few percent, not to 1e-2.  The operator itself is held to
+    # 1e-2 on identical inputs in test_gpu_kernels.py::test_fp8_gemm_both_modes; tokens must still match.
+    _compare(dec, oracle, ids, L, steps, pad, eos, tol=1e-1 if precision == "fp8" else 1e-2)
 
 
 def test_llama2_graph_replay_equals_eager():
