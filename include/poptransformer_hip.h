@@ -74,12 +74,16 @@ int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t st
  *   PTA_NORM_LAYER: pta_layer_norm_ce(X, norm_weight, norm_bias, eps)   (ops/customized.py:69-102)
  *   The fused norm needs M <= 4 and K <= 20480 / M; otherwise the call returns PTA_EUNSUPPORTED and the
  *   caller runs the norm entry point first.
- * After, in this order: Y = Y0 + bias (layers/linear.py:42-46); Y = act(Y); Y = Y + residual (the
- * blocks' residual `ops.add`, e.g. models/llama2/model.py:38-46). */
+ * After, in this order: Y = Y0 + bias (layers/linear.py:42-46); Y = act(Y); Y = Y * mul (the
+ * receptance gate of models/rwkv/ffn.py:58); Y = Y + residual (the blocks' residual `ops.add`, e.g.
+ * models/llama2/model.py:38-46); Y = Y * post_scale when post_scale != 0 (the halving of
+ * models/rwkv/model.py:115-116). */
 typedef struct pta_fusion {
   const pta_half* bias;        /* [N] or NULL                                   */
   const pta_half* residual;    /* [M, N] or NULL; may alias Y                   */
   int act;                     /* PTA_ACT_*                                     */
+  const pta_half* mul;         /* [M, N] or NULL                                */
+  float post_scale;            /* 0 = none                                      */
   int norm;                    /* PTA_NORM_*                                    */
   const pta_half* norm_weight; /* [K]                                           */
   const pta_half* norm_bias;   /* [K], PTA_NORM_LAYER only                      */
@@ -275,6 +279,9 @@ typedef struct pta_weight {
   const void* tiled;   /* from pta_w4_tile / pta_f16_tile / pta_fp8_tile                      */
   const void* scale;   /* INT4: fp16 [N]; FP8: device int32 exponent; FP16: NULL              */
   int N, K;
+  const pta_half* x;   /* NULL, or this weight's own input [M, K] instead of X (the three token-shift
+                          mixes of models/rwkv/attention.py:69-71 feed three Linears)          */
+  int act;             /* PTA_ACT_* applied to this weight's output in a multi-weight launch  */
 } pta_weight;
 
 /* Y_i[M, N_i] = fp16(X' @ W_i) + bias_i for `count` (1..4) weights of one kind and one K in one
@@ -288,6 +295,22 @@ int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_w
 /* out = up * swish(gate), two fp16 ops (models/llama2/mlp.py:22-26): the unfused form of the
  * SwiGLU pair, for gate/up weights that cannot share a launch. */
 int pta_swiglu(const pta_half* gate, const pta_half* up, pta_half* out, size_t n, pta_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * RWKV-4 recurrent step (models/rwkv/attention.py:59-105, models/rwkv/ffn.py:40-59)
+ * ---------------------------------------------------------------------------------- */
+
+/* Token-shift mixes o_i = x*w_i + (1 - w_i)*prev (fp16 ops of `gate`, attention.py:59-64) for one to
+ * three mixing vectors w_i [cols] (w1/w2 may be NULL), then prev <- x.  x, prev, o_i: [rows, cols]. */
+int pta_rwkv_mix(const pta_half* x, pta_half* prev, const pta_half* w0, const pta_half* w1, const pta_half* w2,
+                 pta_half* o0, pta_half* o1, pta_half* o2, int rows, int cols, pta_stream_t stream);
+
+/* The WKV recurrence in fp32 (attention.py:78-100) followed by y = r * fp16(out) (:101-103).
+ * k, v, r, y fp16 [rows, cols]; time_decay, time_first fp16 [cols]; num, den, max_state fp32
+ * [rows, cols], updated in place (initial values 0, 0, -1e30: models/rwkv/model.py:157-187). */
+int pta_rwkv_wkv(const pta_half* k, const pta_half* v, const pta_half* r, const pta_half* time_decay,
+                 const pta_half* time_first, float* num, float* den, float* max_state, pta_half* y, int rows, int cols,
+                 pta_stream_t stream);
 
 #ifdef __cplusplus
 }

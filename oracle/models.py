@@ -381,3 +381,152 @@ class ChatGLM2Oracle:
         logits = self.head(x)
         _, idx = O.topk1(logits, axis=2)
         return idx.reshape(B), logits.reshape(B, -1)
+
+
+# --------------------------------------------------------------------------------------
+# RWKV-4
+# --------------------------------------------------------------------------------------
+def make_rwkv_state_dict(cfg, seed=0, int4=True):
+    """Random-init RWKV-4-shaped checkpoint in the form the reference holds it after
+    RWKVDecodeModel.process_hf_model_state_dict (poptransformer/models/rwkv/model.py:150-155):
+    `attention.output.weight` and `feed_forward.value.weight` of block i divided by
+    2^(i // rescale_every).  Weights N(0, 0.02), time_decay U(-8, -1), time_first U(-1, 1),
+    time_mix_* U(0, 1), LayerNorm gamma 1 / beta 0; Linear weights packed INT4 when `int4`.
+    Keys: models/rwkv/model.py:34-42,81-94,129-148, attention.py:29-57, ffn.py:27-38, embedding.py:26-27."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, f, a, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["attention_hidden_size"], cfg["vocab_size"]
+    sd = {"rwkv.embeddings.weight": _normal(rng, (v, d))}
+
+    def linear(key, out_f, in_f, div=1.0):
+        w = (rng.standard_normal((out_f, in_f), dtype=f32) * 0.02 / div).astype(f16)
+        if int4:
+            sd[key + ".weight"], sd[key + ".weight_scale"] = quantize_int4(w)
+        else:
+            sd[key + ".weight"] = w
+
+    def ln(key):
+        sd[key + ".weight"], sd[key + ".bias"] = np.ones(d, f16), np.zeros(d, f16)
+
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"rwkv.blocks.{i}."
+        div = 2.0 ** (i // cfg["rescale_every"]) if cfg["rescale_every"] > 0 else 1.0
+        if i == 0:
+            ln(p + "pre_ln")
+        ln(p + "ln1")
+        ln(p + "ln2")
+        linear(p + "attention.key", a, d)
+        linear(p + "attention.value", a, d)
+        linear(p + "attention.receptance", a, d)
+        linear(p + "attention.output", d, a, div)
+        sd[p + "attention.time_decay"] = rng.uniform(-8, -1, d).astype(f16)
+        sd[p + "attention.time_first"] = rng.uniform(-1, 1, d).astype(f16)
+        for n in ("key", "value", "receptance"):
+            sd[p + f"attention.time_mix_{n}"] = rng.uniform(0, 1, (1, 1, d)).astype(f16)
+        linear(p + "feed_forward.key", f, d)
+        linear(p + "feed_forward.receptance", d, d)
+        linear(p + "feed_forward.value", d, f, div)
+        for n in ("key", "receptance"):
+            sd[p + f"feed_forward.time_mix_{n}"] = rng.uniform(0, 1, (1, 1, d)).astype(f16)
+    ln("rwkv.ln_out")
+    sd["head.weight"] = _normal(rng, (v, d))
+    return sd
+
+
+def _gate(a, w, b):
+    """BaseRWKVAttention.gate (poptransformer/models/rwkv/attention.py:59-64): fp16 ops."""
+    y1 = (a * w).astype(f16)
+    y2 = (f16(1) - w).astype(f16)
+    y2 = (y2 * b).astype(f16)
+    return (y1 + y2).astype(f16)
+
+
+class RWKVOracle:
+    """RWKVDecodeModel.build_model_graph (poptransformer/models/rwkv/model.py:189-213), RWKVModel.__call__
+    (:96-119), RWKVBlock (:44-53), BaseRWKVAttention (attention.py:66-105), BaseRWKVFeedforward
+    (ffn.py:47-59).  States per block (model.py:157-187): two fp16 token-shift rows and the fp32
+    numerator / denominator / maximum (-1e30).  The WKV arithmetic runs in fp32 as the reference does
+    under precision 'fp16' (attention.py:78-82); the same is assumed for INT4 Linear weights, where
+    the reference's `== 'fp16'` guard would leave fp16 operands next to fp32 states."""
+
+    def __init__(self, sd, cfg, max_length, batch_size):
+        self.cfg, self.L, self.B = cfg, max_length, batch_size
+        self.d = cfg["hidden_size"]
+        self.eps = cfg["layer_norm_epsilon"]
+        self.rescale = cfg["rescale_every"]
+        self.embed = sd["rwkv.embeddings.weight"]
+        self.layers = []
+        B, d = batch_size, self.d
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"rwkv.blocks.{i}."
+            lay = {n: (sd[p + n + ".weight"], sd[p + n + ".bias"]) for n in ("ln1", "ln2")}
+            if i == 0:
+                lay["pre_ln"] = (sd[p + "pre_ln.weight"], sd[p + "pre_ln.bias"])
+            for n in ("key", "value", "receptance", "output"):
+                lay["att_" + n] = _Linear(sd, p + "attention." + n, False)
+            for n in ("key", "receptance", "value"):
+                lay["ffn_" + n] = _Linear(sd, p + "feed_forward." + n, False)
+            lay["time_decay"] = sd[p + "attention.time_decay"]
+            lay["time_first"] = sd[p + "attention.time_first"]
+            for n in ("key", "value", "receptance"):
+                lay["att_mix_" + n] = sd[p + f"attention.time_mix_{n}"]
+            for n in ("key", "receptance"):
+                lay["ffn_mix_" + n] = sd[p + f"feed_forward.time_mix_{n}"]
+            lay["state"] = [np.zeros((B, 1, d), f16), np.zeros((B, 1, d), f16), np.zeros((B, 1, d), f32),
+                            np.zeros((B, 1, d), f32), np.full((B, 1, d), -1e30, f32)]
+            self.layers.append(lay)
+        self.ln_out = (sd["rwkv.ln_out.weight"], sd["rwkv.ln_out.bias"])
+        self.head = _Linear(sd, "head", False)
+
+    def _ln(self, x, wb):
+        return O.layer_norm_ce(x, wb[0], wb[1], self.eps, self.B, 1, self.d)
+
+    def _attention(self, lay, hidden):
+        st = lay["state"]
+        num, den, mx = st[2], st[3], st[4]
+        key = _gate(hidden, lay["att_mix_key"], st[1])
+        value = _gate(hidden, lay["att_mix_value"], st[1])
+        rec = _gate(hidden, lay["att_mix_receptance"], st[1])
+        st[1] = hidden
+        key, value = lay["att_key"](key), lay["att_value"](value)
+        rec = O.sigmoid(lay["att_receptance"](rec))
+        td, k, v, tf = lay["time_decay"].astype(f32), key.astype(f32), value.astype(f32), lay["time_first"].astype(f32)
+        t1 = (k + tf).astype(f32)
+        m_out = np.where(mx > t1, mx, t1)
+        with np.errstate(under="ignore"):
+            e1, e2 = np.exp(mx - m_out, dtype=f32), np.exp(t1 - m_out, dtype=f32)
+            out = ((e1 * num + e2 * v) / (e1 * den + e2)).astype(f32)
+            t2 = (mx - np.exp(td, dtype=f32)).astype(f32)
+            m_st = np.where(t2 > k, t2, k)
+            e1, e2 = np.exp(t2 - m_st, dtype=f32), np.exp(k - m_st, dtype=f32)
+        st[2] = (e1 * num + e2 * v).astype(f32)
+        st[3] = (e1 * den + e2).astype(f32)
+        st[4] = m_st.astype(f32)
+        out = (rec * out.astype(f16)).astype(f16)
+        return lay["att_output"](out)
+
+    def _ffn(self, lay, hidden):
+        st = lay["state"]
+        key = _gate(hidden, lay["ffn_mix_key"], st[0])
+        rec = _gate(hidden, lay["ffn_mix_receptance"], st[0])
+        st[0] = hidden
+        key = lay["ffn_key"](key)
+        key = np.maximum(key, f16(0))
+        key = (key * key).astype(f16)
+        value = lay["ffn_value"](key)
+        rec = O.sigmoid(lay["ffn_receptance"](rec))
+        return (rec * value).astype(f16)
+
+    def step(self, ids, step, mask=None):
+        B = self.B
+        hidden = self.embed[ids.reshape(B, 1)]
+        for i, lay in enumerate(self.layers):
+            if i == 0:
+                hidden = self._ln(hidden, lay["pre_ln"])
+            hidden = (hidden + self._attention(lay, self._ln(hidden, lay["ln1"]))).astype(f16)
+            hidden = (hidden + self._ffn(lay, self._ln(hidden, lay["ln2"]))).astype(f16)
+            if self.rescale > 0 and (i + 1) % self.rescale == 0:
+                hidden = (hidden / f16(2)).astype(f16)
+        hidden = self._ln(hidden, self.ln_out)
+        logits = self.head(hidden)
+        _, idx = O.topk1(logits, axis=2)
+        return idx.reshape(B), logits.reshape(B, -1)

@@ -24,14 +24,16 @@ NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
 
 
 class Weight(ctypes.Structure):
-    _fields_ = [("kind", c_int), ("tiled", c_void_p), ("scale", c_void_p), ("N", c_int), ("K", c_int)]
+    _fields_ = [("kind", c_int), ("tiled", c_void_p), ("scale", c_void_p), ("N", c_int), ("K", c_int),
+                ("x", c_void_p), ("act", c_int)]
 
 
 W_INT4, W_F16, W_F143, W_F152 = 0, 1, 2, 3
 
 
 class Fusion(ctypes.Structure):
-    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("norm", c_int),
+    _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("mul", c_void_p), ("post_scale", c_float),
+                ("norm", c_int),
                 ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float)]
 
 
@@ -74,6 +76,8 @@ SIGNATURES = {
     "pta_linear": (c_int, [c_void_p, c_void_p, c_int, POINTER(Weight), POINTER(c_void_p), POINTER(c_void_p), c_int, c_int,
                            POINTER(Fusion), c_void_p]),
     "pta_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "pta_rwkv_mix": (c_int, [c_void_p] * 8 + [c_int, c_int, c_void_p]),
+    "pta_rwkv_wkv": (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
 }

@@ -11,6 +11,8 @@ struct GemmEpilogue {
   const f16* bias;
   const f16* residual;
   int act;
+  const f16* mul;
+  float post_scale;
   int norm;                 // PTA_NORM_*, applied to the rows of X before the product
   const f16* norm_weight;
   const f16* norm_bias;
@@ -46,18 +48,21 @@ __device__ __forceinline__ f16 apply_act(int act, f16 y) {
 __device__ __forceinline__ f16 apply_epilogue(const GemmEpilogue& e, f16 y, int m, int n, int N) {
   if (e.bias) y = y + e.bias[n];
   y = apply_act(e.act, y);
+  if (e.mul) y = y * e.mul[(size_t)m * N + n];
   if (e.residual) y = y + e.residual[(size_t)m * N + n];
+  if (e.post_scale != 0.0f) y = y * (f16)e.post_scale;
   return y;
 }
 
 static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const char* name) {
-  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, PTA_NORM_NONE, nullptr, nullptr, 0.f};
+  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, nullptr, 0.f, PTA_NORM_NONE, nullptr, nullptr, 0.f};
   if (!in) return PTA_OK;
   PTA_REQUIRE(in->act >= PTA_ACT_NONE && in->act <= PTA_ACT_SIGMOID, "%s: unknown activation %d", name, in->act);
   PTA_REQUIRE(in->norm >= PTA_NORM_NONE && in->norm <= PTA_NORM_LAYER, "%s: unknown norm %d", name, in->norm);
   PTA_REQUIRE(in->norm == PTA_NORM_NONE || in->norm_weight, "%s: fused norm needs norm_weight", name);
   PTA_REQUIRE(in->norm != PTA_NORM_LAYER || in->norm_bias, "%s: fused LayerNorm needs norm_bias", name);
   out->bias = (const f16*)in->bias; out->residual = (const f16*)in->residual; out->act = in->act;
+  out->mul = (const f16*)in->mul; out->post_scale = in->post_scale;
   out->norm = in->norm; out->norm_weight = (const f16*)in->norm_weight; out->norm_bias = (const f16*)in->norm_bias;
   out->norm_eps = in->norm_eps;
   return PTA_OK;
@@ -78,6 +83,8 @@ struct GemmMat {
   const void* tiled;
   const void* scale;   // fp16 [N] (INT4), device int32 exponent (FP8), unused (FP16)
   const f16* bias;     // [N] or null; used when the launch holds several matrices
+  const f16* X;        // this matrix's own input, or null for the shared one
+  int act;             // activation of this matrix's output when the launch holds several
   f16* Y;
   int N;
   int nb_begin;        // first 16-channel block of this matrix in the launch grid
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
   for (int mt = 0; mt < MT; ++mt) {
     int m = mt * 16 + (lane & 15);
     m = m < a.M ? m : a.M - 1;
-    xrow[mt] = a.X + (size_t)m * K + (lane >> 4) * 8;
+    xrow[mt] = (a.mat[mi].X ? a.mat[mi].X : a.X) + (size_t)m * K + (lane >> 4) * 8;
   }
 
   f32x4 acc[NACC][MT];
@@ -196,6 +203,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
     } else {
       f16 y0 = (f16)sum[0];
       if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
+      y0 = apply_act(a.mat[mi].act, y0);
       a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
     }
   }
@@ -251,7 +259,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
     for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
       const int m = i / vec_per_row, c = i % vec_per_row;
       f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (c * 8 < K) v = *reinterpret_cast<const f16x8*>(a.X + (size_t)m * K + c * 8);
+      if (c * 8 < K) v = *reinterpret_cast<const f16x8*>((a.mat[mi].X ? a.mat[mi].X : a.X) + (size_t)m * K + c * 8);
       *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
       if (a.epi.norm != PTA_NORM_NONE) {
         float s1 = 0.f, s2 = 0.f;
@@ -359,6 +367,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
     } else {
       f16 y0 = (f16)sum[0];
       if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
+      y0 = apply_act(a.mat[mi].act, y0);
       a.mat[mi].Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
     }
   }

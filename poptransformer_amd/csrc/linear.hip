@@ -22,8 +22,9 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
   PTA_REQUIRE(count >= 1 && count <= 4, "pta_linear: count must be in [1, 4], got %d", count);
   PTA_REQUIRE(!swiglu || count == 2, "pta_linear: a SwiGLU pair is exactly two weights (gate, up)");
   const int kind = host_w[0].kind, K = host_w[0].K;
-  int rc = check_gemv_common("pta_linear", X, M, K);
+  int rc = check_gemv_common("pta_linear", X ? (const void*)X : (const void*)host_w[0].x, M, K);
   if (rc) return rc;
+  for (int i = 0; i < count; ++i) PTA_REQUIRE(X || host_w[i].x, "pta_linear: entry %d has no input", i);
   PTA_REQUIRE(kind >= PTA_W_INT4 && kind <= PTA_W_F152, "pta_linear: unknown weight kind %d", kind);
   GemmArgs a{};
   a.count = count; a.X = (const f16*)X; a.x_scale = x_scale; a.M = M; a.K = K; a.KT = (K + 127) / 128;
@@ -36,8 +37,11 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
     PTA_REQUIRE(kind == PTA_W_F16 || w.scale, "pta_linear: entry %d needs its scale", i);
     PTA_REQUIRE(pta_aligned(w.tiled, 16), "pta_linear: tiled[%d] must be 16-byte aligned", i);
     PTA_REQUIRE(!swiglu || w.N == host_w[0].N, "pta_linear: the SwiGLU weights must have the same shape");
-    a.mat[i] = GemmMat{w.tiled, w.scale, host_bias ? (const f16*)host_bias[i] : nullptr, (f16*)host_Y[i], w.N,
-                       swiglu ? 0 : nb};
+    PTA_REQUIRE(w.act >= PTA_ACT_NONE && w.act <= PTA_ACT_SIGMOID, "pta_linear: unknown activation %d in entry %d", w.act, i);
+    PTA_REQUIRE(!swiglu || (!w.x && w.act == PTA_ACT_NONE), "pta_linear: the SwiGLU pair shares X and takes no activation");
+    PTA_REQUIRE(!w.x || pta_aligned(w.x, 16), "pta_linear: x[%d] must be 16-byte aligned", i);
+    a.mat[i] = GemmMat{w.tiled, w.scale, host_bias ? (const f16*)host_bias[i] : nullptr, (const f16*)w.x, w.act,
+                       (f16*)host_Y[i], w.N, swiglu ? 0 : nb};
     nb += (w.N + 15) / 16;
   }
   if (swiglu) {
@@ -46,7 +50,7 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
   }
   rc = make_epilogue(fuse, &a.epi, "pta_linear");
   if (rc) return rc;
-  PTA_REQUIRE(count == 1 || (!a.epi.bias && !a.epi.residual && a.epi.act == PTA_ACT_NONE),
+  PTA_REQUIRE(count == 1 || (!a.epi.bias && !a.epi.residual && !a.epi.mul && a.epi.post_scale == 0.0f && a.epi.act == PTA_ACT_NONE),
               "pta_linear: with several weights only the norm fields of `fuse` apply (use host_bias for biases)");
   hipStream_t s = (hipStream_t)stream;
   switch (kind) {
@@ -62,7 +66,7 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
 // ------------------------------------------------------------------------------------------
 extern "C" int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y, int M, int K,
                               int N, const pta_fusion* fuse, pta_stream_t stream) {
-  pta_weight w{PTA_W_INT4, tiled, scale, N, K};
+  pta_weight w{PTA_W_INT4, tiled, scale, N, K, nullptr, PTA_ACT_NONE};
   return pta_linear(X, nullptr, 1, &w, nullptr, &Y, M, 0, fuse, stream);
 }
 
@@ -71,21 +75,22 @@ extern "C" int pta_w4a16_gemm_multi(const pta_half* X, int count, const void* co
                                     int M, int K, const pta_fusion* fuse, pta_stream_t stream) {
   PTA_REQUIRE(count >= 1 && count <= 4 && host_tiled && host_scale && host_N, "pta_w4a16_gemm_multi: bad arguments");
   pta_weight w[4];
-  for (int i = 0; i < count; ++i) w[i] = pta_weight{PTA_W_INT4, host_tiled[i], host_scale[i], host_N[i], K};
+  for (int i = 0; i < count; ++i) w[i] = pta_weight{PTA_W_INT4, host_tiled[i], host_scale[i], host_N[i], K, nullptr, PTA_ACT_NONE};
   return pta_linear(X, nullptr, count, w, nullptr, host_Y, M, 0, fuse, stream);
 }
 
 extern "C" int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_half* scale_gate,
                                      const void* tiled_up, const pta_half* scale_up, pta_half* Y, int M, int K, int F,
                                      const pta_fusion* fuse, pta_stream_t stream) {
-  pta_weight w[2] = {{PTA_W_INT4, tiled_gate, scale_gate, F, K}, {PTA_W_INT4, tiled_up, scale_up, F, K}};
+  pta_weight w[2] = {{PTA_W_INT4, tiled_gate, scale_gate, F, K, nullptr, PTA_ACT_NONE},
+                     {PTA_W_INT4, tiled_up, scale_up, F, K, nullptr, PTA_ACT_NONE}};
   pta_half* ys[2] = {Y, Y};
   return pta_linear(X, nullptr, 2, w, nullptr, ys, M, 1, fuse, stream);
 }
 
 extern "C" int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
                             const pta_fusion* fuse, pta_stream_t stream) {
-  pta_weight w{PTA_W_F16, tiled, nullptr, N, K};
+  pta_weight w{PTA_W_F16, tiled, nullptr, N, K, nullptr, PTA_ACT_NONE};
   return pta_linear(X, nullptr, 1, &w, nullptr, &Y, M, 0, fuse, stream);
 }
 
@@ -111,6 +116,6 @@ extern "C" int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_r
     X = (const f16*)workspace;
     xs = scale_lhs;
   }
-  pta_weight w{format_rhs == PTA_F143 ? PTA_W_F143 : PTA_W_F152, tiled_rhs, scale_rhs, N, K};
+  pta_weight w{format_rhs == PTA_F143 ? PTA_W_F143 : PTA_W_F152, tiled_rhs, scale_rhs, N, K, nullptr, PTA_ACT_NONE};
   return pta_linear((const pta_half*)X, xs, 1, &w, nullptr, &Y, M, 0, fuse, stream);
 }

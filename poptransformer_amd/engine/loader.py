@@ -116,3 +116,38 @@ def chatglm2_spec(cfg, max_len, batch, pad_id=0, eos_id=2, early_stop=False):
     d, h = cfg["hidden_size"], cfg["num_attention_heads"]
     return DecoderSpec("chatglm2", cfg["num_layers"], d, h, cfg["multi_query_group_num"], d // h,
                        cfg["padded_vocab_size"], max_len, batch, cfg["layernorm_epsilon"], pad_id, eos_id, early_stop)
+
+
+def rwkv_weights(sd, cfg, device="cuda"):
+    from .rwkv import RWKVBlockWeights, RWKVWeights
+
+    def ln(key):
+        return (_dev(sd[key + ".weight"], device), _dev(sd[key + ".bias"], device))
+
+    def vec(key):
+        return _dev(np.asarray(sd[key], np.float16).reshape(-1), device)
+
+    blocks = []
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"rwkv.blocks.{i}."
+        blocks.append(RWKVBlockWeights(
+            pre_ln=ln(p + "pre_ln") if i == 0 else None, ln1=ln(p + "ln1"), ln2=ln(p + "ln2"),
+            att_key=linear_from_state_dict(sd, p + "attention.key", False, device),
+            att_value=linear_from_state_dict(sd, p + "attention.value", False, device),
+            att_receptance=linear_from_state_dict(sd, p + "attention.receptance", False, device),
+            att_output=linear_from_state_dict(sd, p + "attention.output", False, device),
+            time_decay=vec(p + "attention.time_decay"), time_first=vec(p + "attention.time_first"),
+            att_mix=[vec(p + f"attention.time_mix_{n}") for n in ("key", "value", "receptance")],
+            ffn_key=linear_from_state_dict(sd, p + "feed_forward.key", False, device),
+            ffn_receptance=linear_from_state_dict(sd, p + "feed_forward.receptance", False, device),
+            ffn_value=linear_from_state_dict(sd, p + "feed_forward.value", False, device),
+            ffn_mix=[vec(p + f"feed_forward.time_mix_{n}") for n in ("key", "receptance")]))
+    return RWKVWeights(embed=_dev(sd["rwkv.embeddings.weight"], device), blocks=blocks, ln_out=ln("rwkv.ln_out"),
+                       head=linear_from_state_dict(sd, "head", False, device))
+
+
+def rwkv_spec(cfg, max_len, batch, pad_id=0, eos_id=-1, early_stop=False):
+    from .rwkv import RWKVSpec
+    return RWKVSpec(cfg["num_hidden_layers"], cfg["hidden_size"], cfg["attention_hidden_size"], cfg["intermediate_size"],
+                    cfg["vocab_size"], max_len, batch, cfg["layer_norm_epsilon"], cfg["rescale_every"], pad_id, eos_id,
+                    early_stop)

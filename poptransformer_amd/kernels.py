@@ -49,10 +49,10 @@ def norm_fusable(M, K):
     return M <= 4 and M * (((K + 127) // 128) * 128 + 8) * 2 <= 40 * 1024
 
 
-def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None):
-    if bias is None and residual is None and act == _lib.ACT_NONE and norm is None:
+def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0):
+    if bias is None and residual is None and act == _lib.ACT_NONE and norm is None and mul is None and not post_scale:
         return None
-    e = Fusion(_p(bias), _p(residual), act, norm.kind if norm else _lib.NORM_NONE,
+    e = Fusion(_p(bias), _p(residual), act, _p(mul), float(post_scale), norm.kind if norm else _lib.NORM_NONE,
                _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0)
     return ctypes.byref(e)
 
@@ -244,25 +244,30 @@ def half_to_fp8_grid(x, scale, fp8_format="F143", out=None):
 
 
 # ------------------------------------------------------------------ general Linear -------
-def _desc(w):
+def _desc(w, x=None, act=_lib.ACT_NONE):
+    xp = x.data_ptr() if x is not None else None
     if isinstance(w, W4Weight):
-        return _lib.Weight(_lib.W_INT4, w.tiled.data_ptr(), w.scale.data_ptr(), w.N, w.K)
+        return _lib.Weight(_lib.W_INT4, w.tiled.data_ptr(), w.scale.data_ptr(), w.N, w.K, xp, act)
     if isinstance(w, F16Weight):
-        return _lib.Weight(_lib.W_F16, w.tiled.data_ptr(), None, w.N, w.K)
+        return _lib.Weight(_lib.W_F16, w.tiled.data_ptr(), None, w.N, w.K, xp, act)
     if isinstance(w, F8Weight):
         return _lib.Weight(_lib.W_F143 if w.format == _lib.F143 else _lib.W_F152, w.tiled.data_ptr(), w.scale.data_ptr(),
-                           w.N, w.K)
+                           w.N, w.K, xp, act)
     raise TypeError(f"not a tiled weight: {type(w)}")
 
 
 def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None, residual=None, act=_lib.ACT_NONE,
-           norm=None):
-    """pta_linear: up to four weights of one kind sharing x.  `biases` is a per-weight list (or None);
-    bias/residual/act apply to the single-weight form only."""
+           norm=None, mul=None, post_scale=0.0, xs=None, acts=None):
+    """pta_linear: up to four weights of one kind.  They share x, or each takes its own input from
+    `xs`.  `biases` / `acts` are per-weight lists (or None); bias / residual / act / mul / post_scale
+    apply to the single-weight form only."""
+    if xs is not None:
+        x = xs[0]
     _need(x, torch.float16, "x", 2)
     M = x.shape[0]
     n = len(weights)
-    descs = (_lib.Weight * n)(*[_desc(w) for w in weights])
+    descs = (_lib.Weight * n)(*[_desc(w, xs[i] if xs is not None else None, acts[i] if acts is not None else _lib.ACT_NONE)
+                                for i, w in enumerate(weights)])
     VP = ctypes.c_void_p * n
     ys = VP(*[o.data_ptr() for o in outs])
     bs = None
@@ -272,7 +277,7 @@ def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None,
         if w.K != x.shape[1]:
             raise ValueError(f"matmul: contracting dimensions differ ({x.shape[1]} vs {w.K})")
     check(_lib.load().pta_linear(_p(x), _p(x_scale), n, descs, bs, ys, M, 1 if swiglu else 0,
-                                 _fusion(bias, residual, act, norm), _stream()))
+                                 _fusion(bias, residual, act, norm, mul, post_scale), _stream()))
     return outs
 
 
@@ -412,3 +417,21 @@ def step_update(container, mask, stop_mask, step, next_ids, ids_out, keep_going,
     check(_lib.load().pta_step_update(_p(container), _p(mask), _p(stop_mask), _p(step), _p(next_ids), _p(ids_out),
                                       _p(keep_going), B, max_len, int(pad_id), int(eos_id), 1 if early_stop else 0,
                                       _stream()))
+
+
+# ------------------------------------------------------------------ RWKV -----------------
+def rwkv_mix(x, prev, ws, outs):
+    """Token-shift mixes for 1..3 mixing vectors; prev is overwritten with x."""
+    rows, cols = x.shape
+    w = list(ws) + [None] * (3 - len(ws))
+    o = list(outs) + [None] * (3 - len(outs))
+    check(_lib.load().pta_rwkv_mix(_p(x), _p(prev), _p(w[0]), _p(w[1]), _p(w[2]), _p(o[0]), _p(o[1]), _p(o[2]), rows, cols,
+                                   _stream()))
+    return outs
+
+
+def rwkv_wkv(k, v, r, time_decay, time_first, num, den, max_state, y):
+    rows, cols = k.shape
+    check(_lib.load().pta_rwkv_wkv(_p(k), _p(v), _p(r), _p(time_decay), _p(time_first), _p(num), _p(den), _p(max_state),
+                                   _p(y), rows, cols, _stream()))
+    return y

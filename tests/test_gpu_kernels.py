@@ -440,6 +440,50 @@ def test_rope_bit_exact(K):
         assert np.array_equal(r[1, :, :, it], v)
 
 
+# ---------------------------------------------------------------- RWKV pieces
+def test_rwkv_mix_bit_exact_and_wkv(K):
+    rng = np.random.default_rng(41)
+    B, d = 3, 256
+    x = rng.standard_normal((B, d)).astype(np.float16)
+    prev = rng.standard_normal((B, d)).astype(np.float16)
+    ws = [rng.uniform(0, 1, d).astype(np.float16) for _ in range(3)]
+    outs = [torch.empty((B, d), dtype=torch.float16, device="cuda") for _ in range(3)]
+    pd = dev(prev)
+    K.rwkv_mix(dev(x), pd, [dev(w) for w in ws], outs)
+    for w, o in zip(ws, outs):
+        assert np.array_equal(host(o).view(np.uint16), OM_gate(x, w, prev).view(np.uint16))
+    assert np.array_equal(host(pd), x)
+    # WKV: three consecutive steps against the fp32 closed form
+    k = [rng.standard_normal((B, d)).astype(np.float16) for _ in range(3)]
+    v = [rng.standard_normal((B, d)).astype(np.float16) for _ in range(3)]
+    r = [rng.uniform(0, 1, (B, d)).astype(np.float16) for _ in range(3)]
+    td = rng.uniform(-8, -1, d).astype(np.float16)
+    tf = rng.uniform(-1, 1, d).astype(np.float16)
+    num = torch.zeros((B, d), dtype=torch.float32, device="cuda")
+    den = torch.zeros_like(num)
+    mx = torch.full_like(num, -1e30)
+    a = np.zeros((B, d), np.float64); b = np.zeros((B, d), np.float64); p = np.full((B, d), -1e30)
+    y = torch.empty((B, d), dtype=torch.float16, device="cuda")
+    for t in range(3):
+        K.rwkv_wkv(dev(k[t]), dev(v[t]), dev(r[t]), dev(td), dev(tf), num, den, mx, y)
+        kk, vv = k[t].astype(np.float64), v[t].astype(np.float64)
+        t1 = kk + tf.astype(np.float64)
+        M = np.maximum(p, t1)
+        out = (np.exp(p - M) * a + np.exp(t1 - M) * vv) / (np.exp(p - M) * b + np.exp(t1 - M))
+        p2 = p - np.exp(td.astype(np.float64))
+        M2 = np.maximum(p2, kk)
+        a, b, p = np.exp(p2 - M2) * a + np.exp(kk - M2) * vv, np.exp(p2 - M2) * b + np.exp(kk - M2), M2
+        ref = r[t].astype(np.float64) * out
+        assert np.abs(host(y).astype(np.float64) - ref).max() <= 2e-3 * max(1.0, np.abs(ref).max())
+        assert np.abs(host(num) - a).max() <= 1e-4 * max(1.0, np.abs(a).max())
+        assert np.abs(host(mx) - p).max() <= 1e-5 * np.abs(p).max()
+
+
+def OM_gate(a, w, b):
+    from oracle.models import _gate
+    return _gate(a, w, b)
+
+
 # ---------------------------------------------------------------- selection & loop
 @pytest.mark.parametrize("rows,n", [(1, 32000), (16, 50257), (3, 65536), (2, 5)])
 def test_argmax(K, rows, n):

@@ -83,6 +83,26 @@ def test_chatglm2_decode_matches_oracle(precision):
     _compare(dec, oracle, ids, L, steps, pad, eos, tol=1e-1 if precision == "fp8" else 1e-2)
 
 
+RWKV_TINY = dict(hidden_size=256, intermediate_size=512, attention_hidden_size=256, layer_norm_epsilon=1e-5,
+                 vocab_size=500, num_hidden_layers=4, rescale_every=2)
+
+
+@pytest.mark.parametrize("B,int4", [(1, True), (3, True), (2, False)])
+def test_rwkv_decode_matches_oracle(B, int4):
+    from poptransformer_amd.engine import loader, rwkv
+    L, steps, pad, eos = 48, 32, 0, 499
+    sd = OM.make_rwkv_state_dict(RWKV_TINY, seed=6, int4=int4)
+    oracle = OM.RWKVOracle(sd, RWKV_TINY, L, B)
+    dec = rwkv.RWKVDecoder(loader.rwkv_spec(RWKV_TINY, L, B, pad, eos), loader.rwkv_weights(sd, RWKV_TINY))
+    ids = _prompt(np.random.default_rng(11), B, L, 9, 490, pad)
+    _compare(dec, oracle, ids, L, steps, pad, eos)
+    # a second generation starts from fresh states
+    dec.capture()
+    c, st = dec.run(ids, steps)
+    ref_c, ref_s = OM.run_decode_loop(OM.RWKVOracle(sd, RWKV_TINY, L, B), ids, L, steps, pad, eos)
+    assert np.array_equal(c, ref_c) and st == ref_s
+
+
 def test_llama2_graph_replay_equals_eager():
     from poptransformer_amd.engine import fused, loader
     B, L, pad, eos = 2, 40, 0, 2

@@ -106,3 +106,41 @@ def test_quantize_int4_roundtrip_error_bound():
     assert p.dtype == np.int8 and p.shape == (8, 32) and s.dtype == f16
     wq = O.int4_to_half(p, s, 1).T.astype(f32)
     assert np.abs(wq - w.astype(f32)).max() <= 0.5 * s.astype(f32).max() * 1.01
+
+
+def test_rwkv_oracle_against_hf():
+    from transformers import RwkvConfig, RwkvForCausalLM
+    torch.manual_seed(2)
+    hf_cfg = RwkvConfig(vocab_size=150, context_length=32, hidden_size=64, num_hidden_layers=4, attention_hidden_size=64,
+                        intermediate_size=128, layer_norm_epsilon=1e-5, rescale_every=2)
+    hf = RwkvForCausalLM(hf_cfg).eval()
+    with torch.no_grad():
+        for n, p in hf.named_parameters():
+            if "time_decay" in n:
+                p.copy_(torch.empty_like(p).uniform_(-6, -1))
+            elif "time_first" in n:
+                p.copy_(torch.empty_like(p).uniform_(-1, 1))
+            elif "time_mix" in n:
+                p.copy_(torch.empty_like(p).uniform_(0.1, 0.9))
+            elif "ln" in n:
+                p.add_(torch.randn_like(p) * 0.05)
+            else:
+                p.mul_(3.0)                                     # make the projections matter
+    cfg = dict(hidden_size=64, intermediate_size=128, attention_hidden_size=64, layer_norm_epsilon=1e-5, vocab_size=150,
+               num_hidden_layers=4, rescale_every=2)
+    # the reference's load-time processing (rwkv/model.py:150-155), applied to a copy
+    sd = {}
+    for k, v in hf.state_dict().items():
+        a = v.detach().numpy().astype(f32).copy()
+        if k.endswith("attention.output.weight") or k.endswith("feed_forward.value.weight"):
+            a /= 2 ** (int(k.split(".")[2]) // 2)
+        sd[k] = a.astype(f16)
+    L, B = 10, 2
+    model = OM.RWKVOracle(sd, cfg, L, B)
+    rng = np.random.default_rng(3)
+    toks = rng.integers(0, 150, size=(B, L)).astype(np.int32)
+    with torch.no_grad():
+        ref_all = hf(torch.from_numpy(toks.astype(np.int64))).logits.numpy()   # eval mode rescales the same way
+    for step in range(L):
+        _, logits = model.step(toks[:, step].reshape(B, 1), step)
+        assert _rel(logits, ref_all[:, step]) < 3e-2, f"step {step}"
