@@ -312,6 +312,60 @@ int pta_rwkv_wkv(const pta_half* k, const pta_half* v, const pta_half* r, const 
                  const pta_half* time_first, float* num, float* den, float* max_state, pta_half* y, int rows, int cols,
                  pta_stream_t stream);
 
+/* ------------------------------------------------------------------------------------
+ * One whole loop iteration in one launch (models/base_model.py:271-355 driving
+ * models/llama2/model.py:162-197: embedding, every decoder layer, final RMSNorm, lm_head,
+ * top-1, container / mask / stop-mask update).  The reference compiles this loop body into one
+ * Poplar program; this entry is its counterpart for INT4 Llama-2 shapes: a single persistent
+ * kernel, one workgroup per compute unit, phases separated by a grid-wide barrier, the weights of
+ * the next phase requested before each barrier.  Results equal those of the per-operator entry
+ * points above run in the reference's order.
+ * ---------------------------------------------------------------------------------- */
+
+typedef struct pta_decode_layer {
+  const void *wq, *wk, *wv, *wo, *wg, *wu, *wd;       /* INT4 weights tiled by pta_w4_tile            */
+  const pta_half *sq, *sk, *sv, *so, *sg, *su, *sd;   /* their per-output-channel scales              */
+  const pta_half *norm1, *norm2;                      /* RMSNorm weights [hidden]                     */
+  pta_half* kv_ring;                                  /* ring of pta_qkv_rope_append for this layer   */
+} pta_decode_layer;
+
+typedef struct pta_decode_model {
+  const pta_decode_layer* layers;                     /* DEVICE array [n_layer]                       */
+  int n_layer;
+  const pta_half* embed;                              /* [vocab, hidden]                              */
+  const pta_half* final_norm;                         /* [hidden]                                     */
+  const void* head;                                   /* lm_head [vocab, hidden] tiled by pta_f16_tile */
+  const pta_half* inv_freq;                           /* rotary inverse frequencies, fp16 [head_dim/2] */
+  int batch, hidden, n_head, head_dim, ffn, vocab, max_len;
+  float eps;
+  int pad_id, eos_id, early_stop;                     /* as pta_step_update                           */
+} pta_decode_model;
+
+typedef struct pta_decode_state {
+  int32_t* container;                                 /* [batch, max_len]                             */
+  pta_half* mask;                                     /* [batch, max_len]                             */
+  int32_t* stop_mask;                                 /* [batch]                                      */
+  int32_t* step;                                      /* [1]                                          */
+  int32_t* keep_going;                                /* [1]; 0 makes the launch a no-op              */
+  int32_t* next_ids;                                  /* [batch] out: the selected tokens             */
+  pta_half *x, *qkv, *ctx, *act, *logits;             /* [batch, hidden | 3 hidden | hidden | ffn | vocab] */
+} pta_decode_state;
+
+/* Bytes of the workspace of pta_llama_decode_step on the current device; 0 for unsupported shapes.
+ * The caller zeroes it once after allocating it; the kernel keeps it consistent afterwards. */
+size_t pta_decode_step_workspace_bytes(int batch, int n_head, int head_dim);
+
+/* Enqueues one loop iteration.  Supports batch <= 4, head_dim 128, hidden = n_head * 128 with
+ * (hidden, ffn) of the 7B and 13B models or a small test shape; PTA_EUNSUPPORTED otherwise.
+ * Needs every compute unit of the device for itself while it runs: the grid barrier waits a bounded
+ * time for all workgroups and, if one never arrives, sets word 1 of the workspace (sticky), leaves
+ * the loop state untouched and ends; pta_decode_step_failed reports it. */
+int pta_llama_decode_step(const pta_decode_model* model, const pta_decode_state* state, void* workspace,
+                          pta_stream_t stream);
+
+/* Copies the failure word of the workspace to *failed (synchronises with `stream`). */
+int pta_decode_step_failed(const void* workspace, int* failed, pta_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -31,6 +31,24 @@ class Weight(ctypes.Structure):
 W_INT4, W_F16, W_F143, W_F152 = 0, 1, 2, 3
 
 
+class DecodeLayer(ctypes.Structure):
+    _fields_ = [(n, c_void_p) for n in ("wq", "wk", "wv", "wo", "wg", "wu", "wd", "sq", "sk", "sv", "so", "sg", "su",
+                                        "sd", "norm1", "norm2", "kv_ring")]
+
+
+class DecodeModel(ctypes.Structure):
+    _fields_ = [("layers", c_void_p), ("n_layer", c_int), ("embed", c_void_p), ("final_norm", c_void_p),
+                ("head", c_void_p), ("inv_freq", c_void_p),
+                ("batch", c_int), ("hidden", c_int), ("n_head", c_int), ("head_dim", c_int), ("ffn", c_int),
+                ("vocab", c_int), ("max_len", c_int), ("eps", c_float),
+                ("pad_id", c_int), ("eos_id", c_int), ("early_stop", c_int)]
+
+
+class DecodeState(ctypes.Structure):
+    _fields_ = [(n, c_void_p) for n in ("container", "mask", "stop_mask", "step", "keep_going", "next_ids", "x", "qkv",
+                                        "ctx", "act", "logits")]
+
+
 class Fusion(ctypes.Structure):
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("mul", c_void_p), ("post_scale", c_float),
                 ("norm", c_int),
@@ -80,6 +98,9 @@ SIGNATURES = {
     "pta_rwkv_wkv": (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
+    "pta_decode_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "pta_llama_decode_step": (c_int, [POINTER(DecodeModel), POINTER(DecodeState), c_void_p, c_void_p]),
+    "pta_decode_step_failed": (c_int, [c_void_p, POINTER(c_int), c_void_p]),
 }
 
 _lib = None

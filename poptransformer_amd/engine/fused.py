@@ -144,6 +144,35 @@ class FusedDecoder:
         # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
         self._fp8_buf = {k: buf(B, k) for k in {d, ffn}}
         self._gate, self._up = buf(B, ffn), buf(B, ffn)
+        self.persistent = None
+
+    def enable_persistent(self):
+        """Run each loop iteration as one persistent launch (pta_llama_decode_step) instead of one
+        launch per operator.  Raises NotImplementedError when the model is not an INT4 Llama-2
+        shape the kernel covers; the per-operator path stays available through `persistent = None`."""
+        s, w = self.spec, self.w
+        if s.family != "llama2" or s.n_kv_head != s.n_head:
+            raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
+        lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
+        if not all(lw.is_int4 and lw.bias is None for lw in lins):
+            raise NotImplementedError("the persistent decode step needs bias-free INT4 Linears")
+        if not isinstance(w.head.w, K.F16Weight) or w.head.bias is not None:
+            raise NotImplementedError("the persistent decode step needs a bias-free fp16 lm_head")
+        layers = []
+        for b, ring in zip(w.blocks, self.rings):
+            q, k, v = b.qkv
+            g, u = b.mlp_in
+            layers.append(dict(wq=q.w.tiled, wk=k.w.tiled, wv=v.w.tiled, wo=b.out.w.tiled, wg=g.w.tiled, wu=u.w.tiled,
+                               wd=b.mlp_out.w.tiled, sq=q.w.scale, sk=k.w.scale, sv=v.w.scale, so=b.out.w.scale,
+                               sg=g.w.scale, su=u.w.scale, sd=b.mlp_out.w.scale, norm1=b.norm1[0], norm2=b.norm2[0],
+                               kv_ring=ring))
+        state = dict(container=self.container, mask=self.mask, stop_mask=self.stop_mask, step=self.step,
+                     keep_going=self.keep_going, next_ids=self.next_ids, x=self.x, qkv=self.qkv, ctx=self.ctx,
+                     act=self.act, logits=self.logits)
+        self.persistent = K.DecodeStep(layers, w.embed, w.final_norm[0], w.head.w.tiled, w.inv_freq, s.batch, s.d_model,
+                                       s.n_head, s.head_dim, w.blocks[0].mlp_out.K, s.vocab, s.max_len, s.eps, s.pad_id,
+                                       s.eos_id, s.early_stop, state)
+        return self
 
     # ------------------------------------------------------------------ one loop iteration
     def _norm(self, x, gb, out):
@@ -191,6 +220,9 @@ class FusedDecoder:
             self._linear(x, lw, o, norm=norm)
 
     def step_fn(self):
+        if self.persistent is not None:
+            self.persistent.launch()
+            return
         s, w = self.spec, self.w
         B = s.batch
         K.embedding(w.embed, self.container, self.x, pos_table=w.pos_embed,
@@ -283,4 +315,7 @@ class FusedDecoder:
             if self.spec.early_stop and int(self.keep_going.item()) == 0:
                 break
         torch.cuda.synchronize()
+        if self.persistent is not None and self.persistent.failed():
+            raise RuntimeError("persistent decode step: a workgroup never reached the grid barrier (the kernel needs "
+                               "every compute unit of the device while it runs); the loop state was not advanced")
         return self.container.cpu().numpy(), int(self.step.item())

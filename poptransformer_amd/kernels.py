@@ -435,3 +435,38 @@ def rwkv_wkv(k, v, r, time_decay, time_first, num, den, max_state, y):
     check(_lib.load().pta_rwkv_wkv(_p(k), _p(v), _p(r), _p(time_decay), _p(time_first), _p(num), _p(den), _p(max_state),
                                    _p(y), rows, cols, _stream()))
     return y
+
+
+class DecodeStep:
+    """One whole loop iteration of an INT4 Llama-2-shaped decoder in a single persistent launch
+    (pta_llama_decode_step).  Holds the device copies of the layer descriptors and the workspace;
+    raises NotImplementedError for shapes the kernel does not cover."""
+
+    def __init__(self, layers, embed, final_norm, head, inv_freq, batch, hidden, n_head, head_dim, ffn, vocab, max_len,
+                 eps, pad_id, eos_id, early_stop, state):
+        lib = _lib.load()
+        nbytes = lib.pta_decode_step_workspace_bytes(batch, n_head, head_dim)
+        if nbytes == 0:
+            raise NotImplementedError(f"decode step kernel: unsupported batch {batch} / head size {head_dim}")
+        dev = embed.device
+        self.workspace = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        arr = (_lib.DecodeLayer * len(layers))()
+        for dst, src in zip(arr, layers):
+            for name, t in src.items():
+                setattr(dst, name, t.data_ptr())
+        host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
+        self.layers = host.to(dev)
+        self._keep = (layers, embed, final_norm, head, inv_freq, state)
+        self.model = _lib.DecodeModel(self.layers.data_ptr(), len(layers), embed.data_ptr(), final_norm.data_ptr(),
+                                      head.data_ptr(), inv_freq.data_ptr(), batch, hidden, n_head, head_dim, ffn, vocab,
+                                      max_len, eps, pad_id, eos_id, 1 if early_stop else 0)
+        self.state = _lib.DecodeState(**{k: v.data_ptr() for k, v in state.items()})
+
+    def launch(self):
+        check(_lib.load().pta_llama_decode_step(ctypes.byref(self.model), ctypes.byref(self.state), _p(self.workspace),
+                                                _stream()))
+
+    def failed(self):
+        flag = ctypes.c_int(0)
+        check(_lib.load().pta_decode_step_failed(_p(self.workspace), ctypes.byref(flag), _stream()))
+        return bool(flag.value)
