@@ -7,9 +7,13 @@ attention over the cache, residuals), final norm, fp16 lm_head, greedy selection
 bookkeeping.  The default run follows the headline configuration: batch 1, a 128-token prompt
 consumed token by token (the untimed warm-up), then 256 timed new tokens, KV cache length 2048.
 
-Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel (the fused INT4
-gate/up projection) measured with events on its own stream, and a CPU baseline (the numpy
-restatement of the same graph on the host cores, on a reduced number of layers).
+By default the iteration runs as one persistent launch (pta_llama_decode_step, batch <= 4);
+``--executor operators`` runs it as one launch per operator instead.
+
+Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel measured with events
+on the stream it runs on (the persistent decode-step kernel: one launch moves the whole step's
+bytes; or, with the per-operator executor, the fused INT4 gate/up projection), and a CPU baseline
+(the numpy restatement of the same graph on the host cores, on a reduced number of layers).
 """
 import argparse
 import json
@@ -87,6 +91,8 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=128)
     ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
+                    help="default: persistent when the batch fits it (<= 4), else operators")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -106,6 +112,9 @@ def main():
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
+    executor = args.executor or ("persistent" if B <= 4 else "operators")
+    if executor == "persistent":
+        dec.enable_persistent()
     dec.capture()
 
     rng = np.random.Generator(np.random.PCG64(1234))
@@ -125,30 +134,52 @@ def main():
     mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(args.warmup, args.warmup + args.steps)])
     step_frac = mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9)
 
-    # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
-    # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
-    # (1.4 GB in total, so no launch finds its weights in a cache).
-    d, f = cfg["hidden_size"], cfg["intermediate_size"]
     stream = torch.cuda.Stream()
-    reps = 10
-    with torch.cuda.stream(stream):
-        for blk in weights.blocks:
-            K.w4a16_gemm_swiglu(dec.h, blk.mlp_in[0].w, blk.mlp_in[1].w, dec.act)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        g = torch.cuda.CUDAGraph()
-        stream.synchronize()
-        with torch.cuda.graph(g, stream=stream):
+    if executor == "persistent":
+        if dec.persistent.failed():
+            print("the persistent decode step reported a failure", file=sys.stderr)
+            sys.exit(1)
+        # Dominant kernel: the decode-step kernel itself, one launch per step.  Timed with events on the
+        # stream it is launched on, continuing the generation (so the context keeps growing as it does in
+        # the timed region above); its algorithmic bytes are the step's.
+        reps = min(64, MAX_LEN - 2 - args.warmup - args.steps)
+        t_first = args.warmup + args.steps
+        with torch.cuda.stream(stream):
+            stream.wait_stream(torch.cuda.current_stream())
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                dec.persistent.launch()
+            e1.record(stream)
+        torch.cuda.synchronize()
+        kernel_s = e0.elapsed_time(e1) * 1e-3 / reps
+        kernel_bytes = float(np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(t_first, t_first + reps)]))
+        kernel_name = "decode_step_kernel<2, 6, 3, %d> (whole decode step)" % (1 if B == 1 else 4)
+    else:
+        # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
+        # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
+        # (1.4 GB in total, so no launch finds its weights in a cache).
+        d, f = cfg["hidden_size"], cfg["intermediate_size"]
+        reps = 10
+        with torch.cuda.stream(stream):
             for blk in weights.blocks:
                 K.w4a16_gemm_swiglu(dec.h, blk.mlp_in[0].w, blk.mlp_in[1].w, dec.act)
-        g.replay()
-        e0.record(stream)
-        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            g = torch.cuda.CUDAGraph()
+            stream.synchronize()
+            with torch.cuda.graph(g, stream=stream):
+                for blk in weights.blocks:
+                    K.w4a16_gemm_swiglu(dec.h, blk.mlp_in[0].w, blk.mlp_in[1].w, dec.act)
             g.replay()
-        e1.record(stream)
-    torch.cuda.synchronize()
-    launches = reps * len(weights.blocks)
-    kernel_s = e0.elapsed_time(e1) * 1e-3 / launches
-    kernel_bytes = 2 * (d * f // 2 + 2 * f) + B * d * 2 + B * f * 2
+            e0.record(stream)
+            for _ in range(reps):
+                g.replay()
+            e1.record(stream)
+        torch.cuda.synchronize()
+        launches = reps * len(weights.blocks)
+        kernel_s = e0.elapsed_time(e1) * 1e-3 / launches
+        kernel_bytes = 2 * (d * f // 2 + 2 * f) + B * d * 2 + B * f * 2
+        kernel_name = "gemv_lds_kernel<FmtW4, 8, true> (INT4 gate/up + SwiGLU)"
     achieved = kernel_bytes / kernel_s / 1e9
 
     out = {
@@ -158,9 +189,9 @@ def main():
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"Llama2-7B-shape INT4 greedy decode, batch {B}, prompt {prompt} consumed token by token, "
                                f"context {args.warmup}..{args.warmup + args.steps - 1}, fp16 KV cache length {MAX_LEN}",
-                   "batch": B, "kv_cache_len": MAX_LEN},
+                   "batch": B, "kv_cache_len": MAX_LEN, "executor": executor},
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
-        "roofline": {"bound": "hbm", "kernel": "gemv_mfma_kernel<FmtW4, 1, 8, true> (INT4 gate/up + SwiGLU)",
+        "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": None, "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }

@@ -318,8 +318,8 @@ int pta_rwkv_wkv(const pta_half* k, const pta_half* v, const pta_half* r, const 
  * top-1, container / mask / stop-mask update).  The reference compiles this loop body into one
  * Poplar program; this entry is its counterpart for INT4 Llama-2 shapes: a single persistent
  * kernel, one workgroup per compute unit, phases separated by a grid-wide barrier, the weights of
- * the next phase requested before each barrier.  Results equal those of the per-operator entry
- * points above run in the reference's order.
+ * later phases requested early.  Results equal those of the per-operator entry points above run in the
+ * reference's order, up to the order in which attention partial sums are merged.
  * ---------------------------------------------------------------------------------- */
 
 typedef struct pta_decode_layer {
@@ -348,18 +348,20 @@ typedef struct pta_decode_state {
   int32_t* step;                                      /* [1]                                          */
   int32_t* keep_going;                                /* [1]; 0 makes the launch a no-op              */
   int32_t* next_ids;                                  /* [batch] out: the selected tokens             */
-  pta_half *x, *qkv, *ctx, *act, *logits;             /* [batch, hidden | 3 hidden | hidden | ffn | vocab] */
+  pta_half* logits;                                   /* [batch, vocab] out, 16-byte aligned          */
 } pta_decode_state;
 
-/* Bytes of the workspace of pta_llama_decode_step on the current device; 0 for unsupported shapes.
- * The caller zeroes it once after allocating it; the kernel keeps it consistent afterwards. */
-size_t pta_decode_step_workspace_bytes(int batch, int n_head, int head_dim);
+/* Bytes of the workspace of pta_llama_decode_step for this model on the current device; 0 for
+ * unsupported shapes.  The workspace holds one slot per intermediate vector of an iteration (the
+ * residual stream after each half layer, q|k|v, attention output and partials, SwiGLU output) and a
+ * few synchronisation words.  The caller zeroes it once after allocating it (256-byte aligned). */
+size_t pta_decode_step_workspace_bytes(const pta_decode_model* model);
 
 /* Enqueues one loop iteration.  Supports batch <= 4, head_dim 128, hidden = n_head * 128 with
- * (hidden, ffn) of the 7B and 13B models or a small test shape; PTA_EUNSUPPORTED otherwise.
- * Needs every compute unit of the device for itself while it runs: the grid barrier waits a bounded
- * time for all workgroups and, if one never arrives, sets word 1 of the workspace (sticky), leaves
- * the loop state untouched and ends; pta_decode_step_failed reports it. */
+ * (hidden, ffn) of the 7B model or a small test shape; PTA_EUNSUPPORTED otherwise.
+ * Needs every compute unit of the device for itself while it runs: workgroups wait for each
+ * other's results, every wait is bounded, and if one gives up it sets word 1 of the workspace
+ * (sticky), the loop state is left untouched and the kernel ends; pta_decode_step_failed reports it. */
 int pta_llama_decode_step(const pta_decode_model* model, const pta_decode_state* state, void* workspace,
                           pta_stream_t stream);
 

@@ -45,8 +45,7 @@ class DecodeModel(ctypes.Structure):
 
 
 class DecodeState(ctypes.Structure):
-    _fields_ = [(n, c_void_p) for n in ("container", "mask", "stop_mask", "step", "keep_going", "next_ids", "x", "qkv",
-                                        "ctx", "act", "logits")]
+    _fields_ = [(n, c_void_p) for n in ("container", "mask", "stop_mask", "step", "keep_going", "next_ids", "logits")]
 
 
 class Fusion(ctypes.Structure):
@@ -98,7 +97,7 @@ SIGNATURES = {
     "pta_rwkv_wkv": (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),
-    "pta_decode_step_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "pta_decode_step_workspace_bytes": (c_size_t, [POINTER(DecodeModel)]),
     "pta_llama_decode_step": (c_int, [POINTER(DecodeModel), POINTER(DecodeState), c_void_p, c_void_p]),
     "pta_decode_step_failed": (c_int, [c_void_p, POINTER(c_int), c_void_p]),
 }

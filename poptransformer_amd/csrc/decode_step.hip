@@ -6,32 +6,31 @@
 // [down + residual], once per layer, then [RMSNorm + lm_head] -> [top-1 + container update].
 // Launched as separate kernels, every phase pays a launch boundary and a cold start of the weight
 // stream; at batch 1 a 7B layer's 101 MB of weights stream in 13 us and the boundaries take longer
-// than that.  Here one workgroup per compute unit stays resident for the whole iteration, phases
-// are separated by a grid barrier, and every wave holds the weight tiles of the next phase(s) in
-// registers: they are requested one phase (or more) before they are used, so HBM streams while
-// the grid synchronises and the phases themselves only wait for activations.
+// than that.  Here one workgroup per compute unit stays resident for the whole iteration and every
+// wave holds the weight tiles of the next phase(s) in registers: they are requested a phase or
+// more before they are used, so HBM streams while the phases wait for each other's results.
 //
 // Numerics are those of the per-operator entry points (formats.h, norm.hip, attention.hip,
 // select.hip), which the parity tests compare against the CPU restatement; this file only changes
 // when things happen (and the order in which attention partials are merged).
 //
-// Memory ordering between workgroups.  Results that another workgroup reads in the same launch are
-// written with agent-scope stores (they go through the writer's L2 to memory) and read with
-// agent-scope loads (they do not hit stale lines); a writer only has to wait until its stores have
-// completed before it signals.  A write-back or invalidation of the whole L2 per barrier, which is
-// what fences at agent scope cost, measured 5-20 us here and is avoided.
+// How phases hand over results.  Every intermediate vector of the iteration (the residual stream
+// after each half layer, q|k|v, the attention output, the SwiGLU output, attention partials, the
+// logits) has a slot of its own in the workspace.  At the start of a launch all slots are filled
+// with a bit pattern no result can have (all ones: a NaN that the stores below never write), one
+// grid barrier follows, and from then on a consumer simply loads the values it needs until none
+// of them is the filler: data and "ready" travel in the same load, there is no flag to wait for
+// first and no barrier between phases.  Producers write with agent-scope stores (through the
+// writer's L2 to memory), consumers read with agent-scope loads (no stale lines), so neither side
+// needs a cache write-back or invalidation, which cost 5-20 us per use here.  Every wait is
+// bounded: after DS_SPIN_LIMIT polls a wave sets the sticky error word of the workspace, every
+// workgroup that sees it stops, and the loop state is left as it was.
 //
-// Grid barrier.  sync[0] holds the epoch base, sync[1] an error flag, sync[16 + g] the arrival
-// word of workgroup g.  The waves that wrote results wait for their stores, the workgroup meets,
-// thread 0 publishes the epoch in its arrival word, wave 0 polls all arrival words, and the
-// workgroup meets again.  The poll is bounded: if an epoch has not arrived after DS_SPIN_LIMIT
-// polls the (sticky) error flag is set, every workgroup passes its remaining barriers without
-// waiting, and the kernel ends without advancing the loop.
-//
-// Loads return in order within a wave, so a wave that waits for a small activation load also waits
-// for every weight tile it requested before; each phase therefore requests its activations first
-// and the next weights second, and all waves request weights at the same program points, which
-// lets the compiler count exactly how many requests may stay in flight at each use.
+// A compute unit returns loads in the order it received them from all of its waves, so a small
+// activation load issued behind a burst of weight requests waits for those.  Each phase therefore
+// first obtains its activations and only then requests weights for later phases; the attention
+// phase, which is all latency, requests none.  All waves request weights at the same program
+// points, which lets the compiler count exactly how many requests may stay in flight at each use.
 #include "common.h"
 #include "formats.h"
 
@@ -39,15 +38,17 @@ namespace {
 
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
-constexpr int DS_STORE_WAVES = 4;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
 constexpr int DS_MAXB = 4;
 constexpr int DS_D = 128;                                   // head size
 constexpr int DS_MAX_SPLIT = 16;
+constexpr int DS_PART = DS_D + 2;                           // floats of one attention partial
 constexpr int DS_RED = DS_WAVES * 3 * 16 * DS_MAXB;         // floats in one reduction buffer
 constexpr int DS_ATT_FLOATS = 3 * DS_D / 2 + 2 * DS_WAVES + DS_WAVES * DS_D;
 constexpr int DS_TAIL_FLOATS = DS_WAVES * DS_MAXB + 64 + 4; // norm sums | selection scratch | flags
 constexpr int DS_LAYER_WORDS = sizeof(pta_decode_layer) / 4;
+constexpr uint16_t DS_EMPTY16 = 0xFFFFu;                    // filler of fp16 slots
+constexpr uint32_t DS_EMPTY32 = 0xFFFFFFFFu;                // filler of fp32 slots
 
 // indices of the pointers in pta_decode_layer
 enum { P_WQ, P_WK, P_WV, P_WO, P_WG, P_WU, P_WD, P_SQ, P_SK, P_SV, P_SO, P_SG, P_SU, P_SD, P_N1, P_N2, P_KV };
@@ -64,9 +65,14 @@ struct DsArgs {
   float eps;
   int32_t* container; f16* mask; int32_t* stop_mask; int32_t* step; int32_t* keep_going; int32_t* next_ids;
   int pad_id, eos_id, early_stop;
-  f16* x; f16* qkv; f16* ctx; f16* act; f16* logits;
-  float* attn_part;      // [B*H, nsplit, D + 2]
-  unsigned* tickets;     // [B*H], zero between launches
+  f16* logits;
+  // slots in the workspace
+  f16* xres;             // [2 n_layer + 1][B, d]: residual stream after the embedding and after each half layer
+  f16* qkv;              // [n_layer][B, 3d]
+  f16* ctx;              // [n_layer][B, d]
+  f16* act;              // [n_layer][B, ffn]
+  float* part;           // [n_layer][B*H, nsplit, DS_PART]
+  size_t fill_bytes;     // qkv .. end of part, contiguous from xres + B*d (the first residual is not filled)
   unsigned* sync;
   int nsplit;
   int region0;           // bytes of the activation / attention area at the start of LDS
@@ -78,13 +84,6 @@ struct DsArgs {
 #else
 #define TRACE(i) do {} while (0)
 #endif
-
-struct Grid {
-  unsigned* sync;
-  unsigned epoch;
-  int G, wg;
-  bool dead;
-};
 
 // The asm statements make the thread index opaque at each use, so that what a phase derives from
 // it is recomputed there (a few integer instructions) instead of being kept in registers across
@@ -108,58 +107,97 @@ __device__ __forceinline__ const DS_GLOBAL T* as_global(const T* p) { return (co
 template <class T>
 __device__ __forceinline__ DS_GLOBAL T* as_global(T* p) { return (DS_GLOBAL T*)p; }
 
+// results: agent-scope stores that never write the filler (a NaN with another payload replaces it)
 __device__ __forceinline__ void put(f16* p, f16 v) {
-  __hip_atomic_store((DS_GLOBAL uint16_t*)p, bitcast<uint16_t>(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  uint16_t bits = bitcast<uint16_t>(v);
+  bits = bits == DS_EMPTY16 ? (uint16_t)0xFE00u : bits;
+  __hip_atomic_store((DS_GLOBAL uint16_t*)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void put(float* p, float v) {
-  __hip_atomic_store((DS_GLOBAL float*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  uint32_t bits = bitcast<uint32_t>(v);
+  bits = bits == DS_EMPTY32 ? 0xFFC00000u : bits;
+  __hip_atomic_store((DS_GLOBAL uint32_t*)p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ float get(const float* p) {
-  return __hip_atomic_load((const DS_GLOBAL float*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ uint32_t get_bits(const float* p) {
+  return __hip_atomic_load((const DS_GLOBAL uint32_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ f16 get(const f16* p) {
-  return bitcast<f16>(__hip_atomic_load((const DS_GLOBAL uint16_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+__device__ __forceinline__ uint16_t get_bits(const f16* p) {
+  return __hip_atomic_load((const DS_GLOBAL uint16_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// 16 bytes at agent scope, through a buffer descriptor because only buffer loads take the scope
+// 16 bytes at agent scope, through a buffer descriptor because only buffer accesses take the scope
 // bits together with a 128-bit width
-__device__ __forceinline__ f16x8 get8(const f16* base, size_t bytes, int byte_offset) {
-  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16*>(base), 0, (int)bytes, 0x00020000);
-  return bitcast<f16x8>(__builtin_amdgcn_raw_buffer_load_b128(r, byte_offset, 0, 16 /* sc1 */));
+__device__ __forceinline__ u32x4 get16(const void* base, size_t bytes, size_t byte_offset) {
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, 16 /* sc1 */);
+}
+__device__ __forceinline__ void put16(void* base, size_t bytes, size_t byte_offset, u32x4 v) {
+  const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(base, 0, (int)bytes, 0x00020000);
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)byte_offset, 0, 16 /* sc1 */);
+}
+__device__ __forceinline__ bool has_empty16(u32x4 v) {
+  bool e = false;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) e = e || (v[i] & 0xFFFFu) == DS_EMPTY16 || (v[i] >> 16) == DS_EMPTY16;
+  return e;
 }
 
-// the agent-scope stores of this wave have completed; called before the grid barrier (or a ticket)
-// by the waves that store results, i.e. the first DS_STORE_WAVES of a workgroup
-__device__ __forceinline__ void release_results() {
-  if (wave_id() < DS_STORE_WAVES) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+// Bounded waiting of one wave.  `give_up` turns true when the wave has polled DS_SPIN_LIMIT times
+// or another workgroup has reported a failure; the wave then sets the error word and the
+// workgroup-wide flag in LDS and stops waiting.
+struct Waiter {
+  unsigned* err;     // sync[1]
+  int* lds_dead;
+  unsigned spins;
+  __device__ __forceinline__ bool give_up() {
+    ++spins;
+    bool stop = spins > DS_SPIN_LIMIT;
+    if ((spins & 63u) == 0)
+      stop = stop || __hip_atomic_load((DS_GLOBAL unsigned*)err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+    if (stop) {
+      __hip_atomic_store((DS_GLOBAL unsigned*)err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *lds_dead = 1;
+    }
+    return stop;
+  }
+};
+
+// wave-uniform wait for one fp16 / fp32 value per lane (lanes with on == false do not wait)
+__device__ __forceinline__ f16 wait_value(const f16* p, bool on, Waiter& w) {
+  uint16_t bits = 0;
+  for (;;) {
+    if (on) bits = get_bits(p);
+    if (!__any(on && bits == DS_EMPTY16) || w.give_up()) break;
+  }
+  return bitcast<f16>(bits);
+}
+__device__ __forceinline__ float wait_value(const float* p, bool on, Waiter& w) {
+  uint32_t bits = 0;
+  for (;;) {
+    if (on) bits = get_bits(p);
+    if (!__any(on && bits == DS_EMPTY32) || w.give_up()) break;
+  }
+  return bitcast<float>(bits);
 }
 
-__device__ __forceinline__ void grid_barrier(Grid& g, int* lds_flag) {
+// The one grid barrier of a launch (after the slots have been filled).  sync[0] holds the epoch
+// base, sync[1] the error word, sync[16 + g] the arrival word of workgroup g.
+__device__ __forceinline__ void grid_barrier(unsigned* sync, unsigned epoch, int G, int wg, Waiter& w) {
   const int wave = wave_id(), lane = lane_id();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's agent-scope stores have completed
   wg_sync();
-  if (!g.dead) {
-    if (thread_id() == 0)
-      __hip_atomic_store(g.sync + 16 + g.wg, g.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (wave == 0) {
-      unsigned spins = 0;
-      int bad = 0;
-      for (;;) {
-        // the arrival words and the error flag travel in one batch of loads: one round trip per poll
-        const unsigned err = __hip_atomic_load(g.sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        bool ok = true;
-        for (int i = lane; i < g.G; i += 64) {
-          const unsigned v = __hip_atomic_load(g.sync + 16 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          ok = ok && ((int)(v - g.epoch) >= 0);
-        }
-        if (__all(ok)) break;
-        if (err != 0 || ++spins > DS_SPIN_LIMIT) { bad = 1; break; }
+  if (thread_id() == 0)
+    __hip_atomic_store((DS_GLOBAL unsigned*)(sync + 16 + wg), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (wave == 0) {
+    for (;;) {
+      bool ok = true;
+      for (int i = lane; i < G; i += 64) {
+        const unsigned v = __hip_atomic_load((DS_GLOBAL unsigned*)(sync + 16 + i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && ((int)(v - epoch) >= 0);
       }
-      if (bad && lane == 0) __hip_atomic_store(g.sync + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (lane == 0) *lds_flag = bad;
+      if (__all(ok) || w.give_up()) break;
     }
   }
   wg_sync();
-  if (!g.dead && *lds_flag) g.dead = true;
-  g.epoch += 1;
 }
 
 // The 17 pointers of one layer as scalars: lane l reads descriptor word l from LDS (one read for
@@ -225,12 +263,13 @@ __device__ __forceinline__ void load_unit(Unit<Fmt, NRB, TPW>& t, const Mat (&m)
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 
 // out[r][m, n] = sum_k xs[m, k] * W_r[n, k] for unit u, whose tiles are in t.  `res` is the residual
-// element of this thread (EPI_RESIDUAL), read at the start of the phase.
-template <class Fmt, int NRB, int TPW, int EPI>
-__device__ __forceinline__ void gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* const (&out)[NRB], int ostride, f16 res,
-                                          int u, int n_units, int N, int KT, int M, const f16* xs, int xstride,
-                                          float* red, int& red_buf) {
-  if (u >= n_units) return;
+// element of this thread (EPI_RESIDUAL); the value the thread stored is returned (it is the
+// residual of the same thread in the next residual phase).
+template <class Fmt, int NRB, int TPW, int EPI, int MAXB>
+__device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* const (&out)[NRB], int ostride, f16 res,
+                                         int u, int n_units, int N, int KT, int M, const f16* xs, int xstride,
+                                         float* red, int& red_buf) {
+  if (u >= n_units) return res;
   const int wave = wave_id(), lane = lane_id();
   int mrow = lane & 15;
   mrow = mrow < M ? mrow : M - 1;
@@ -261,17 +300,20 @@ __device__ __forceinline__ void gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* con
         rb[((wave * NRB + r) * 16 + (lane >> 4) * 4 + q) * DS_MAXB + (lane & 15)] = acc[r][q];
   }
   wg_sync();
+  f16 y = res;
   {
+    // thread (r * M + m_) * 16 + ch finishes channel ch of row m_ of matrix r (M <= 4: no division)
     const int tid = thread_id();
-    const int per = 16 * M;
-    const int total = (EPI == EPI_SWIGLU ? 1 : NRB) * per;
+    const int total = (EPI == EPI_SWIGLU ? 1 : NRB) * 16 * M;
     if (tid < total) {
-      const int r = tid / per, ch = (tid % per) / M, m_ = tid % M;
+      const int q = tid >> 4, ch = tid & 15;
+      const int r = (q >= M ? 1 : 0) + (q >= 2 * M ? 1 : 0);
+      const int m_ = q - r * M;
       const int n = u * 16 + ch;
       if (n < N) {
         if (EPI == EPI_SWIGLU) {
           float sg = 0.f, su = 0.f;
-#pragma unroll
+#pragma unroll 4
           for (int w = 0; w < DS_WAVES; ++w) {
             sg += rb[((w * NRB + 0) * 16 + ch) * DS_MAXB + m_];
             su += rb[((w * NRB + (NRB > 1 ? 1 : 0)) * 16 + ch) * DS_MAXB + m_];
@@ -279,9 +321,9 @@ __device__ __forceinline__ void gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* con
           put(out[0] + (size_t)m_ * ostride + n, (f16)su * swish_f16((f16)sg));
         } else {
           float s = 0.f;
-#pragma unroll
+#pragma unroll 8
           for (int w = 0; w < DS_WAVES; ++w) s += rb[((w * NRB + r) * 16 + ch) * DS_MAXB + m_];
-          f16 y = (f16)s;
+          y = (f16)s;
           if (EPI == EPI_RESIDUAL) y = y + res;
           put(out[r] + (size_t)m_ * ostride + n, y);
         }
@@ -289,111 +331,111 @@ __device__ __forceinline__ void gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* con
     }
   }
   red_buf ^= 1;
+  return y;
 }
 
-// the residual element the epilogue thread of unit u adds (same thread mapping as gemv_unit)
-__device__ __forceinline__ f16 residual_at(const f16* residual, int u, int N, int M) {
-  const int tid = thread_id();
-  if (tid >= 16 * M) return (f16)0.0f;
-  const int n = u * 16 + tid / M;
-  return n < N ? get(residual + (size_t)(tid % M) * N + n) : (f16)0.0f;
-}
+// i / per for i < 4 * per, without a division
+__device__ __forceinline__ int row_of(int i, int per) { return (i >= per ? 1 : 0) + (i >= 2 * per ? 1 : 0) + (i >= 3 * per ? 1 : 0); }
 
-// Activations of a phase, first half: every thread requests its 16-byte vectors of X (fp16 [M, K]).
-template <int NS>
-struct Staged {
-  f16x8 v[NS];
-};
-template <int NS>
-__device__ __forceinline__ void stage_request(Staged<NS>& s, const f16* X, int M, int K, int KT) {
+// Activations of a phase.  Every thread loads its 16-byte vectors of X (fp16 [M, K]) until none of
+// their elements is the filler, then the vectors go to LDS (zero from K up to KT*128), RMS-
+// normalised on the way when norm_w (in LDS) is given, as pta_rmsnorm does it
+// (layers/rms_layer_norm.py:26-36).  Returns false when the wait was given up.
+template <int NS, int MAXB>
+__device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* xs, int xstride, const f16* norm_w,
+                                      float eps, float* scratch, Waiter& w) {
   const int vec_per_row = KT * 16, total = M * vec_per_row;
+  const int lane = lane_id(), wave = wave_id();
+  u32x4 v[NS];
+  bool need[NS];
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
     const int i = thread_id() + k * DS_THREADS;
-    const int m = i / vec_per_row, c = i % vec_per_row;
-    s.v[k] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-    if (i < total && c * 8 < K) s.v[k] = get8(X, (size_t)M * K * 2, (m * K + c * 8) * 2);
+    v[k] = u32x4{0, 0, 0, 0};
+    need[k] = i < total && (i - row_of(i, vec_per_row) * vec_per_row) * 8 < K;
   }
-}
-// Second half: the vectors go to LDS (zero from K up to KT*128), RMS-normalised on the way when
-// norm_w (in LDS) is given, as pta_rmsnorm does it (layers/rms_layer_norm.py:26-36).
-template <int NS>
-__device__ __forceinline__ void stage_commit(const Staged<NS>& s, int M, int K, int KT, f16* xs, int xstride,
-                                             const f16* norm_w, float eps, float* scratch) {
-  const int vec_per_row = KT * 16, total = M * vec_per_row;
-  const int lane = lane_id(), wave = wave_id();
-  if (!norm_w) {
+  for (;;) {
+    bool pending = false;
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      if (need[k]) {
+        const int i = thread_id() + k * DS_THREADS;
+        const int m = row_of(i, vec_per_row);
+        v[k] = get16(X, (size_t)M * K * 2, ((size_t)m * K + (size_t)(i - m * vec_per_row) * 8) * 2);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      if (need[k]) {
+        if (has_empty16(v[k])) pending = true;
+        else need[k] = false;
+      }
+    }
+    if (!__any(pending) || w.give_up()) break;
+  }
+  float pq[MAXB];
+#pragma unroll
+  for (int mm = 0; mm < MAXB; ++mm) pq[mm] = 0.f;
+  if (norm_w) {
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
       const int i = thread_id() + k * DS_THREADS;
-      if (i < total) *reinterpret_cast<f16x8*>(xs + (size_t)(i / vec_per_row) * xstride + (i % vec_per_row) * 8) = s.v[k];
+      if (i < total) {
+        const int m = row_of(i, vec_per_row);
+        const f16x8 h = bitcast<f16x8>(v[k]);
+        float s2 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { const float f = (float)h[e]; s2 = __builtin_fmaf(f, f, s2); }
+#pragma unroll
+        for (int mm = 0; mm < MAXB; ++mm) if (mm == m) pq[mm] += s2;
+      }
+    }
+#pragma unroll
+    for (int mm = 0; mm < MAXB; ++mm) pq[mm] = wave_sum(pq[mm]);
+    if (lane == 0) {
+#pragma unroll
+      for (int mm = 0; mm < MAXB; ++mm) scratch[wave * DS_MAXB + mm] = pq[mm];
     }
     wg_sync();
-    return;
   }
-  float pq[DS_MAXB] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int k = 0; k < NS; ++k) {
-    const int i = thread_id() + k * DS_THREADS;
-    if (i < total) {
-      const int m = i / vec_per_row;
-      float s2 = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) { const float f = (float)s.v[k][e]; s2 = __builtin_fmaf(f, f, s2); }
-#pragma unroll
-      for (int mm = 0; mm < DS_MAXB; ++mm) if (mm == m) pq[mm] += s2;
-    }
-  }
-#pragma unroll
-  for (int mm = 0; mm < DS_MAXB; ++mm) pq[mm] = wave_sum(pq[mm]);
-  if (lane == 0) {
-#pragma unroll
-    for (int mm = 0; mm < DS_MAXB; ++mm) scratch[wave * DS_MAXB + mm] = pq[mm];
-  }
-  wg_sync();
   const float inv_n = 1.0f / (float)K;
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
     const int i = thread_id() + k * DS_THREADS;
     if (i < total) {
-      const int m = i / vec_per_row, c = i % vec_per_row;
-      f16x8 v = s.v[k];
-      if (c * 8 < K) {
+      const int m = row_of(i, vec_per_row), c = i - m * vec_per_row;
+      f16x8 h = bitcast<f16x8>(v[k]);
+      if (norm_w && c * 8 < K) {
         float sq = 0.f;
 #pragma unroll
-        for (int w = 0; w < DS_WAVES; ++w) sq += scratch[w * DS_MAXB + m];
+        for (int ww = 0; ww < DS_WAVES; ++ww) sq += scratch[ww * DS_MAXB + m];
         const f16 r16 = (f16)(1.0f / sqrtf(sq * inv_n + eps));
         const f16x8 gm = *reinterpret_cast<const f16x8*>(norm_w + c * 8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = (v[e] * r16) * gm[e];
+        for (int e = 0; e < 8; ++e) h[e] = (h[e] * r16) * gm[e];
       }
-      *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+      *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = h;
     }
   }
   wg_sync();
+  return *w.lds_dead == 0;
 }
 
-// RMSNorm weights travel global -> register (requested a phase early) -> LDS (committed at the
-// end of that phase, after the stage that used the previous weights)
-__device__ __forceinline__ f16x8 normw_request(const f16* w, int d) {
-  const int i = thread_id();
-  return i * 8 < d ? *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(w) + i * 8) : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-}
-__device__ __forceinline__ void normw_commit(f16x8 v, f16* lds_w, int d) {
-  const int i = thread_id();
-  if (i * 8 < d) *reinterpret_cast<f16x8*>(lds_w + i * 8) = v;
+// RMSNorm weights go from global memory straight into LDS (no registers), requested at the end of
+// the phase before the one that normalises with them; the wait of that phase's `stage` covers them,
+// because a wave's loads complete in order.  Wave w moves weights [512 w, 512 w + 512): a whole KiB of
+// LDS per wave (lanes beyond d repeat the last vector), so the LDS array is d rounded up to 512.
+__device__ __forceinline__ void normw_fetch(const f16* w, f16* lds_w, int d) {
+  const int wave = wave_id(), lane = lane_id();
+  if (wave * 512 < d) {
+    int i = wave * 512 + lane * 8;
+    i = i + 8 <= d ? i : d - 8;      // d is a multiple of 128
+    __builtin_amdgcn_global_load_lds((const DS_GLOBAL void*)(as_global(w) + i),
+                                     (__attribute__((address_space(3))) void*)(lds_w + wave * 512), 16, 0, 0);
+  }
 }
 
 // ------------------------------------------------------------------------------------------ attention phase
-// rotate-half rotary of one element, as rope_llama in attention.hip (models/llama2/attention.py:83-97);
-// cs holds fp16(cos(angle_i)) and fp16(sin(angle_i)) of this step
-__device__ __forceinline__ f16 rope_at(const f16* x, int d, const f16* cs) {
-  const int half = DS_D >> 1;
-  const int i = d < half ? d : d - half;
-  const f16 rot = d < half ? -get(x + d + half) : get(x + d - half);
-  return get(x + d) * cs[i] + rot * cs[half + i];
-}
-
 // merges the online-softmax state of the lane `o` lanes away into this lane's
 __device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8], int o) {
   const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
@@ -406,19 +448,23 @@ __device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8],
   m = mn;
 }
 
-// One (sequence, head, split) unit: rotary of q and of the new k, append of the new K/V row to the
-// ring by the split whose range holds it, online-softmax attention over this split's rows, partial
-// result to global memory; the last split of a head to finish combines the partials into ctx.
-__device__ __forceinline__ void attention_unit(const DsArgs& a, f16* kring_base, int unit, int step, float* lds,
-                                               const f16* cs, int* lds_i) {
-  constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP;
+// One (sequence, head, split) unit: rotary of q and of the new k (rotate-half, as rope_llama in
+// attention.hip, models/llama2/attention.py:83-97; cs holds fp16 cos and sin of this step's
+// angles), append of the new K/V row to the ring by the split whose range holds it, online-softmax
+// attention over this split's rows.  Split 0 of a head collects the partials of the other splits
+// that have rows and writes the head's output.
+__device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kring_base, int unit, int step, float* lds,
+                                               const f16* cs, Waiter& w) {
+  constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2;
   const int wave = wave_id(), lane = lane_id();
   const int bh = unit / a.nsplit, split = unit % a.nsplit;
   const int b = bh / a.H, h = bh % a.H;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
   const int pos = step % a.max_len;
   const int chunk = ((valid + a.nsplit - 1) / a.nsplit + 63) & ~63;
+  const int nact = (valid + chunk - 1) / chunk;       // splits that have rows
   const int c0 = split * chunk;
+  if (c0 >= valid) return;
   const int c1 = c0 + chunk < valid ? c0 + chunk : valid;
   f16* q_s = reinterpret_cast<f16*>(lds);            // [D] rotated q
   f16* k_s = q_s + D;                                 // [D] rotated new k
@@ -426,31 +472,32 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, f16* kring_base,
   float* sm_m = lds + 3 * D / 2;                      // [DS_WAVES]
   float* sm_l = sm_m + DS_WAVES;
   float* sm_acc = sm_l + DS_WAVES;                    // [DS_WAVES][D]
-  const f16* qrow = a.qkv + (size_t)b * 3 * a.d + h * D;
-  const f16* krow = qrow + a.d;
-  const f16* vrow = qrow + 2 * a.d;
+  const f16* qrow = a.qkv + ((size_t)li * a.B + b) * 3 * a.d + h * D;
   f16* kring = kring_base + ((size_t)b * a.H + h) * a.max_len * D;
   f16* vring = kring + (size_t)a.B * a.H * a.max_len * D;
   const bool owner = pos >= c0 && pos < c0 + chunk;
   {
+    // waves 0-1: q, waves 2-3: k, waves 4-5: v; a rotated element needs x[d] and x[d +- D/2]
     const int tid = thread_id();
-    if (tid < D) {
-      q_s[tid] = rope_at(qrow, tid, cs);
-    } else if (tid < 2 * D) {
-      const int d_ = tid - D;
-      const f16 kr = rope_at(krow, d_, cs);
-      k_s[d_] = kr;
-      if (owner) as_global(kring)[(size_t)pos * D + d_] = kr;
-    } else if (tid < 3 * D) {
-      const int d_ = tid - 2 * D;
-      const f16 vv = get(vrow + d_);
-      v_s[d_] = vv;
-      if (owner) as_global(vring)[(size_t)pos * D + d_] = vv;
+    const int which = tid / D, d_ = tid % D;
+    const bool on = tid < 3 * D;
+    const f16* row = qrow + (size_t)(which < 3 ? which : 0) * a.d;
+    const f16 x0 = wait_value(row + d_, on, w);
+    const f16 x1 = wait_value(row + (d_ < HALF ? d_ + HALF : d_ - HALF), on && which < 2, w);
+    if (on) {
+      f16 y = x0;
+      if (which < 2) {
+        const int i = d_ < HALF ? d_ : d_ - HALF;
+        const f16 rot = d_ < HALF ? -x1 : x1;
+        y = x0 * cs[i] + rot * cs[HALF + i];
+      }
+      q_s[which * D + d_] = y;
+      if (which == 1 && owner) as_global(kring)[(size_t)pos * D + d_] = y;
+      if (which == 2 && owner) as_global(vring)[(size_t)pos * D + d_] = y;
     }
   }
   wg_sync();
-  float* part = a.attn_part + ((size_t)bh * a.nsplit + split) * (D + 2);
-  if (c0 < valid) {
+  {
     const int grp = lane / LPP, sub = lane % LPP, d0 = sub * 8;
     float qf[8];
 #pragma unroll
@@ -495,57 +542,38 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, f16* kring_base,
 #pragma unroll
       for (int e = 0; e < 8; ++e) sm_acc[wave * D + d0 + e] = acc[e];
     }
-    wg_sync();
-    if (thread_id() < D) {
-      const int d_ = thread_id();
-      float Mx = -INFINITY;
-#pragma unroll
-      for (int i = 0; i < DS_WAVES; ++i) Mx = fmaxf(Mx, sm_m[i]);
-      float Ls = 0.f, As = 0.f;
-#pragma unroll
-      for (int i = 0; i < DS_WAVES; ++i) {
-        const float w = sm_m[i] == -INFINITY ? 0.f : __expf(sm_m[i] - Mx);
-        Ls = __builtin_fmaf(sm_l[i], w, Ls);
-        As = __builtin_fmaf(sm_acc[i * D + d_], w, As);
-      }
-      put(part + 2 + d_, As);
-      if (d_ == 0) { put(part, Mx); put(part + 1, Ls); }
-    }
-  } else if (thread_id() == 0) {
-    put(part, -INFINITY); put(part + 1, 0.f);      // an empty split contributes nothing
-  }
-  // ticket: the last split of this head to arrive combines all partials into ctx
-  release_results();
-  wg_sync();
-  if (thread_id() == 0) {
-    const unsigned t = __hip_atomic_fetch_add(a.tickets + bh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const int last = (t == (unsigned)a.nsplit - 1) ? 1 : 0;
-    if (last) __hip_atomic_store(a.tickets + bh, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    *lds_i = last;
   }
   wg_sync();
-  if (*lds_i && thread_id() < D) {
+  if (thread_id() < D) {      // waves 0 and 1
     const int d_ = thread_id();
-    const float* p = a.attn_part + (size_t)bh * a.nsplit * (D + 2);
-    float pm[DS_MAX_SPLIT], pl[DS_MAX_SPLIT], pa[DS_MAX_SPLIT];
-#pragma unroll
-    for (int s = 0; s < DS_MAX_SPLIT; ++s) {       // all loads in one batch
-      const bool on = s < a.nsplit;
-      const float* ps = p + (size_t)(on ? s : 0) * (D + 2);
-      pm[s] = get(ps); pl[s] = get(ps + 1); pa[s] = get(ps + 2 + d_);
-      if (!on) pm[s] = -INFINITY;
-    }
     float Mx = -INFINITY;
 #pragma unroll
-    for (int s = 0; s < DS_MAX_SPLIT; ++s) Mx = fmaxf(Mx, pm[s]);
+    for (int i = 0; i < DS_WAVES; ++i) Mx = fmaxf(Mx, sm_m[i]);
     float Ls = 0.f, As = 0.f;
 #pragma unroll
-    for (int s = 0; s < DS_MAX_SPLIT; ++s) {
-      const float w = pm[s] == -INFINITY ? 0.f : __expf(pm[s] - Mx);
-      Ls = __builtin_fmaf(pl[s], w, Ls);
-      As = __builtin_fmaf(pm[s] == -INFINITY ? 0.f : pa[s], w, As);
+    for (int i = 0; i < DS_WAVES; ++i) {
+      const float wgt = sm_m[i] == -INFINITY ? 0.f : __expf(sm_m[i] - Mx);
+      Ls = __builtin_fmaf(sm_l[i], wgt, Ls);
+      As = __builtin_fmaf(sm_acc[i * D + d_], wgt, As);
     }
-    put(a.ctx + (size_t)b * a.d + h * D + d_, (f16)(As / Ls));
+    float* part = a.part + (((size_t)li * a.B * a.H + bh) * a.nsplit) * DS_PART;
+    if (split != 0) {
+      float* mine = part + (size_t)split * DS_PART;
+      put(mine + 2 + d_, As);
+      if (d_ == 0) { put(mine, Mx); put(mine + 1, Ls); }
+    } else {
+      // the other splits' (max, denominator, numerator[d_]) in ascending order of split
+      for (int s = 1; s < nact; ++s) {
+        const float* ps = part + (size_t)s * DS_PART;
+        const float ms = wait_value(ps, true, w), ls = wait_value(ps + 1, true, w), as = wait_value(ps + 2 + d_, true, w);
+        const float mn = fmaxf(Mx, ms);
+        const float ca = __expf(Mx - mn), cb = __expf(ms - mn);
+        Ls = Ls * ca + ls * cb;
+        As = As * ca + as * cb;
+        Mx = mn;
+      }
+      put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
+    }
   }
   wg_sync();
 }
@@ -553,7 +581,8 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, f16* kring_base,
 // ------------------------------------------------------------------------------------------ selection and bookkeeping
 // Top-1 per sequence (lowest index among equals), then the container / mask / stop-mask update of
 // models/base_model.py:313-355 exactly as step_update_kernel in select.hip; workgroup 0 only.
-__device__ __forceinline__ void select_and_advance(const DsArgs& a, float* lds) {
+// Returns false when the wait for the logits was given up (nothing is updated then).
+__device__ __forceinline__ bool select_and_advance(const DsArgs& a, float* lds, Waiter& w) {
   float* sv = lds;
   int* si = reinterpret_cast<int*>(lds + DS_WAVES);
   int* ids = si + DS_WAVES;
@@ -562,18 +591,19 @@ __device__ __forceinline__ void select_and_advance(const DsArgs& a, float* lds) 
     const f16* xr = a.logits + (size_t)b * a.vocab;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i0 = thread_id() * 8; i0 < a.vocab; i0 += DS_THREADS * 8) {
-      if (i0 + 8 <= a.vocab) {
-        const f16x8 v8 = get8(xr, (size_t)a.vocab * 2, i0 * 2);
+    for (int i0 = thread_id() * 8; __any(i0 < a.vocab); i0 += DS_THREADS * 8) {
+      const bool on = i0 < a.vocab;      // vocab is a multiple of 8
+      u32x4 v = {0, 0, 0, 0};
+      for (;;) {
+        if (on) v = get16(xr, (size_t)a.vocab * 2, (size_t)i0 * 2);
+        if (!__any(on && has_empty16(v)) || w.give_up()) break;
+      }
+      if (on) {
+        const f16x8 h = bitcast<f16x8>(v);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const float v = (float)v8[e];
-          if (v > best) { best = v; bi = i0 + e; }
-        }
-      } else {
-        for (int i = i0; i < a.vocab; ++i) {
-          const float v = (float)get(xr + i);
-          if (v > best) { best = v; bi = i; }
+          const float f = (float)h[e];
+          if (f > best) { best = f; bi = i0 + e; }
         }
       }
     }
@@ -586,12 +616,13 @@ __device__ __forceinline__ void select_and_advance(const DsArgs& a, float* lds) 
     if (lane == 0) { sv[wave] = best; si[wave] = bi; }
     wg_sync();
     if (thread_id() == 0) {
-      for (int w = 1; w < DS_WAVES; ++w)
-        if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
+      for (int ww = 1; ww < DS_WAVES; ++ww)
+        if (sv[ww] > best || (sv[ww] == best && si[ww] < bi)) { best = sv[ww]; bi = si[ww]; }
       ids[b] = bi == 0x7fffffff ? 0 : bi;
     }
     wg_sync();
   }
+  if (*w.lds_dead != 0) return false;
   if (thread_id() == 0) {
     const int ns = *a.step + 1;
     int stopped_before = 0;
@@ -610,58 +641,71 @@ __device__ __forceinline__ void select_and_advance(const DsArgs& a, float* lds) 
     *a.keep_going = a.early_stop ? (stopped_before < a.B ? 1 : 0) : 1;
     *a.step = ns;
   }
+  return true;
 }
 
 // ------------------------------------------------------------------------------------------ the kernel
-// TPW_D / TPW_F: K tiles per wave for K = hidden / ffn; U_F: gate/up row-blocks per workgroup.
-// hidden row-blocks (q/k/v, o_proj, down) are at most one per workgroup.
-// MAXB: largest batch the instance stages (vectors per thread: NS_D for K = hidden, NS_F for K = ffn).
+// TPW_D / TPW_F: K tiles per wave for K = hidden / ffn; U_F: gate/up row-blocks per workgroup;
+// MAXB: largest batch the instance serves.  Hidden row-blocks (q/k/v, o_proj, down) are at most
+// one per workgroup.
 template <int TPW_D, int TPW_F, int U_F, int MAXB>
 __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   constexpr int NS_D = (MAXB * TPW_D * DS_WAVES * 16 + DS_THREADS - 1) / DS_THREADS;
   constexpr int NS_F = (MAXB * TPW_F * DS_WAVES * 16 + DS_THREADS - 1) / DS_THREADS;
   extern __shared__ __align__(16) unsigned char smem[];
-  // once the loop condition has gone false a further iteration leaves everything as it is
+  // once the loop condition has gone false a further iteration leaves everything as it is; so does
+  // every launch after one that failed (the error word is sticky)
   if (*a.keep_going == 0) return;
+  if (__hip_atomic_load((DS_GLOBAL unsigned*)(a.sync + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
   const int KT_D = (a.d + 127) / 128, KT_F = (a.ffn + 127) / 128;
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
   f16* xs = reinterpret_cast<f16*>(smem);
   float* att_lds = reinterpret_cast<float*>(smem);           // the attention phase reuses the activation area
   float* red = reinterpret_cast<float*>(smem + a.region0);
   float* scratch = red + 2 * DS_RED;                          // norm sums, then selection scratch, then flags
-  int* lds_flag = reinterpret_cast<int*>(scratch + DS_WAVES * DS_MAXB + 64);
-  f16* normw = reinterpret_cast<f16*>(scratch + DS_TAIL_FLOATS);   // [d]
-  f16* cs = normw + ((a.d + 7) & ~7);                              // [D]: cos, sin of this step's angles
+  int* lds_dead = reinterpret_cast<int*>(scratch + DS_WAVES * DS_MAXB + 64);
+  f16* normw = reinterpret_cast<f16*>(scratch + DS_TAIL_FLOATS);   // [d rounded up to 512]: normw_fetch writes whole KiB
+  f16* cs = normw + ((a.d + 511) & ~511);                          // [D]: cos, sin of this step's angles
   uint32_t* lds_layers = reinterpret_cast<uint32_t*>(cs + DS_D);   // [n_layer] descriptors
 
   const int M = a.B;
   const int step = *a.step;
   const int nb_d = (a.d + 15) / 16, nb_f = (a.ffn + 15) / 16, nb_v = (a.vocab + 15) / 16;
-  Grid g;
-  g.sync = a.sync; g.G = gridDim.x; g.wg = blockIdx.x; g.dead = false;
-  g.epoch = __hip_atomic_load(a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  const int G = gridDim.x, wg = blockIdx.x;
+  struct { int wg; } g{wg};       // for TRACE
+  (void)g;
+  const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  Waiter w{a.sync + 1, lds_dead, 0};
   int red_buf = 0;
+  const size_t xslot = (size_t)M * a.d;      // halves of one residual-stream slot
 
-  // ---- set-up: descriptors and this step's rotary factors into LDS, embedding rows into x
+  // ---- set-up: fill the slots, descriptors and this step's rotary factors into LDS, embedding rows
   {
     const int tid = thread_id();
+    if (tid == 0) *lds_dead = 0;
+    const u32x4 filler = {DS_EMPTY32, DS_EMPTY32, DS_EMPTY32, DS_EMPTY32};
+    char* fill = reinterpret_cast<char*>(a.xres + xslot);
+    for (size_t off = ((size_t)wg * DS_THREADS + tid) * 16; off < a.fill_bytes; off += (size_t)G * DS_THREADS * 16) {
+      const size_t win = off & ~(((size_t)1 << 30) - 1);     // a buffer descriptor spans less than 4 GiB
+      put16(fill + win, a.fill_bytes - win < ((size_t)1 << 31) ? a.fill_bytes - win : ((size_t)1 << 31), off - win, filler);
+    }
+    for (size_t i = ((size_t)wg * DS_THREADS + tid) * 8; i < (size_t)M * a.vocab; i += (size_t)G * DS_THREADS * 8)
+      put16(a.logits, (size_t)M * a.vocab * 2, i * 2, filler);
     for (int i = tid; i < a.n_layer * DS_LAYER_WORDS; i += DS_THREADS) lds_layers[i] = a.layers[i];
     if (tid < DS_D / 2) {
       const f16 ang = (f16)((float)(f16)(float)step * (float)a.inv_freq[tid]);
       cs[tid] = (f16)cosf((float)ang);
       cs[DS_D / 2 + tid] = (f16)sinf((float)ang);
     }
-    if (tid == 0) { lds_flag[0] = 0; lds_flag[1] = 0; }
-    // x[b] = embed[container[b, step]] (layers/embedding.py:34-36)
+    // xres[0][b] = embed[container[b, step]] (layers/embedding.py:34-36)
     const int col = step < a.max_len ? step : a.max_len - 1;
-    for (int i = g.wg * DS_THREADS + tid; i < M * a.d; i += g.G * DS_THREADS) {
+    for (int i = wg * DS_THREADS + tid; i < M * a.d; i += G * DS_THREADS) {
       const int b = i / a.d, c = i % a.d;
       int id = a.container[(size_t)b * a.max_len + col];
       id = id < 0 ? 0 : (id >= a.vocab ? a.vocab - 1 : id);
-      put(a.x + i, a.embed[(size_t)id * a.d + c]);
+      put(a.xres + i, a.embed[(size_t)id * a.d + c]);
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // every wave stored here
   wg_sync();
 
   Unit<FmtW4, 3, TPW_D> t_qkv;
@@ -670,142 +714,124 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   Unit<FmtW4, 1, TPW_F> t_d;
   {
     const LayerPtrs L0 = layer_ptrs(lds_layers, 0);
-    normw_commit(normw_request(L0.get<const f16>(P_N1), a.d), normw, a.d);
+    normw_fetch(L0.get<const f16>(P_N1), normw, a.d);
     const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
-    load_unit(t_qkv, m3, g.wg, nb_d, a.d, KT_D);
+    load_unit(t_qkv, m3, wg, nb_d, a.d, KT_D);
   }
-  grid_barrier(g, lds_flag);
+  grid_barrier(a.sync, epoch, G, wg, w);
+  bool alive = *lds_dead == 0;
 
-  // Within a phase the order is: request the activations, wait for them, and only then request
-  // weights for later phases.  A compute unit returns loads in the order it received them from all
-  // of its waves, so an activation load issued behind a burst of weight requests would wait for
-  // those; issued first it takes half a microsecond.  Weights requested in one phase land while it
-  // computes, publishes and synchronises; the attention phase, all latency, requests none.
-  for (int li = 0; li < a.n_layer && !g.dead; ++li) {
+  // the residual element of this thread's output channel (epilogue mapping of gemv_unit, N = d)
+  f16 res = (f16)0.0f;
+  if (alive) {
+    const int tid = thread_id();
+    const int m_ = tid >> 4, n = wg * 16 + (tid & 15);
+    const bool on = m_ < M && n < a.d;
+    res = wait_value(a.xres + (on ? (size_t)m_ * a.d + n : 0), on, w);
+  }
+
+  for (int li = 0; li < a.n_layer && alive; ++li) {
     const LayerPtrs L = layer_ptrs(lds_layers, li);
     const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
-    Staged<NS_D> st;
-    Staged<NS_F> st_f;
-    // ---- RMSNorm + q/k/v; a row of the [B, 3d] buffer holds q | k | v.
+    f16* const x_in = a.xres + (size_t)(2 * li) * xslot;        // residual stream entering the layer
+    f16* const x_mid = x_in + xslot;                             // after attention
+    f16* const x_out = x_mid + xslot;                            // after the MLP
+    // ---- RMSNorm + q/k/v; a row of the [B, 3d] slot holds q | k | v.
     //      Requests o_proj and the first two gate/up units.
     TRACE(0);
-    stage_request(st, a.x, M, a.d, KT_D);
-    stage_commit(st, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch);
+    alive = stage<NS_D, MAXB>(x_in, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
+    if (!alive) break;
     {
       const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
-      load_unit(t_o, mo, g.wg, nb_d, a.d, KT_D);
+      load_unit(t_o, mo, wg, nb_d, a.d, KT_D);
 #pragma unroll
-      for (int k = 0; k < U_F && k < 2; ++k) load_unit(t_gu[k], mgu, g.wg + k * g.G, nb_f, a.ffn, KT_D);
+      for (int k = 0; k < U_F && k < 2; ++k) load_unit(t_gu[k], mgu, wg + k * G, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
     {
-      f16* const o3[3] = {a.qkv, a.qkv + a.d, a.qkv + 2 * a.d};
-      gemv_unit<FmtW4, 3, TPW_D, EPI_STORE>(t_qkv, o3, 3 * a.d, (f16)0.0f, g.wg, nb_d, a.d, KT_D, M, xs, xstride, red,
-                                            red_buf);
+      f16* q = a.qkv + (size_t)li * M * 3 * a.d;
+      f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
+      gemv_unit<FmtW4, 3, TPW_D, EPI_STORE, MAXB>(t_qkv, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs, xstride,
+                                                  red, red_buf);
     }
     TRACE(2);
-    release_results();
-    TRACE(3);
-    grid_barrier(g, lds_flag);
-    TRACE(4);
     // ---- rotary + KV append + attention
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
-      for (int u = g.wg; u < units; u += g.G) attention_unit(a, kring, u, step, att_lds, cs, lds_flag + 1);
+      for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
     }
-    TRACE(5);
-    release_results();
-    TRACE(6);
-    grid_barrier(g, lds_flag);
-    TRACE(7);
+    TRACE(3);
     // ---- o_proj + residual.  Requests the remaining gate/up units and the RMSNorm weights of the MLP.
-    f16 res;
-    f16x8 nw;
-    stage_request(st, a.ctx, M, a.d, KT_D);
-    res = residual_at(a.x, g.wg, a.d, M);
-    stage_commit(st, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch);
-    nw = normw_request(L.get<const f16>(P_N2), a.d);
+    alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
+    if (!alive) break;
 #pragma unroll
-    for (int k = 2; k < U_F; ++k) load_unit(t_gu[k], mgu, g.wg + k * g.G, nb_f, a.ffn, KT_D);
+    for (int k = 2; k < U_F; ++k) load_unit(t_gu[k], mgu, wg + k * G, nb_f, a.ffn, KT_D);
+    TRACE(4);
+    {
+      f16* const o1[1] = {x_mid};
+      res = gemv_unit<FmtW4, 1, TPW_D, EPI_RESIDUAL, MAXB>(t_o, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride, red,
+                                                          red_buf);
+    }
+    normw_fetch(L.get<const f16>(P_N2), normw, a.d);
+    TRACE(5);
+    // ---- RMSNorm + gate/up + SwiGLU.  Requests down once the first unit has been multiplied.
+    alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
+    if (!alive) break;
+    TRACE(6);
+    {
+      f16* act = a.act + (size_t)li * M * a.ffn;
+      f16* const o2[2] = {act, act};
+#pragma unroll
+      for (int k = 0; k < U_F; ++k) {
+        gemv_unit<FmtW4, 2, TPW_D, EPI_SWIGLU, MAXB>(t_gu[k], o2, a.ffn, (f16)0.0f, wg + k * G, nb_f, a.ffn, KT_D, M, xs,
+                                                     xstride, red, red_buf);
+        if (k == (U_F > 1 ? 1 : 0)) {      // registers of the units multiplied so far are free now
+          const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
+          load_unit(t_d, md, wg, nb_d, a.d, KT_F);
+        }
+      }
+    }
+    TRACE(7);
+    // ---- down + residual.  Requests the q/k/v of the next layer and the next RMSNorm weights.
+    alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w);
+    if (!alive) break;
+    const bool more = li + 1 < a.n_layer;
+    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
+    {
+      const Mat m3[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
+      load_unit(t_qkv, m3, wg, nb_d, a.d, KT_D);
+    }
     TRACE(8);
     {
-      f16* const o1[1] = {a.x};
-      gemv_unit<FmtW4, 1, TPW_D, EPI_RESIDUAL>(t_o, o1, a.d, res, g.wg, nb_d, a.d, KT_D, M, xs, xstride, red, red_buf);
+      f16* const o1[1] = {x_out};
+      res = gemv_unit<FmtW4, 1, TPW_F, EPI_RESIDUAL, MAXB>(t_d, o1, a.d, res, wg, nb_d, a.d, KT_F, M, xs, xstride, red,
+                                                          red_buf);
     }
-    normw_commit(nw, normw, a.d);
+    normw_fetch(more ? Ln.get<const f16>(P_N1) : a.final_norm, normw, a.d);
     TRACE(9);
-    release_results();
-    TRACE(10);
-    grid_barrier(g, lds_flag);
-    TRACE(11);
-    // ---- RMSNorm + gate/up + SwiGLU.  Requests down.
-    stage_request(st, a.x, M, a.d, KT_D);
-    stage_commit(st, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch);
-    {
-      const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
-      load_unit(t_d, md, g.wg, nb_d, a.d, KT_F);
-    }
-    TRACE(12);
-    {
-      f16* const o2[2] = {a.act, a.act};
-#pragma unroll
-      for (int k = 0; k < U_F; ++k)
-        gemv_unit<FmtW4, 2, TPW_D, EPI_SWIGLU>(t_gu[k], o2, a.ffn, (f16)0.0f, g.wg + k * g.G, nb_f, a.ffn, KT_D, M, xs,
-                                               xstride, red, red_buf);
-    }
-    TRACE(13);
-    release_results();
-    TRACE(14);
-    grid_barrier(g, lds_flag);
-    TRACE(15);
-    // ---- down + residual.  Requests the q/k/v of the next layer and the next RMSNorm weights.
-    stage_request(st_f, a.act, M, a.ffn, KT_F);
-    res = residual_at(a.x, g.wg, a.d, M);
-    stage_commit(st_f, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch);
-    {
-      const bool more = li + 1 < a.n_layer;
-      const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
-      nw = normw_request(more ? Ln.get<const f16>(P_N1) : a.final_norm, a.d);
-      const Mat m3[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
-      load_unit(t_qkv, m3, g.wg, nb_d, a.d, KT_D);
-    }
-    TRACE(16);
-    {
-      f16* const o1[1] = {a.x};
-      gemv_unit<FmtW4, 1, TPW_F, EPI_RESIDUAL>(t_d, o1, a.d, res, g.wg, nb_d, a.d, KT_F, M, xs, xstride, red, red_buf);
-    }
-    normw_commit(nw, normw, a.d);
-    TRACE(17);
-    release_results();
-    TRACE(18);
-    grid_barrier(g, lds_flag);
-    TRACE(19);
   }
   // ---- final RMSNorm + lm_head, streamed unit by unit with the next unit's tiles in flight
-  if (!g.dead) {
+  if (alive) alive = stage<NS_D, MAXB>(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, KT_D, xs, xstride, normw, a.eps,
+                                       scratch, w);
+  if (alive) {
     const Mat m1[1] = {{a.head, nullptr}};
     f16* const o1[1] = {a.logits};
-    Staged<NS_D> st;
-    stage_request(st, a.x, M, a.d, KT_D);
     Unit<FmtF16, 1, TPW_D> cur;
-    load_unit(cur, m1, g.wg, nb_v, a.vocab, KT_D);
-    stage_commit(st, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch);
-    for (int u = g.wg; u < nb_v; u += g.G) {
+    load_unit(cur, m1, wg, nb_v, a.vocab, KT_D);
+    for (int u = wg; u < nb_v; u += G) {
       Unit<FmtF16, 1, TPW_D> nxt;
-      load_unit(nxt, m1, u + g.G, nb_v, a.vocab, KT_D);
-      gemv_unit<FmtF16, 1, TPW_D, EPI_STORE>(cur, o1, a.vocab, (f16)0.0f, u, nb_v, a.vocab, KT_D, M, xs, xstride, red,
-                                             red_buf);
+      load_unit(nxt, m1, u + G, nb_v, a.vocab, KT_D);
+      gemv_unit<FmtF16, 1, TPW_D, EPI_STORE, MAXB>(cur, o1, a.vocab, (f16)0.0f, u, nb_v, a.vocab, KT_D, M, xs, xstride,
+                                                   red, red_buf);
       cur = nxt;
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  grid_barrier(g, lds_flag);
   // ---- selection and bookkeeping
-  if (g.wg == 0) {
-    if (!g.dead) select_and_advance(a, scratch + DS_WAVES * DS_MAXB);
+  if (wg == 0) {
+    if (alive) select_and_advance(a, scratch + DS_WAVES * DS_MAXB, w);
     if (thread_id() == 0)   // epoch base of the next launch
-      __hip_atomic_store(a.sync, g.epoch - 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store((DS_GLOBAL unsigned*)a.sync, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 }
 
@@ -829,14 +855,41 @@ int device_cus(int* cus) {
   return 0;
 }
 
+int splits_for(int cus, int B, int H) {
+  const int n = cus / (B * H);
+  return n < 1 ? 1 : (n > DS_MAX_SPLIT ? DS_MAX_SPLIT : n);
+}
+
+// byte offsets of the workspace parts
+struct Layout {
+  size_t sync, xres, qkv, ctx, act, part, trace, total;
+};
+Layout layout_for(const pta_decode_model* m, int cus) {
+  const size_t B = m->batch, d = m->hidden, L = m->n_layer, f = m->ffn, H = m->n_head;
+  Layout l;
+  l.sync = 0;
+  l.xres = align256((size_t)(16 + cus) * 4);
+  l.qkv = l.xres + align256((2 * L + 1) * B * d * 2);
+  l.ctx = l.qkv + align256(L * B * 3 * d * 2);
+  l.act = l.ctx + align256(L * B * d * 2);
+  l.part = l.act + align256(L * B * f * 2);
+  l.trace = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
+  l.total = l.trace + (size_t)cus * 256;
+  return l;
+}
+
+bool shape_ok(const pta_decode_model* m) {
+  return m && m->batch >= 1 && m->batch <= DS_MAXB && m->hidden > 0 && m->n_head > 0 && m->ffn > 0 && m->vocab > 0 &&
+         m->max_len > 0 && m->n_layer > 0 && m->head_dim == DS_D && m->hidden == m->n_head * DS_D && m->ffn % 8 == 0 &&
+         m->vocab % 8 == 0;
+}
+
 }  // namespace
 
-extern "C" size_t pta_decode_step_workspace_bytes(int batch, int n_head, int head_dim) {
+extern "C" size_t pta_decode_step_workspace_bytes(const pta_decode_model* model) {
   int cus = 0;
-  if (batch <= 0 || batch > DS_MAXB || n_head <= 0 || head_dim != DS_D || device_cus(&cus) != 0) return 0;
-  // sync words | tickets | attention partials | per-workgroup timestamps of instrumented builds
-  return align256((size_t)(16 + cus) * 4) + align256((size_t)batch * n_head * 4) +
-         align256((size_t)batch * n_head * DS_MAX_SPLIT * (DS_D + 2) * 4) + (size_t)cus * 256;
+  if (!shape_ok(model) || device_cus(&cus) != 0) return 0;
+  return layout_for(model, cus).total;
 }
 
 extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
@@ -844,9 +897,10 @@ extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_deco
   PTA_REQUIRE(mdl && st && workspace, "pta_llama_decode_step: null pointer");
   PTA_REQUIRE(mdl->layers && mdl->n_layer > 0 && mdl->embed && mdl->final_norm && mdl->head && mdl->inv_freq,
               "pta_llama_decode_step: incomplete model");
-  PTA_REQUIRE(st->container && st->mask && st->stop_mask && st->step && st->keep_going && st->next_ids && st->x &&
-                  st->qkv && st->ctx && st->act && st->logits,
+  PTA_REQUIRE(st->container && st->mask && st->stop_mask && st->step && st->keep_going && st->next_ids && st->logits,
               "pta_llama_decode_step: incomplete state");
+  PTA_REQUIRE(pta_aligned(workspace, 256) && pta_aligned(st->logits, 16),
+              "pta_llama_decode_step: the workspace must be 256-byte aligned and the logits 16-byte aligned");
   const int B = mdl->batch, d = mdl->hidden, H = mdl->n_head, ffn = mdl->ffn;
   PTA_REQUIRE(B >= 1 && d > 0 && H > 0 && ffn > 0 && mdl->vocab > 0 && mdl->max_len > 0,
               "pta_llama_decode_step: empty shape");
@@ -859,14 +913,16 @@ extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_deco
   Variant* var = nullptr;
   for (Variant& v : g_variants)
     if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B <= v.maxb && !var) var = &v;
-  if (B > DS_MAXB || mdl->head_dim != DS_D || d != H * DS_D || ffn % 8 != 0 || mdl->vocab % 8 != 0 || nb_d > cus || !var) {
+  if (!shape_ok(mdl) || nb_d > cus || !var) {
     pta_set_error("pta_llama_decode_step: supports batch <= %d, head size %d, hidden = heads * head size <= %d, ffn "
-                  "and vocabulary sizes that are multiples of 8, and the (hidden, ffn) of the 7B model or small test shapes "
-                  "(got batch %d, head size %d, hidden %d, heads %d, ffn %d)",
-                  DS_MAXB, DS_D, 16 * cus, B, mdl->head_dim, d, H, ffn);
+                  "and vocabulary sizes that are multiples of 8, and the (hidden, ffn) of the 7B model or small test "
+                  "shapes (got batch %d, head size %d, hidden %d, heads %d, ffn %d, vocabulary %d)",
+                  DS_MAXB, DS_D, 16 * cus, B, mdl->head_dim, d, H, ffn, mdl->vocab);
     return PTA_EUNSUPPORTED;
   }
 
+  const Layout lay = layout_for(mdl, cus);
+  char* ws = (char*)workspace;
   DsArgs a{};
   a.layers = reinterpret_cast<const uint32_t*>(mdl->layers);
   a.n_layer = mdl->n_layer;
@@ -876,21 +932,22 @@ extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_deco
   a.container = st->container; a.mask = (f16*)st->mask; a.stop_mask = st->stop_mask; a.step = st->step;
   a.keep_going = st->keep_going; a.next_ids = st->next_ids;
   a.pad_id = mdl->pad_id; a.eos_id = mdl->eos_id; a.early_stop = mdl->early_stop;
-  a.x = (f16*)st->x; a.qkv = (f16*)st->qkv; a.ctx = (f16*)st->ctx; a.act = (f16*)st->act; a.logits = (f16*)st->logits;
-  const size_t sync_b = align256((size_t)(16 + cus) * 4), tick_b = align256((size_t)B * H * 4);
-  a.sync = (unsigned*)workspace;
-  a.tickets = (unsigned*)((char*)workspace + sync_b);
-  a.attn_part = (float*)((char*)workspace + sync_b + tick_b);
-  a.trace = (unsigned long long*)((char*)workspace + sync_b + tick_b +
-                                  align256((size_t)B * H * DS_MAX_SPLIT * (DS_D + 2) * 4));
-  int nsplit = cus / (B * H);
-  a.nsplit = nsplit < 1 ? 1 : (nsplit > DS_MAX_SPLIT ? DS_MAX_SPLIT : nsplit);
+  a.logits = (f16*)st->logits;
+  a.sync = (unsigned*)(ws + lay.sync);
+  a.xres = (f16*)(ws + lay.xres);
+  a.qkv = (f16*)(ws + lay.qkv);
+  a.ctx = (f16*)(ws + lay.ctx);
+  a.act = (f16*)(ws + lay.act);
+  a.part = (float*)(ws + lay.part);
+  a.trace = (unsigned long long*)(ws + lay.trace);
+  a.fill_bytes = lay.trace - (lay.xres + (size_t)B * d * 2);   // everything after the first residual slot
+  a.nsplit = splits_for(cus, B, H);
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
   size_t region0 = (size_t)B * xstride * 2;
   if (region0 < (size_t)DS_ATT_FLOATS * 4) region0 = (size_t)DS_ATT_FLOATS * 4;
   region0 = (region0 + 15) & ~(size_t)15;
   a.region0 = (int)region0;
-  const size_t lds = region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 7) & ~7) * 2 + DS_D * 2 +
+  const size_t lds = region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
                      (size_t)mdl->n_layer * sizeof(pta_decode_layer);
   PTA_REQUIRE(lds <= 160 * 1024, "pta_llama_decode_step: %zu bytes of LDS exceed a compute unit's 160 KiB", lds);
 

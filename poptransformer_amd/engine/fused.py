@@ -167,8 +167,7 @@ class FusedDecoder:
                                sg=g.w.scale, su=u.w.scale, sd=b.mlp_out.w.scale, norm1=b.norm1[0], norm2=b.norm2[0],
                                kv_ring=ring))
         state = dict(container=self.container, mask=self.mask, stop_mask=self.stop_mask, step=self.step,
-                     keep_going=self.keep_going, next_ids=self.next_ids, x=self.x, qkv=self.qkv, ctx=self.ctx,
-                     act=self.act, logits=self.logits)
+                     keep_going=self.keep_going, next_ids=self.next_ids, logits=self.logits)
         self.persistent = K.DecodeStep(layers, w.embed, w.final_norm[0], w.head.w.tiled, w.inv_freq, s.batch, s.d_model,
                                        s.n_head, s.head_dim, w.blocks[0].mlp_out.K, s.vocab, s.max_len, s.eps, s.pad_id,
                                        s.eos_id, s.early_stop, state)

@@ -445,21 +445,21 @@ class DecodeStep:
     def __init__(self, layers, embed, final_norm, head, inv_freq, batch, hidden, n_head, head_dim, ffn, vocab, max_len,
                  eps, pad_id, eos_id, early_stop, state):
         lib = _lib.load()
-        nbytes = lib.pta_decode_step_workspace_bytes(batch, n_head, head_dim)
-        if nbytes == 0:
-            raise NotImplementedError(f"decode step kernel: unsupported batch {batch} / head size {head_dim}")
         dev = embed.device
-        self.workspace = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         arr = (_lib.DecodeLayer * len(layers))()
         for dst, src in zip(arr, layers):
             for name, t in src.items():
                 setattr(dst, name, t.data_ptr())
-        host = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8)
-        self.layers = host.to(dev)
+        self.layers = torch.frombuffer(bytearray(bytes(arr)), dtype=torch.uint8).to(dev)
         self._keep = (layers, embed, final_norm, head, inv_freq, state)
         self.model = _lib.DecodeModel(self.layers.data_ptr(), len(layers), embed.data_ptr(), final_norm.data_ptr(),
                                       head.data_ptr(), inv_freq.data_ptr(), batch, hidden, n_head, head_dim, ffn, vocab,
                                       max_len, eps, pad_id, eos_id, 1 if early_stop else 0)
+        nbytes = lib.pta_decode_step_workspace_bytes(ctypes.byref(self.model))
+        if nbytes == 0:
+            raise NotImplementedError(f"decode step kernel: unsupported shape (batch {batch}, head size {head_dim}, "
+                                      f"hidden {hidden}, ffn {ffn}, vocabulary {vocab})")
+        self.workspace = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
         self.state = _lib.DecodeState(**{k: v.data_ptr() for k, v in state.items()})
 
     def launch(self):
