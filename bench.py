@@ -85,6 +85,50 @@ def cpu_baseline(seconds_budget=20.0):
                       f"layer time scaled x{LLAMA2_7B['num_hidden_layers'] // layers}"}
 
 
+PMC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "llama2_7b_int4_b1_decode_step_pmc.txt")
+
+
+def summarize_pmc(fetch_csv, write_csv):
+    """FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of the decode-step kernel, each scaled by what the
+    same counter reads for the 1 GiB calibration kernel of --copy-calibration."""
+    import csv
+
+    def per_kernel(path, counter):
+        vals = {}
+        for r in csv.DictReader(open(path)):
+            if r["Counter_Name"] == counter:
+                vals.setdefault(r["Kernel_Name"], []).append(float(r["Counter_Value"]))
+        return vals
+
+    out = {}
+    for counter, path in (("FETCH_SIZE", fetch_csv), ("WRITE_SIZE", write_csv)):
+        vals = per_kernel(path, counter)
+        step = [v for k, v in vals.items() if "decode_step_kernel" in k]
+        cal = [v for k, v in vals.items() if "neg_kernel" in k or "NegFunctor" in k or "neg" in k.lower()]
+        if not step or not cal:
+            raise SystemExit(f"{path}: decode-step or calibration kernel not found")
+        step, cal = step[0], cal[0]
+        cal_kib = sum(cal) / len(cal)
+        factor = (1 << 20) / cal_kib                      # the calibration kernel moves 1 GiB = 2^20 KiB each way
+        mean_kib = sum(step) / len(step)
+        out[counter] = mean_kib * factor * 1024
+        print(f"{counter}: decode_step_kernel mean {mean_kib:.1f} KiB over {len(step)} launches "
+              f"(min {min(step):.1f}, max {max(step):.1f}); calibration kernel reads {cal_kib:.1f} KiB for 2^20 KiB "
+              f"-> factor {factor:.4f} -> {out[counter]:.0f} bytes per launch")
+    print(f"traffic_bytes_per_launch = {out['FETCH_SIZE'] + out['WRITE_SIZE']:.0f}")
+
+
+def recorded_traffic():
+    """HBM bytes per launch of the decode-step kernel from the committed counter summary, or None."""
+    try:
+        for line in open(PMC_SUMMARY):
+            if line.startswith("traffic_bytes_per_launch"):
+                return float(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -94,7 +138,16 @@ def main():
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
                     help="default: persistent when the batch fits it (<= 4), else operators")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
+                         "of known traffic for scaling hardware counters (FETCH_SIZE / WRITE_SIZE) collected over this run")
+    ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: print the traffic summary of two rocprofv3 --pmc runs of this script "
+                         "(counter_collection.csv of the FETCH_SIZE run and of the WRITE_SIZE run, both with --copy-calibration)")
     args = ap.parse_args()
+    if args.summarize_pmc:
+        summarize_pmc(*args.summarize_pmc)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
@@ -193,8 +246,15 @@ def main():
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
+                     "traffic": recorded_traffic() if executor == "persistent" and B == 1 else None,
+                     "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, dtype=torch.float16, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.neg(src, out=dst)
+        torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
