@@ -28,9 +28,13 @@
 //
 // A compute unit returns loads in the order it received them from all of its waves, so a small
 // activation load issued behind a burst of weight requests waits for those.  Each phase therefore
-// first obtains its activations and only then requests weights for later phases; the attention
-// phase, which is all latency, requests none.  All waves request weights at the same program
-// points, which lets the compiler count exactly how many requests may stay in flight at each use.
+// first obtains its activations and only then requests weights for later phases.  A compute unit
+// also accepts only a few tens of KiB of requests at a time: a wave that requests more is held at
+// the request until earlier data has arrived, and the workgroup's barrier behind the phase's product
+// waits for that wave.  The requests are therefore spread over the phases (64-96 KiB per workgroup
+// and phase at the 7B shape) instead of being issued where registers first become free.  Every
+// tile has a fixed place in one register array for the whole layer loop, so that no requested tile
+// is ever moved between registers (a move waits for the load and for the burst around it).
 #include "common.h"
 #include "formats.h"
 
@@ -262,35 +266,13 @@ __device__ __forceinline__ void load_unit(Unit<Fmt, NRB, TPW>& t, const Mat (&m)
 
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 
-// out[r][m, n] = sum_k xs[m, k] * W_r[n, k] for unit u, whose tiles are in t.  `res` is the residual
-// element of this thread (EPI_RESIDUAL); the value the thread stored is returned (it is the
-// residual of the same thread in the next residual phase).
-template <class Fmt, int NRB, int TPW, int EPI, int MAXB>
-__device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* const (&out)[NRB], int ostride, f16 res,
-                                         int u, int n_units, int N, int KT, int M, const f16* xs, int xstride,
-                                         float* red, int& red_buf) {
-  if (u >= n_units) return res;
+// The partial sums of the useful accumulator columns (activation rows m < M) of all waves meet in
+// LDS; `res` is the residual element of this thread (EPI_RESIDUAL), and the value the thread
+// stored is returned (it is the residual of the same thread in the next residual phase).
+template <int NRB, int EPI>
+__device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (&out)[NRB], int ostride, f16 res, int u,
+                                           int N, int M, float* red, int& red_buf) {
   const int wave = wave_id(), lane = lane_id();
-  int mrow = lane & 15;
-  mrow = mrow < M ? mrow : M - 1;
-  const f16* xl = xs + (size_t)mrow * xstride + (lane >> 4) * 8;
-  f32x4 acc[NRB];
-#pragma unroll
-  for (int r = 0; r < NRB; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int i = 0; i < TPW; ++i) {
-    const int kt = wave + i * DS_WAVES;
-    if (kt < KT) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
-#pragma unroll
-        for (int r = 0; r < NRB; ++r)
-          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(t.w[r][i], j, t.sc[r]), xb, acc[r], 0, 0, 0);
-      }
-    }
-  }
-  // the partial sums of the useful accumulator columns (activation rows m < M) meet in LDS
   float* rb = red + red_buf * DS_RED;
   if ((lane & 15) < M) {
 #pragma unroll
@@ -332,6 +314,93 @@ __device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* cons
   }
   red_buf ^= 1;
   return y;
+}
+
+// out[r][m, n] = sum_k xs[m, k] * W_r[n, k] for unit u, whose tiles are in t.  `res` is the residual
+// element of this thread (EPI_RESIDUAL); the value the thread stored is returned (it is the
+// residual of the same thread in the next residual phase).
+template <class Fmt, int NRB, int TPW, int EPI, int MAXB>
+__device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* const (&out)[NRB], int ostride, f16 res,
+                                         int u, int n_units, int N, int KT, int M, const f16* xs, int xstride,
+                                         float* red, int& red_buf) {
+  if (u >= n_units) return res;
+  const int wave = wave_id(), lane = lane_id();
+  int mrow = lane & 15;
+  mrow = mrow < M ? mrow : M - 1;
+  const f16* xl = xs + (size_t)mrow * xstride + (lane >> 4) * 8;
+  f32x4 acc[NRB];
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) {
+    const int kt = wave + i * DS_WAVES;
+    if (kt < KT) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
+#pragma unroll
+        for (int r = 0; r < NRB; ++r)
+          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(t.w[r][i], j, t.sc[r]), xb, acc[r], 0, 0, 0);
+      }
+    }
+  }
+  return finish_unit<NRB, EPI>(acc, out, ostride, res, u, N, M, red, red_buf);
+}
+
+// The INT4 tiles of the layer phases live in ONE register array with a fixed place for every unit
+// (the map is in the kernel), and so do their scales.  A place is written by the loads of the unit
+// that owns it at that point of the layer and read by that unit's products, always under the same
+// compile-time index, so no value ever has to move between registers: a move of a requested tile
+// would have to wait for its load, and with it for the whole burst of requests around it.
+template <int NRB, int TPW, int BASE, int SCBASE, int NSLOT, int NSC>
+__device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], const Mat (&m)[NRB], int u, int n_units,
+                                           int N, int KT) {
+  static_assert(BASE + NRB * TPW <= NSLOT && SCBASE + NRB <= NSC, "unit outside the register array");
+  const int wave = wave_id(), lane = lane_id();
+  u = u < n_units ? u : n_units - 1;
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) {
+    const DS_GLOBAL u32x4* p = as_global(m[r].tiled) + (size_t)u * KT * 64 + lane;
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+      int kt = wave + i * DS_WAVES;
+      kt = kt < KT ? kt : KT - 1;
+      S[BASE + r * TPW + i] = __builtin_nontemporal_load(p + (size_t)kt * 64);
+    }
+    int row = u * 16 + (lane & 15);
+    row = row < N ? row : N - 1;
+    const f16 sv = as_global(m[r].scale)[row];
+    SC[SCBASE + r] = f16x2{sv, sv};
+  }
+}
+
+template <int NRB, int TPW, int EPI, int MAXB, int BASE, int SCBASE, int NSLOT, int NSC>
+__device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB],
+                                          int ostride, f16 res, int u, int n_units, int N, int KT, int M, const f16* xs,
+                                          int xstride, float* red, int& red_buf) {
+  if (u >= n_units) return res;
+  const int wave = wave_id(), lane = lane_id();
+  int mrow = lane & 15;
+  mrow = mrow < M ? mrow : M - 1;
+  const f16* xl = xs + (size_t)mrow * xstride + (lane >> 4) * 8;
+  f32x4 acc[NRB];
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < TPW; ++i) {
+    const int kt = wave + i * DS_WAVES;
+    if (kt < KT) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
+#pragma unroll
+        for (int r = 0; r < NRB; ++r)
+          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(S[BASE + r * TPW + i][j], SC[SCBASE + r]), xb, acc[r],
+                                                          0, 0, 0);
+      }
+    }
+  }
+  return finish_unit<NRB, EPI>(acc, out, ostride, res, u, N, M, red, red_buf);
 }
 
 // i / per for i < 4 * per, without a division
@@ -708,15 +777,23 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   }
   wg_sync();
 
-  Unit<FmtW4, 3, TPW_D> t_qkv;
-  Unit<FmtW4, 1, TPW_D> t_o;
-  Unit<FmtW4, 2, TPW_D> t_gu[U_F];
-  Unit<FmtW4, 1, TPW_F> t_d;
+  // Places of the units in the tile array.  q/k/v, o_proj and the first two gate/up units are
+  // held together; the third gate/up unit is requested when q/k/v have been multiplied and takes
+  // their place; down is requested when the first two gate/up units have been multiplied and
+  // takes theirs; the next layer's q/k/v return to the start.
+  constexpr int NSLOT = 8 * TPW_D;
+  constexpr int S_QKV = 0, S_O = 3 * TPW_D, S_GU0 = 4 * TPW_D, S_GU2 = 0, S_D = 4 * TPW_D;
+  constexpr int NSC = 8;
+  constexpr int C_QKV = 0, C_O = 3, C_GU0 = 4, C_GU2 = 0, C_D = 4;
+  static_assert(U_F <= 3, "at most three gate/up units per workgroup");
+  static_assert(TPW_F <= 4 * TPW_D, "the down tiles take the place of two gate/up units");
+  u32x4 S[NSLOT];
+  f16x2 SC[NSC];
   {
     const LayerPtrs L0 = layer_ptrs(lds_layers, 0);
     normw_fetch(L0.get<const f16>(P_N1), normw, a.d);
     const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
-    load_unit(t_qkv, m3, wg, nb_d, a.d, KT_D);
+    load_slots<3, TPW_D, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
   }
   grid_barrier(a.sync, epoch, G, wg, w);
   bool alive = *lds_dead == 0;
@@ -737,22 +814,21 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     f16* const x_mid = x_in + xslot;                             // after attention
     f16* const x_out = x_mid + xslot;                            // after the MLP
     // ---- RMSNorm + q/k/v; a row of the [B, 3d] slot holds q | k | v.
-    //      Requests o_proj and the first two gate/up units.
+    //      Requests o_proj and the first gate/up unit.
     TRACE(0);
     alive = stage<NS_D, MAXB>(x_in, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
     if (!alive) break;
     {
       const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
-      load_unit(t_o, mo, wg, nb_d, a.d, KT_D);
-#pragma unroll
-      for (int k = 0; k < U_F && k < 2; ++k) load_unit(t_gu[k], mgu, wg + k * G, nb_f, a.ffn, KT_D);
+      load_slots<1, TPW_D, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
+      load_slots<2, TPW_D, S_GU0, C_GU0>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
     {
       f16* q = a.qkv + (size_t)li * M * 3 * a.d;
       f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
-      gemv_unit<FmtW4, 3, TPW_D, EPI_STORE, MAXB>(t_qkv, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs, xstride,
-                                                  red, red_buf);
+      gemv_slots<3, TPW_D, EPI_STORE, MAXB, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs,
+                                                          xstride, red, red_buf);
     }
     TRACE(2);
     // ---- rotary + KV append + attention
@@ -760,18 +836,20 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
       for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
+      // the second gate/up unit: requested here and not with the first, so that no phase requests much
+      // more than the others (see the note on requests at the top of the file)
+      if constexpr (U_F > 1) load_slots<2, TPW_D, S_GU0 + 2 * TPW_D, C_GU0 + 2>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
-    // ---- o_proj + residual.  Requests the remaining gate/up units and the RMSNorm weights of the MLP.
+    // ---- o_proj + residual.  Requests the third gate/up unit and the RMSNorm weights of the MLP.
     alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
-#pragma unroll
-    for (int k = 2; k < U_F; ++k) load_unit(t_gu[k], mgu, wg + k * G, nb_f, a.ffn, KT_D);
+    if constexpr (U_F > 2) load_slots<2, TPW_D, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     TRACE(4);
     {
       f16* const o1[1] = {x_mid};
-      res = gemv_unit<FmtW4, 1, TPW_D, EPI_RESIDUAL, MAXB>(t_o, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride, red,
-                                                          red_buf);
+      res = gemv_slots<1, TPW_D, EPI_RESIDUAL, MAXB, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride,
+                                                               red, red_buf);
     }
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
@@ -782,15 +860,18 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     {
       f16* act = a.act + (size_t)li * M * a.ffn;
       f16* const o2[2] = {act, act};
-#pragma unroll
-      for (int k = 0; k < U_F; ++k) {
-        gemv_unit<FmtW4, 2, TPW_D, EPI_SWIGLU, MAXB>(t_gu[k], o2, a.ffn, (f16)0.0f, wg + k * G, nb_f, a.ffn, KT_D, M, xs,
-                                                     xstride, red, red_buf);
-        if (k == (U_F > 1 ? 1 : 0)) {      // registers of the units multiplied so far are free now
-          const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
-          load_unit(t_d, md, wg, nb_d, a.d, KT_F);
-        }
+      gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xs,
+                                                           xstride, red, red_buf);
+      if constexpr (U_F > 1)
+        gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU0 + 2 * TPW_D, C_GU0 + 2>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f,
+                                                                             a.ffn, KT_D, M, xs, xstride, red, red_buf);
+      {      // the places of the units multiplied so far are free now
+        const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
+        load_slots<1, TPW_F, S_D, C_D>(S, SC, md, wg, nb_d, a.d, KT_F);
       }
+      if constexpr (U_F > 2)
+        gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D,
+                                                             M, xs, xstride, red, red_buf);
     }
     TRACE(7);
     // ---- down + residual.  Requests the q/k/v of the next layer and the next RMSNorm weights.
@@ -800,13 +881,13 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
     {
       const Mat m3[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
-      load_unit(t_qkv, m3, wg, nb_d, a.d, KT_D);
+      load_slots<3, TPW_D, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
     }
     TRACE(8);
     {
       f16* const o1[1] = {x_out};
-      res = gemv_unit<FmtW4, 1, TPW_F, EPI_RESIDUAL, MAXB>(t_d, o1, a.d, res, wg, nb_d, a.d, KT_F, M, xs, xstride, red,
-                                                          red_buf);
+      res = gemv_slots<1, TPW_F, EPI_RESIDUAL, MAXB, S_D, C_D>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_F, M, xs, xstride,
+                                                               red, red_buf);
     }
     normw_fetch(more ? Ln.get<const f16>(P_N1) : a.final_norm, normw, a.d);
     TRACE(9);
@@ -817,14 +898,16 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   if (alive) {
     const Mat m1[1] = {{a.head, nullptr}};
     f16* const o1[1] = {a.logits};
-    Unit<FmtF16, 1, TPW_D> cur;
-    load_unit(cur, m1, wg, nb_v, a.vocab, KT_D);
-    for (int u = wg; u < nb_v; u += G) {
-      Unit<FmtF16, 1, TPW_D> nxt;
-      load_unit(nxt, m1, u + G, nb_v, a.vocab, KT_D);
-      gemv_unit<FmtF16, 1, TPW_D, EPI_STORE, MAXB>(cur, o1, a.vocab, (f16)0.0f, u, nb_v, a.vocab, KT_D, M, xs, xstride,
+    // two units in turn, each requested while the other is multiplied, each in registers of its own
+    Unit<FmtF16, 1, TPW_D> even, odd;
+    load_unit(even, m1, wg, nb_v, a.vocab, KT_D);
+    for (int u = wg; u < nb_v; u += 2 * G) {
+      load_unit(odd, m1, u + G, nb_v, a.vocab, KT_D);
+      gemv_unit<FmtF16, 1, TPW_D, EPI_STORE, MAXB>(even, o1, a.vocab, (f16)0.0f, u, nb_v, a.vocab, KT_D, M, xs, xstride,
                                                    red, red_buf);
-      cur = nxt;
+      load_unit(even, m1, u + 2 * G, nb_v, a.vocab, KT_D);
+      gemv_unit<FmtF16, 1, TPW_D, EPI_STORE, MAXB>(odd, o1, a.vocab, (f16)0.0f, u + G, nb_v, a.vocab, KT_D, M, xs, xstride,
+                                                   red, red_buf);
     }
   }
   // ---- selection and bookkeeping
