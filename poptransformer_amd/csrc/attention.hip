@@ -100,9 +100,16 @@ extern "C" int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const p
 
 // ------------------------------------------------------------------------------------------
 // Split-K decode attention with online softmax.
+//
+// The grid is fixed when the call is recorded (it may be replayed from a graph while the context
+// grows), so the number of splits per (sequence, head) is chosen from the batch alone - enough
+// workgroups to fill the machine, no more - and each split's range of cache rows is derived on the
+// device from the current step: chunk = ceil(valid / nsplit), rounded up to a multiple of 16 rows
+// and at least 32.  Splits beyond the valid rows exit at once.
 // ------------------------------------------------------------------------------------------
 constexpr int ATT_THREADS = 256;
 constexpr int ATT_WAVES = ATT_THREADS / 64;
+constexpr int ATT_UNROLL = 4;      // cache rows per lane group whose loads are in flight together
 
 struct AttnArgs {
   const f16* q;       // [B, Hq, D]
@@ -111,26 +118,34 @@ struct AttnArgs {
   const int32_t* step;
   float* part;        // [B*Hq, nsplit, D + 2]: running max, denominator, numerator
   f16* out;           // [B, Hq*D]
-  int B, Hq, Hkv, max_len, chunk, nsplit;
+  int B, Hq, Hkv, max_len, nsplit;
   int use_scale;
   f16 scale;
 };
 
+__device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
+  int c = (valid + nsplit - 1) / nsplit;
+  c = (c + 15) & ~15;
+  return c < 32 ? 32 : c;
+}
+
 // Partial attention of one (sequence, query head) over one chunk of cache rows.
-// LPP = D/8 lanes share a cache row (16 bytes each); a wave covers 64/LPP rows per load.
+// LPP = D/8 lanes share a cache row (16 bytes each); a wave covers 64/LPP rows per load, and
+// requests ATT_UNROLL such loads of K and of V before it uses the first.
 template <int D>
 __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   constexpr int LPP = D / 8;
   constexpr int PPW = 64 / LPP;
-  constexpr int NG = ATT_WAVES * PPW;
-  __shared__ float sm_m[NG], sm_l[NG];
-  __shared__ float sm_acc[NG][D];
+  constexpr int STRIDE = ATT_WAVES * PPW;
+  __shared__ float sm_m[ATT_WAVES], sm_l[ATT_WAVES];
+  __shared__ float sm_acc[ATT_WAVES][D];
   const int split = blockIdx.x, bh = blockIdx.y;
   const int step = *a.step;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
-  const int c0 = split * a.chunk;
+  const int chunk = attn_chunk(valid, a.nsplit);
+  const int c0 = split * chunk;
   if (c0 >= valid) return;
-  const int c1 = c0 + a.chunk < valid ? c0 + a.chunk : valid;
+  const int c1 = c0 + chunk < valid ? c0 + chunk : valid;
   const int b = bh / a.Hq, h = bh % a.Hq;
   const int hk = h / (a.Hq / a.Hkv);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -150,42 +165,73 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
 
-  for (int p0 = c0 + wave * PPW; p0 < c1; p0 += ATT_WAVES * PPW) {
-    const int p = p0 + grp;
-    const bool on = p < c1;
-    const int pc = on ? p : c1 - 1;
-    const f16x8 k8 = *reinterpret_cast<const f16x8*>(kb + (size_t)pc * D);
-    const f16x8 v8 = *reinterpret_cast<const f16x8*>(vb + (size_t)pc * D);
-    float s = 0.f;
+  for (int p0 = c0 + wave * PPW + grp; p0 < c1 + grp; p0 += STRIDE * ATT_UNROLL) {
+    f16x8 k8[ATT_UNROLL], v8[ATT_UNROLL];
+    bool on[ATT_UNROLL];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
+    for (int u = 0; u < ATT_UNROLL; ++u) {
+      const int p = p0 + u * STRIDE;
+      on[u] = p < c1;
+      const int pc = on[u] ? p : c1 - 1;
+      k8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (size_t)pc * D));
+      v8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(vb + (size_t)pc * D));
+    }
+    float x[ATT_UNROLL];
+    float mn = m;
 #pragma unroll
-    for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-    f16 s16 = (f16)s;                       // fp16 output of the q.K^T MatMul
-    if (a.use_scale) s16 = s16 * a.scale;   // fp16 multiply by fp16(1/sqrt(D))
-    const float x = on ? (float)s16 : -INFINITY;
-    const float mn = fmaxf(m, x);
-    const float corr = m == -INFINITY ? 0.f : __expf(m - mn);  // nothing accumulated yet
-    const float pe = on ? __expf(x - mn) : 0.f;
-    l = l * corr + pe;
+    for (int u = 0; u < ATT_UNROLL; ++u) {
+      float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
-    m = mn;
+      for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[u][e], s);
+#pragma unroll
+      for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      f16 s16 = (f16)s;                       // fp16 output of the q.K^T MatMul
+      if (a.use_scale) s16 = s16 * a.scale;   // fp16 multiply by fp16(1/sqrt(D))
+      x[u] = on[u] ? (float)s16 : -INFINITY;
+      mn = fmaxf(mn, x[u]);
+    }
+    if (mn != -INFINITY) {                    // some row of this group so far is valid
+      const float corr = m == -INFINITY ? 0.f : __expf(m - mn);
+      l *= corr;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] *= corr;
+#pragma unroll
+      for (int u = 0; u < ATT_UNROLL; ++u) {
+        const float pe = on[u] ? __expf(x[u] - mn) : 0.f;
+        l += pe;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[u][e], acc[e]);
+      }
+      m = mn;
+    }
   }
 
-  const int g = wave * PPW + grp;
-  if (sub == 0) { sm_m[g] = m; sm_l[g] = l; }
+  // the row groups of a wave merge in registers, the waves in LDS
 #pragma unroll
-  for (int e = 0; e < 8; ++e) sm_acc[g][d0 + e] = acc[e];
+  for (int o = LPP; o < 64; o <<= 1) {
+    const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
+    const float mn = fmaxf(m, mo);
+    const float ca = m == -INFINITY ? 0.f : __expf(m - mn);
+    const float cb = mo == -INFINITY ? 0.f : __expf(mo - mn);
+    l = l * ca + lo * cb;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = acc[e] * ca + __shfl_xor(acc[e], o, 64) * cb;
+    m = mn;
+  }
+  if (lane == 0) { sm_m[wave] = m; sm_l[wave] = l; }
+  if (lane < LPP) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sm_acc[wave][d0 + e] = acc[e];
+  }
   __syncthreads();
   float* out = a.part + ((size_t)bh * a.nsplit + split) * (D + 2);
   for (int d = threadIdx.x; d < D; d += ATT_THREADS) {
     float M = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < NG; ++i) M = fmaxf(M, sm_m[i]);
+    for (int i = 0; i < ATT_WAVES; ++i) M = fmaxf(M, sm_m[i]);
     float L = 0.f, A = 0.f;
 #pragma unroll
-    for (int i = 0; i < NG; ++i) {
+    for (int i = 0; i < ATT_WAVES; ++i) {
       const float w = sm_m[i] == -INFINITY ? 0.f : __expf(sm_m[i] - M);
       L = __builtin_fmaf(sm_l[i], w, L);
       A = __builtin_fmaf(sm_acc[i][d], w, A);
@@ -200,7 +246,8 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
   const int bh = blockIdx.x, d = threadIdx.x;
   const int step = *a.step;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
-  const int nact = (valid + a.chunk - 1) / a.chunk;
+  const int chunk = attn_chunk(valid, a.nsplit);
+  const int nact = (valid + chunk - 1) / chunk;
   const float* p = a.part + (size_t)bh * a.nsplit * (D + 2);
   float M = -INFINITY;
   for (int s = 0; s < nact; ++s) M = fmaxf(M, p[(size_t)s * (D + 2)]);
@@ -212,6 +259,15 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
     A = __builtin_fmaf(ps[2 + d], w, A);
   }
   a.out[(size_t)bh * D + d] = (f16)(A / L);
+}
+
+// splits per (sequence, head): about 1024 workgroups in all, never more than one per 64 cache rows
+// (which is what the workspace is sized for)
+static int attn_splits(int B, int Hq, int max_len) {
+  const int cap = (max_len + 63) / 64;
+  int n = (1024 + B * Hq - 1) / (B * Hq);
+  n = n < 1 ? 1 : n;
+  return n > cap ? cap : n;
 }
 
 extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int max_len) {
@@ -232,7 +288,7 @@ extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, 
   AttnArgs a{};
   a.q = (const f16*)q; a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
   a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
-  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.chunk = 64; a.nsplit = (max_len + 63) / 64;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len);
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(a.nsplit, B * Hq);
