@@ -129,6 +129,57 @@ def recorded_traffic():
     return None
 
 
+def gemm_workload(args):
+    """Single-operator INT4 weight-only GEMV/GEMM: X[M, 4096] fp16 by W[4096, 11008] packed INT4 with
+    per-output-channel fp16 scales -> fp16 [M, 11008].  A step is one launch; 48 copies of the weight
+    (1 GiB in all) are used in turn so that no launch finds its weight in a cache."""
+    import torch
+    from poptransformer_amd import kernels as K
+    M, Kd, N, copies = args.batch, 4096, 11008, 48
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn(M, Kd, device="cuda", dtype=torch.float16, generator=gen)
+    ws = []
+    for _ in range(copies):
+        packed = torch.randint(0, 256, (N, Kd // 2), device="cuda", dtype=torch.uint8, generator=gen).view(torch.int8)
+        scale = (torch.rand(N, device="cuda", generator=gen) * 0.015 + 0.005).to(torch.float16)
+        ws.append(K.W4Weight(packed, scale))
+        del packed
+    out = torch.empty(M, N, device="cuda", dtype=torch.float16)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for w in ws:
+            K.w4a16_gemm(x, w, out=out)
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for w in ws:
+                K.w4a16_gemm(x, w, out=out)
+        rounds_w = max(1, args.warmup // copies)
+        rounds = max(1, args.steps // copies)
+        for _ in range(rounds_w):
+            g.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(rounds):
+            g.replay()
+        e1.record(stream)
+    torch.cuda.synchronize()
+    steps = rounds * copies
+    sec = e0.elapsed_time(e1) * 1e-3 / steps
+    nbytes = Kd * N // 2 + 2 * N + 2 * M * Kd + 2 * M * N
+    achieved = nbytes / sec / 1e9
+    print(json.dumps({
+        "metric": "INT4 weight-only GEMV/GEMM launches/s", "value": 1.0 / sec, "unit": "launches/s", "n_gpus": 1,
+        "steps": steps, "warmup": rounds_w * copies, "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
+        "config": {"workload": f"single-operator W4A16: X[{M},4096] fp16 by W[4096,11008] packed INT4, fp16 scales", "M": M},
+        "roofline": {"bound": "hbm", "kernel": "pta_w4a16_gemm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": sec * 1e6,
+                     "tflops": 2.0 * M * Kd * N / sec / 1e12},
+    }))
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,6 +188,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
                     help="default: persistent when the batch fits it (<= 4), else operators")
+    ap.add_argument("--workload", choices=["decode", "gemm"], default="decode",
+                    help="decode: the Llama2-7B-shape INT4 decode loop (the headline); gemm: the single INT4 "
+                         "weight-only operator at M = --batch rows")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -162,6 +216,9 @@ def main():
     if not torch.cuda.is_available():
         print("no GPU visible", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "gemm":
+        gemm_workload(args)
+        return
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
@@ -232,7 +289,9 @@ def main():
         launches = reps * len(weights.blocks)
         kernel_s = e0.elapsed_time(e1) * 1e-3 / launches
         kernel_bytes = 2 * (d * f // 2 + 2 * f) + B * d * 2 + B * f * 2
-        kernel_name = "gemv_lds_kernel<FmtW4, 8, true> (INT4 gate/up + SwiGLU)"
+        kernel_name = ("gemv_lds_kernel<FmtW4, 8, true>" if B <= 4 else
+                       "gemv_wide_kernel<FmtW4, 3, true>" if B <= 16 else "gemv_mfma_kernel<FmtW4, MT, 8, true>") + \
+            " (INT4 gate/up + SwiGLU)"
     achieved = kernel_bytes / kernel_s / 1e9
 
     out = {

@@ -105,7 +105,7 @@ extern "C" int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const p
 // grows), so the number of splits per (sequence, head) is chosen from the batch alone - enough
 // workgroups to fill the machine, no more - and each split's range of cache rows is derived on the
 // device from the current step: chunk = ceil(valid / nsplit), rounded up to a multiple of 16 rows
-// and at least 32.  Splits beyond the valid rows exit at once.
+// and at least 64.  Splits beyond the valid rows exit at once.
 // ------------------------------------------------------------------------------------------
 constexpr int ATT_THREADS = 256;
 constexpr int ATT_WAVES = ATT_THREADS / 64;
@@ -126,7 +126,7 @@ struct AttnArgs {
 __device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
   int c = (valid + nsplit - 1) / nsplit;
   c = (c + 15) & ~15;
-  return c < 32 ? 32 : c;
+  return c < 64 ? 64 : c;
 }
 
 // Partial attention of one (sequence, query head) over one chunk of cache rows.
