@@ -180,6 +180,69 @@ def gemm_workload(args):
 
 
 
+CHATGLM2_6B = dict(num_layers=28, hidden_size=4096, num_attention_heads=32, multi_query_group_num=2, ffn_hidden_size=13696,
+                   padded_vocab_size=65024, layernorm_epsilon=1e-5)
+RWKV4_7B = dict(num_hidden_layers=32, hidden_size=4096, attention_hidden_size=4096, intermediate_size=16384,
+                vocab_size=65536, layer_norm_epsilon=1e-5, rescale_every=6)
+
+
+def other_model_workload(args):
+    """ChatGLM2-6B-shape FP8 decode (F143 weights and activations, fp16 KV cache of length 4096) or
+    RWKV-4-7B-shape INT4 recurrent decode, one launch per operator replayed from a HIP graph.  The prompt is
+    consumed token by token in the untimed warm-up.  Reported like the headline, without a kernel leg."""
+    import torch
+    from poptransformer_amd.engine import fused, loader, rwkv, synthetic
+    B = args.batch
+    rng = np.random.Generator(np.random.PCG64(1234))
+    if args.workload == "chatglm2":
+        cfg, max_len = CHATGLM2_6B, 4096
+        weights = synthetic.chatglm2_synthetic_weights(cfg, "fp8", seed=0)
+        dec = fused.FusedDecoder(loader.chatglm2_spec(cfg, max_len, B, pad_id=0, eos_id=2), weights)
+        hd = cfg["hidden_size"] // cfg["num_attention_heads"]
+        per_pos = B * cfg["num_layers"] * 2 * cfg["multi_query_group_num"] * hd * 2
+        wbytes, vocab = weights.nbytes(), cfg["padded_vocab_size"]
+        name = "ChatGLM2-6B-shape FP8 (F143 weights and activations, F143 lm_head) greedy decode"
+        dtype = "fp8 (F143) weights and activations decoded to f16, f32 accumulation"
+
+        def step_bytes(t):
+            return wbytes + per_pos * (t + 1) + B * cfg["hidden_size"] * 2
+    else:
+        cfg, max_len = RWKV4_7B, args.warmup + args.steps + 2
+        weights = synthetic.rwkv_synthetic_weights(cfg, seed=0)
+        dec = rwkv.RWKVDecoder(loader.rwkv_spec(cfg, max_len, B, pad_id=0, eos_id=-1), weights)
+        wbytes, vocab = weights.nbytes(), cfg["vocab_size"]
+        state = B * 2 * cfg["num_hidden_layers"] * (2 * 2 + 3 * 4) * cfg["hidden_size"]
+        name = "RWKV-4-7B-shape INT4 recurrent decode"
+        dtype = "int4 weights, f16 activations, f32 accumulation and WKV state"
+
+        def step_bytes(t):
+            return wbytes + state + B * cfg["hidden_size"] * 2
+    if args.warmup + args.steps + 1 > max_len:
+        print(f"warmup + steps must stay below the sequence length {max_len}", file=sys.stderr)
+        sys.exit(2)
+    dec.capture()
+    ids = np.zeros((B, max_len), np.int32)
+    ids[:, :args.warmup] = rng.integers(3, vocab, size=(B, args.warmup))
+    dec.reset(ids)
+    dec.run_steps(args.warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.run_steps(args.steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_bytes = float(np.mean([step_bytes(t) for t in range(args.warmup, args.warmup + args.steps)]))
+    print(json.dumps({
+        "metric": "decode tokens/s + % of HBM roofline", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": f"{name}, batch {B}, prompt {args.warmup} consumed token by token, "
+                               f"{args.steps} new tokens", "batch": B, "executor": "operators"},
+        "step_algorithmic_bytes": mean_bytes,
+        "step_roofline_frac": mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9),
+    }))
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -188,9 +251,10 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
                     help="default: persistent when the batch fits it (<= 4), else operators")
-    ap.add_argument("--workload", choices=["decode", "gemm"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemm", "chatglm2", "rwkv"], default="decode",
                     help="decode: the Llama2-7B-shape INT4 decode loop (the headline); gemm: the single INT4 "
-                         "weight-only operator at M = --batch rows")
+                         "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
+                         "rwkv: RWKV-4-7B-shape INT4 recurrent decode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -205,7 +269,7 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
-    if args.warmup + args.steps + 1 > MAX_LEN:
+    if args.workload == "decode" and args.warmup + args.steps + 1 > MAX_LEN:
         print(f"warmup + steps must stay below the KV cache length {MAX_LEN}", file=sys.stderr)
         sys.exit(2)
 
@@ -218,6 +282,9 @@ def main():
         sys.exit(1)
     if args.workload == "gemm":
         gemm_workload(args)
+        return
+    if args.workload in ("chatglm2", "rwkv"):
+        other_model_workload(args)
         return
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)

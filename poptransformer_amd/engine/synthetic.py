@@ -53,3 +53,73 @@ def llama2_synthetic_weights(cfg, seed=0, device="cuda"):
     torch.cuda.synchronize()
     return ModelWeights(embed=embed, pos_embed=None, blocks=blocks, final_norm=(ones.clone(), None), head=head,
                         inv_freq=inv_freq)
+
+
+def _f8_scale_for(w):
+    """Power-of-two exponent e such that max|w| * 2^-e lies in (120, 240] (the largest F143 value is 240)."""
+    m = float(w.abs().amax())
+    return int(np.ceil(np.log2(m / 240.0))) if m > 0 else 0
+
+
+def _linear_f143(gen, out_f, in_f, device, act_fp8, bias=False):
+    from .loader import f143_encode_device
+    w = (torch.randn((out_f, in_f), generator=gen, device=device, dtype=torch.float32) * 0.02).half()
+    e = _f8_scale_for(w)
+    w8, sc = f143_encode_device(w, e)
+    b = torch.zeros(out_f, dtype=torch.float16, device=device) if bias else None
+    return LinearWeights(K.F8Weight(w8, sc, "F143"), b, act_fp8=act_fp8, scale_value=e)
+
+
+def chatglm2_synthetic_weights(cfg, precision="fp8", seed=0, device="cuda"):
+    """ChatGLM2-shaped weights, every Linear cast to F143 with a per-tensor power-of-two scale
+    (precision "fp8": activations are cast to F143 too; "fp8_weight": they stay fp16)."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    d, f, v = cfg["hidden_size"], cfg["ffn_hidden_size"], cfg["padded_vocab_size"]
+    hd = d // cfg["num_attention_heads"]
+    kv = 2 * cfg["multi_query_group_num"] * hd
+    ones = torch.ones(d, dtype=torch.float16, device=device)
+    act8 = precision == "fp8"
+    blocks = []
+    for _ in range(cfg["num_layers"]):
+        blocks.append(BlockWeights(
+            norm1=(ones.clone(), None), norm2=(ones.clone(), None),
+            qkv=[_linear_f143(gen, d, d, device, act8, bias=True), _linear_f143(gen, kv, d, device, act8, bias=True)],
+            out=_linear_f143(gen, d, d, device, act8),
+            mlp_in=[_linear_f143(gen, f, d, device, act8) for _ in range(2)],
+            mlp_out=_linear_f143(gen, d, f, device, act8)))
+    embed = (torch.randn((v, d), generator=gen, device=device, dtype=torch.float32) * 0.02).half()
+    rot = hd // 2
+    inv_freq = torch.from_numpy(np.array([1.0 / (10000 ** (i / rot)) for i in range(0, rot, 2)]).astype(np.float32)).to(device)
+    head = _linear_f143(gen, v, d, device, act8)
+    torch.cuda.synchronize()
+    return ModelWeights(embed=embed, pos_embed=None, blocks=blocks, final_norm=(ones.clone(), None), head=head,
+                        inv_freq=inv_freq)
+
+
+def rwkv_synthetic_weights(cfg, seed=0, device="cuda"):
+    """RWKV-4-shaped weights: INT4 Linear weights, time_decay U(-8, -1), time_first U(-1, 1), time_mix U(0, 1)."""
+    from .rwkv import RWKVBlockWeights, RWKVWeights
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    d, a, f, v = cfg["hidden_size"], cfg["attention_hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+
+    def ln(n):
+        return (torch.ones(n, dtype=torch.float16, device=device), torch.zeros(n, dtype=torch.float16, device=device))
+
+    def uni(n, lo, hi):
+        return (torch.rand(n, generator=gen, device=device) * (hi - lo) + lo).half()
+
+    blocks = []
+    for i in range(cfg["num_hidden_layers"]):
+        blocks.append(RWKVBlockWeights(
+            pre_ln=ln(d) if i == 0 else None, ln1=ln(d), ln2=ln(d),
+            att_key=_linear_int4(gen, a, d, device), att_value=_linear_int4(gen, a, d, device),
+            att_receptance=_linear_int4(gen, a, d, device), att_output=_linear_int4(gen, d, a, device),
+            time_decay=uni(a, -8.0, -1.0), time_first=uni(a, -1.0, 1.0), att_mix=[uni(d, 0.0, 1.0) for _ in range(3)],
+            ffn_key=_linear_int4(gen, f, d, device), ffn_receptance=_linear_int4(gen, d, d, device),
+            ffn_value=_linear_int4(gen, d, f, device), ffn_mix=[uni(d, 0.0, 1.0) for _ in range(2)]))
+    embed = (torch.randn((v, d), generator=gen, device=device, dtype=torch.float32) * 0.02).half()
+    head = LinearWeights(K.F16Weight((torch.randn((v, d), generator=gen, device=device, dtype=torch.float32) * 0.02).half()))
+    torch.cuda.synchronize()
+    return RWKVWeights(embed=embed, blocks=blocks, ln_out=ln(d), head=head)
