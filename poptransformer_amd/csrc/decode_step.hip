@@ -352,25 +352,27 @@ __device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* cons
 // that owns it at that point of the layer and read by that unit's products, always under the same
 // compile-time index, so no value ever has to move between registers: a move of a requested tile
 // would have to wait for its load, and with it for the whole burst of requests around it.
-template <int NRB, int TPW, int BASE, int SCBASE, int NSLOT, int NSC>
+// Requests tiles [FIRST, FIRST + COUNT) of unit u (tile r * TPW + i is tile i of matrix r), and the
+// scales of the matrices whose first tile is among them.
+template <int NRB, int TPW, int BASE, int SCBASE, int FIRST = 0, int COUNT = NRB * TPW, int NSLOT, int NSC>
 __device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], const Mat (&m)[NRB], int u, int n_units,
                                            int N, int KT) {
   static_assert(BASE + NRB * TPW <= NSLOT && SCBASE + NRB <= NSC, "unit outside the register array");
+  static_assert(FIRST >= 0 && COUNT >= 0 && FIRST + COUNT <= NRB * TPW, "tiles outside the unit");
   const int wave = wave_id(), lane = lane_id();
   u = u < n_units ? u : n_units - 1;
 #pragma unroll
-  for (int r = 0; r < NRB; ++r) {
-    const DS_GLOBAL u32x4* p = as_global(m[r].tiled) + (size_t)u * KT * 64 + lane;
-#pragma unroll
-    for (int i = 0; i < TPW; ++i) {
-      int kt = wave + i * DS_WAVES;
-      kt = kt < KT ? kt : KT - 1;
-      S[BASE + r * TPW + i] = __builtin_nontemporal_load(p + (size_t)kt * 64);
+  for (int t = FIRST; t < FIRST + COUNT; ++t) {
+    const int r = t / TPW, i = t % TPW;
+    int kt = wave + i * DS_WAVES;
+    kt = kt < KT ? kt : KT - 1;
+    S[BASE + t] = __builtin_nontemporal_load(as_global(m[r].tiled) + ((size_t)u * KT + kt) * 64 + lane);
+    if (i == 0) {
+      int row = u * 16 + (lane & 15);
+      row = row < N ? row : N - 1;
+      const f16 sv = as_global(m[r].scale)[row];
+      SC[SCBASE + r] = f16x2{sv, sv};
     }
-    int row = u * 16 + (lane & 15);
-    row = row < N ? row : N - 1;
-    const f16 sv = as_global(m[r].scale)[row];
-    SC[SCBASE + r] = f16x2{sv, sv};
   }
 }
 
@@ -395,8 +397,8 @@ __device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (
         const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
 #pragma unroll
         for (int r = 0; r < NRB; ++r)
-          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant8(S[BASE + r * TPW + i][j], SC[SCBASE + r]), xb, acc[r],
-                                                          0, 0, 0);
+          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant_step(S[BASE + r * TPW + i], j, SC[SCBASE + r]), xb,
+                                                          acc[r], 0, 0, 0);
       }
     }
   }
@@ -777,23 +779,28 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   }
   wg_sync();
 
-  // Places of the units in the tile array.  q/k/v, o_proj and the first two gate/up units are
-  // held together; the third gate/up unit is requested when q/k/v have been multiplied and takes
-  // their place; down is requested when the first two gate/up units have been multiplied and
-  // takes theirs; the next layer's q/k/v return to the start.
-  constexpr int NSLOT = 8 * TPW_D;
-  constexpr int S_QKV = 0, S_O = 3 * TPW_D, S_GU0 = 4 * TPW_D, S_GU2 = 0, S_D = 4 * TPW_D;
-  constexpr int NSC = 8;
-  constexpr int C_QKV = 0, C_O = 3, C_GU0 = 4, C_GU2 = 0, C_D = 4;
+  // Places of the units in the tile array (T = TPW_D tiles per wave and matrix): q | k | v at
+  // [0, 3T), o_proj at [3T, 4T), the first and second gate/up units at [4T, 6T) and [6T, 8T); the
+  // third gate/up unit takes [0, 2T) once q/k/v have been multiplied, down takes [3T, 3T + TPW_F)
+  // (o_proj's place and the start of the first gate/up unit's) as those are multiplied, and the
+  // next layer's v, q, k return to their places as these become free.  No request point asks for
+  // more than 2T tiles per wave (64 KiB per workgroup at the 7B shape): that is what a compute unit
+  // accepts without holding the requesting waves.
+  constexpr int T = TPW_D;
+  constexpr int NSLOT = 8 * T;
+  constexpr int S_QKV = 0, S_O = 3 * T, S_GU0 = 4 * T, S_GU1 = 6 * T, S_GU2 = 0, S_D = 3 * T;
+  constexpr int NSC = 9;
+  constexpr int C_QKV = 0, C_O = 3, C_GU0 = 4, C_GU1 = 6, C_GU2 = 0, C_D = 8;
+  constexpr int D_EARLY = TPW_F < T ? TPW_F : T;        // down tiles that fit o_proj's place
   static_assert(U_F <= 3, "at most three gate/up units per workgroup");
-  static_assert(TPW_F <= 4 * TPW_D, "the down tiles take the place of two gate/up units");
+  static_assert(TPW_F <= 3 * T, "the down tiles end where the first gate/up unit ends");
   u32x4 S[NSLOT];
   f16x2 SC[NSC];
   {
     const LayerPtrs L0 = layer_ptrs(lds_layers, 0);
     normw_fetch(L0.get<const f16>(P_N1), normw, a.d);
     const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
-    load_slots<3, TPW_D, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
+    load_slots<3, T, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
   }
   grid_barrier(a.sync, epoch, G, wg, w);
   bool alive = *lds_dead == 0;
@@ -809,80 +816,80 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
 
   for (int li = 0; li < a.n_layer && alive; ++li) {
     const LayerPtrs L = layer_ptrs(lds_layers, li);
+    const bool more = li + 1 < a.n_layer;
+    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
     const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
+    const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
+    const Mat m3n[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
     f16* const x_in = a.xres + (size_t)(2 * li) * xslot;        // residual stream entering the layer
     f16* const x_mid = x_in + xslot;                             // after attention
     f16* const x_out = x_mid + xslot;                            // after the MLP
     // ---- RMSNorm + q/k/v; a row of the [B, 3d] slot holds q | k | v.
-    //      Requests o_proj and the first gate/up unit.
+    //      Requests o_proj and the gate half of the first gate/up unit before the product, the up half after it.
     TRACE(0);
     alive = stage<NS_D, MAXB>(x_in, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
     if (!alive) break;
     {
       const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
-      load_slots<1, TPW_D, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
-      load_slots<2, TPW_D, S_GU0, C_GU0>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+      load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
+      load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
     {
       f16* q = a.qkv + (size_t)li * M * 3 * a.d;
       f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
-      gemv_slots<3, TPW_D, EPI_STORE, MAXB, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs,
-                                                          xstride, red, red_buf);
+      gemv_slots<3, T, EPI_STORE, MAXB, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs, xstride,
+                                                      red, red_buf);
     }
+    load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     TRACE(2);
-    // ---- rotary + KV append + attention
+    // ---- rotary + KV append + attention.  Requests the second gate/up unit when it is done.
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
       for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
-      // the second gate/up unit: requested here and not with the first, so that no phase requests much
-      // more than the others (see the note on requests at the top of the file)
-      if constexpr (U_F > 1) load_slots<2, TPW_D, S_GU0 + 2 * TPW_D, C_GU0 + 2>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
+      if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
-    // ---- o_proj + residual.  Requests the third gate/up unit and the RMSNorm weights of the MLP.
+    // ---- o_proj + residual.  Requests the third gate/up unit before the product; after it the first
+    //      down tiles (o_proj's place), the next layer's v and the RMSNorm weights of the MLP.
     alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
-    if constexpr (U_F > 2) load_slots<2, TPW_D, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
+    if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     TRACE(4);
     {
       f16* const o1[1] = {x_mid};
-      res = gemv_slots<1, TPW_D, EPI_RESIDUAL, MAXB, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride,
-                                                               red, red_buf);
+      res = gemv_slots<1, T, EPI_RESIDUAL, MAXB, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride, red,
+                                                           red_buf);
     }
+    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
-    // ---- RMSNorm + gate/up + SwiGLU.  Requests down once the first unit has been multiplied.
+    // ---- RMSNorm + gate/up + SwiGLU.  Requests the remaining down tiles once the first unit has been
+    //      multiplied (they take its place), and the next layer's q after the last unit.
     alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
     if (!alive) break;
     TRACE(6);
     {
       f16* act = a.act + (size_t)li * M * a.ffn;
       f16* const o2[2] = {act, act};
-      gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xs,
-                                                           xstride, red, red_buf);
+      gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xs, xstride,
+                                                       red, red_buf);
+      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
       if constexpr (U_F > 1)
-        gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU0 + 2 * TPW_D, C_GU0 + 2>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f,
-                                                                             a.ffn, KT_D, M, xs, xstride, red, red_buf);
-      {      // the places of the units multiplied so far are free now
-        const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
-        load_slots<1, TPW_F, S_D, C_D>(S, SC, md, wg, nb_d, a.d, KT_F);
-      }
+        gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU1, C_GU1>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xs,
+                                                         xstride, red, red_buf);
       if constexpr (U_F > 2)
-        gemv_slots<2, TPW_D, EPI_SWIGLU, MAXB, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D,
-                                                             M, xs, xstride, red, red_buf);
+        gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xs,
+                                                         xstride, red, red_buf);
     }
+    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
-    // ---- down + residual.  Requests the q/k/v of the next layer and the next RMSNorm weights.
+    // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
     alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
-    const bool more = li + 1 < a.n_layer;
-    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
-    {
-      const Mat m3[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
-      load_slots<3, TPW_D, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
-    }
+    load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
       f16* const o1[1] = {x_out};

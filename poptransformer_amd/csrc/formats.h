@@ -7,9 +7,11 @@
 // Fused W4A16 GEMV/GEMM.
 // ------------------------------------------------------------------------------------------
 
-// One tiled dword -> 8 fp16 weights, each fp16(q * s) with a single rounding (the product of
-// an integer in [-8, 7] held exactly in fp16 and the fp16 scale), which is what the
-// reference's `half(nibble) * scale` computes.
+// The four dwords of a lane -> the 8 fp16 weights of MFMA step m (features m*32 + (l/16)*8 + 0..7
+// of channel l%16), each fp16(q * s) with a single rounding (the product of an integer in [-8, 7]
+// held exactly in fp16 and the fp16 scale), which is what the reference's `half(nibble) * scale`
+// computes.  Dword d holds features 2d (low half) and 2d + 1 (high half) of every step, step m in
+// nibble m of each half, stored offset-binary (q + 8).
 // (a & mask) | orv in one VALU instruction.  The mask travels in an SGPR and the OR value in a
 // VGPR: a VOP3 encoding on this target takes no literal and at most one scalar operand.
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
@@ -18,23 +20,26 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t o
   return r;
 }
 
-__device__ __forceinline__ f16x8 dequant8(uint32_t w, f16x2 s2) {
+__device__ __forceinline__ f16x8 dequant_step(u32x4 w, int m, f16x2 s2) {
   const uint32_t MAGIC = 0x64006400u;  // fp16 1024.0 in both halves
   const f16x2 c1032 = {(f16)1032.0f, (f16)1032.0f};
   const f16x2 c16th = {(f16)0.0625f, (f16)0.0625f};
   const f16x2 c72 = {(f16)-72.0f, (f16)-72.0f};
-  const uint32_t w8 = w >> 8;
-  f16x2 p0 = bitcast<f16x2>(and_or(w, 0x000f000fu, MAGIC));   // 1024 + u      (features 0,1)
-  f16x2 p1 = bitcast<f16x2>(and_or(w, 0x00f000f0u, MAGIC));   // 1024 + 16 u   (features 2,3)
-  f16x2 p2 = bitcast<f16x2>(and_or(w8, 0x000f000fu, MAGIC));  // features 4,5
-  f16x2 p3 = bitcast<f16x2>(and_or(w8, 0x00f000f0u, MAGIC));  // features 6,7
-  p0 = (p0 - c1032) * s2;                                  // exact integer, then one rounding
-  p2 = (p2 - c1032) * s2;
-  p1 = __builtin_elementwise_fma(p1, c16th, c72) * s2;     // (1024 + 16u)/16 - 72 = u - 8, exact
-  p3 = __builtin_elementwise_fma(p3, c16th, c72) * s2;
   f16x8 r;
-  r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
-  r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const uint32_t wd = m >= 2 ? w[d] >> 8 : w[d];
+    f16x2 p;
+    if (m & 1) {
+      p = bitcast<f16x2>(and_or(wd, 0x00f000f0u, MAGIC));       // 1024 + 16 u
+      p = __builtin_elementwise_fma(p, c16th, c72) * s2;        // (1024 + 16u)/16 - 72 = u - 8, exact; one rounding
+    } else {
+      p = bitcast<f16x2>(and_or(wd, 0x000f000fu, MAGIC));       // 1024 + u
+      p = (p - c1032) * s2;                                     // exact integer, then one rounding
+    }
+    r[2 * d] = p[0];
+    r[2 * d + 1] = p[1];
+  }
   return r;
 }
 
@@ -47,7 +52,7 @@ struct FmtW4 {
     return f16x2{s, s};
   }
   static __device__ __forceinline__ f16x8 a_operand(const u32x4 (&raw)[1], int j, Scale s) {
-    return dequant8(raw[0][j], s);
+    return dequant_step(raw[0], j, s);
   }
   static __device__ __forceinline__ float finish(float acc, Scale) { return acc; }
 };

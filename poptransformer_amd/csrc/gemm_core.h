@@ -374,20 +374,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Variant for 4 < M <= 16 when all matrices of the launch share X: one workgroup of 16 waves per
+// Variant for 4 < M <= 64 when all matrices of the launch share X: one workgroup of 16 waves per
 // compute unit's worth of work.  A workgroup owns NB 16-channel blocks (blocks g, g + G, ... of
 // the launch's G workgroups); wave w takes the feature tiles w, w + 16, ... of ALL of them, so the
-// activation fragment of a tile (the B operand, 4 KiB at M = 16 against 1 KiB of INT4 weights) is
-// read once and used NB times, and every wave has NB weight tiles per feature tile in flight.
+// activation fragments of a tile (the B operands: 4 KiB per 16 rows, against 1 KiB of INT4
+// weights) are read once and used NB times, and every wave has NB weight tiles per feature tile
+// in flight.  MT = number of 16-row groups of X.
 // ------------------------------------------------------------------------------------------
 constexpr int WIDE_WAVES = 16;
 
-template <class Fmt, int NB, bool PAIR>
+template <class Fmt, int MT, int NB, bool PAIR>
 __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, int total_nb) {
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int KV = Fmt::kVec;
   extern __shared__ __align__(16) unsigned char smem[];
-  float* red = reinterpret_cast<float*>(smem);          // [WIDE_WAVES][NB][NACC][256]
+  float* red = reinterpret_cast<float*>(smem);          // [WIDE_WAVES][NB][NACC][MT][256]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int G = gridDim.x;
   const int K = a.K, KT = a.KT;
@@ -415,105 +416,164 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
       wp[b][g] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb[b] * KT * (64 * KV) + lane;
     }
   }
-  int mrow = lane & 15;
-  mrow = mrow < a.M ? mrow : a.M - 1;                   // padding rows compute values that are never stored
-  const f16* xrow = a.X + (size_t)mrow * K + (lane >> 4) * 8;
-
-  f32x4 acc[NB][NACC];
+  const f16* xrow[MT];
 #pragma unroll
-  for (int b = 0; b < NB; ++b)
-#pragma unroll
-    for (int g = 0; g < NACC; ++g) acc[b][g] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // UN feature tiles per step, all of their loads requested before the first product (a tile
-  // beyond KT repeats the last one with zero activations)
-  constexpr int UN = NB * NACC * KV <= 4 ? 2 : 1;
-  for (int kt0 = wave; kt0 < KT; kt0 += WIDE_WAVES * UN) {
-    u32x4 w[UN][NB][NACC][KV];
-    f16x8 xb[UN][4];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-      const int kt_ = kt0 + u * WIDE_WAVES;
-      const bool there = kt_ < KT;
-      const int kt = there ? kt_ : KT - 1;
-#pragma unroll
-      for (int b = 0; b < NB; ++b)
-#pragma unroll
-        for (int g = 0; g < NACC; ++g)
-#pragma unroll
-          for (int v = 0; v < KV; ++v)
-            w[u][b][g][v] = __builtin_nontemporal_load(wp[b][g] + ((size_t)kt * KV + v) * 64);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int k = kt * 128 + j * 32;
-        const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        xb[u][j] = there && k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xrow + k) : z;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UN; ++u)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int b = 0; b < NB; ++b)
-#pragma unroll
-          for (int g = 0; g < NACC; ++g)
-            acc[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(w[u][b][g], j, sc[b][g]), xb[u][j],
-                                                               acc[b][g], 0, 0, 0);
+  for (int mt = 0; mt < MT; ++mt) {
+    int mrow = mt * 16 + (lane & 15);
+    mrow = mrow < a.M ? mrow : a.M - 1;                 // padding rows compute values that are never stored
+    xrow[mt] = a.X + (size_t)mrow * K + (lane >> 4) * 8;
   }
 
-  // The accumulator of lane l holds channels (l/16)*4 + r, r = 0..3, for activation row l%16.
+  f32x4 acc[NB][NACC][MT];
 #pragma unroll
   for (int b = 0; b < NB; ++b)
 #pragma unroll
     for (int g = 0; g < NACC; ++g)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[((((wave * NB + b) * NACC + g) * 4 + r) * 64) + lane] = acc[b][g][r];
+      for (int mt = 0; mt < MT; ++mt) acc[b][g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if constexpr (MT == 1) {
+    // UN feature tiles per step, all of their loads requested before the first product (a tile
+    // beyond KT repeats the last one with zero activations)
+    constexpr int UN = NB * NACC * KV <= 4 ? 2 : 1;
+    for (int kt0 = wave; kt0 < KT; kt0 += WIDE_WAVES * UN) {
+      u32x4 w[UN][NB][NACC][KV];
+      f16x8 xb[UN][4];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int kt_ = kt0 + u * WIDE_WAVES;
+        const bool there = kt_ < KT;
+        const int kt = there ? kt_ : KT - 1;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+          for (int g = 0; g < NACC; ++g)
+#pragma unroll
+            for (int v = 0; v < KV; ++v)
+              w[u][b][g][v] = __builtin_nontemporal_load(wp[b][g] + ((size_t)kt * KV + v) * 64);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = kt * 128 + j * 32;
+          const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+          xb[u][j] = there && k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xrow[0] + k) : z;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g = 0; g < NACC; ++g)
+              acc[b][g][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(w[u][b][g], j, sc[b][g]), xb[u][j],
+                                                                    acc[b][g][0], 0, 0, 0);
+    }
+  } else {
+    // several row groups: the activation fragments of one 32-feature slice at a time (16 bytes per
+    // lane and row group), each used for all blocks before the next slice is read
+    for (int kt = wave; kt < KT; kt += WIDE_WAVES) {
+      u32x4 w[NB][NACC][KV];
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int g = 0; g < NACC; ++g)
+#pragma unroll
+          for (int v = 0; v < KV; ++v) w[b][g][v] = __builtin_nontemporal_load(wp[b][g] + ((size_t)kt * KV + v) * 64);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = kt * 128 + j * 32;
+        const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        f16x8 xb[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          xb[mt] = k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xrow[mt] + k) : z;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+          for (int g = 0; g < NACC; ++g) {
+            const f16x8 av = Fmt::a_operand(w[b][g], j, sc[b][g]);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              acc[b][g][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[mt], acc[b][g][mt], 0, 0, 0);
+          }
+      }
+    }
+  }
+
+  // The accumulator of lane l holds channels (l/16)*4 + r, r = 0..3, for activation row l%16 of its group.
+#pragma unroll
+  for (int b = 0; b < NB; ++b)
+#pragma unroll
+    for (int g = 0; g < NACC; ++g)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          red[((((wave * NB + b) * NACC + g) * MT + mt) * 4 + r) * 64 + lane] = acc[b][g][mt][r];
   __syncthreads();
-  // thread t finishes output (row (t / 16) % 16, channel t % 16) of block t / 256
-  static_assert(NB * 256 <= WIDE_WAVES * 64, "one output per thread");
+  // The 256 outputs (16 rows x 16 channels) of (block b, row group mt) are finished by the quarter
+  // (b * MT + mt) % 4 of the workgroup, thread t of it taking row (t / 16) % 16, channel t % 16.
+  const int quarter = threadIdx.x >> 8;
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
-    if ((int)(threadIdx.x >> 8) != b) continue;
-    const int nn = threadIdx.x & 15, m = (threadIdx.x >> 4) & 15;
-    const GemmMat& mt = a.mat[PAIR ? 0 : mi[b]];
-    const int N = mt.N, n = nb[b] * 16 + nn;
-    if ((int)blockIdx.x + b * G >= total_nb || m >= a.M || n >= N) continue;
-    const int r = nn & 3, ln = (nn >> 2) * 16 + m;
-    float sum[NACC];
 #pragma unroll
-    for (int g = 0; g < NACC; ++g) {
-      float t = 0.f;
+    for (int mt = 0; mt < MT; ++mt) {
+      if (((b * MT + mt) & 3) != quarter) continue;
+      const int nn = threadIdx.x & 15, m = mt * 16 + ((threadIdx.x >> 4) & 15);
+      const GemmMat& mat = a.mat[PAIR ? 0 : mi[b]];
+      const int N = mat.N, n = nb[b] * 16 + nn;
+      if ((int)blockIdx.x + b * G >= total_nb || m >= a.M || n >= N) continue;
+      const int r = nn & 3, ln = (nn >> 2) * 16 + (m & 15);
+      float sum[NACC];
 #pragma unroll
-      for (int w = 0; w < WIDE_WAVES; ++w) t += red[((((w * NB + b) * NACC + g) * 4 + r) * 64) + ln];
-      sum[g] = Fmt::finish(t, sc[b][g]);      // no format's finish uses the per-channel part of the scale
-    }
-    if (PAIR) {
-      const f16 gate = (f16)sum[0];
-      const f16 up = (f16)sum[1];
-      mt.Y[(size_t)m * N + n] = up * swish_f16(gate);
-    } else {
-      f16 y0 = (f16)sum[0];
-      if (mt.bias) y0 = y0 + mt.bias[n];
-      y0 = apply_act(mt.act, y0);
-      mt.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
+      for (int g = 0; g < NACC; ++g) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < WIDE_WAVES; ++w) t += red[((((w * NB + b) * NACC + g) * MT + mt) * 4 + r) * 64 + ln];
+        sum[g] = Fmt::finish(t, sc[b][g]);      // no format's finish uses the per-channel part of the scale
+      }
+      if (PAIR) {
+        const f16 gate = (f16)sum[0];
+        const f16 up = (f16)sum[1];
+        mat.Y[(size_t)m * N + n] = up * swish_f16(gate);
+      } else {
+        f16 y0 = (f16)sum[0];
+        if (mat.bias) y0 = y0 + mat.bias[n];
+        y0 = apply_act(mat.act, y0);
+        mat.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
+      }
     }
   }
 }
 
-template <class Fmt, int NB, bool PAIR>
+template <class Fmt, int MT, int NB, bool PAIR>
 static int launch_gemv_wide(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   static bool ready = false;
-  const size_t smem = (size_t)WIDE_WAVES * NB * (PAIR ? 2 : 1) * 256 * sizeof(float);
+  const size_t smem = (size_t)WIDE_WAVES * NB * (PAIR ? 2 : 1) * MT * 256 * sizeof(float);
+  static_assert(WIDE_WAVES * NB * (PAIR ? 2 : 1) * MT * 1024 <= 128 * 1024, "reduction buffer beyond 128 KiB of LDS");
   if (!ready) {
-    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemv_wide_kernel<Fmt, NB, PAIR>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem) == hipSuccess,
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemv_wide_kernel<Fmt, MT, NB, PAIR>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess,
                 "%s: cannot reserve %zu bytes of LDS", name, smem);
     ready = true;
   }
-  hipLaunchKernelGGL((gemv_wide_kernel<Fmt, NB, PAIR>), dim3((total_nb + NB - 1) / NB), dim3(WIDE_WAVES * 64), smem, s, a,
-                     total_nb);
+  hipLaunchKernelGGL((gemv_wide_kernel<Fmt, MT, NB, PAIR>), dim3((total_nb + NB - 1) / NB), dim3(WIDE_WAVES * 64), smem, s,
+                     a, total_nb);
   return PTA_OK;
+}
+
+// blocks per workgroup: the launch's share per compute unit, capped by what the registers of a wave
+// (weight tiles in flight) and the LDS reduction buffer (8 KiB-groups of partial sums) hold
+template <class Fmt, int MT, bool PAIR>
+static int launch_gemv_wide_for(const GemmArgs& a, int total_nb, int per_cu, hipStream_t s, const char* name) {
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int cap_regs = Fmt::kVec * NACC <= 4 ? 3 : 2;
+  constexpr int cap_lds = 8 / (NACC * MT) >= 1 ? 8 / (NACC * MT) : 1;
+  constexpr int cap = cap_regs < cap_lds ? cap_regs : cap_lds;
+  if (per_cu <= 1 || cap == 1) return launch_gemv_wide<Fmt, MT, 1, PAIR>(a, total_nb, s, name);
+  if (per_cu == 2 || cap == 2) return launch_gemv_wide<Fmt, MT, cap >= 2 ? 2 : 1, PAIR>(a, total_nb, s, name);
+  return launch_gemv_wide<Fmt, MT, cap >= 3 ? 3 : 1, PAIR>(a, total_nb, s, name);
 }
 
 static inline int device_compute_units() {
@@ -562,24 +622,20 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
   if (a.M <= 4 && xbytes <= 40 * 1024) {
     if (a.KT >= 16 && total_nb <= 1024 && !PAIR) launch_gemv_lds<Fmt, 16, PAIR>(a, total_nb, s);
     else launch_gemv_lds<Fmt, 8, PAIR>(a, total_nb, s);
-  } else if (a.M <= 16) {
+  } else {
     bool shared_x = true;
     for (int i = 0; i < a.count; ++i) shared_x = shared_x && a.mat[i].X == nullptr;
     const int per_cu = (total_nb + device_compute_units() - 1) / device_compute_units();
     if (shared_x && a.KT >= 8) {
       int rc;
-      // three blocks per workgroup only where their tiles fit the registers of a wave
-      constexpr bool three = Fmt::kVec * (PAIR ? 2 : 1) <= 4;
-      if (per_cu <= 1) rc = launch_gemv_wide<Fmt, 1, PAIR>(a, total_nb, s, name);
-      else if (per_cu == 2 || !three) rc = launch_gemv_wide<Fmt, 2, PAIR>(a, total_nb, s, name);
-      else rc = launch_gemv_wide<Fmt, three ? 3 : 2, PAIR>(a, total_nb, s, name);
+      if (a.M <= 16) rc = launch_gemv_wide_for<Fmt, 1, PAIR>(a, total_nb, per_cu, s, name);
+      else if (a.M <= 32) rc = launch_gemv_wide_for<Fmt, 2, PAIR>(a, total_nb, per_cu, s, name);
+      else rc = launch_gemv_wide_for<Fmt, 4, PAIR>(a, total_nb, per_cu, s, name);
       if (rc) return rc;
-    } else {
-      launch_gemv<Fmt, 1, PAIR>(a, total_nb, s);
-    }
+    } else if (a.M <= 16) launch_gemv<Fmt, 1, PAIR>(a, total_nb, s);
+    else if (a.M <= 32) launch_gemv<Fmt, 2, PAIR>(a, total_nb, s);
+    else launch_gemv<Fmt, 4, PAIR>(a, total_nb, s);
   }
-  else if (a.M <= 32) launch_gemv<Fmt, 2, PAIR>(a, total_nb, s);
-  else launch_gemv<Fmt, 4, PAIR>(a, total_nb, s);
   PTA_CHECK_LAUNCH(name);
   return PTA_OK;
 }

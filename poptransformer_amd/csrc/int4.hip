@@ -78,38 +78,40 @@ extern "C" int pta_int4_to_half(const int8_t* packed, const pta_half* scale, pta
 // Load-time tiling.
 //
 // A tile covers 16 output channels x 128 input features and is 1 KiB, stored so that lane l
-// of a wave finds its 16 bytes at byte offset 16*l: dword j (0..3) of that lane holds the 8
-// weights of channel (l % 16) for features  kt*128 + j*32 + (l/16)*8 + 0..7, i.e. exactly the
-// A operand of one 16x16x32 MFMA.  Tiles of one 16-channel block are contiguous over kt, so a
-// block streams one contiguous range.  Inside a dword weight i sits in nibble slot
-// (i & 1) * 4 + (i >> 1) and is stored offset-binary (q + 8): with that order two AND/OR
-// operations per shifted dword yield fp16 pairs of consecutive features.
-// Padding rows / features hold the code of zero.
+// of a wave finds its 16 bytes at byte offset 16*l.  The A operand of MFMA step m (0..3) of a
+// tile is, for lane l, the 8 weights of channel (l % 16) for features
+// kt*128 + m*32 + (l/16)*8 + 0..7.  Dword d (0..3) of the lane holds features 2d (in its low
+// half) and 2d + 1 (in its high half) of all four steps, step m in nibble m of each half,
+// stored offset-binary (q + 8): one AND|OR per dword and step yields an fp16 pair of
+// consecutive features, and all weights of one step sit at the same bit position of their
+// half.  Tiles of one 16-channel block are contiguous over kt, so a block streams one
+// contiguous range.  Padding rows / features hold the code of zero.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void w4_tile_kernel(const int8_t* __restrict__ P,
                                                       uint32_t* __restrict__ tiled, int N, int K,
                                                       int KT, size_t total_dwords) {
   const size_t d = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (d >= total_dwords) return;
-  const int j = (int)(d & 3);
+  const int dw = (int)(d & 3);
   const int lane = (int)((d >> 2) & 63);
   const size_t tile = d >> 8;
   const int kt = (int)(tile % KT);
   const int nb = (int)(tile / KT);
   const int row = nb * 16 + (lane & 15);
-  const int k0 = kt * 128 + j * 32 + (lane >> 4) * 8;
   uint32_t w = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int k = k0 + i;
-    uint32_t u = 8;  // q = 0
-    if (row < N && k < K) {
-      const int8_t b = P[(size_t)row * (K / 2) + (k >> 1)];
-      const int q = (k & 1) ? nib_lo(b) : nib_hi(b);
-      u = (uint32_t)(q + 8);
+  for (int m = 0; m < 4; ++m) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int k = kt * 128 + m * 32 + (lane >> 4) * 8 + 2 * dw + h;
+      uint32_t u = 8;  // q = 0
+      if (row < N && k < K) {
+        const int8_t b = P[(size_t)row * (K / 2) + (k >> 1)];
+        const int q = (k & 1) ? nib_lo(b) : nib_hi(b);
+        u = (uint32_t)(q + 8);
+      }
+      w |= u << (16 * h + 4 * m);
     }
-    const int slot = (i & 1) * 4 + (i >> 1);
-    w |= u << (4 * slot);
   }
   tiled[d] = w;
 }
