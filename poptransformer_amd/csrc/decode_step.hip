@@ -49,7 +49,8 @@ constexpr int DS_MAX_SPLIT = 16;
 constexpr int DS_PART = DS_D + 2;                           // floats of one attention partial
 constexpr int DS_RED = DS_WAVES * 3 * 16 * DS_MAXB;         // floats in one reduction buffer
 constexpr int DS_ATT_FLOATS = 3 * DS_D / 2 + 2 * DS_WAVES + DS_WAVES * DS_D;
-constexpr int DS_TAIL_FLOATS = DS_WAVES * DS_MAXB + 64 + 4; // norm sums | selection scratch | flags
+constexpr int DS_XSUM = DS_WAVES * DS_MAXB + 64 + 4;        // offset of the per-wave sums of the staged activations
+constexpr int DS_TAIL_FLOATS = DS_XSUM + DS_WAVES * DS_MAXB; // norm sums | selection scratch | flags | activation sums
 constexpr int DS_LAYER_WORDS = sizeof(pta_decode_layer) / 4;
 constexpr uint16_t DS_EMPTY16 = 0xFFFFu;                    // filler of fp16 slots
 constexpr uint32_t DS_EMPTY32 = 0xFFFFFFFFu;                // filler of fp32 slots
@@ -183,6 +184,32 @@ __device__ __forceinline__ float wait_value(const float* p, bool on, Waiter& w) 
   return bitcast<float>(bits);
 }
 
+// the same for two fp16 values per lane whose loads travel together (one round trip, not two)
+__device__ __forceinline__ void wait_pair(const f16* p0, bool on0, const f16* p1, bool on1, f16& v0, f16& v1, Waiter& w) {
+  uint16_t b0 = 0, b1 = 0;
+  for (;;) {
+    if (on0) b0 = get_bits(p0);
+    if (on1) b1 = get_bits(p1);
+    if (!__any((on0 && b0 == DS_EMPTY16) || (on1 && b1 == DS_EMPTY16)) || w.give_up()) break;
+  }
+  v0 = bitcast<f16>(b0);
+  v1 = bitcast<f16>(b1);
+}
+// and for three fp32 values per lane
+__device__ __forceinline__ void wait_triple(const float* p0, const float* p1, const float* p2, bool on2, float& v0, float& v1,
+                                            float& v2, Waiter& w) {
+  uint32_t b0 = 0, b1 = 0, b2 = 0;
+  for (;;) {
+    b0 = get_bits(p0);
+    b1 = get_bits(p1);
+    if (on2) b2 = get_bits(p2);
+    if (!__any(b0 == DS_EMPTY32 || b1 == DS_EMPTY32 || (on2 && b2 == DS_EMPTY32)) || w.give_up()) break;
+  }
+  v0 = bitcast<float>(b0);
+  v1 = bitcast<float>(b1);
+  v2 = bitcast<float>(b2);
+}
+
 // The one grid barrier of a launch (after the slots have been filled).  sync[0] holds the epoch
 // base, sync[1] the error word, sync[16 + g] the arrival word of workgroup g.
 __device__ __forceinline__ void grid_barrier(unsigned* sync, unsigned epoch, int G, int wg, Waiter& w) {
@@ -269,9 +296,14 @@ enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_SWIGLU = 2 };
 // The partial sums of the useful accumulator columns (activation rows m < M) of all waves meet in
 // LDS; `res` is the residual element of this thread (EPI_RESIDUAL), and the value the thread
 // stored is returned (it is the residual of the same thread in the next residual phase).
-template <int NRB, int EPI>
+struct NoScales {};
+// SCALED: the sums are over stored codes q + 8; 8 * sum(x) (xsum: per-wave partial sums of the staged
+// activations) comes off and the channel's scale (SC[scbase + r] of the finishing lane, whose
+// channel is lane % 16) is applied before the rounding to fp16.
+template <int NRB, int EPI, bool SCALED = false, class Scales = NoScales>
 __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (&out)[NRB], int ostride, f16 res, int u,
-                                           int N, int M, float* red, int& red_buf) {
+                                           int N, int M, float* red, int& red_buf, const float* xsum = nullptr,
+                                           const Scales& SC = Scales{}, int scbase = 0) {
   const int wave = wave_id(), lane = lane_id();
   float* rb = red + red_buf * DS_RED;
   if ((lane & 15) < M) {
@@ -293,6 +325,14 @@ __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (
       const int m_ = q - r * M;
       const int n = u * 16 + ch;
       if (n < N) {
+        float off = 0.f, scale[NRB];
+        if constexpr (SCALED) {
+#pragma unroll 8
+          for (int w = 0; w < DS_WAVES; ++w) off += xsum[w * DS_MAXB + m_];
+          off *= 8.0f;
+#pragma unroll
+          for (int i = 0; i < NRB; ++i) scale[i] = (float)SC[scbase + i][0];
+        }
         if (EPI == EPI_SWIGLU) {
           float sg = 0.f, su = 0.f;
 #pragma unroll 4
@@ -300,11 +340,18 @@ __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (
             sg += rb[((w * NRB + 0) * 16 + ch) * DS_MAXB + m_];
             su += rb[((w * NRB + (NRB > 1 ? 1 : 0)) * 16 + ch) * DS_MAXB + m_];
           }
+          if constexpr (SCALED) { sg = (sg - off) * scale[0]; su = (su - off) * scale[NRB > 1 ? 1 : 0]; }
           put(out[0] + (size_t)m_ * ostride + n, (f16)su * swish_f16((f16)sg));
         } else {
           float s = 0.f;
 #pragma unroll 8
           for (int w = 0; w < DS_WAVES; ++w) s += rb[((w * NRB + r) * 16 + ch) * DS_MAXB + m_];
+          if constexpr (SCALED) {
+            float sc = scale[0];
+#pragma unroll
+            for (int i = 1; i < NRB; ++i) sc = r == i ? scale[i] : sc;
+            s = (s - off) * sc;
+          }
           y = (f16)s;
           if (EPI == EPI_RESIDUAL) y = y + res;
           put(out[r] + (size_t)m_ * ostride + n, y);
@@ -376,33 +423,49 @@ __device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], 
   }
 }
 
+// out[r][m, n] = fp16(s_r[n] * sum_k xs[m, k] * q_r[n, k]) for unit u: the scale is applied once, to
+// the fp32 sum, where the per-operator kernels multiply by fp16(q * s) (the reference materialises
+// that matrix, ops/customized.py:115-125 into ops/popart.py:55-67); the two differ by the rounding of
+// the 4096..11008 products q * s to fp16, far below the rounding of the fp16 result.  It makes the
+// weights cost 5 VALU instructions per 8 instead of 13, and this phase is bound by exactly those.
+// A stored code c = q + 8 masked in place is the fp16 subnormal c * 2^-24 (nibble 0 or 2 of a
+// half, after a shift by 8 for the latter) or c * 2^-20 (nibble 1 or 3); the matrix unit takes
+// subnormal operands at their exact value.  Steps of equal weight share an accumulator;
+// sum_k x * (c - 8) = 2^24 acc_even + 2^20 acc_odd - 8 sum_k x, with sum_k x from `stage`.
 template <int NRB, int TPW, int EPI, int MAXB, int BASE, int SCBASE, int NSLOT, int NSC>
 __device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB],
                                           int ostride, f16 res, int u, int n_units, int N, int KT, int M, const f16* xs,
-                                          int xstride, float* red, int& red_buf) {
+                                          int xstride, float* red, int& red_buf, const float* xsum) {
   if (u >= n_units) return res;
   const int wave = wave_id(), lane = lane_id();
   int mrow = lane & 15;
   mrow = mrow < M ? mrow : M - 1;
   const f16* xl = xs + (size_t)mrow * xstride + (lane >> 4) * 8;
-  f32x4 acc[NRB];
+  f32x4 acc[NRB][2];
 #pragma unroll
-  for (int r = 0; r < NRB; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < NRB; ++r) acc[r][0] = acc[r][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int i = 0; i < TPW; ++i) {
     const int kt = wave + i * DS_WAVES;
     if (kt < KT) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + j * 32);
+      for (int m = 0; m < 4; ++m) {
+        const f16x8 xb = *reinterpret_cast<const f16x8*>(xl + kt * 128 + m * 32);
 #pragma unroll
-        for (int r = 0; r < NRB; ++r)
-          acc[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(dequant_step(S[BASE + r * TPW + i], j, SC[SCBASE + r]), xb,
-                                                          acc[r], 0, 0, 0);
+        for (int r = 0; r < NRB; ++r) {
+          const u32x4 w = S[BASE + r * TPW + i];
+          u32x4 c;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) c[d] = (m >= 2 ? w[d] >> 8 : w[d]) & ((m & 1) ? 0x00f000f0u : 0x000f000fu);
+          acc[r][m & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<f16x8>(c), xb, acc[r][m & 1], 0, 0, 0);
+        }
       }
     }
   }
-  return finish_unit<NRB, EPI>(acc, out, ostride, res, u, N, M, red, red_buf);
+  f32x4 sum[NRB];
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) sum[r] = acc[r][0] * 16777216.0f + acc[r][1] * 1048576.0f;
+  return finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
 }
 
 // i / per for i < 4 * per, without a division
@@ -470,6 +533,9 @@ __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* x
     wg_sync();
   }
   const float inv_n = 1.0f / (float)K;
+  float ps[MAXB];      // sums of the values this thread puts into LDS, per activation row
+#pragma unroll
+  for (int mm = 0; mm < MAXB; ++mm) ps[mm] = 0.f;
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
     const int i = thread_id() + k * DS_THREADS;
@@ -486,7 +552,19 @@ __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* x
         for (int e = 0; e < 8; ++e) h[e] = (h[e] * r16) * gm[e];
       }
       *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = h;
+      float s1 = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s1 += (float)h[e];
+#pragma unroll
+      for (int mm = 0; mm < MAXB; ++mm) if (mm == m) ps[mm] += s1;
     }
+  }
+  // The INT4 products below multiply by the stored codes q + 8 and take 8 * sum(x) off at the end.
+#pragma unroll
+  for (int mm = 0; mm < MAXB; ++mm) ps[mm] = wave_sum(ps[mm]);
+  if (lane == 0) {
+#pragma unroll
+    for (int mm = 0; mm < MAXB; ++mm) scratch[DS_XSUM + wave * DS_MAXB + mm] = ps[mm];
   }
   wg_sync();
   return *w.lds_dead == 0;
@@ -553,8 +631,8 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
     const int which = tid / D, d_ = tid % D;
     const bool on = tid < 3 * D;
     const f16* row = qrow + (size_t)(which < 3 ? which : 0) * a.d;
-    const f16 x0 = wait_value(row + d_, on, w);
-    const f16 x1 = wait_value(row + (d_ < HALF ? d_ + HALF : d_ - HALF), on && which < 2, w);
+    f16 x0, x1;
+    wait_pair(row + d_, on, row + (d_ < HALF ? d_ + HALF : d_ - HALF), on && which < 2, x0, x1, w);
     if (on) {
       f16 y = x0;
       if (which < 2) {
@@ -615,28 +693,43 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
     }
   }
   wg_sync();
-  if (thread_id() < D) {      // waves 0 and 1
+  float Mx = -INFINITY, Ls = 0.f, As = 0.f;
+  float* part = a.part + (((size_t)li * a.B * a.H + bh) * a.nsplit) * DS_PART;
+  if (thread_id() < D) {      // waves 0 and 1: this workgroup's own partial
     const int d_ = thread_id();
-    float Mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < DS_WAVES; ++i) Mx = fmaxf(Mx, sm_m[i]);
-    float Ls = 0.f, As = 0.f;
 #pragma unroll
     for (int i = 0; i < DS_WAVES; ++i) {
       const float wgt = sm_m[i] == -INFINITY ? 0.f : __expf(sm_m[i] - Mx);
       Ls = __builtin_fmaf(sm_l[i], wgt, Ls);
       As = __builtin_fmaf(sm_acc[i * D + d_], wgt, As);
     }
-    float* part = a.part + (((size_t)li * a.B * a.H + bh) * a.nsplit) * DS_PART;
     if (split != 0) {
       float* mine = part + (size_t)split * DS_PART;
       put(mine + 2 + d_, As);
       if (d_ == 0) { put(mine, Mx); put(mine + 1, Ls); }
-    } else {
-      // the other splits' (max, denominator, numerator[d_]) in ascending order of split
+    }
+  }
+  if (split == 0) {
+    // The partials of the other splits that have rows: wave s fetches split s (all at the same time:
+    // one round trip for all of them), they meet in LDS and merge in ascending order of split.
+    static_assert(DS_MAX_SPLIT <= DS_WAVES && D == 128, "one wave per split, two numerator elements per lane");
+    wg_sync();                // the per-wave state in LDS has been read
+    if (wave >= 1 && wave < nact) {
+      const float* ps = part + (size_t)wave * DS_PART;
+      float a0, a1, ml;
+      wait_triple(ps + 2 + lane, ps + 2 + 64 + lane, ps + (lane & 1), lane < 2, a0, a1, ml, w);
+      sm_acc[wave * D + lane] = a0;
+      sm_acc[wave * D + 64 + lane] = a1;
+      if (lane == 0) sm_m[wave] = ml;
+      if (lane == 1) sm_l[wave] = ml;
+    }
+    wg_sync();
+    if (thread_id() < D) {
+      const int d_ = thread_id();
       for (int s = 1; s < nact; ++s) {
-        const float* ps = part + (size_t)s * DS_PART;
-        const float ms = wait_value(ps, true, w), ls = wait_value(ps + 1, true, w), as = wait_value(ps + 2 + d_, true, w);
+        const float ms = sm_m[s], ls = sm_l[s], as = sm_acc[s * D + d_];
         const float mn = fmaxf(Mx, ms);
         const float ca = __expf(Mx - mn), cb = __expf(ms - mn);
         Ls = Ls * ca + ls * cb;
@@ -839,7 +932,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       f16* q = a.qkv + (size_t)li * M * 3 * a.d;
       f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
       gemv_slots<3, T, EPI_STORE, MAXB, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs, xstride,
-                                                      red, red_buf);
+                                                      red, red_buf, scratch + DS_XSUM);
     }
     load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     TRACE(2);
@@ -860,7 +953,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     {
       f16* const o1[1] = {x_mid};
       res = gemv_slots<1, T, EPI_RESIDUAL, MAXB, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride, red,
-                                                           red_buf);
+                                                           red_buf, scratch + DS_XSUM);
     }
     load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
     load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
@@ -875,14 +968,14 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       f16* act = a.act + (size_t)li * M * a.ffn;
       f16* const o2[2] = {act, act};
       gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xs, xstride,
-                                                       red, red_buf);
+                                                       red, red_buf, scratch + DS_XSUM);
       load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
       if constexpr (U_F > 1)
         gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU1, C_GU1>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xs,
-                                                         xstride, red, red_buf);
+                                                         xstride, red, red_buf, scratch + DS_XSUM);
       if constexpr (U_F > 2)
         gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xs,
-                                                         xstride, red, red_buf);
+                                                         xstride, red, red_buf, scratch + DS_XSUM);
     }
     load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
@@ -894,7 +987,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     {
       f16* const o1[1] = {x_out};
       res = gemv_slots<1, TPW_F, EPI_RESIDUAL, MAXB, S_D, C_D>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_F, M, xs, xstride,
-                                                               red, red_buf);
+                                                               red, red_buf, scratch + DS_XSUM);
     }
     normw_fetch(more ? Ln.get<const f16>(P_N1) : a.final_norm, normw, a.d);
     TRACE(9);
