@@ -361,7 +361,11 @@ size_t pta_decode_step_workspace_bytes(const pta_decode_model* model);
  * (hidden, ffn) of the 7B model or a small test shape; PTA_EUNSUPPORTED otherwise.
  * Needs every compute unit of the device for itself while it runs: workgroups wait for each
  * other's results, every wait is bounded, and if one gives up it sets word 1 of the workspace
- * (sticky), the loop state is left untouched and the kernel ends; pta_decode_step_failed reports it. */
+ * (sticky), the loop state is left untouched and the kernel ends; pta_decode_step_failed reports it.
+ * Numerics: every rounding point is that of the per-operator entry points, except that an INT4
+ * projection is fp16(scale * sum(x * q)) - the scale applied once to the fp32 sum - where
+ * pta_w4a16_gemm computes fp16(sum(x * fp16(q * scale))); the results agree to the last fp16 bit or
+ * differ in it. */
 int pta_llama_decode_step(const pta_decode_model* model, const pta_decode_state* state, void* workspace,
                           pta_stream_t stream);
 

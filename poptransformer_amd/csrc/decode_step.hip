@@ -10,9 +10,10 @@
 // wave holds the weight tiles of the next phase(s) in registers: they are requested a phase or
 // more before they are used, so HBM streams while the phases wait for each other's results.
 //
-// Numerics are those of the per-operator entry points (formats.h, norm.hip, attention.hip,
-// select.hip), which the parity tests compare against the CPU restatement; this file only changes
-// when things happen (and the order in which attention partials are merged).
+// Numerics are those of the per-operator entry points (norm.hip, attention.hip, select.hip), which
+// the parity tests compare against the CPU restatement, with two differences: the order in which
+// attention partials are merged, and the INT4 products, which apply the scale once to the fp32 sum
+// instead of multiplying by fp16(q * s) (see gemv_slots).  The lm_head (fp16) is as in formats.h.
 //
 // How phases hand over results.  Every intermediate vector of the iteration (the residual stream
 // after each half layer, q|k|v, the attention output, the SwiGLU output, attention partials, the
