@@ -48,7 +48,7 @@ constexpr int DS_MAXB = 4;
 constexpr int DS_D = 128;                                   // head size
 constexpr int DS_MAX_SPLIT = 16;
 constexpr int DS_PART = DS_D + 2;                           // floats of one attention partial
-constexpr int DS_RED = DS_WAVES * 3 * 16 * DS_MAXB;         // floats in one reduction buffer
+constexpr int DS_RED = DS_WAVES * 6 * 16 * DS_MAXB;         // floats in one reduction buffer (up to six matrices)
 constexpr int DS_ATT_FLOATS = 3 * DS_D / 2 + 2 * DS_WAVES + DS_WAVES * DS_D;
 constexpr int DS_XSUM = DS_WAVES * DS_MAXB + 64 + 4;        // offset of the per-wave sums of the staged activations
 constexpr int DS_TAIL_FLOATS = DS_XSUM + DS_WAVES * DS_MAXB; // norm sums | selection scratch | flags | activation sums
@@ -433,11 +433,12 @@ __device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], 
 // half, after a shift by 8 for the latter) or c * 2^-20 (nibble 1 or 3); the matrix unit takes
 // subnormal operands at their exact value.  Steps of equal weight share an accumulator;
 // sum_k x * (c - 8) = 2^24 acc_even + 2^20 acc_odd - 8 sum_k x, with sum_k x from `stage`.
-template <int NRB, int TPW, int EPI, int MAXB, int BASE, int SCBASE, int NSLOT, int NSC>
-__device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB],
-                                          int ostride, f16 res, int u, int n_units, int N, int KT, int M, const f16* xs,
-                                          int xstride, float* red, int& red_buf, const float* xsum) {
-  if (u >= n_units) return res;
+template <int NRB, int TPW, int BASE, int NSLOT>
+__device__ __forceinline__ void slots_product(const u32x4 (&S)[NSLOT], f32x4 (&sum)[NRB], int u, int n_units, int KT, int M,
+                                              const f16* xs, int xstride) {
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) sum[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (u >= n_units) return;
   const int wave = wave_id(), lane = lane_id();
   int mrow = lane & 15;
   mrow = mrow < M ? mrow : M - 1;
@@ -463,10 +464,68 @@ __device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (
       }
     }
   }
-  f32x4 sum[NRB];
 #pragma unroll
   for (int r = 0; r < NRB; ++r) sum[r] = acc[r][0] * 16777216.0f + acc[r][1] * 1048576.0f;
+}
+
+template <int NRB, int TPW, int EPI, int MAXB, int BASE, int SCBASE, int NSLOT, int NSC>
+__device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB],
+                                          int ostride, f16 res, int u, int n_units, int N, int KT, int M, const f16* xs,
+                                          int xstride, float* red, int& red_buf, const float* xsum) {
+  if (u >= n_units) return res;
+  f32x4 sum[NRB];
+  slots_product<NRB, TPW, BASE>(S, sum, u, n_units, KT, M, xs, xstride);
   return finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+}
+
+// The gate/up units of a workgroup (units wg, wg + G, ...) finish together: one meeting of the partial
+// sums in LDS and one round of stores for all of them.  A wave puts the gate / up sums of unit k into
+// LDS as soon as it has them (stash_gate_up); sg[k] / su[k] are the scales of this lane's channel.
+template <int U_F>
+__device__ __forceinline__ void stash_gate_up(const f32x4 (&sum)[2], int k, int M, float* red, int red_buf) {
+  const int wave = wave_id(), lane = lane_id();
+  float* rb = red + red_buf * DS_RED;
+  if ((lane & 15) < M) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        rb[((wave * (2 * U_F) + 2 * k + r) * 16 + (lane >> 4) * 4 + q) * DS_MAXB + (lane & 15)] = sum[r][q];
+  }
+}
+
+template <int U_F, int MAXB>
+__device__ __forceinline__ void finish_gate_up(const float (&sg)[U_F], const float (&su)[U_F], f16* act, int ffn, int wg, int G,
+                                               int nb_f, int M, float* red, int& red_buf, const float* xsum) {
+  float* rb = red + red_buf * DS_RED;
+  wg_sync();
+  // thread (k * M + m_) * 16 + ch finishes channel ch of row m_ of unit k
+  const int tid = thread_id();
+  const int per = 16 * M;
+  if (tid < U_F * per) {
+    const int k = (tid >= per ? 1 : 0) + (tid >= 2 * per ? 1 : 0);
+    const int m_ = (tid - k * per) >> 4, ch = tid & 15;
+    const int u = wg + k * G, n = u * 16 + ch;
+    if (u < nb_f && n < ffn) {
+      float off = 0.f;
+#pragma unroll 8
+      for (int w = 0; w < DS_WAVES; ++w) off += xsum[w * DS_MAXB + m_];
+      off *= 8.0f;
+      float g = 0.f, v = 0.f;
+#pragma unroll 4
+      for (int w = 0; w < DS_WAVES; ++w) {
+        g += rb[((w * (2 * U_F) + 2 * k) * 16 + ch) * DS_MAXB + m_];
+        v += rb[((w * (2 * U_F) + 2 * k + 1) * 16 + ch) * DS_MAXB + m_];
+      }
+      float cg = sg[0], cu = su[0];
+#pragma unroll
+      for (int i = 1; i < U_F; ++i) { cg = k == i ? sg[i] : cg; cu = k == i ? su[i] : cu; }
+      g = (g - off) * cg;
+      v = (v - off) * cu;
+      put(act + (size_t)m_ * ffn + n, (f16)v * swish_f16((f16)g));
+    }
+  }
+  red_buf ^= 1;
 }
 
 // i / per for i < 4 * per, without a division
@@ -967,16 +1026,23 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     TRACE(6);
     {
       f16* act = a.act + (size_t)li * M * a.ffn;
-      f16* const o2[2] = {act, act};
-      gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xs, xstride,
-                                                       red, red_buf, scratch + DS_XSUM);
+      f32x4 gsum[2];
+      slots_product<2, T, S_GU0>(S, gsum, wg, nb_f, KT_D, M, xs, xstride);
+      stash_gate_up<U_F>(gsum, 0, M, red, red_buf);
       load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-      if constexpr (U_F > 1)
-        gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU1, C_GU1>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xs,
-                                                         xstride, red, red_buf, scratch + DS_XSUM);
-      if constexpr (U_F > 2)
-        gemv_slots<2, T, EPI_SWIGLU, MAXB, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xs,
-                                                         xstride, red, red_buf, scratch + DS_XSUM);
+      if constexpr (U_F > 1) {
+        slots_product<2, T, S_GU1>(S, gsum, wg + G, nb_f, KT_D, M, xs, xstride);
+        stash_gate_up<U_F>(gsum, 1, M, red, red_buf);
+      }
+      if constexpr (U_F > 2) {
+        slots_product<2, T, S_GU2>(S, gsum, wg + 2 * G, nb_f, KT_D, M, xs, xstride);
+        stash_gate_up<U_F>(gsum, 2, M, red, red_buf);
+      }
+      float sg[U_F], su[U_F];
+      sg[0] = (float)SC[C_GU0][0]; su[0] = (float)SC[C_GU0 + 1][0];
+      if constexpr (U_F > 1) { sg[1] = (float)SC[C_GU1][0]; su[1] = (float)SC[C_GU1 + 1][0]; }
+      if constexpr (U_F > 2) { sg[2] = (float)SC[C_GU2][0]; su[2] = (float)SC[C_GU2 + 1][0]; }
+      finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
     load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
