@@ -576,6 +576,196 @@ static int launch_gemv_wide_for(const GemmArgs& a, int total_nb, int per_cu, hip
   return launch_gemv_wide<Fmt, MT, cap >= 3 ? 3 : 1, PAIR>(a, total_nb, s, name);
 }
 
+// ------------------------------------------------------------------------------------------
+// Variant for 16 < M <= 64: the activation rows of a feature tile are staged in LDS once per
+// workgroup and shared by its waves, so that the B operands (4 KiB per 16 rows and tile, against
+// 1 KiB of INT4 weights) come from LDS and not from the L2.
+// A workgroup of 8 waves owns 2 * (8 / KQ) weight streams of 16 channels (consecutive channel blocks
+// of one matrix; or, for a SwiGLU pair, the gate and the up weights of 8 / KQ channel blocks) and
+// all rows; its waves form KQ groups that take the feature tiles g, g + KQ, ... each; a wave
+// multiplies two streams, so every B fragment it reads from LDS feeds two MFMAs.  The X tiles of
+// step i + 1 are fetched (global -> registers -> LDS, double-buffered) while step i is multiplied,
+// and so are the weight tiles.  The partial sums of the KQ groups meet in LDS (the staging area).
+// ------------------------------------------------------------------------------------------
+constexpr int TILE_WAVES = 8;
+constexpr int TILE_XSTRIDE = 128 + 8;      // halves per staged row: 16 consecutive rows hit 16 different bank groups
+
+template <class Fmt, int MT, int KQ, bool PAIR>
+__global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) {
+  constexpr int KV = Fmt::kVec;
+  constexpr int WPG = TILE_WAVES / KQ;          // waves per K group
+  constexpr int ROWS = MT * 16;
+  constexpr int XBUF = ROWS * TILE_XSTRIDE;     // halves of one staged tile
+  constexpr int VPT = ROWS * 16 / (WPG * 64);   // 16-byte vectors of a tile per thread of its group
+  static_assert(VPT >= 1 && ROWS * 16 % (WPG * 64) == 0, "staging must divide evenly");
+  extern __shared__ __align__(16) unsigned char smem[];
+  f16* xs = reinterpret_cast<f16*>(smem);       // [KQ][2][ROWS][TILE_XSTRIDE]
+  float* red = reinterpret_cast<float*>(smem);  // after the product: [TILE_WAVES][2][MT][256]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int kq = wave / WPG, wg_ = wave % WPG;  // K group, wave within the group
+  const int tig = wg_ * 64 + lane;              // thread index within the group
+  const int K = a.K, KT = a.KT, M = a.M;
+
+  // the two weight streams of this wave
+  int mi = 0;
+  const int first_blk = PAIR ? (int)blockIdx.x * WPG : (int)blockIdx.x * 2 * WPG;
+  if (!PAIR) {
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (i < a.count && first_blk >= a.mat[i].nb_begin) mi = i;
+  }
+  int nb[2];
+  typename Fmt::Scale sc[2];
+  const u32x4* wp[2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {
+    const GemmMat& m = a.mat[PAIR ? st : mi];
+    nb[st] = PAIR ? first_blk + wg_ : first_blk - m.nb_begin + 2 * wg_ + st;
+    sc[st] = Fmt::load_scale(m.scale, a.x_scale, nb[st] * 16 + (lane & 15), m.N);
+    wp[st] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb[st] * KT * (64 * KV) + lane;
+  }
+  const f16* X = a.mat[mi].X ? a.mat[mi].X : a.X;
+
+  f32x4 acc[2][MT];
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[st][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // thread tig of a group stages vectors tig, tig + WPG*64, ... of the tile: vector v = row * 16 + c
+  auto fetch_x = [&](int kt, u32x4 (&xv)[VPT]) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int v = tig + i * WPG * 64;
+      const int row = v >> 4, c = v & 15;
+      const int k = kt * 128 + c * 8;
+      xv[i] = (row < M && k < K && kt < KT) ? *reinterpret_cast<const u32x4*>(X + (size_t)row * K + k) : u32x4{0, 0, 0, 0};
+    }
+  };
+  auto store_x = [&](f16* buf, const u32x4 (&xv)[VPT]) {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const int v = tig + i * WPG * 64;
+      *reinterpret_cast<u32x4*>(buf + (v >> 4) * TILE_XSTRIDE + (v & 15) * 8) = xv[i];
+    }
+  };
+  auto fetch_w = [&](int kt, u32x4 (&w)[2][KV]) {
+    const int ktc = kt < KT ? kt : KT - 1;
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int v = 0; v < KV; ++v) w[st][v] = __builtin_nontemporal_load(wp[st] + ((size_t)ktc * KV + v) * 64);
+  };
+
+  f16* xbuf = xs + (size_t)kq * 2 * XBUF;
+  const int steps = (KT + KQ - 1) / KQ;
+  u32x4 w_cur[2][KV], w_nxt[2][KV], xv[VPT];
+  fetch_w(kq, w_cur);
+  fetch_x(kq, xv);
+  store_x(xbuf, xv);
+  __syncthreads();
+  for (int i = 0; i < steps; ++i) {
+    const int kt = kq + i * KQ, ktn = kt + KQ;
+    const bool more = i + 1 < steps;
+    if (more) { fetch_w(ktn, w_nxt); fetch_x(ktn, xv); }
+    const f16* cur = xbuf + (i & 1) * XBUF + (lane & 15) * TILE_XSTRIDE + (lane >> 4) * 8;
+    if (kt < KT) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        f16x8 xb[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xb[mt] = *reinterpret_cast<const f16x8*>(cur + mt * 16 * TILE_XSTRIDE + m * 32);
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const f16x8 av = Fmt::a_operand(w_cur[st], m, sc[st]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[st][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[mt], acc[st][mt], 0, 0, 0);
+        }
+      }
+    }
+    if (more) {
+      store_x(xbuf + ((i + 1) & 1) * XBUF, xv);
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int v = 0; v < KV; ++v) w_cur[st][v] = w_nxt[st][v];
+    }
+    __syncthreads();
+  }
+
+  // partial sums of the K groups meet in LDS (the staging area is free after the last barrier)
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(((wave * 2 + st) * MT + mt) * 4 + r) * 64 + lane] = acc[st][mt][r];
+  __syncthreads();
+  // outputs of the workgroup: WPG wave slots x 2 streams x MT row groups x 256; PAIR: one output per stream pair
+  constexpr int OUTS = WPG * (PAIR ? 1 : 2) * MT * 256;
+  for (int o = threadIdx.x; o < OUTS; o += TILE_WAVES * 64) {
+    const int nn = o & 15, m16 = (o >> 4) & 15;
+    int rest = o >> 8;
+    const int mt = rest % MT; rest /= MT;
+    const int st = PAIR ? 0 : rest & 1;
+    const int wslot = PAIR ? rest : rest >> 1;
+    const int m = mt * 16 + m16;
+    const GemmMat& mat = a.mat[PAIR ? 0 : mi];
+    const int N = mat.N;
+    const int blk = PAIR ? first_blk + wslot : first_blk - mat.nb_begin + 2 * wslot + st;
+    const int n = blk * 16 + nn;
+    if (m >= M || n >= N) continue;
+    const int r = nn & 3, ln = (nn >> 2) * 16 + m16;
+    float sum[2] = {0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < (PAIR ? 2 : 1); ++g) {
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < KQ; ++q) t += red[((((q * WPG + wslot) * 2 + (PAIR ? g : st)) * MT + mt) * 4 + r) * 64 + ln];
+      sum[g] = Fmt::finish(t, sc[0]);      // no format's finish uses the per-channel part of the scale
+    }
+    if (PAIR) {
+      const f16 gate = (f16)sum[0];
+      const f16 up = (f16)sum[1];
+      mat.Y[(size_t)m * N + n] = up * swish_f16(gate);
+    } else {
+      f16 y0 = (f16)sum[0];
+      if (mat.bias) y0 = y0 + mat.bias[n];
+      y0 = apply_act(mat.act, y0);
+      mat.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
+    }
+  }
+}
+
+template <class Fmt, int MT, int KQ, bool PAIR>
+static int launch_gemm_tile(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  static bool ready = false;
+  constexpr int WPG = TILE_WAVES / KQ;
+  const size_t stage = (size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2;
+  const size_t redb = (size_t)TILE_WAVES * 2 * MT * 256 * 4;
+  const size_t smem = stage > redb ? stage : redb;
+  static_assert((size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2 <= 160 * 1024, "staging beyond the LDS of a compute unit");
+  if (!ready) {
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_tile_kernel<Fmt, MT, KQ, PAIR>,
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess,
+                "%s: cannot reserve %zu bytes of LDS", name, smem);
+    ready = true;
+  }
+  const int per_wg = PAIR ? WPG : 2 * WPG;
+  hipLaunchKernelGGL((gemm_tile_kernel<Fmt, MT, KQ, PAIR>), dim3(total_nb / per_wg), dim3(TILE_WAVES * 64), smem, s, a);
+  return PTA_OK;
+}
+
+// whether the launch fits gemm_tile_kernel with `per_wg` channel blocks per workgroup: every matrix
+// a whole number of workgroups, enough feature tiles for the K groups
+static inline bool tile_fits(const GemmArgs& a, int per_wg, int kq, bool pair) {
+  if (a.KT < 2 * kq) return false;
+  if (pair) return ((a.mat[0].N + 15) / 16) % per_wg == 0;
+  for (int i = 0; i < a.count; ++i)
+    if (((a.mat[i].N + 15) / 16) % per_wg != 0) return false;
+  return true;
+}
+
 static inline int device_compute_units() {
   static int cus = 0;
   if (cus == 0) {
@@ -626,6 +816,20 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
     bool shared_x = true;
     for (int i = 0; i < a.count; ++i) shared_x = shared_x && a.mat[i].X == nullptr;
     const int per_cu = (total_nb + device_compute_units() - 1) / device_compute_units();
+    if (a.M > 16 && a.epi.norm == PTA_NORM_NONE) {
+      // the staged kernel where its workgroups fill the machine: 2 streams x 4 K groups (4 channel blocks,
+      // or 2 SwiGLU pairs, per workgroup); for M <= 32 also 8 K groups (half as many blocks per workgroup)
+      const int cus = device_compute_units();
+      const int wgs4 = total_nb / (PAIR ? 2 : 4), wgs8 = total_nb / (PAIR ? 1 : 2);
+      int rc = 1;
+      if (tile_fits(a, PAIR ? 2 : 4, 4, PAIR) && 2 * wgs4 >= cus) {
+        rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(a, total_nb, s, name);
+      } else if (a.M <= 32 && tile_fits(a, PAIR ? 1 : 2, 8, PAIR) && 2 * wgs8 >= cus) {
+        rc = launch_gemm_tile<Fmt, 2, 8, PAIR>(a, total_nb, s, name);
+      }
+      if (rc < 0) return rc;
+      if (rc == 0) { PTA_CHECK_LAUNCH(name); return PTA_OK; }
+    }
     if (shared_x && a.KT >= 8) {
       int rc;
       if (a.M <= 16) rc = launch_gemv_wide_for<Fmt, 1, PAIR>(a, total_nb, per_cu, s, name);

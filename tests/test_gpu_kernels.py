@@ -100,6 +100,54 @@ def test_w4a16_gemm_exact_integers(K):
     assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 64])
+@pytest.mark.parametrize("Kdim,N", [(1024, 8192), (1160, 4096), (4096, 8192)])
+def test_w4a16_gemm_many_rows_wide_outputs(K, M, Kdim, N):
+    """More than 16 rows and enough output channels to fill the machine: the kernel that stages the
+    activation rows in LDS (4096 channels only up to 32 rows; 1160 features = a ragged last tile)."""
+    x, packed, scale = _w4_case(M * 3 + Kdim + N, M, Kdim, N)
+    w = K.W4Weight(dev(packed), dev(scale))
+    got = host(K.w4a16_gemm(dev(x), w))
+    ref = O.w4a16_matmul(x, packed, scale)
+    assert rel_err(got, ref) <= 1e-2
+    ref64 = x.astype(np.float64) @ O.int4_to_half(packed, scale, 1).astype(np.float64)
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
+
+
+def test_w4a16_gemm_many_rows_exact_integers(K):
+    rng = np.random.default_rng(6)
+    M, Kdim, N = 40, 1024, 8192
+    x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
+    q = rng.integers(-8, 8, size=(N, Kdim))
+    w = K.W4Weight(dev(O.pack_int4(q)), dev(np.ones(N, np.float16)))
+    got = host(K.w4a16_gemm(dev(x), w)).astype(np.int64)
+    assert np.array_equal(got, x.astype(np.int64) @ q.T.astype(np.int64))
+
+
+def test_w4a16_gemm_many_rows_multi_swiglu_epilogue(K):
+    rng = np.random.default_rng(8)
+    M, Kdim = 33, 1024
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    mats = []
+    for N in (4096, 2048, 2048):
+        mats.append((rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8),
+                     rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)))
+    ws = [K.W4Weight(dev(p), dev(s)) for p, s in mats]
+    for (p, s), o in zip(mats, K.w4a16_gemm_multi(dev(x), ws)):
+        assert rel_err(host(o), O.w4a16_matmul(x, p, s)) <= 1e-2
+    N = 8192
+    (pg, sg), (pu, su) = [(rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8),
+                           rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)) for _ in range(2)]
+    got = host(K.w4a16_gemm_swiglu(dev(x), K.W4Weight(dev(pg), dev(sg)), K.W4Weight(dev(pu), dev(su))))
+    ref = (O.w4a16_matmul(x, pu, su) * O.swish(O.w4a16_matmul(x, pg, sg))).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    got = host(K.w4a16_gemm(dev(x), K.W4Weight(dev(pg), dev(sg)), bias=dev(bias), residual=dev(res)))
+    ref = ((O.w4a16_matmul(x, pg, sg) + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+
+
 def test_w4a16_gemm_epilogue(K):
     x, packed, scale = _w4_case(11, 3, 512, 96)
     rng = np.random.default_rng(12)
@@ -178,6 +226,15 @@ def test_f16_gemm(K, M, Kdim, N):
     assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-4
 
 
+def test_f16_gemm_many_rows_wide_outputs(K):
+    rng = np.random.default_rng(21)
+    M, Kdim, N = 24, 1024, 8192
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    w = (rng.standard_normal((N, Kdim)) * 0.02).astype(np.float16)
+    got = host(K.f16_gemm(dev(x), K.F16Weight(dev(w))))
+    assert rel_err(got, O.matmul(x, w.T)) <= 1e-2
+
+
 def test_f16_gemm_gelu_bias(K):
     rng = np.random.default_rng(9)
     x = rng.standard_normal((2, 256)).astype(np.float16)
@@ -237,6 +294,16 @@ def test_fp8_gemm_both_modes(K, M, Kdim, N, fmt):
     # same weights given in [N, K] orientation tile identically
     fw2 = K.F8Weight(dev(np.ascontiguousarray(w8.T)), sd, fmt, kn=False)
     assert torch.equal(fw.tiled, fw2.tiled)
+
+
+def test_fp8_gemm_many_rows_wide_outputs(K):
+    rng = np.random.default_rng(22)
+    M, Kdim, N = 48, 1024, 8192
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    w8 = O.f8_encode((rng.standard_normal((Kdim, N)) * 0.02).astype(np.float32), "F143", -1)
+    fw = K.F8Weight(dev(w8), dev(np.array([-1], np.int32)), "F143", kn=True)
+    got = host(K.fp8_gemm(dev(x), fw, K.fp8_gemm_workspace(M, Kdim, "cuda")))
+    assert rel_err(got, O.fp8_matmul(x, w8, [-1], [-1], "F143", "F143")) <= 1e-2
 
 
 def test_fp8_gemm_exact_on_representable_values(K):
