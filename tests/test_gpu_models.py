@@ -117,3 +117,18 @@ def test_llama2_graph_replay_equals_eager():
     for _ in range(2):                      # the second run checks that replays start from a clean state
         c_graph, s_graph = graphed.run(ids, L)
         assert np.array_equal(c_graph, c_eager) and s_graph == s_eager
+
+
+def test_llama2_checkpoint_from_disk(tmp_path):
+    """fp16 Hugging Face-style checkpoint on disk (sharded safetensors) -> quantised to the INT4 layout ->
+    decoder: the tokens are those of the oracle on the same quantised weights."""
+    from poptransformer_amd.engine import fused, loader
+    from poptransformer_amd.utils import checkpoint
+    B, L, steps, pad, eos = 2, 48, 32, 0, 2
+    checkpoint.save_state_dict(OM.make_llama2_state_dict(LLAMA_TINY, seed=31, int4=False), str(tmp_path),
+                               max_shard_bytes=256 * 1024)
+    sd = checkpoint.quantize_state_dict_int4(checkpoint.load_state_dict(str(tmp_path)))
+    assert sd["model.layers.0.mlp.down_proj.weight"].dtype == np.int8 and "lm_head.weight_scale" not in sd
+    ids = _prompt(np.random.default_rng(17), B, L, 5, LLAMA_TINY["vocab_size"], pad)
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_TINY, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_TINY))
+    _compare(dec, OM.Llama2Oracle(sd, LLAMA_TINY, L, B), ids, L, steps, pad, eos)
