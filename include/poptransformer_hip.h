@@ -217,6 +217,15 @@ int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32
  * of the largest logit of row r, the lowest index among equals; values (optional) receives it. */
 int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, pta_stream_t stream);
 
+/* ops.topk(k) over the last axis (ops/popart.py:135-137; layers/lm_head.py:52-53,89): ids[r, j] and
+ * values[r, j] (optional) are the j-th largest logit of row r; equal values come in ascending order of
+ * index.  1 <= k <= n. */
+int pta_topk(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, int k, pta_stream_t stream);
+
+/* The slice of ops.random_sample (ops/popart.py:25-29): out[r] = candidates[r, *pick] for candidates
+ * int32 [rows, k] and a device index `pick` (clamped into [0, k)), the same column for every row. */
+int pta_take_column(const int32_t* candidates, const int32_t* pick, int32_t* out, int rows, int k, pta_stream_t stream);
+
 /* Embedding rows (layers/embedding.py:34-36); with pos_table also GPT-2's wte[id] + wpe[*pos]
  * (models/gpt2/embedding.py:31-36).  out [rows, cols].  Row b uses
  * id = ids[b*ids_stride + (ids_index ? *ids_index : 0)], so the `dynamic_slice(container, step)`

@@ -81,6 +81,8 @@ SIGNATURES = {
     "pta_decode_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_void_p]),
     "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "pta_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "pta_take_column": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "pta_embedding": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "pta_half_to_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "pta_fp8_to_half": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_void_p]),

@@ -46,6 +46,83 @@ extern "C" int pta_argmax(const pta_half* logits, int32_t* ids, pta_half* values
   return PTA_OK;
 }
 
+// ops.topk(k) over the last axis (ops/popart.py:135-137; layers/lm_head.py:52-53,89 with topk > 1):
+// the k largest logits of a row in descending order, equal values in ascending order of index (ONNX
+// TopK).  One workgroup per row; pass j finds the largest element that comes after pick j - 1 in that
+// order, so no state beyond the previous pick is kept and equal values are handled exactly.
+__global__ __launch_bounds__(AM_THREADS) void topk_kernel(const f16* __restrict__ x, int32_t* __restrict__ idx,
+                                                          f16* __restrict__ val, int n, int k) {
+  __shared__ float sv[AM_THREADS / 64];
+  __shared__ int si[AM_THREADS / 64];
+  __shared__ float pv;
+  __shared__ int pi;
+  const f16* xr = x + (size_t)blockIdx.x * n;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float last_v = INFINITY;
+  int last_i = -1;
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += AM_THREADS) {
+      const float v = (float)xr[i];
+      const bool after = v < last_v || (v == last_v && i > last_i);      // NaN compares false: never picked
+      if (after && (v > best || (v == best && i < bi))) { best = v; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if (lane == 0) { sv[wave] = best; si[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < AM_THREADS / 64; ++w)
+        if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
+      // fewer than k comparable values (NaN rows, or -inf repeated): index 0 with value -inf
+      idx[(size_t)blockIdx.x * k + j] = bi == 0x7fffffff ? 0 : bi;
+      if (val) val[(size_t)blockIdx.x * k + j] = (f16)best;
+      pv = best;
+      pi = bi;
+    }
+    __syncthreads();
+    last_v = pv;
+    last_i = pi;
+    __syncthreads();
+  }
+}
+
+extern "C" int pta_topk(const pta_half* logits, int32_t* ids, pta_half* values, int rows, int n, int k, pta_stream_t stream) {
+  PTA_REQUIRE(logits && ids, "pta_topk: null pointer");
+  PTA_REQUIRE(rows > 0 && n > 0, "pta_topk: empty input [%d,%d]", rows, n);
+  PTA_REQUIRE(k >= 1 && k <= n, "pta_topk: k must be in [1, %d], got %d", n, k);
+  hipLaunchKernelGGL(topk_kernel, dim3(rows), dim3(AM_THREADS), 0, (hipStream_t)stream, (const f16*)logits, ids,
+                     (f16*)values, n, k);
+  PTA_CHECK_LAUNCH("pta_topk");
+  return PTA_OK;
+}
+
+// ops.random_sample (ops/popart.py:25-29): next[r] = candidates[r, *pick], the same column of the top-k
+// candidates for every row (the reference draws one index per step: the argmax of k normal draws).
+__global__ void take_column_kernel(const int32_t* __restrict__ cand, const int32_t* __restrict__ pick,
+                                   int32_t* __restrict__ out, int rows, int k) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  int c = *pick;
+  c = c < 0 ? 0 : (c >= k ? k - 1 : c);
+  out[r] = cand[(size_t)r * k + c];
+}
+
+extern "C" int pta_take_column(const int32_t* candidates, const int32_t* pick, int32_t* out, int rows, int k,
+                               pta_stream_t stream) {
+  PTA_REQUIRE(candidates && pick && out, "pta_take_column: null pointer");
+  PTA_REQUIRE(rows > 0 && k > 0, "pta_take_column: empty input [%d,%d]", rows, k);
+  hipLaunchKernelGGL(take_column_kernel, dim3((rows + 255) / 256), dim3(256), 0, (hipStream_t)stream, candidates, pick,
+                     out, rows, k);
+  PTA_CHECK_LAUNCH("pta_take_column");
+  return PTA_OK;
+}
+
 // out[b, :] = table[id_b, :] (+ pos_table[*pos, :] in fp16 when pos_table is given), with
 // id_b = ids[b * ids_stride + (ids_index ? *ids_index : 0)]: the column `step` of the id container
 // (dynamic_slice of models/llama2/model.py:168) is read in place.

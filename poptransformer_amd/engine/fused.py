@@ -36,6 +36,7 @@ class DecoderSpec:
     pad_id: int = 0
     eos_id: int = -1
     early_stop: bool = False
+    topk: int = 1                    # > 1: the next token is one of the top-k, drawn as ops.random_sample does
 
     @property
     def norm(self):
@@ -128,6 +129,11 @@ class FusedDecoder:
         self.act = buf(B, ffn)
         self.logits = buf(B, s.vocab)
         self.next_ids = buf(B, dtype=i32)
+        if s.topk > 1:
+            if s.topk > s.vocab:
+                raise ValueError(f"topk = {s.topk} exceeds the vocabulary size {s.vocab}")
+            self._topk_ids, self._topk_vals = buf(B, s.topk, dtype=i32), buf(B, s.topk)
+            self._draws, self._pick = buf(1, s.topk), buf(1, dtype=i32)
         self.container = buf(B, s.max_len, dtype=i32)
         self.mask = buf(B, s.max_len)
         self.stop_mask = buf(B, dtype=i32)
@@ -151,6 +157,8 @@ class FusedDecoder:
         launch per operator.  Raises NotImplementedError when the model is not an INT4 Llama-2
         shape the kernel covers; the per-operator path stays available through `persistent = None`."""
         s, w = self.spec, self.w
+        if s.topk != 1:
+            raise NotImplementedError("the persistent decode step selects greedily (topk = 1)")
         if s.family != "llama2" or s.n_kv_head != s.n_head:
             raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
         lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
@@ -245,7 +253,15 @@ class FusedDecoder:
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)
         h, nrm = self._normed(self.x, w.final_norm)
         self._linear(h, w.head, self.logits, norm=nrm)
-        K.argmax(self.logits, self.next_ids)
+        if s.topk == 1:
+            K.argmax(self.logits, self.next_ids)
+        else:
+            # layers/lm_head.py:52-53 -> ops.random_sample (ops/popart.py:25-29): the top-k ids, then the column
+            # chosen by the argmax of k normal draws, one draw per step for the whole batch
+            K.topk(self.logits, s.topk, self._topk_ids, self._topk_vals)
+            self._draws.normal_()
+            K.argmax(self._draws, self._pick)
+            K.take_column(self._topk_ids, self._pick, self.next_ids)
         K.step_update(self.container, self.mask, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
                       s.pad_id, s.eos_id, s.early_stop)
 

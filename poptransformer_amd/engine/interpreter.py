@@ -224,6 +224,10 @@ class Interpreter:
             vals = torch.empty(xc.shape[:-1], dtype=torch.float16, device=x.device)
             idx = K.argmax(xc, values=vals).reshape(xc.shape[:-1])
             return [vals.unsqueeze(-1), idx.unsqueeze(-1)]
+        if x.dtype == torch.float16 and axis in (-1, x.dim() - 1):
+            xc = x.contiguous()
+            vals, idx = K.topk(xc, k)
+            return [vals.reshape(*xc.shape[:-1], k), idx.reshape(*xc.shape[:-1], k)]
         v, i = torch.topk(x, k, dim=axis)
         return [v, i.to(torch.int32)]
     def _aiOnnx_randomnormal(self, n, env):

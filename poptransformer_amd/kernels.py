@@ -395,6 +395,32 @@ def argmax(logits, ids=None, values=None):
     return ids
 
 
+def topk(logits, k, ids=None, values=None):
+    """The k largest entries of every row of the last axis, descending, equal values by ascending index."""
+    _need(logits, torch.float16, "logits")
+    n = logits.shape[-1]
+    rows = logits.numel() // n
+    if not 1 <= k <= n:
+        raise ValueError(f"topk: k must be in [1, {n}], got {k}")
+    if ids is None:
+        ids = torch.empty((rows, k), dtype=_i32, device=logits.device)
+    if values is None:
+        values = torch.empty((rows, k), dtype=torch.float16, device=logits.device)
+    check(_lib.load().pta_topk(_p(logits), _p(ids), _p(values), rows, n, k, _stream()))
+    return values, ids
+
+
+def take_column(candidates, pick, out=None):
+    """out[r] = candidates[r, pick[0]] (pick: device int32)."""
+    _need(candidates, _i32, "candidates", 2)
+    _need(pick, _i32, "pick")
+    rows, k = candidates.shape
+    if out is None:
+        out = torch.empty(rows, dtype=_i32, device=candidates.device)
+    check(_lib.load().pta_take_column(_p(candidates), _p(pick), _p(out), rows, k, _stream()))
+    return out
+
+
 def embedding(table, ids, out=None, pos_table=None, pos=None, ids_index=None):
     """Rows of `table`.  ids int32 [rows] or, with ids_index (device int32 scalar), a container
     [rows, L] of which column *ids_index is used."""

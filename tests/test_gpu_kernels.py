@@ -599,3 +599,28 @@ def test_step_update_matches_loop_simulator(K, early_stop):
         assert int(host(step)) == state["step"]
         assert bool(host(keep)) == keep_ref
         assert np.array_equal(host(ids_out), upd)
+
+
+# ---------------------------------------------------------------- top-k and sampling
+@pytest.mark.parametrize("rows,n,k", [(1, 50257, 5), (3, 1000, 1), (2, 64, 64), (4, 32000, 40)])
+def test_topk_matches_a_stable_sort(K, rows, n, k):
+    rng = np.random.default_rng(rows + n + k)
+    x = rng.standard_normal((rows, n)).astype(np.float16)
+    x[:, ::7] = x[:, 3:4]                      # many equal values: ties resolve to the lower index
+    vals, ids = K.topk(dev(x), k)
+    vals, ids = host(vals), host(ids)
+    order = np.argsort(-x.astype(np.float32), axis=1, kind="stable")[:, :k]
+    assert np.array_equal(ids, order)
+    assert np.array_equal(vals, np.take_along_axis(x, order, axis=1))
+
+
+def test_topk_guards_and_take_column(K):
+    x = dev(np.zeros((2, 8), np.float16))
+    with pytest.raises(ValueError):
+        K.topk(x, 9)
+    with pytest.raises(ValueError):
+        K.topk(x, 0)
+    cand = dev(np.arange(12, dtype=np.int32).reshape(3, 4))
+    for pick, col in ((0, 0), (3, 3), (7, 3), (-2, 0)):     # out-of-range picks are clamped
+        got = host(K.take_column(cand, dev(np.array([pick], np.int32))))
+        assert np.array_equal(got, np.arange(12).reshape(3, 4)[:, col])

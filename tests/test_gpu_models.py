@@ -132,3 +132,31 @@ def test_llama2_checkpoint_from_disk(tmp_path):
     ids = _prompt(np.random.default_rng(17), B, L, 5, LLAMA_TINY["vocab_size"], pad)
     dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_TINY, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_TINY))
     _compare(dec, OM.Llama2Oracle(sd, LLAMA_TINY, L, B), ids, L, steps, pad, eos)
+
+
+def test_llama2_top_k_sampling_draws_from_the_top_k():
+    """topk > 1 (layers/lm_head.py:52-53): every generated token is one of the k best of that step's logits, all
+    rows of the batch use the same draw, and over many steps every rank is drawn (the reference's generator and
+    its stream are not reproduced: which rank is drawn at a step is not comparable)."""
+    from poptransformer_amd.engine import fused, loader
+    B, L, k, pad, eos = 2, 64, 4, 0, -1
+    sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=1, int4=True)
+    spec = loader.llama2_spec(LLAMA_TINY, L, B, pad, eos)
+    spec.topk = k
+    dec = fused.FusedDecoder(spec, loader.llama2_weights(sd, LLAMA_TINY))
+    ids = _prompt(np.random.default_rng(3), B, L, 4, LLAMA_TINY["vocab_size"], pad)
+    torch.manual_seed(0)
+    dec.capture()
+    dec.reset(ids)
+    ranks = []
+    for it in range(L - 2):
+        dec.run_steps(1)
+        torch.cuda.synchronize()
+        logits = dec.logits.cpu().numpy().astype(np.float32)
+        order = np.argsort(-logits, axis=1, kind="stable")[:, :k]
+        nxt = dec.next_ids.cpu().numpy()
+        r = [int(np.where(order[b] == nxt[b])[0][0]) for b in range(B)]     # raises if not among the top k
+        assert len(set(r)) == 1
+        ranks.append(r[0])
+    assert set(ranks) == set(range(k))
+    assert max(np.bincount(ranks)) < 0.6 * len(ranks)
