@@ -209,6 +209,15 @@ int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32
                          pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
                          pta_stream_t stream);
 
+/* pta_qkv_rope_append and pta_decode_attention in one pass: every attention workgroup rotates its own
+ * query head from the raw projection rows, and the workgroups whose rows hold this step's position
+ * rotate the new key, use it and the new value directly and write them to the ring.  Arguments as in
+ * those two calls; the result is bit-identical to calling them one after the other. */
+int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                             int v_stride, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                             void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
+                             int use_scale, pta_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Token selection and loop bookkeeping
  * ---------------------------------------------------------------------------------- */

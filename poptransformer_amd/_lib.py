@@ -78,6 +78,8 @@ SIGNATURES = {
     "pta_qkv_rope_append": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "pta_decode_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "pta_decode_attention_qkv": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "pta_decode_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_void_p]),
     "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),

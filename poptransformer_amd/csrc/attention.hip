@@ -121,6 +121,12 @@ struct AttnArgs {
   int B, Hq, Hkv, max_len, nsplit;
   int use_scale;
   f16 scale;
+  // fused preparation (pta_decode_attention_qkv): raw projection rows instead of q [B, Hq, D]
+  const f16* q_raw; const f16* k_raw; const f16* v_raw;
+  int q_stride, k_stride, v_stride;
+  f16* kring_w; f16* vring_w;
+  const void* inv_freq;
+  int rope;
 };
 
 __device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
@@ -132,13 +138,18 @@ __device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
 // Partial attention of one (sequence, query head) over one chunk of cache rows.
 // LPP = D/8 lanes share a cache row (16 bytes each); a wave covers 64/LPP rows per load, and
 // requests ATT_UNROLL such loads of K and of V before it uses the first.
-template <int D>
+// FUSED: the workgroup prepares its own operands from the raw projection rows - the rotary embedding
+// of its query head, and, when its range of rows holds this step's position, of the new key; that
+// key and the new value are used from LDS and written to the ring (by the first query head of the
+// KV group), so that no separate preparation pass runs before the attention.
+template <int D, bool FUSED>
 __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   constexpr int LPP = D / 8;
   constexpr int PPW = 64 / LPP;
   constexpr int STRIDE = ATT_WAVES * PPW;
   __shared__ float sm_m[ATT_WAVES], sm_l[ATT_WAVES];
   __shared__ float sm_acc[ATT_WAVES][D];
+  __shared__ __align__(16) f16 sm_qkv[FUSED ? 3 * D : 8];
   const int split = blockIdx.x, bh = blockIdx.y;
   const int step = *a.step;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
@@ -152,9 +163,31 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   const int grp = lane / LPP, sub = lane % LPP;
   const int d0 = sub * 8;
 
+  const int pos = step % a.max_len;
+  bool owner = false;
+  if constexpr (FUSED) {
+    owner = pos >= c0 && pos < c1;
+    for (int t = threadIdx.x; t < (owner ? 3 * D : D); t += ATT_THREADS) {
+      const int which = t / D, d = t % D;
+      const f16* x = which == 0 ? a.q_raw + (size_t)b * a.q_stride + h * D
+                                : (which == 1 ? a.k_raw + (size_t)b * a.k_stride + hk * D : a.v_raw + (size_t)b * a.v_stride + hk * D);
+      f16* y = sm_qkv + which * D;
+      if (which == 2 || a.rope == PTA_ROPE_NONE) y[d] = x[d];
+      else if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
+      else rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
+    }
+    __syncthreads();
+    if (owner && h % (a.Hq / a.Hkv) == 0) {
+      for (int t = threadIdx.x; t < 2 * D; t += ATT_THREADS) {
+        f16* ring = t < D ? a.kring_w : a.vring_w;
+        ring[(((size_t)b * a.Hkv + hk) * a.max_len + pos) * D + t % D] = sm_qkv[D + t];
+      }
+    }
+  }
   float qf[8];
   {
-    const f16x8 q8 = *reinterpret_cast<const f16x8*>(a.q + (size_t)bh * D + d0);
+    const f16x8 q8 = FUSED ? *reinterpret_cast<const f16x8*>(sm_qkv + d0)
+                           : *reinterpret_cast<const f16x8*>(a.q + (size_t)bh * D + d0);
 #pragma unroll
     for (int e = 0; e < 8; ++e) qf[e] = (float)q8[e];
   }
@@ -173,8 +206,13 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       const int p = p0 + u * STRIDE;
       on[u] = p < c1;
       const int pc = on[u] ? p : c1 - 1;
-      k8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (size_t)pc * D));
-      v8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(vb + (size_t)pc * D));
+      if (FUSED && pc == pos) {      // this step's row: its ring copy is being written by this launch
+        k8[u] = *reinterpret_cast<const f16x8*>(sm_qkv + D + d0);
+        v8[u] = *reinterpret_cast<const f16x8*>(sm_qkv + 2 * D + d0);
+      } else {
+        k8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (size_t)pc * D));
+        v8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(vb + (size_t)pc * D));
+      }
     }
     float x[ATT_UNROLL];
     float mn = m;
@@ -293,12 +331,45 @@ extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, 
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(a.nsplit, B * Hq);
   if (D == 128) {
-    hipLaunchKernelGGL(attn_partial_kernel<128>, grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL((attn_partial_kernel<128, false>), grid, dim3(ATT_THREADS), 0, s, a);
     hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * Hq), dim3(128), 0, s, a);
   } else {
-    hipLaunchKernelGGL(attn_partial_kernel<64>, grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL((attn_partial_kernel<64, false>), grid, dim3(ATT_THREADS), 0, s, a);
     hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * Hq), dim3(64), 0, s, a);
   }
   PTA_CHECK_LAUNCH("pta_decode_attention");
+  return PTA_OK;
+}
+
+extern "C" int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                                        int v_stride, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                                        void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
+                                        int use_scale, pta_stream_t stream) {
+  PTA_REQUIRE(q && k && v && kv_ring && step && workspace && out, "pta_decode_attention_qkv: null pointer");
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_decode_attention_qkv: bad head counts %d/%d", Hq, Hkv);
+  PTA_REQUIRE(D == 64 || D == 128, "pta_decode_attention_qkv: head size must be 64 or 128, got %d", D);
+  PTA_REQUIRE(max_len > 0, "pta_decode_attention_qkv: max_len = %d", max_len);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "pta_decode_attention_qkv: unknown rope mode %d", rope);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "pta_decode_attention_qkv: inv_freq is required for rotary modes");
+  PTA_REQUIRE(pta_aligned(kv_ring, 16), "pta_decode_attention_qkv: kv_ring must be 16-byte aligned");
+  AttnArgs a{};
+  a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
+  a.kring_w = (f16*)kv_ring; a.vring_w = (f16*)kv_ring + (size_t)B * Hkv * max_len * D;
+  a.q_raw = (const f16*)q; a.k_raw = (const f16*)k; a.v_raw = (const f16*)v;
+  a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
+  a.inv_freq = inv_freq; a.rope = rope;
+  a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len);
+  a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(a.nsplit, B * Hq);
+  if (D == 128) {
+    hipLaunchKernelGGL((attn_partial_kernel<128, true>), grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * Hq), dim3(128), 0, s, a);
+  } else {
+    hipLaunchKernelGGL((attn_partial_kernel<64, true>), grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * Hq), dim3(64), 0, s, a);
+  }
+  PTA_CHECK_LAUNCH("pta_decode_attention_qkv");
   return PTA_OK;
 }

@@ -240,10 +240,8 @@ class FusedDecoder:
             h, nrm = self._normed(self.x, blk.norm1)
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
-            K.qkv_rope_append(qp, kp, vp, self.q_rot, self.rings[li], self.step, w.inv_freq, B, s.n_head,
-                              s.n_kv_head, s.head_dim, s.max_len, s.rope, qs, ks, vs)
-            K.decode_attention(self.q_rot, self.rings[li], self.step, self.attn_ws, self.ctx, B, s.n_head,
-                               s.n_kv_head, s.head_dim, s.max_len, s.scale_scores)
+            K.decode_attention_qkv(qp, kp, vp, self.rings[li], self.step, w.inv_freq, self.attn_ws, self.ctx, B,
+                                   s.n_head, s.n_kv_head, s.head_dim, s.max_len, s.rope, s.scale_scores, qs, ks, vs)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2)
             if len(blk.mlp_in) == 2:

@@ -384,6 +384,18 @@ def decode_attention(q, kv_ring, step, workspace, out, B, Hq, Hkv, D, max_len, u
     return out
 
 
+def decode_attention_qkv(q, k, v, kv_ring, step, inv_freq, workspace, out, B, Hq, Hkv, D, max_len, rope, use_scale,
+                         q_stride=None, k_stride=None, v_stride=None):
+    """qkv_rope_append + decode_attention in one pass (bit-identical to the two calls)."""
+    q_stride = Hq * D if q_stride is None else q_stride
+    k_stride = Hkv * D if k_stride is None else k_stride
+    v_stride = Hkv * D if v_stride is None else v_stride
+    check(_lib.load().pta_decode_attention_qkv(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(kv_ring), _p(step),
+                                               _p(inv_freq), _p(workspace), _p(out), B, Hq, Hkv, D, max_len, rope,
+                                               1 if use_scale else 0, _stream()))
+    return out
+
+
 # ------------------------------------------------------------------ selection ------------
 def argmax(logits, ids=None, values=None):
     _need(logits, torch.float16, "logits")

@@ -482,6 +482,38 @@ def test_rope_append_attention(K, family, B, Hq, Hkv, D, max_len, steps):
         assert rel_err(got, refs[it]) <= 1e-2, f"step {it}"
 
 
+@pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 130), ("gpt2", 1, 12, 12, 64, 40, 45),
+                                                             ("glm2", 3, 8, 2, 128, 150, 90)])
+def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, Hkv, D, max_len, steps):
+    """pta_decode_attention_qkv (rotary + append inside the attention pass) against the two separate calls: the
+    same context vectors and the same ring, bit for bit, at every step including those after the ring has
+    wrapped, with grouped KV heads and with strided q | k | v rows."""
+    from poptransformer_amd import _lib
+    rng = np.random.default_rng(B * 5 + Hq + D)
+    rope = {"llama": _lib.ROPE_LLAMA, "glm2": _lib.ROPE_GLM2, "gpt2": _lib.ROPE_NONE}[family]
+    inv = None
+    if family == "llama":
+        inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    elif family == "glm2":
+        inv = dev(np.array([1.0 / (10000 ** (i / (D // 2))) for i in range(0, D // 2, 2)]).astype(np.float32))
+    row = (Hq + 2 * Hkv) * D
+    rings = [torch.zeros((2 * B * Hkv, max_len, D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    wss = [K.decode_attention_workspace(B, Hq, D, max_len, "cuda") for _ in range(2)]
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float16, device="cuda")
+    outs = [torch.empty((B, Hq * D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in range(steps):
+        qkv = dev(rng.standard_normal((B, row)).astype(np.float16))          # one row holds q | k | v
+        q, k, v = qkv, qkv[:, Hq * D:], qkv[:, (Hq + Hkv) * D:]
+        step.fill_(it)
+        K.qkv_rope_append(q, k, v, q_rot, rings[0], step, inv, B, Hq, Hkv, D, max_len, rope, row, row, row)
+        K.decode_attention(q_rot, rings[0], step, wss[0], outs[0], B, Hq, Hkv, D, max_len, family != "gpt2")
+        K.decode_attention_qkv(q, k, v, rings[1], step, inv, wss[1], outs[1], B, Hq, Hkv, D, max_len, rope,
+                               family != "gpt2", row, row, row)
+        assert torch.equal(outs[0], outs[1]), f"context differs at step {it}"
+    assert torch.equal(rings[0], rings[1])
+
+
 def test_rope_bit_exact(K):
     """q after rotary embedding and the appended key row are pure fp16 elementwise work: bit-exact."""
     from poptransformer_amd import _lib
