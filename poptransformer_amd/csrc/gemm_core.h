@@ -383,8 +383,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 // ------------------------------------------------------------------------------------------
 constexpr int WIDE_WAVES = 16;
 
-template <class Fmt, int MT, int NB, bool PAIR>
+template <class Fmt, int MT, int NB, bool PAIR, bool NORM = false>
 __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, int total_nb) {
+  static_assert(!NORM || MT == 1, "the fused norm covers up to 16 rows");
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int KV = Fmt::kVec;
   extern __shared__ __align__(16) unsigned char smem[];
@@ -432,6 +433,45 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[b][g][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Fused norm (MT == 1): a first pass over this wave's activation fragments gives the row sums (lane l
+  // holds row l % 16, features (l / 16) * 8 + 0..7 of every 32), they meet over the lane groups and, in
+  // LDS, over the waves; the product pass then normalises every fragment it loads, with the numerics of
+  // pta_rmsnorm / pta_layer_norm_ce (rows > 1 variant).
+  f16 n_mean = (f16)0.0f, n_r = (f16)1.0f;
+  if constexpr (NORM) {
+    {
+      float s1 = 0.f, s2 = 0.f;
+      for (int kt = wave; kt < KT; kt += WIDE_WAVES)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = kt * 128 + j * 32;
+          if (k + (lane >> 4) * 8 < K) {
+            const f16x8 v = *reinterpret_cast<const f16x8*>(xrow[0] + k);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s1 += f; s2 = __builtin_fmaf(f, f, s2); }
+          }
+        }
+      s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
+      s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
+      if (lane < 16) { red[(wave * 16 + lane) * 2] = s1; red[(wave * 16 + lane) * 2 + 1] = s2; }
+      __syncthreads();
+      float sum = 0.f, sq = 0.f;
+#pragma unroll
+      for (int w = 0; w < WIDE_WAVES; ++w) { sum += red[(w * 16 + (lane & 15)) * 2]; sq += red[(w * 16 + (lane & 15)) * 2 + 1]; }
+      __syncthreads();      // the buffer is reused for the partial sums of the product
+      const float inv_n = 1.0f / (float)K;
+      if (a.epi.norm == PTA_NORM_RMS) {
+        n_r = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
+      } else {
+        const float mean = sum * inv_n;
+        n_mean = (f16)mean;
+        float var;
+        if (a.M == 1) var = sq * inv_n - mean * mean + a.epi.norm_eps;          // single-row NormCE
+        else { const float mf = (float)n_mean; var = fmaxf(sq * inv_n - mf * mf, 0.0f) + a.epi.norm_eps; }
+        n_r = (f16)(1.0f / sqrtf(var));
+      }
+    }
+  }
   if constexpr (MT == 1) {
     // UN feature tiles per step, all of their loads requested before the first product (a tile
     // beyond KT repeats the last one with zero activations)
@@ -455,7 +495,19 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
         for (int j = 0; j < 4; ++j) {
           const int k = kt * 128 + j * 32;
           const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-          xb[u][j] = there && k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xrow[0] + k) : z;
+          const bool in = there && k + (lane >> 4) * 8 < K;
+          xb[u][j] = in ? *reinterpret_cast<const f16x8*>(xrow[0] + k) : z;
+          if (NORM && in) {
+            const f16x8 gm = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + k + (lane >> 4) * 8);
+            if (a.epi.norm == PTA_NORM_RMS) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) xb[u][j][e] = (xb[u][j][e] * n_r) * gm[e];
+            } else {
+              const f16x8 bt = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + k + (lane >> 4) * 8);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) xb[u][j][e] = ((xb[u][j][e] - n_mean) * n_r) * gm[e] + bt[e];
+            }
+          }
         }
       }
 #pragma unroll
@@ -547,33 +599,33 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
   }
 }
 
-template <class Fmt, int MT, int NB, bool PAIR>
+template <class Fmt, int MT, int NB, bool PAIR, bool NORM = false>
 static int launch_gemv_wide(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   static bool ready = false;
   const size_t smem = (size_t)WIDE_WAVES * NB * (PAIR ? 2 : 1) * MT * 256 * sizeof(float);
   static_assert(WIDE_WAVES * NB * (PAIR ? 2 : 1) * MT * 1024 <= 128 * 1024, "reduction buffer beyond 128 KiB of LDS");
   if (!ready) {
-    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemv_wide_kernel<Fmt, MT, NB, PAIR>,
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemv_wide_kernel<Fmt, MT, NB, PAIR, NORM>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess,
                 "%s: cannot reserve %zu bytes of LDS", name, smem);
     ready = true;
   }
-  hipLaunchKernelGGL((gemv_wide_kernel<Fmt, MT, NB, PAIR>), dim3((total_nb + NB - 1) / NB), dim3(WIDE_WAVES * 64), smem, s,
+  hipLaunchKernelGGL((gemv_wide_kernel<Fmt, MT, NB, PAIR, NORM>), dim3((total_nb + NB - 1) / NB), dim3(WIDE_WAVES * 64), smem, s,
                      a, total_nb);
   return PTA_OK;
 }
 
 // blocks per workgroup: the launch's share per compute unit, capped by what the registers of a wave
 // (weight tiles in flight) and the LDS reduction buffer (8 KiB-groups of partial sums) hold
-template <class Fmt, int MT, bool PAIR>
+template <class Fmt, int MT, bool PAIR, bool NORM = false>
 static int launch_gemv_wide_for(const GemmArgs& a, int total_nb, int per_cu, hipStream_t s, const char* name) {
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int cap_regs = Fmt::kVec * NACC <= 4 ? 3 : 2;
   constexpr int cap_lds = 8 / (NACC * MT) >= 1 ? 8 / (NACC * MT) : 1;
   constexpr int cap = cap_regs < cap_lds ? cap_regs : cap_lds;
-  if (per_cu <= 1 || cap == 1) return launch_gemv_wide<Fmt, MT, 1, PAIR>(a, total_nb, s, name);
-  if (per_cu == 2 || cap == 2) return launch_gemv_wide<Fmt, MT, cap >= 2 ? 2 : 1, PAIR>(a, total_nb, s, name);
-  return launch_gemv_wide<Fmt, MT, cap >= 3 ? 3 : 1, PAIR>(a, total_nb, s, name);
+  if (per_cu <= 1 || cap == 1) return launch_gemv_wide<Fmt, MT, 1, PAIR, NORM>(a, total_nb, s, name);
+  if (per_cu == 2 || cap == 2) return launch_gemv_wide<Fmt, MT, cap >= 2 ? 2 : 1, PAIR, NORM>(a, total_nb, s, name);
+  return launch_gemv_wide<Fmt, MT, cap >= 3 ? 3 : 1, PAIR, NORM>(a, total_nb, s, name);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -805,8 +857,13 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   const size_t xbytes = (size_t)a.M * (a.KT * 128 + 8) * 2;
-  if (a.epi.norm != PTA_NORM_NONE && !(a.M <= 4 && xbytes <= 40 * 1024)) {
-    pta_set_error("%s: the fused norm needs M <= 4 and M*K <= 20480 (got M=%d K=%d)", name, a.M, a.K);
+  bool all_shared_x = true;
+  for (int i = 0; i < a.count; ++i) all_shared_x = all_shared_x && a.mat[i].X == nullptr;
+  const bool norm_small = a.M <= 4 && xbytes <= 40 * 1024;
+  const bool norm_wide = a.M <= 16 && all_shared_x && a.KT >= 8;
+  if (a.epi.norm != PTA_NORM_NONE && !norm_small && !norm_wide) {
+    pta_set_error("%s: the fused norm needs M <= 4 with M*K <= 20480, or M <= 16 with one shared X and K >= 1024 "
+                  "(got M=%d K=%d)", name, a.M, a.K);
     return PTA_EUNSUPPORTED;
   }
   if (a.M <= 4 && xbytes <= 40 * 1024) {
@@ -832,7 +889,8 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
     }
     if (shared_x && a.KT >= 8) {
       int rc;
-      if (a.M <= 16) rc = launch_gemv_wide_for<Fmt, 1, PAIR>(a, total_nb, per_cu, s, name);
+      if (a.M <= 16 && a.epi.norm != PTA_NORM_NONE) rc = launch_gemv_wide_for<Fmt, 1, PAIR, true>(a, total_nb, per_cu, s, name);
+      else if (a.M <= 16) rc = launch_gemv_wide_for<Fmt, 1, PAIR>(a, total_nb, per_cu, s, name);
       else if (a.M <= 32) rc = launch_gemv_wide_for<Fmt, 2, PAIR>(a, total_nb, per_cu, s, name);
       else rc = launch_gemv_wide_for<Fmt, 4, PAIR>(a, total_nb, per_cu, s, name);
       if (rc) return rc;

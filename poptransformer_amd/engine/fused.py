@@ -144,8 +144,10 @@ class FusedDecoder:
         self.attn_ws = K.decode_attention_workspace(B, s.n_head, s.head_dim, s.max_len, device)
         self.graph = None
         self._stream = torch.cuda.Stream()
-        # Measured on MI355X at d = 4096: the norm inside the GEMM costs every workgroup a pass over X
-        # and two barriers (+5 us per launch), the stand-alone norm kernel 2.4 us, so it stays separate.
+        # Measured on MI355X at d = 4096: the norm inside the GEMM costs every workgroup a pass over X and two
+        # barriers: +5 us per launch at batch <= 4 (the stand-alone norm kernel takes 2.4 us) and +5 us per
+        # launch at batch 16 as well (stand-alone 4.4 us, but two of the three GEMMs that follow a norm each
+        # pay for it), so it stays separate.  The kernels support it (M <= 16); tests cover it.
         self.fuse_norm = False
         # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
         self._fp8_buf = {k: buf(B, k) for k in {d, ffn}}
@@ -187,10 +189,11 @@ class FusedDecoder:
             return K.rmsnorm(x, gb[0], self.spec.eps, out)
         return K.layer_norm_ce(x, gb[0], gb[1], self.spec.eps, out)
 
-    def _normed(self, x, gb):
-        """Input and fused-norm argument for a GEMM that consumes norm(x): the norm runs inside the
-        GEMM when the shape allows it, as a kernel of its own into self.h otherwise."""
-        if self.fuse_norm:
+    def _normed(self, x, gb, consumers):
+        """Input and fused-norm argument for the Linears `consumers` of norm(x): the norm runs inside the
+        GEMM when the shape allows it, as a kernel of its own into self.h otherwise (always when a consumer
+        casts its input to FP8 first: the cast needs the normalised values)."""
+        if self.fuse_norm and not any(lw.is_fp8 and lw.act_fp8 for lw in consumers):
             return x, K.Norm(gb[0], gb[1], self.spec.eps)
         self._norm(x, gb, self.h)
         return self.h, None
@@ -237,19 +240,19 @@ class FusedDecoder:
         for li, blk in enumerate(w.blocks):
             if not hasattr(self, "_qkv_views"):
                 self._prepare_qkv_views(blk)
-            h, nrm = self._normed(self.x, blk.norm1)
+            h, nrm = self._normed(self.x, blk.norm1, blk.qkv)
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
             K.decode_attention_qkv(qp, kp, vp, self.rings[li], self.step, w.inv_freq, self.attn_ws, self.ctx, B,
                                    s.n_head, s.n_kv_head, s.head_dim, s.max_len, s.rope, s.scale_scores, qs, ks, vs)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
-            h, nrm = self._normed(self.x, blk.norm2)
+            h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:
                 self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True)
             else:
                 self._linear(h, blk.mlp_in[0], self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)
-        h, nrm = self._normed(self.x, w.final_norm)
+        h, nrm = self._normed(self.x, w.final_norm, [w.head])
         self._linear(h, w.head, self.logits, norm=nrm)
         if s.topk == 1:
             K.argmax(self.logits, self.next_ids)

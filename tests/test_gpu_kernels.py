@@ -204,6 +204,34 @@ def test_gemm_fused_norms(K, M):
         K.w4a16_gemm(dev(np.zeros((16, 768), np.float16)), w, norm=K.Norm(gd, None, 1e-5))
 
 
+@pytest.mark.parametrize("M", [5, 16])
+@pytest.mark.parametrize("Kdim,N", [(1160, 96), (4096, 4096)])
+def test_gemm_fused_norms_up_to_16_rows(K, M, Kdim, N):
+    """5..16 rows: the norm inside the GEMM (row sums in a pass of their own over the fragments each wave
+    loads anyway) equals the norm entry point followed by the GEMM; 1160 features end in a ragged tile."""
+    x, packed, scale = _w4_case(31 + M, M, Kdim, N)
+    rng = np.random.default_rng(23 + Kdim)
+    g = rng.uniform(0.5, 1.5, Kdim).astype(np.float16)
+    b = (rng.standard_normal(Kdim) * 0.1).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    xd, gd, bd = dev(x), dev(g), dev(b)
+    two = host(K.w4a16_gemm(K.rmsnorm(xd, gd, 1e-5), w))
+    one = host(K.w4a16_gemm(xd, w, norm=K.Norm(gd, None, 1e-5)))
+    assert rel_err(one, two) <= 2e-3
+    assert rel_err(one, O.w4a16_matmul(O.rms_norm(x, g, 1e-5), packed, scale)) <= 1e-2
+    two = host(K.w4a16_gemm(K.layer_norm_ce(xd, gd, bd, 1e-5), w))
+    one = host(K.w4a16_gemm(xd, w, norm=K.Norm(gd, bd, 1e-5)))
+    assert rel_err(one, two) <= 2e-3
+    assert rel_err(one, O.w4a16_matmul(O.layer_norm_ce(x, g, b, 1e-5, M, 1, Kdim), packed, scale)) <= 1e-2
+    # a SwiGLU pair and several weights in one launch, each with the norm inside
+    _, pu, su = _w4_case(77, M, Kdim, N)
+    wu = K.W4Weight(dev(pu), dev(su))
+    h = K.rmsnorm(xd, gd, 1e-5)
+    assert rel_err(host(K.w4a16_gemm_swiglu(xd, w, wu, norm=K.Norm(gd, None, 1e-5))), host(K.w4a16_gemm_swiglu(h, w, wu))) <= 2e-3
+    for o1, o2 in zip(K.w4a16_gemm_multi(xd, [w, wu], norm=K.Norm(gd, None, 1e-5)), K.w4a16_gemm_multi(h, [w, wu])):
+        assert rel_err(host(o1), host(o2)) <= 2e-3
+
+
 def test_w4a16_guards(K):
     x, packed, scale = _w4_case(1, 1, 128, 16)
     w = K.W4Weight(dev(packed), dev(scale))

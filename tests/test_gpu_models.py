@@ -160,3 +160,21 @@ def test_llama2_top_k_sampling_draws_from_the_top_k():
         ranks.append(r[0])
     assert set(ranks) == set(range(k))
     assert max(np.bincount(ranks)) < 0.6 * len(ranks)
+
+
+LLAMA_WIDE = dict(vocab_size=640, hidden_size=1024, rms_norm_eps=1e-5, num_attention_heads=8,
+                  intermediate_size=1408, num_hidden_layers=2)
+
+
+@pytest.mark.parametrize("B", [6, 16])
+def test_llama2_int4_decode_batch_up_to_16(B):
+    """Hidden size 1024 and 5..16 sequences: the projections run on the kernel that shares activation fragments
+    between channel blocks, with the norm as a kernel of its own and with the norm inside the GEMM."""
+    from poptransformer_amd.engine import fused, loader
+    L, steps, pad, eos = 40, 32, 0, 2
+    sd = OM.make_llama2_state_dict(LLAMA_WIDE, seed=5, int4=True)
+    ids = _prompt(np.random.default_rng(9), B, L, 6, LLAMA_WIDE["vocab_size"], pad)
+    for fuse in (False, True):
+        dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_WIDE, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_WIDE))
+        dec.fuse_norm = fuse
+        _compare(dec, OM.Llama2Oracle(sd, LLAMA_WIDE, L, B), ids, L, steps, pad, eos)
