@@ -14,6 +14,11 @@ Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel meas
 on the stream it runs on (the persistent decode-step kernel: one launch moves the whole step's
 bytes; or, with the per-operator executor, the fused INT4 gate/up projection), and a CPU baseline
 (the numpy restatement of the same graph on the host cores, on a reduced number of layers).
+
+Other workloads (``--workload``), each printing one line of the same form: ``gemm`` = the single INT4
+weight-only operator X[M, 4096] by W[4096, 11008] at M = ``--batch``; ``chatglm2`` = ChatGLM2-6B-shape FP8
+decode; ``rwkv`` = RWKV-4-7B-shape INT4 recurrent decode.  ``--copy-calibration`` and ``--summarize-pmc``
+serve the hardware-counter measurement of the HBM traffic (see their help).
 """
 import argparse
 import json
