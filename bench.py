@@ -17,7 +17,8 @@ bytes; or, with the per-operator executor, the fused INT4 gate/up projection), a
 
 Other workloads (``--workload``), each printing one line of the same form: ``gemm`` = the single INT4
 weight-only operator X[M, 4096] by W[4096, 11008] at M = ``--batch``; ``chatglm2`` = ChatGLM2-6B-shape FP8
-decode; ``rwkv`` = RWKV-4-7B-shape INT4 recurrent decode.  ``--copy-calibration`` and ``--summarize-pmc``
+decode; ``rwkv`` = RWKV-4-7B-shape INT4 recurrent decode; ``prompt`` = the prompt of the headline model taken in
+passes of up to 64 rows (a step is one pass) instead of one position per loop iteration.  ``--copy-calibration`` and ``--summarize-pmc``
 serve the hardware-counter measurement of the HBM traffic (see their help).
 """
 import argparse
@@ -248,6 +249,52 @@ def other_model_workload(args):
 
 
 
+def prompt_workload(args):
+    """The prompt of the Llama2-7B-shape INT4 model in passes (FusedDecoder.consume_prompt): a step is one pass of
+    64 // batch consecutive positions of every sequence through the 32 blocks (no head: the loop discards the
+    tokens of these positions).  --steps passes are timed after one untimed run of the same prompt; the number of
+    passes is capped by the KV cache length."""
+    import torch
+    from poptransformer_amd.engine import fused, loader, synthetic
+    B, cfg = args.batch, LLAMA2_7B
+    if B > 64:
+        print("the prompt passes take at most 64 rows: batch <= 64", file=sys.stderr)
+        sys.exit(2)
+    R = 64 // B
+    passes = max(1, min(args.steps, (MAX_LEN - 2) // R))
+    n = passes * R
+    weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
+    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
+    rng = np.random.Generator(np.random.PCG64(1234))
+    ids = np.zeros((B, MAX_LEN), np.int32)
+    ids[:, :n + 1] = rng.integers(3, cfg["vocab_size"], size=(B, n + 1))
+    dec.reset(ids)
+    dec.consume_prompt(n)                      # untimed: allocates the row buffers, warms every code path
+    dec.reset(ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.consume_prompt(n)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    d, f, nl = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
+    per_layer = (4 * d * d + 3 * d * f) // 2 + 2 * (4 * d + 2 * f + d) + 2 * 2 * d
+    # per pass: every block's weights once, the pass's K/V rows written, the cache read once per sequence
+    kv = float(np.mean([B * nl * 2 * d * 2 * (p * R + R) + B * nl * 2 * d * 2 * R for p in range(passes)]))
+    pass_bytes = nl * per_layer + kv + 2 * B * R * d
+    flops = 2.0 * B * R * nl * (4 * d * d + 3 * d * f)
+    print(json.dumps({
+        "metric": "prompt tokens/s", "value": B * n / dt, "unit": "tokens/s", "n_gpus": 1, "steps": passes, "warmup": passes,
+        "ms_per_step": dt / passes * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
+        "config": {"workload": f"Llama2-7B-shape INT4 prompt of {n} positions per sequence in {passes} passes of {R} positions, "
+                               f"batch {B}, KV cache length {MAX_LEN}", "batch": B, "rows_per_pass": B * R,
+                   "executor": "operators"},
+        "step_algorithmic_bytes": pass_bytes,
+        "step_roofline_frac": pass_bytes / (dt / passes) / (HBM_PEAK_GBS * 1e9),
+        "projection_tflops": flops / (dt / passes) / 1e12,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -256,10 +303,11 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
                     help="default: persistent when the batch fits it (<= 4), else operators")
-    ap.add_argument("--workload", choices=["decode", "gemm", "chatglm2", "rwkv"], default="decode",
+    ap.add_argument("--workload", choices=["decode", "gemm", "chatglm2", "rwkv", "prompt"], default="decode",
                     help="decode: the Llama2-7B-shape INT4 decode loop (the headline); gemm: the single INT4 "
                          "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
-                         "rwkv: RWKV-4-7B-shape INT4 recurrent decode")
+                         "rwkv: RWKV-4-7B-shape INT4 recurrent decode; prompt: the headline model's prompt in passes "
+                         "of up to 64 rows (--steps passes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -290,6 +338,9 @@ def main():
         return
     if args.workload in ("chatglm2", "rwkv"):
         other_model_workload(args)
+        return
+    if args.workload == "prompt":
+        prompt_workload(args)
         return
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)

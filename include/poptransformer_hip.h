@@ -218,6 +218,21 @@ int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_hal
                              void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
                              int use_scale, pta_stream_t stream);
 
+/* The same two operators over `rows` consecutive positions of every sequence at once - the prompt.
+ * The reference feeds a prompt through its loop one token per iteration (the container keeps the
+ * prompt's ids, models/base_model.py:313-318); its two-stage ChatGLM graphs run the same layers with
+ * sequence_length > 1 for the prompt (models/chatglm/attention.py:89-140).  Row r of sequence b (row
+ * b*rows + r of q, k, v, q_out, out) stands at position *step + r: it is rotated for that position,
+ * appended there, and attends to positions 0 .. *step + r, which is what `rows` iterations of the loop
+ * compute.  *step + rows must not exceed max_len (no wrap inside one call).  The attention workspace
+ * is pta_decode_attention_workspace_bytes(B*rows, ...) bytes. */
+int pta_prompt_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                           int v_stride, pta_half* q_out, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                           int B, int rows, int Hq, int Hkv, int D, int max_len, int rope, pta_stream_t stream);
+int pta_prompt_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                         pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
+                         pta_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Token selection and loop bookkeeping
  * ---------------------------------------------------------------------------------- */

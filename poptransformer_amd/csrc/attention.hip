@@ -22,6 +22,7 @@ struct QkvArgs {
   const int32_t* step;
   const void* inv_freq;                       // fp16 [D/2] (PTA_ROPE_LLAMA) or fp32 [D/4] (PTA_ROPE_GLM2)
   int B, Hq, Hkv, D, max_len, rope;
+  int rows;                                   // consecutive positions per sequence (1 in the decode step)
 };
 
 // Llama: angle = fp16(fp16(step) * inv_freq16) (an fp16 MatMul of a 1x1 by a 1xD/2 matrix,
@@ -52,15 +53,16 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
   const int D = a.D;
   const int per_b = (a.Hq + 2 * a.Hkv) * D;
   const int idx = blockIdx.x * 256 + threadIdx.x;
-  if (idx >= a.B * per_b) return;
-  const int b = idx / per_b;
+  if (idx >= a.B * a.rows * per_b) return;
+  const int row = idx / per_b;                // row of the projection outputs: sequence-major, then position
+  const int b = row / a.rows;
   int r = idx % per_b;
-  const int step = *a.step;
+  const int step = *a.step + row % a.rows;
   const int pos = step % a.max_len;
   if (r < a.Hq * D) {
     const int h = r / D, d = r % D;
-    const f16* x = a.q + (size_t)b * a.q_stride + h * D;
-    f16* y = a.q_out + ((size_t)b * a.Hq + h) * D;
+    const f16* x = a.q + (size_t)row * a.q_stride + h * D;
+    f16* y = a.q_out + ((size_t)row * a.Hq + h) * D;
     if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
     else if (a.rope == PTA_ROPE_GLM2) rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
     else y[d] = x[d];
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
   r -= a.Hq * D;
   if (r < a.Hkv * D) {
     const int h = r / D, d = r % D;
-    const f16* x = a.k + (size_t)b * a.k_stride + h * D;
+    const f16* x = a.k + (size_t)row * a.k_stride + h * D;
     f16* y = a.kring + (((size_t)b * a.Hkv + h) * a.max_len + pos) * D;
     if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
     else if (a.rope == PTA_ROPE_GLM2) rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
@@ -78,24 +80,41 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
   }
   r -= a.Hkv * D;
   const int h = r / D, d = r % D;
-  a.vring[(((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d] = a.v[(size_t)b * a.v_stride + h * D + d];
+  a.vring[(((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d] = a.v[(size_t)row * a.v_stride + h * D + d];
+}
+
+static int rope_append_rows(const char* name, const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
+                            int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring, const int32_t* step,
+                            const void* inv_freq, int B, int rows, int Hq, int Hkv, int D, int max_len, int rope,
+                            pta_stream_t stream) {
+  PTA_REQUIRE(q && k && v && q_out && kv_ring && step, "%s: null pointer", name);
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
+  PTA_REQUIRE(D > 0 && D % 4 == 0 && max_len > 0, "%s: bad head size %d or max_len %d", name, D, max_len);
+  PTA_REQUIRE(rows > 0 && rows <= max_len, "%s: rows = %d must lie in [1, max_len = %d]", name, rows, max_len);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "%s: unknown rope mode %d", name, rope);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "%s: inv_freq is required for rotary modes", name);
+  QkvArgs a{(const f16*)q, (const f16*)k, (const f16*)v, q_stride, k_stride, v_stride, (f16*)q_out,
+            (f16*)kv_ring, (f16*)kv_ring + (size_t)B * Hkv * max_len * D, step, inv_freq, B, Hq, Hkv, D, max_len, rope, rows};
+  const long total = (long)B * rows * (Hq + 2 * Hkv) * D;
+  hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
+  PTA_CHECK_LAUNCH(name);
+  return PTA_OK;
 }
 
 extern "C" int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
                                    int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring,
                                    const int32_t* step, const void* inv_freq, int B, int Hq, int Hkv, int D,
                                    int max_len, int rope, pta_stream_t stream) {
-  PTA_REQUIRE(q && k && v && q_out && kv_ring && step, "pta_qkv_rope_append: null pointer");
-  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_qkv_rope_append: bad head counts %d/%d", Hq, Hkv);
-  PTA_REQUIRE(D > 0 && D % 4 == 0 && max_len > 0, "pta_qkv_rope_append: bad head size %d or max_len %d", D, max_len);
-  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "pta_qkv_rope_append: unknown rope mode %d", rope);
-  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "pta_qkv_rope_append: inv_freq is required for rotary modes");
-  QkvArgs a{(const f16*)q, (const f16*)k, (const f16*)v, q_stride, k_stride, v_stride, (f16*)q_out,
-            (f16*)kv_ring, (f16*)kv_ring + (size_t)B * Hkv * max_len * D, step, inv_freq, B, Hq, Hkv, D, max_len, rope};
-  const int total = B * (Hq + 2 * Hkv) * D;
-  hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((total + 255) / 256), dim3(256), 0, (hipStream_t)stream, a);
-  PTA_CHECK_LAUNCH("pta_qkv_rope_append");
-  return PTA_OK;
+  return rope_append_rows("pta_qkv_rope_append", q, k, v, q_stride, k_stride, v_stride, q_out, kv_ring, step, inv_freq, B, 1,
+                          Hq, Hkv, D, max_len, rope, stream);
+}
+
+extern "C" int pta_prompt_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
+                                      int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring,
+                                      const int32_t* step, const void* inv_freq, int B, int rows, int Hq, int Hkv,
+                                      int D, int max_len, int rope, pta_stream_t stream) {
+  return rope_append_rows("pta_prompt_rope_append", q, k, v, q_stride, k_stride, v_stride, q_out, kv_ring, step, inv_freq, B,
+                          rows, Hq, Hkv, D, max_len, rope, stream);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -119,6 +138,7 @@ struct AttnArgs {
   float* part;        // [B*Hq, nsplit, D + 2]: running max, denominator, numerator
   f16* out;           // [B, Hq*D]
   int B, Hq, Hkv, max_len, nsplit;
+  int rows;           // consecutive positions per sequence (1 in the decode step): row r of a sequence sits at step + r
   int use_scale;
   f16 scale;
   // fused preparation (pta_decode_attention_qkv): raw projection rows instead of q [B, Hq, D]
@@ -150,14 +170,14 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   __shared__ float sm_m[ATT_WAVES], sm_l[ATT_WAVES];
   __shared__ float sm_acc[ATT_WAVES][D];
   __shared__ __align__(16) f16 sm_qkv[FUSED ? 3 * D : 8];
-  const int split = blockIdx.x, bh = blockIdx.y;
-  const int step = *a.step;
+  const int split = blockIdx.x, bh = blockIdx.y;      // bh = (sequence * rows + row) * Hq + head
+  const int step = *a.step + (bh / a.Hq) % a.rows;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
   const int chunk = attn_chunk(valid, a.nsplit);
   const int c0 = split * chunk;
   if (c0 >= valid) return;
   const int c1 = c0 + chunk < valid ? c0 + chunk : valid;
-  const int b = bh / a.Hq, h = bh % a.Hq;
+  const int b = bh / (a.Hq * a.rows), h = bh % a.Hq;
   const int hk = h / (a.Hq / a.Hkv);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int grp = lane / LPP, sub = lane % LPP;
@@ -282,7 +302,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
 template <int D>
 __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
   const int bh = blockIdx.x, d = threadIdx.x;
-  const int step = *a.step;
+  const int step = *a.step + (bh / a.Hq) % a.rows;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
   const int chunk = attn_chunk(valid, a.nsplit);
   const int nact = (valid + chunk - 1) / chunk;
@@ -315,30 +335,43 @@ extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int
   return (size_t)B * Hq * nsplit * (D + 2) * sizeof(float);
 }
 
-extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
-                                    pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
-                                    pta_stream_t stream) {
-  PTA_REQUIRE(q && kv_ring && step && workspace && out, "pta_decode_attention: null pointer");
-  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_decode_attention: bad head counts %d/%d", Hq, Hkv);
-  PTA_REQUIRE(D == 64 || D == 128, "pta_decode_attention: head size must be 64 or 128, got %d", D);
-  PTA_REQUIRE(max_len > 0, "pta_decode_attention: max_len = %d", max_len);
-  PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "pta_decode_attention: q and kv_ring must be 16-byte aligned");
+static int attention_rows(const char* name, const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                          pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
+                          pta_stream_t stream) {
+  PTA_REQUIRE(q && kv_ring && step && workspace && out, "%s: null pointer", name);
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
+  PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
+  PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
+  PTA_REQUIRE(rows > 0 && rows <= max_len && (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
+  PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "%s: q and kv_ring must be 16-byte aligned", name);
   AttnArgs a{};
   a.q = (const f16*)q; a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
   a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
-  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len);
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B * rows, Hq, max_len); a.rows = rows;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(a.nsplit, B * Hq);
+  dim3 grid(a.nsplit, B * rows * Hq);
   if (D == 128) {
     hipLaunchKernelGGL((attn_partial_kernel<128, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * Hq), dim3(128), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * rows * Hq), dim3(128), 0, s, a);
   } else {
     hipLaunchKernelGGL((attn_partial_kernel<64, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * Hq), dim3(64), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * rows * Hq), dim3(64), 0, s, a);
   }
-  PTA_CHECK_LAUNCH("pta_decode_attention");
+  PTA_CHECK_LAUNCH(name);
   return PTA_OK;
+}
+
+extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                                    pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
+                                    pta_stream_t stream) {
+  return attention_rows("pta_decode_attention", q, kv_ring, step, workspace, out, B, 1, Hq, Hkv, D, max_len, use_scale, stream);
+}
+
+extern "C" int pta_prompt_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+                                    pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
+                                    pta_stream_t stream) {
+  return attention_rows("pta_prompt_attention", q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale, stream);
 }
 
 extern "C" int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
@@ -359,7 +392,7 @@ extern "C" int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, co
   a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
   a.inv_freq = inv_freq; a.rope = rope;
   a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
-  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len);
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len); a.rows = 1;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(a.nsplit, B * Hq);

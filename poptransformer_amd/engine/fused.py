@@ -269,7 +269,7 @@ class FusedDecoder:
     def _prepare_qkv_views(self, blk):
         """Output buffers of the projections and the (pointer, row stride) views of q, k, v."""
         s = self.spec
-        B, Hq, Hkv, D = s.batch, s.n_head, s.n_kv_head, s.head_dim
+        B, Hq, Hkv, D = getattr(self, "_rows", s.batch), s.n_head, s.n_kv_head, s.head_dim
         f16 = torch.float16
         if len(blk.qkv) == 1:           # GPT-2: one row holds q | k | v
             row = (Hq + 2 * Hkv) * D
@@ -291,12 +291,61 @@ class FusedDecoder:
         ids = torch.as_tensor(np.asarray(input_ids, np.int32))
         if tuple(ids.shape) != (s.batch, s.max_len):
             raise ValueError(f"input_ids must be [{s.batch}, {s.max_len}], got {tuple(ids.shape)}")
+        self._host_ids = ids.numpy().copy()
         self.container.copy_(ids)
         self.mask.fill_(-10000.0)
         self.mask[:, 0] = 0
         self.stop_mask.zero_()
         self.step.zero_()
         self.keep_going.fill_(1)
+
+    def prompt_positions(self):
+        """How many leading loop iterations only read the prompt: their `next_ids` are dropped because the
+        container already holds a token at the next position (models/base_model.py:313-318), and no
+        sequence meets its end token there.  These are the positions `consume_prompt` may take at once."""
+        s, ids = self.spec, self._host_ids
+        n = s.max_len - 1
+        for row in ids:
+            later = row[1:]
+            pads = np.nonzero(later == s.pad_id)[0]
+            ends = np.nonzero(later == s.eos_id)[0]
+            n = min(n, int(pads[0]) if len(pads) else s.max_len - 1, int(ends[0]) if len(ends) else s.max_len - 1)
+        return max(n, 0)
+
+    def consume_prompt(self, n=None, rows_per_pass=None):
+        """Runs the first `n` loop iterations (default: `prompt_positions()`) as passes over up to
+        `rows_per_pass` consecutive positions of every sequence at once instead of one position per iteration.
+        Each weight matrix is then read once per pass instead of once per position.  The KV rings and the loop
+        state end up as `n` iterations of the loop leave them; the logits of these positions are not computed
+        (the loop would discard their tokens).  Call after `reset`.  Returns n."""
+        from .prompt import PromptPass
+        s = self.spec
+        limit = self.prompt_positions()
+        n = limit if n is None else int(n)
+        if n < 0 or n > limit:
+            raise ValueError(f"consume_prompt: n = {n} outside [0, {limit}] (the prompt's own positions before any end token)")
+        if int(self.step.item()) != 0:
+            raise RuntimeError("consume_prompt must follow reset()")
+        if n == 0:
+            return 0
+        R = max(1, 64 // s.batch) if rows_per_pass is None else int(rows_per_pass)
+        if R < 1 or R * s.batch > 64:
+            raise ValueError(f"consume_prompt: rows_per_pass * batch must lie in [1, 64], got {R} * {s.batch}")
+        if not hasattr(self, "_prompt_passes"):
+            self._prompt_passes = {}
+        with torch.cuda.stream(self._stream):
+            p0 = 0
+            while p0 < n:
+                rc = min(R, n - p0)
+                if rc not in self._prompt_passes:
+                    self._prompt_passes[rc] = PromptPass(self, rc)
+                self._prompt_passes[rc].run(p0)
+                p0 += rc
+            # the state n iterations leave behind (pta_step_update n times): positions 0..n open, no stop
+            self.mask[:, :n + 1] = 0
+            self.step.fill_(n)
+        self._stream.synchronize()
+        return n
 
     def capture(self):
         """Record one loop iteration into a HIP graph (after an eager iteration has warmed up

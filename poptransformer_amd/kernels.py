@@ -396,6 +396,29 @@ def decode_attention_qkv(q, k, v, kv_ring, step, inv_freq, workspace, out, B, Hq
     return out
 
 
+def prompt_rope_append(q, k, v, q_out, kv_ring, step, inv_freq, B, rows, Hq, Hkv, D, max_len, rope,
+                       q_stride=None, k_stride=None, v_stride=None):
+    """qkv_rope_append over `rows` consecutive positions per sequence (row b*rows + r stands at step + r)."""
+    _need(step, _i32, "step")
+    q_stride = Hq * D if q_stride is None else q_stride
+    k_stride = Hkv * D if k_stride is None else k_stride
+    v_stride = Hkv * D if v_stride is None else v_stride
+    check(_lib.load().pta_prompt_rope_append(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(q_out), _p(kv_ring),
+                                             _p(step), _p(inv_freq), B, rows, Hq, Hkv, D, max_len, rope, _stream()))
+
+
+def prompt_attention(q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale):
+    """decode_attention over `rows` consecutive positions per sequence; row r attends to positions 0..step+r.
+    workspace: decode_attention_workspace(B * rows, ...)."""
+    _need(step, _i32, "step")
+    need = _lib.load().pta_decode_attention_workspace_bytes(B * rows, Hq, D, max_len)
+    if workspace.numel() * workspace.element_size() < need:
+        raise ValueError(f"prompt_attention: the workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
+    check(_lib.load().pta_prompt_attention(_p(q), _p(kv_ring), _p(step), _p(workspace), _p(out), B, rows, Hq, Hkv, D,
+                                           max_len, 1 if use_scale else 0, _stream()))
+    return out
+
+
 # ------------------------------------------------------------------ selection ------------
 def argmax(logits, ids=None, values=None):
     _need(logits, torch.float16, "logits")

@@ -542,6 +542,55 @@ def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, H
     assert torch.equal(rings[0], rings[1])
 
 
+@pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,first,rows", [("llama", 2, 4, 4, 128, 160, 0, 32), ("llama", 1, 4, 4, 128, 160, 70, 64),
+                                                                  ("gpt2", 3, 4, 4, 64, 64, 5, 21), ("glm2", 2, 8, 2, 128, 200, 64, 17)])
+def test_prompt_rows_equal_the_loop(K, family, B, Hq, Hkv, D, max_len, first, rows):
+    """pta_prompt_rope_append + pta_prompt_attention over `rows` positions at once against the oracle's
+    position-by-position attention (1e-2) and against the per-position calls: the ring is bit-identical, the
+    context vectors agree to rounding (the split of the cache rows over workgroups differs)."""
+    from poptransformer_amd import _lib
+    rng = np.random.default_rng(B + rows + D)
+    steps = first + rows
+    qs = [(rng.standard_normal((B, Hq, D)) * (0.3 if family == "gpt2" else 1.0)).astype(np.float16) for _ in range(steps)]
+    ks = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(steps)]
+    vs = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(steps)]
+    refs = _attention_reference(family, qs, ks, vs, max_len, D)
+    rope = {"llama": _lib.ROPE_LLAMA, "glm2": _lib.ROPE_GLM2, "gpt2": _lib.ROPE_NONE}[family]
+    inv = None
+    if family == "llama":
+        inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    elif family == "glm2":
+        inv = dev(np.array([1.0 / (10000 ** (i / (D // 2))) for i in range(0, D // 2, 2)]).astype(np.float32))
+    rings = [torch.zeros((2 * B * Hkv, max_len, D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    ws = K.decode_attention_workspace(B, Hq, D, max_len, "cuda")
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float16, device="cuda")
+    out = torch.empty((B, Hq * D), dtype=torch.float16, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    loop_out = []
+    for it in range(steps):                       # ring 0: the loop, one position per call
+        step.fill_(it)
+        K.qkv_rope_append(dev(qs[it]), dev(ks[it]), dev(vs[it]), q_rot, rings[0], step, inv, B, Hq, Hkv, D, max_len, rope)
+        K.decode_attention(q_rot, rings[0], step, ws, out, B, Hq, Hkv, D, max_len, family != "gpt2")
+        loop_out.append(host(out))
+        if it < first:                            # ring 1 receives the positions before the pass the same way
+            K.qkv_rope_append(dev(qs[it]), dev(ks[it]), dev(vs[it]), q_rot, rings[1], step, inv, B, Hq, Hkv, D, max_len, rope)
+    # rows of the pass: sequence-major, then position
+    stack = lambda xs: dev(np.stack(xs[first:], axis=1).reshape(B * rows, -1))
+    q_rows = torch.empty((B * rows, Hq, D), dtype=torch.float16, device="cuda")
+    out_rows = torch.empty((B * rows, Hq * D), dtype=torch.float16, device="cuda")
+    ws_rows = K.decode_attention_workspace(B * rows, Hq, D, max_len, "cuda")
+    step.fill_(first)
+    K.prompt_rope_append(stack(qs), stack(ks), stack(vs), q_rows, rings[1], step, inv, B, rows, Hq, Hkv, D, max_len, rope)
+    K.prompt_attention(q_rows, rings[1], step, ws_rows, out_rows, B, rows, Hq, Hkv, D, max_len, family != "gpt2")
+    assert torch.equal(rings[0], rings[1])
+    got = host(out_rows).reshape(B, rows, Hq * D)
+    for r in range(rows):
+        assert rel_err(got[:, r], refs[first + r]) <= 1e-2, f"row {r} against the oracle"
+        assert rel_err(got[:, r], loop_out[first + r]) <= 2e-3, f"row {r} against the loop"
+    with pytest.raises(ValueError):
+        K.prompt_attention(q_rows, rings[1], step, ws, out_rows, B, rows, Hq, Hkv, D, max_len, True)   # workspace of one row
+
+
 def test_rope_bit_exact(K):
     """q after rotary embedding and the appended key row are pure fp16 elementwise work: bit-exact."""
     from poptransformer_amd import _lib

@@ -178,3 +178,93 @@ def test_llama2_int4_decode_batch_up_to_16(B):
         dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_WIDE, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_WIDE))
         dec.fuse_norm = fuse
         _compare(dec, OM.Llama2Oracle(sd, LLAMA_WIDE, L, B), ids, L, steps, pad, eos)
+
+
+def _prompt_then_loop(dec, ids, steps, rows_per_pass=None):
+    dec.reset(ids)
+    n = dec.consume_prompt(rows_per_pass=rows_per_pass)
+    dec.run_steps(steps - n)
+    torch.cuda.synchronize()
+    return n
+
+
+@pytest.mark.parametrize("family,B,plen,rows_per_pass", [("llama2", 1, 41, None), ("llama2", 3, 30, 7), ("gpt2", 2, 25, None),
+                                                          ("chatglm2", 2, 29, 16), ("chatglm2_fp8_weight", 2, 29, None),
+                                                          ("chatglm2_fp8", 2, 29, None)])
+def test_prompt_in_passes_equals_the_loop(family, B, plen, rows_per_pass):
+    """The prompt taken several positions per pass (consume_prompt), then the loop: the container, the step and
+    the tokens are those of the oracle's position-by-position loop, and the KV rings hold what the loop leaves
+    there to fp16 rounding.  Prompts of different lengths: the passes stop at the shortest."""
+    from poptransformer_amd.engine import fused, loader
+    L, steps, pad, eos = 64, 56, 0, 2
+    if family == "llama2":
+        sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=1, int4=True)
+        oracle = OM.Llama2Oracle(sd, LLAMA_TINY, L, B)
+        make = lambda: fused.FusedDecoder(loader.llama2_spec(LLAMA_TINY, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_TINY))
+        vocab = LLAMA_TINY["vocab_size"]
+    elif family == "gpt2":
+        pad, eos = 999, 998
+        sd = OM.make_gpt2_state_dict(GPT2_TINY, seed=2)
+        oracle = OM.GPT2Oracle(sd, GPT2_TINY, L, B)
+        make = lambda: fused.FusedDecoder(loader.gpt2_spec(GPT2_TINY, L, B, pad, eos), loader.gpt2_weights(sd, GPT2_TINY))
+        vocab = 900
+    else:
+        precision = family[9:] or "fp16"
+        sd = OM.make_chatglm2_state_dict(GLM2_TINY, seed=4)
+        scales = {k[:-7]: OM.fp8_weight_scale(v) for k, v in sd.items() if k.endswith("dense.weight") or "h_to_4h_1" in k}
+        oracle = OM.ChatGLM2Oracle(sd, GLM2_TINY, L, B, precision, scales)
+        make = lambda: fused.FusedDecoder(loader.chatglm2_spec(GLM2_TINY, L, B, pad, eos),
+                                          loader.chatglm2_weights(sd, GLM2_TINY, precision, scales))
+        vocab = GLM2_TINY["padded_vocab_size"]
+    ids = _prompt(np.random.default_rng(21), B, L, plen, vocab, pad)
+    if B > 1:
+        ids[B - 1, plen - 4:] = pad                                  # one shorter prompt
+    ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos)
+    loop = make()
+    c_loop, s_loop = loop.run(ids, steps)
+    dec = make()
+    n = _prompt_then_loop(dec, ids, steps, rows_per_pass)
+    assert n == (plen - 1 if B == 1 else plen - 5)
+    assert int(dec.step.item()) == ref_step == s_loop
+    assert torch.equal(dec.mask, loop.mask) and torch.equal(dec.stop_mask, loop.stop_mask)
+    if family.endswith("fp8"):
+        # FP8 activations (3 mantissa bits): a one-ulp fp16 difference between the many-row and the one-row
+        # GEMM flips an FP8 rounding now and then, a 6 % step in that element, and these tiny random models
+        # then pick other tokens later on.  Checked here: the prompt's part of the KV rings, to that step.
+        for a, b in zip(dec.rings, loop.rings):
+            a, b = a[:, :n].float(), b[:, :n].float()
+            assert ((a - b).abs().max() / b.abs().max()).item() <= 1e-1
+        return
+    assert np.array_equal(c_loop, ref_container)
+    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+    for a, b in zip(dec.rings, loop.rings):
+        err = (a.float() - b.float()).abs().max().item() / b.float().abs().max().item()
+        assert err <= 1e-2, f"KV ring differs from the loop's by {err}"
+    # a second generation on the same decoder, graph-captured loop after the passes
+    dec.capture()
+    _prompt_then_loop(dec, ids, steps, rows_per_pass)
+    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+
+
+def test_prompt_passes_stop_before_an_end_token_and_check_their_arguments():
+    from poptransformer_amd.engine import fused, loader
+    B, L, pad, eos = 2, 48, 0, 2
+    sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=1, int4=True)
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_TINY, L, B, pad, eos, early_stop=True), loader.llama2_weights(sd, LLAMA_TINY))
+    ids = _prompt(np.random.default_rng(3), B, L, 20, LLAMA_TINY["vocab_size"], pad)
+    ids[ids == eos] = eos + 1
+    ids[1, 9] = eos                                   # an end token inside the second prompt
+    dec.reset(ids)
+    assert dec.prompt_positions() == 8                # iterations 0..7 read positions 1..8: no end token yet
+    with pytest.raises(ValueError):
+        dec.consume_prompt(9)
+    with pytest.raises(ValueError):
+        dec.consume_prompt(4, rows_per_pass=40)       # 80 rows
+    assert dec.consume_prompt(8) == 8
+    with pytest.raises(RuntimeError):
+        dec.consume_prompt(1)                         # only directly after reset
+    oracle = OM.Llama2Oracle(sd, LLAMA_TINY, L, B)
+    ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, 40, pad, eos, early_stop=True)
+    dec.run_steps(32)
+    torch.cuda.synchronize()
+    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
