@@ -77,7 +77,11 @@ int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t st
  * After, in this order: Y = Y0 + bias (layers/linear.py:42-46); Y = act(Y); Y = Y * mul (the
  * receptance gate of models/rwkv/ffn.py:58); Y = Y + residual (the blocks' residual `ops.add`, e.g.
  * models/llama2/model.py:38-46); Y = Y * post_scale when post_scale != 0 (the halving of
- * models/rwkv/model.py:115-116). */
+ * models/rwkv/model.py:115-116).
+ * workspace (optional): scratch of pta_linear_workspace_bytes(M, N) bytes, 16-byte aligned.  With it, a
+ * single-weight launch of more than 32 rows whose channel count alone cannot fill the machine also
+ * splits K across workgroups (fp32 partial sums in the workspace, summed by a second kernel that
+ * applies the epilogue).  Calls sharing one workspace must not overlap. */
 typedef struct pta_fusion {
   const pta_half* bias;        /* [N] or NULL                                   */
   const pta_half* residual;    /* [M, N] or NULL; may alias Y                   */
@@ -88,7 +92,11 @@ typedef struct pta_fusion {
   const pta_half* norm_weight; /* [K]                                           */
   const pta_half* norm_bias;   /* [K], PTA_NORM_LAYER only                      */
   float norm_eps;
+  void* workspace;             /* NULL, or scratch for a K split across workgroups */
+  size_t workspace_bytes;
 } pta_fusion;
+
+size_t pta_linear_workspace_bytes(int M, int N);
 
 enum { PTA_NORM_NONE = 0, PTA_NORM_RMS = 1, PTA_NORM_LAYER = 2 };
 enum { PTA_ACT_NONE = 0, PTA_ACT_GELU_TANH = 1, PTA_ACT_RELU_SQUARE = 2, PTA_ACT_SIGMOID = 3 };

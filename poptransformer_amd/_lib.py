@@ -51,7 +51,8 @@ class DecodeState(ctypes.Structure):
 class Fusion(ctypes.Structure):
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("mul", c_void_p), ("post_scale", c_float),
                 ("norm", c_int),
-                ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float)]
+                ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float),
+                ("workspace", c_void_p), ("workspace_bytes", c_size_t)]
 
 
 # name -> (restype, argtypes); the order follows include/poptransformer_hip.h
@@ -86,6 +87,7 @@ SIGNATURES = {
                                        c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "pta_prompt_attention": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                      c_int, c_int, c_int, c_void_p]),
+    "pta_linear_workspace_bytes": (c_size_t, [c_int, c_int]),
     "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "pta_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "pta_take_column": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),

@@ -98,7 +98,13 @@ struct GemmArgs {
   int M, K, KT;
   GemmEpilogue epi;
   // PAIR mode (SwiGLU): mat[0] is the gate weight, mat[1] the up weight, output in mat[0].Y.
+  // K split across workgroups (gemm_tile_kernel, one matrix): slice blockIdx.y of `ksplit` writes its fp32
+  // sums to part[slice][M][N]; splitk_finish_kernel adds the slices and applies the epilogue.
+  float* part;
+  size_t part_bytes;
+  int ksplit;          // 0 or 1: no split
 };
+constexpr int GEMM_MAX_KSPLIT = 4;
 
 template <class Fmt, int MT, int NW, bool PAIR>
 __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
@@ -656,7 +662,12 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kq = wave / WPG, wg_ = wave % WPG;  // K group, wave within the group
   const int tig = wg_ * 64 + lane;              // thread index within the group
-  const int K = a.K, KT = a.KT, M = a.M;
+  const int K = a.K, M = a.M;
+  // feature tiles of this workgroup: all of them, or slice blockIdx.y of a K split
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  const int per_slice = (a.KT + nsl - 1) / nsl;
+  const int kt_first = (int)blockIdx.y * per_slice;
+  const int KT = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;     // end of the slice
 
   // the two weight streams of this wave
   int mi = 0;
@@ -674,7 +685,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     const GemmMat& m = a.mat[PAIR ? st : mi];
     nb[st] = PAIR ? first_blk + wg_ : first_blk - m.nb_begin + 2 * wg_ + st;
     sc[st] = Fmt::load_scale(m.scale, a.x_scale, nb[st] * 16 + (lane & 15), m.N);
-    wp[st] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb[st] * KT * (64 * KV) + lane;
+    wp[st] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb[st] * a.KT * (64 * KV) + lane;
   }
   const f16* X = a.mat[mi].X ? a.mat[mi].X : a.X;
 
@@ -710,14 +721,14 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
   };
 
   f16* xbuf = xs + (size_t)kq * 2 * XBUF;
-  const int steps = (KT + KQ - 1) / KQ;
+  const int steps = (KT - kt_first + KQ - 1) / KQ;
   u32x4 w_cur[2][KV], w_nxt[2][KV], xv[VPT];
-  fetch_w(kq, w_cur);
-  fetch_x(kq, xv);
+  fetch_w(kt_first + kq, w_cur);
+  fetch_x(kt_first + kq, xv);
   store_x(xbuf, xv);
   __syncthreads();
   for (int i = 0; i < steps; ++i) {
-    const int kt = kq + i * KQ, ktn = kt + KQ;
+    const int kt = kt_first + kq + i * KQ, ktn = kt + KQ;
     const bool more = i + 1 < steps;
     if (more) { fetch_w(ktn, w_nxt); fetch_x(ktn, xv); }
     const f16* cur = xbuf + (i & 1) * XBUF + (lane & 15) * TILE_XSTRIDE + (lane >> 4) * 8;
@@ -774,8 +785,14 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
       float t = 0.f;
 #pragma unroll
       for (int q = 0; q < KQ; ++q) t += red[((((q * WPG + wslot) * 2 + (PAIR ? g : st)) * MT + mt) * 4 + r) * 64 + ln];
-      sum[g] = Fmt::finish(t, sc[0]);      // no format's finish uses the per-channel part of the scale
+      sum[g] = t;
     }
+    if (!PAIR && nsl > 1) {                // a slice of a K split: the raw fp32 sum; the finishing kernel does the rest
+      a.part[((size_t)blockIdx.y * M + m) * N + n] = sum[0];
+      continue;
+    }
+#pragma unroll
+    for (int g = 0; g < (PAIR ? 2 : 1); ++g) sum[g] = Fmt::finish(sum[g], sc[0]);   // no format's finish uses the per-channel part
     if (PAIR) {
       const f16 gate = (f16)sum[0];
       const f16 up = (f16)sum[1];
@@ -787,6 +804,24 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
       mat.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
     }
   }
+}
+
+// Second half of a K split: adds the slices' fp32 sums of one matrix and applies what the one-kernel form
+// applies to its sum (the format's scale, bias, activation, epilogue).
+template <class Fmt>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a) {
+  const GemmMat& mat = a.mat[0];
+  const int N = mat.N;
+  const size_t total = (size_t)a.M * N;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int m = (int)(i / N), n = (int)(i % N);
+  float t = 0.f;
+  for (int sl = 0; sl < a.ksplit; ++sl) t += a.part[(size_t)sl * total + i];
+  f16 y0 = (f16)Fmt::finish(t, Fmt::load_scale(mat.scale, a.x_scale, n, N));
+  if (mat.bias) y0 = y0 + mat.bias[n];
+  y0 = apply_act(mat.act, y0);
+  mat.Y[i] = apply_epilogue(a.epi, y0, m, n, N);
 }
 
 template <class Fmt, int MT, int KQ, bool PAIR>
@@ -804,7 +839,12 @@ static int launch_gemm_tile(const GemmArgs& a, int total_nb, hipStream_t s, cons
     ready = true;
   }
   const int per_wg = PAIR ? WPG : 2 * WPG;
-  hipLaunchKernelGGL((gemm_tile_kernel<Fmt, MT, KQ, PAIR>), dim3(total_nb / per_wg), dim3(TILE_WAVES * 64), smem, s, a);
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  hipLaunchKernelGGL((gemm_tile_kernel<Fmt, MT, KQ, PAIR>), dim3(total_nb / per_wg, nsl), dim3(TILE_WAVES * 64), smem, s, a);
+  if (nsl > 1) {
+    const size_t total = (size_t)a.M * a.mat[0].N;
+    hipLaunchKernelGGL(splitk_finish_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+  }
   return PTA_OK;
 }
 
@@ -879,7 +919,16 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
       const int cus = device_compute_units();
       const int wgs4 = total_nb / (PAIR ? 2 : 4), wgs8 = total_nb / (PAIR ? 1 : 2);
       int rc = 1;
-      if (tile_fits(a, PAIR ? 2 : 4, 4, PAIR) && 2 * wgs4 >= cus) {
+      // one matrix, more than 32 rows, too few channel blocks to fill the machine, scratch at hand: split K too
+      int nsl = wgs4 > 0 ? cus / wgs4 : 1;
+      nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
+      while (nsl > 1 && a.KT < nsl * 8) --nsl;
+      if (!PAIR && a.count == 1 && a.M > 32 && a.part && nsl > 1 && tile_fits(a, 4, 4, false) &&
+          a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) {
+        GemmArgs b = a;
+        b.ksplit = nsl;
+        rc = launch_gemm_tile<Fmt, 4, 4, PAIR>(b, total_nb, s, name);
+      } else if (tile_fits(a, PAIR ? 2 : 4, 4, PAIR) && 2 * wgs4 >= cus) {
         rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(a, total_nb, s, name);
       } else if (a.M <= 32 && tile_fits(a, PAIR ? 1 : 2, 8, PAIR) && 2 * wgs8 >= cus) {
         rc = launch_gemm_tile<Fmt, 2, 8, PAIR>(a, total_nb, s, name);

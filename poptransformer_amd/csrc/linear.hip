@@ -50,6 +50,11 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
   }
   rc = make_epilogue(fuse, &a.epi, "pta_linear");
   if (rc) return rc;
+  if (fuse && fuse->workspace) {
+    PTA_REQUIRE(pta_aligned(fuse->workspace, 16), "pta_linear: the workspace must be 16-byte aligned");
+    a.part = (float*)fuse->workspace;
+    a.part_bytes = fuse->workspace_bytes;
+  }
   PTA_REQUIRE(count == 1 || (!a.epi.bias && !a.epi.residual && !a.epi.mul && a.epi.post_scale == 0.0f && a.epi.act == PTA_ACT_NONE),
               "pta_linear: with several weights only the norm fields of `fuse` apply (use host_bias for biases)");
   hipStream_t s = (hipStream_t)stream;
@@ -59,6 +64,11 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
     case PTA_W_F143: return run_linear<FmtF8<0>>(a, nb, swiglu, s, "pta_linear");
     default: return run_linear<FmtF8<1>>(a, nb, swiglu, s, "pta_linear");
   }
+}
+
+extern "C" size_t pta_linear_workspace_bytes(int M, int N) {
+  if (M <= 0 || N <= 0) return 0;
+  return (size_t)GEMM_MAX_KSPLIT * M * N * sizeof(float);
 }
 
 // ------------------------------------------------------------------------------------------

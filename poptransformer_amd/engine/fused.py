@@ -211,7 +211,8 @@ class FusedDecoder:
 
     def _linear(self, x, lw, out, residual=None, act=_lib.ACT_NONE, norm=None):
         xin, xs, norm = self._lhs(x, lw, norm)
-        K.linear(xin, [lw.w], [out], x_scale=xs, bias=lw.bias, residual=residual, act=act, norm=norm)
+        K.linear(xin, [lw.w], [out], x_scale=xs, bias=lw.bias, residual=residual, act=act, norm=norm,
+                 workspace=getattr(self, "_lin_ws", None))
         return out
 
     def _linear_group(self, x, lws, outs, norm=None, swiglu=False):

@@ -47,6 +47,8 @@ class PromptPass(FusedDecoder):
         self.attn_ws = K.decode_attention_workspace(M, s.n_head, s.head_dim, s.max_len, self.dev)
         self.fuse_norm = False
         self.persistent = None
+        # scratch for the K split of the projections with few output channels (attention output, MLP down)
+        self._lin_ws = K.linear_workspace(M, max(d, ffn), self.dev)
 
     def run(self, p0):
         """Positions p0 .. p0+rows-1 of every sequence (row b*rows + r is sequence b at p0 + r).  The pass

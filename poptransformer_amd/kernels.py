@@ -49,12 +49,19 @@ def norm_fusable(M, K):
     return M <= 4 and M * (((K + 127) // 128) * 128 + 8) * 2 <= 40 * 1024
 
 
-def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0):
-    if bias is None and residual is None and act == _lib.ACT_NONE and norm is None and mul is None and not post_scale:
+def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0, workspace=None):
+    if (bias is None and residual is None and act == _lib.ACT_NONE and norm is None and mul is None and not post_scale
+            and workspace is None):
         return None
     e = Fusion(_p(bias), _p(residual), act, _p(mul), float(post_scale), norm.kind if norm else _lib.NORM_NONE,
-               _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0)
+               _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0,
+               _p(workspace), workspace.numel() * workspace.element_size() if workspace is not None else 0)
     return ctypes.byref(e)
+
+
+def linear_workspace(M, N, device):
+    """Scratch that lets a single-weight `linear` of more than 32 rows split K across workgroups."""
+    return torch.empty(_lib.load().pta_linear_workspace_bytes(M, N), dtype=torch.uint8, device=device)
 
 
 # ------------------------------------------------------------------ INT4 -----------------
@@ -94,7 +101,7 @@ class W4Weight:
         return self.N * self.K // 2 + self.N * 2
 
 
-def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm=None):
+def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm=None, workspace=None):
     _need(x, torch.float16, "x", 2)
     M, K = x.shape
     if K != w.K:
@@ -102,7 +109,7 @@ def w4a16_gemm(x, w, bias=None, residual=None, act=_lib.ACT_NONE, out=None, norm
     if out is None:
         out = torch.empty((M, w.N), dtype=torch.float16, device=x.device)
     check(_lib.load().pta_w4a16_gemm(_p(x), _p(w.tiled), _p(w.scale), _p(out), M, K, w.N,
-                                     _fusion(bias, residual, act, norm), _stream()))
+                                     _fusion(bias, residual, act, norm, workspace=workspace), _stream()))
     return out
 
 
@@ -257,7 +264,7 @@ def _desc(w, x=None, act=_lib.ACT_NONE):
 
 
 def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None, residual=None, act=_lib.ACT_NONE,
-           norm=None, mul=None, post_scale=0.0, xs=None, acts=None):
+           norm=None, mul=None, post_scale=0.0, xs=None, acts=None, workspace=None):
     """pta_linear: up to four weights of one kind.  They share x, or each takes its own input from
     `xs`.  `biases` / `acts` are per-weight lists (or None); bias / residual / act / mul / post_scale
     apply to the single-weight form only."""
@@ -277,7 +284,7 @@ def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None,
         if w.K != x.shape[1]:
             raise ValueError(f"matmul: contracting dimensions differ ({x.shape[1]} vs {w.K})")
     check(_lib.load().pta_linear(_p(x), _p(x_scale), n, descs, bs, ys, M, 1 if swiglu else 0,
-                                 _fusion(bias, residual, act, norm, mul, post_scale), _stream()))
+                                 _fusion(bias, residual, act, norm, mul, post_scale, workspace), _stream()))
     return outs
 
 

@@ -114,6 +114,31 @@ def test_w4a16_gemm_many_rows_wide_outputs(K, M, Kdim, N):
     assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
 
 
+@pytest.mark.parametrize("M", [33, 64])
+@pytest.mark.parametrize("Kdim,N", [(4096, 1024), (11008, 4096), (2872, 2048)])
+def test_w4a16_gemm_many_rows_few_outputs_split_k(K, M, Kdim, N):
+    """More than 32 rows and too few output channels to fill the machine: with a workspace the launch also
+    splits the features across workgroups (2872 features = 23 tiles, the last ragged: slices of unequal length)
+    and a second kernel adds the slices and applies bias and residual.  Against the oracle, and against the
+    launch without workspace (same sums in another order)."""
+    x, packed, scale = _w4_case(M + Kdim + N, M, Kdim, N)
+    rng = np.random.default_rng(M + N)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    ws = K.linear_workspace(M, N, "cuda")
+    ws.fill_(0xFF)                                        # NaN patterns: every slice must be written before it is read
+    y = dev(res.copy())
+    K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=y, out=y, workspace=ws)       # the residual aliases the output
+    got = host(y)
+    ref = ((O.w4a16_matmul(x, packed, scale) + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+    plain = host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res)))
+    assert rel_err(got, plain) <= 2e-3
+    small = torch.empty(64, dtype=torch.uint8, device="cuda")                      # too small: the one-kernel form runs
+    assert rel_err(host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res), workspace=small)), ref) <= 1e-2
+
+
 def test_w4a16_gemm_many_rows_exact_integers(K):
     rng = np.random.default_rng(6)
     M, Kdim, N = 40, 1024, 8192
