@@ -35,13 +35,13 @@ MAX_LEN = 2048
 HBM_PEAK_GBS = 8000.0
 
 
-def algorithmic_step_bytes(cfg, B, t):
+def algorithmic_step_bytes(cfg, B, t, kv_bytes=2):
     """Bytes one decode step must move at context t: every weight once (INT4 + scales, norm
-    weights, fp16 lm_head), the KV rows written and read, the embedding rows."""
+    weights, fp16 lm_head), the KV rows written and read (kv_bytes per element), the embedding rows."""
     d, f, v, n = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"], cfg["num_hidden_layers"]
     per_layer = (4 * d * d + 3 * d * f) // 2 + 2 * (4 * d + 2 * f + d)
     weights = n * per_layer + 2 * (2 * n + 1) * d + 2 * v * d
-    kv = B * 2 * n * d * 2 * (t + 1)
+    kv = B * 2 * n * d * kv_bytes * (t + 1)
     return weights + kv + B * d * 2
 
 
@@ -308,6 +308,8 @@ def main():
                          "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
                          "rwkv: RWKV-4-7B-shape INT4 recurrent decode; prompt: the headline model's prompt in passes "
                          "of up to 64 rows (--steps passes)")
+    ap.add_argument("--fp8-cache", action="store_true",
+                    help="decode workload, operators executor: keep the KV cache as F143 bytes (KVCacheOp with fp8 = true)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -344,8 +346,8 @@ def main():
         return
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
-    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
-    executor = args.executor or ("persistent" if B <= 4 else "operators")
+    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
+    executor = args.executor or ("persistent" if B <= 4 and not args.fp8_cache else "operators")
     if executor == "persistent":
         dec.enable_persistent()
     dec.capture()
@@ -364,7 +366,8 @@ def main():
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = B * args.steps / dt
-    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(args.warmup, args.warmup + args.steps)])
+    kvb = 1 if args.fp8_cache else 2
+    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t, kvb) for t in range(args.warmup, args.warmup + args.steps)])
     step_frac = mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9)
 
     stream = torch.cuda.Stream()
@@ -423,7 +426,8 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"Llama2-7B-shape INT4 greedy decode, batch {B}, prompt {prompt} consumed token by token, "
-                               f"context {args.warmup}..{args.warmup + args.steps - 1}, fp16 KV cache length {MAX_LEN}",
+                               f"context {args.warmup}..{args.warmup + args.steps - 1}, {'FP8 (F143)' if args.fp8_cache else 'fp16'} KV cache "
+                               f"length {MAX_LEN}",
                    "batch": B, "kv_cache_len": MAX_LEN, "executor": executor},
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
         "roofline": {"bound": "hbm", "kernel": kernel_name,

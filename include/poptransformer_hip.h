@@ -241,6 +241,23 @@ int pta_prompt_attention(const pta_half* q, const pta_half* kv_ring, const int32
                          pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
                          pta_stream_t stream);
 
+/* The same with an FP8 KV cache: KVCacheOp with fp8 = true casts the rows to F143 bytes with the constant
+ * metadata scale 1 before they are stored and casts the whole cache back to fp16 when it is read
+ * (custom_ops/kv_cache.cpp:43-74,103-105; `fp8_cache` of models/llama2/attention.py:18-24).  kv_ring is
+ * uint8 [2*B*Hkv, max_len, D]: a row holds encode_F143(value * 2^-kv_scale), attention uses
+ * decode(byte) * 2^kv_scale.  rows = 1 is the decode step. */
+int pta_prompt_rope_append_f8(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                              int v_stride, pta_half* q_out, uint8_t* kv_ring, const int32_t* step,
+                              const void* inv_freq, int B, int rows, int Hq, int Hkv, int D, int max_len, int rope,
+                              int kv_scale, pta_stream_t stream);
+int pta_prompt_attention_f8(const pta_half* q, const uint8_t* kv_ring, const int32_t* step, void* workspace,
+                            pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
+                            int kv_scale, pta_stream_t stream);
+int pta_decode_attention_qkv_f8(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                                int v_stride, uint8_t* kv_ring, const int32_t* step, const void* inv_freq,
+                                void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
+                                int use_scale, int kv_scale, pta_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Token selection and loop bookkeeping
  * ---------------------------------------------------------------------------------- */

@@ -137,9 +137,12 @@ def run_decode_loop(model, input_ids, max_length, max_loop, pad_id, eos_id, earl
 class Llama2Oracle:
     """LLAMA2DecModel.build_model_graph (poptransformer/models/llama2/model.py:162-197) for
     sequence_length == 1: embedding gather, per block RMSNorm -> attention -> add -> RMSNorm ->
-    SwiGLU MLP -> add (model.py:38-46), final RMSNorm, LMHead top-1 (layers/lm_head.py:47-57)."""
+    SwiGLU MLP -> add (model.py:38-46), final RMSNorm, LMHead top-1 (layers/lm_head.py:47-57).
+    fp8_cache: the `fp8_cache` argument of models/llama2/attention.py:18-24 taken to mean what the KVCache
+    op does with fp8 = true (custom_ops/kv_cache.cpp:102-104,183-185); the reference's Python never sets
+    the attribute (ops/customized.py:32 passes False)."""
 
-    def __init__(self, sd, cfg, max_length, batch_size):
+    def __init__(self, sd, cfg, max_length, batch_size, fp8_cache=False):
         self.cfg, self.L, self.B = cfg, max_length, batch_size
         self.d, self.H = cfg["hidden_size"], cfg["num_attention_heads"]
         self.D = self.d // self.H
@@ -154,7 +157,7 @@ class Llama2Oracle:
                 "v": _Linear(sd, p + "self_attn.v_proj", False), "o": _Linear(sd, p + "self_attn.o_proj", False),
                 "gate": _Linear(sd, p + "mlp.gate_proj", False), "up": _Linear(sd, p + "mlp.up_proj", False),
                 "down": _Linear(sd, p + "mlp.down_proj", False),
-                "cache": O.KVCache(max_length, 3, 1),
+                "cache": O.KVCache(max_length, 3, 1, fp8=fp8_cache),
             })
         self.norm = sd["model.norm.weight"]
         self.head = _Linear(sd, "lm_head", False)

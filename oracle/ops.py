@@ -119,16 +119,21 @@ class KVCache:
     """KVCacheOpx::grow (custom_ops/kv_cache.cpp:94-187): a persistent tensor with the sequence
     axis extended to max_len.  Each call: clone = zeros if step == 0 else cache (:118-125);
     cache = concat(input, clone[0 : max_len - step_len]) along the sequence axis (:127-132);
-    the op's output is the cache."""
+    the op's output is the cache.  With fp8 (:102-104, :183-185) the input is first cast to F143 bytes
+    with the constant metadata scale 1 (CastToUint8, :43-53), the persistent tensor holds bytes, and the
+    output is the whole cache cast back to fp16 (CastUint8ToFP16, :56-74)."""
+    FP8_SCALE = 1
 
-    def __init__(self, max_len, sequence_axis=1, step_len=1):
-        self.max_len, self.axis, self.step_len = max_len, sequence_axis, step_len
+    def __init__(self, max_len, sequence_axis=1, step_len=1, fp8=False):
+        self.max_len, self.axis, self.step_len, self.fp8 = max_len, sequence_axis, step_len, fp8
         self.cache = None
 
     def __call__(self, step, updater):
         updater = np.asarray(updater)
         if updater.shape[self.axis] != self.step_len:
             raise ValueError("updater sequence length != step_len")
+        if self.fp8:
+            updater = f8_encode(updater, "F143", self.FP8_SCALE)
         if self.cache is None:
             shape = list(updater.shape)
             shape[self.axis] = self.max_len
@@ -136,6 +141,8 @@ class KVCache:
         clone = np.zeros_like(self.cache) if int(step) == 0 else self.cache.copy()
         keep = np.take(clone, range(0, self.max_len - self.step_len), axis=self.axis)
         self.cache = np.concatenate([updater, keep], axis=self.axis)
+        if self.fp8:
+            return f8_decode(self.cache, "F143", self.FP8_SCALE, f16)
         return self.cache
 
 

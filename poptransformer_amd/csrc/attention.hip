@@ -10,6 +10,7 @@
 // output, fp16 multiply by 1/sqrt(D)) are reproduced; probabilities stay fp32 up to the final
 // fp16 rounding of the context vector.
 #include "common.h"
+#include "formats.h"
 
 // ------------------------------------------------------------------------------------------
 // q/k rotary embedding + KV ring append.
@@ -23,30 +24,51 @@ struct QkvArgs {
   const void* inv_freq;                       // fp16 [D/2] (PTA_ROPE_LLAMA) or fp32 [D/4] (PTA_ROPE_GLM2)
   int B, Hq, Hkv, D, max_len, rope;
   int rows;                                   // consecutive positions per sequence (1 in the decode step)
+  int kv8, kv_scale;                          // kv8: the rings hold F143 bytes (kring / vring point at bytes)
 };
 
 // Llama: angle = fp16(fp16(step) * inv_freq16) (an fp16 MatMul of a 1x1 by a 1xD/2 matrix,
 // llama2/attention.py:28-38), sin/cos rounded to fp16, rotate-half over the whole head
 // (llama2/attention.py:40-56): y = fp16(fp16(x*cos) + fp16(rot(x)*sin)).
-__device__ __forceinline__ void rope_llama(const f16* x, f16* y, int d, int D, int step, const f16* inv_freq) {
+__device__ __forceinline__ f16 rope_llama_value(const f16* x, int d, int D, int step, const f16* inv_freq) {
   const int half = D >> 1;
   const int i = d < half ? d : d - half;
   const f16 ang = (f16)((float)(f16)(float)step * (float)inv_freq[i]);
   const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
   const f16 rot = d < half ? -x[d + half] : x[d - half];
-  y[d] = x[d] * c + rot * s;
+  return x[d] * c + rot * s;
+}
+__device__ __forceinline__ void rope_llama(const f16* x, f16* y, int d, int D, int step, const f16* inv_freq) {
+  y[d] = rope_llama_value(x, d, D, step, inv_freq);
 }
 
 // ChatGLM2: only the first D/2 features of a head rotate, as interleaved pairs (2j, 2j+1) with
 // angle fp16(fp32(step) * inv_freq32[j]) (chatglm2/attention.py:77-164).
-__device__ __forceinline__ void rope_glm2(const f16* x, f16* y, int d, int D, int step, const float* inv_freq) {
+__device__ __forceinline__ f16 rope_glm2_value(const f16* x, int d, int D, int step, const float* inv_freq) {
   const int rot_dim = D >> 1;
-  if (d >= rot_dim) { y[d] = x[d]; return; }
+  if (d >= rot_dim) return x[d];
   const int j = d >> 1;
   const f16 ang = (f16)((float)step * inv_freq[j]);
   const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
   const f16 rot = (d & 1) ? x[d - 1] : -x[d + 1];
-  y[d] = x[d] * c + rot * s;
+  return x[d] * c + rot * s;
+}
+__device__ __forceinline__ void rope_glm2(const f16* x, f16* y, int d, int D, int step, const float* inv_freq) {
+  y[d] = rope_glm2_value(x, d, D, step, inv_freq);
+}
+
+__device__ __forceinline__ f16 rope_value(int rope, const f16* x, int d, int D, int step, const void* inv_freq) {
+  if (rope == PTA_ROPE_LLAMA) return rope_llama_value(x, d, D, step, (const f16*)inv_freq);
+  if (rope == PTA_ROPE_GLM2) return rope_glm2_value(x, d, D, step, (const float*)inv_freq);
+  return x[d];
+}
+
+// FP8 KV cache (KVCacheOp with fp8 = true, custom_ops/kv_cache.cpp:43-74,103-105): rows are stored as F143
+// bytes of value * 2^-kv_scale (the reference's metadata scale is the constant 1) and read back as
+// decode(byte) * 2^kv_scale, which fp16 holds exactly.
+__device__ __forceinline__ uint8_t kv8_encode(f16 v, int kv_scale) { return F8<0>::encode(ldexpf((float)v, -kv_scale)); }
+__device__ __forceinline__ f16 kv8_round(f16 v, int kv_scale) {
+  return (f16)ldexpf(F8<0>::decode(kv8_encode(v, kv_scale)), kv_scale);
 }
 
 __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
@@ -72,29 +94,35 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
   if (r < a.Hkv * D) {
     const int h = r / D, d = r % D;
     const f16* x = a.k + (size_t)row * a.k_stride + h * D;
-    f16* y = a.kring + (((size_t)b * a.Hkv + h) * a.max_len + pos) * D;
-    if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
-    else if (a.rope == PTA_ROPE_GLM2) rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
-    else y[d] = x[d];
+    const size_t at = (((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d;
+    const f16 y = rope_value(a.rope, x, d, D, step, a.inv_freq);
+    if (a.kv8) reinterpret_cast<uint8_t*>(a.kring)[at] = kv8_encode(y, a.kv_scale);
+    else a.kring[at] = y;
     return;
   }
   r -= a.Hkv * D;
   const int h = r / D, d = r % D;
-  a.vring[(((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d] = a.v[(size_t)row * a.v_stride + h * D + d];
+  const size_t at = (((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d;
+  const f16 y = a.v[(size_t)row * a.v_stride + h * D + d];
+  if (a.kv8) reinterpret_cast<uint8_t*>(a.vring)[at] = kv8_encode(y, a.kv_scale);
+  else a.vring[at] = y;
 }
 
 static int rope_append_rows(const char* name, const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
                             int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring, const int32_t* step,
                             const void* inv_freq, int B, int rows, int Hq, int Hkv, int D, int max_len, int rope,
-                            pta_stream_t stream) {
+                            int kv8, int kv_scale, pta_stream_t stream) {
   PTA_REQUIRE(q && k && v && q_out && kv_ring && step, "%s: null pointer", name);
+  PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
   PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
   PTA_REQUIRE(D > 0 && D % 4 == 0 && max_len > 0, "%s: bad head size %d or max_len %d", name, D, max_len);
   PTA_REQUIRE(rows > 0 && rows <= max_len, "%s: rows = %d must lie in [1, max_len = %d]", name, rows, max_len);
   PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "%s: unknown rope mode %d", name, rope);
   PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "%s: inv_freq is required for rotary modes", name);
+  const size_t ring_elems = (size_t)B * Hkv * max_len * D;
+  f16* vring = kv8 ? (f16*)((uint8_t*)kv_ring + ring_elems) : (f16*)kv_ring + ring_elems;
   QkvArgs a{(const f16*)q, (const f16*)k, (const f16*)v, q_stride, k_stride, v_stride, (f16*)q_out,
-            (f16*)kv_ring, (f16*)kv_ring + (size_t)B * Hkv * max_len * D, step, inv_freq, B, Hq, Hkv, D, max_len, rope, rows};
+            (f16*)kv_ring, vring, step, inv_freq, B, Hq, Hkv, D, max_len, rope, rows, kv8 ? 1 : 0, kv_scale};
   const long total = (long)B * rows * (Hq + 2 * Hkv) * D;
   hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
   PTA_CHECK_LAUNCH(name);
@@ -106,7 +134,7 @@ extern "C" int pta_qkv_rope_append(const pta_half* q, const pta_half* k, const p
                                    const int32_t* step, const void* inv_freq, int B, int Hq, int Hkv, int D,
                                    int max_len, int rope, pta_stream_t stream) {
   return rope_append_rows("pta_qkv_rope_append", q, k, v, q_stride, k_stride, v_stride, q_out, kv_ring, step, inv_freq, B, 1,
-                          Hq, Hkv, D, max_len, rope, stream);
+                          Hq, Hkv, D, max_len, rope, 0, 0, stream);
 }
 
 extern "C" int pta_prompt_rope_append(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
@@ -114,7 +142,15 @@ extern "C" int pta_prompt_rope_append(const pta_half* q, const pta_half* k, cons
                                       const int32_t* step, const void* inv_freq, int B, int rows, int Hq, int Hkv,
                                       int D, int max_len, int rope, pta_stream_t stream) {
   return rope_append_rows("pta_prompt_rope_append", q, k, v, q_stride, k_stride, v_stride, q_out, kv_ring, step, inv_freq, B,
-                          rows, Hq, Hkv, D, max_len, rope, stream);
+                          rows, Hq, Hkv, D, max_len, rope, 0, 0, stream);
+}
+
+extern "C" int pta_prompt_rope_append_f8(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
+                                         int k_stride, int v_stride, pta_half* q_out, uint8_t* kv_ring,
+                                         const int32_t* step, const void* inv_freq, int B, int rows, int Hq, int Hkv,
+                                         int D, int max_len, int rope, int kv_scale, pta_stream_t stream) {
+  return rope_append_rows("pta_prompt_rope_append_f8", q, k, v, q_stride, k_stride, v_stride, q_out, (pta_half*)kv_ring, step,
+                          inv_freq, B, rows, Hq, Hkv, D, max_len, rope, 1, kv_scale, stream);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -139,6 +175,7 @@ struct AttnArgs {
   f16* out;           // [B, Hq*D]
   int B, Hq, Hkv, max_len, nsplit;
   int rows;           // consecutive positions per sequence (1 in the decode step): row r of a sequence sits at step + r
+  int kv_scale;       // FP8 rings (KV8 kernels): rows hold F143 bytes of value * 2^-kv_scale
   int use_scale;
   f16 scale;
   // fused preparation (pta_decode_attention_qkv): raw projection rows instead of q [B, Hq, D]
@@ -162,7 +199,9 @@ __device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
 // of its query head, and, when its range of rows holds this step's position, of the new key; that
 // key and the new value are used from LDS and written to the ring (by the first query head of the
 // KV group), so that no separate preparation pass runs before the attention.
-template <int D, bool FUSED>
+// KV8: the rings hold F143 bytes (8 per lane and row); they are decoded in registers and the power of two of the
+// cache scale is applied to the fp32 score and numerator, which is exact.
+template <int D, bool FUSED, bool KV8>
 __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   constexpr int LPP = D / 8;
   constexpr int PPW = 64 / LPP;
@@ -170,6 +209,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
   __shared__ float sm_m[ATT_WAVES], sm_l[ATT_WAVES];
   __shared__ float sm_acc[ATT_WAVES][D];
   __shared__ __align__(16) f16 sm_qkv[FUSED ? 3 * D : 8];
+  __shared__ __align__(16) uint8_t sm_code[FUSED && KV8 ? 2 * D : 16];
+  const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
   const int split = blockIdx.x, bh = blockIdx.y;      // bh = (sequence * rows + row) * Hq + head
   const int step = *a.step + (bh / a.Hq) % a.rows;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
@@ -191,16 +232,20 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       const int which = t / D, d = t % D;
       const f16* x = which == 0 ? a.q_raw + (size_t)b * a.q_stride + h * D
                                 : (which == 1 ? a.k_raw + (size_t)b * a.k_stride + hk * D : a.v_raw + (size_t)b * a.v_stride + hk * D);
-      f16* y = sm_qkv + which * D;
-      if (which == 2 || a.rope == PTA_ROPE_NONE) y[d] = x[d];
-      else if (a.rope == PTA_ROPE_LLAMA) rope_llama(x, y, d, D, step, (const f16*)a.inv_freq);
-      else rope_glm2(x, y, d, D, step, (const float*)a.inv_freq);
+      f16 y = which == 2 ? x[d] : rope_value(a.rope, x, d, D, step, a.inv_freq);
+      if (KV8 && which != 0) {          // the new row as the cache will hold it: its byte, and decode(byte) for this pass
+        const uint8_t code = kv8_encode(y, a.kv_scale);
+        sm_code[t - D] = code;
+        y = (f16)F8<0>::decode(code);
+      }
+      sm_qkv[t] = y;
     }
     __syncthreads();
     if (owner && h % (a.Hq / a.Hkv) == 0) {
       for (int t = threadIdx.x; t < 2 * D; t += ATT_THREADS) {
-        f16* ring = t < D ? a.kring_w : a.vring_w;
-        ring[(((size_t)b * a.Hkv + hk) * a.max_len + pos) * D + t % D] = sm_qkv[D + t];
+        const size_t at = (((size_t)b * a.Hkv + hk) * a.max_len + pos) * D + t % D;
+        if (KV8) reinterpret_cast<uint8_t*>(t < D ? a.kring_w : a.vring_w)[at] = sm_code[t];
+        else (t < D ? a.kring_w : a.vring_w)[at] = sm_qkv[D + t];
       }
     }
   }
@@ -211,8 +256,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) qf[e] = (float)q8[e];
   }
-  const f16* kb = a.kring + ((size_t)b * a.Hkv + hk) * a.max_len * D + d0;
-  const f16* vb = a.vring + ((size_t)b * a.Hkv + hk) * a.max_len * D + d0;
+  const size_t ring_at = ((size_t)b * a.Hkv + hk) * a.max_len * D + d0;
+  const f16* kb = a.kring + ring_at;
+  const f16* vb = a.vring + ring_at;
+  const uint8_t* kb8 = reinterpret_cast<const uint8_t*>(a.kring) + ring_at;
+  const uint8_t* vb8 = reinterpret_cast<const uint8_t*>(a.vring) + ring_at;
 
   float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
@@ -229,6 +277,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       if (FUSED && pc == pos) {      // this step's row: its ring copy is being written by this launch
         k8[u] = *reinterpret_cast<const f16x8*>(sm_qkv + D + d0);
         v8[u] = *reinterpret_cast<const f16x8*>(sm_qkv + 2 * D + d0);
+      } else if constexpr (KV8) {
+        const u32x2 kr = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(kb8 + (size_t)pc * D));
+        const u32x2 vr = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vb8 + (size_t)pc * D));
+        k8[u] = f143_decode8(kr[0], kr[1]);
+        v8[u] = f143_decode8(vr[0], vr[1]);
       } else {
         k8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kb + (size_t)pc * D));
         v8[u] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(vb + (size_t)pc * D));
@@ -243,6 +296,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[u][e], s);
 #pragma unroll
       for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      if (KV8) s *= kv_mul;
       f16 s16 = (f16)s;                       // fp16 output of the q.K^T MatMul
       if (a.use_scale) s16 = s16 * a.scale;   // fp16 multiply by fp16(1/sqrt(D))
       x[u] = on[u] ? (float)s16 : -INFINITY;
@@ -294,7 +348,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       L = __builtin_fmaf(sm_l[i], w, L);
       A = __builtin_fmaf(sm_acc[i][d], w, A);
     }
-    out[2 + d] = A;
+    out[2 + d] = KV8 ? A * kv_mul : A;
     if (d == 0) { out[0] = M; out[1] = L; }
   }
 }
@@ -335,29 +389,39 @@ extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int
   return (size_t)B * Hq * nsplit * (D + 2) * sizeof(float);
 }
 
-static int attention_rows(const char* name, const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
+template <bool FUSED>
+static void launch_attention(const AttnArgs& a, int D, bool kv8, int heads_rows, hipStream_t s) {
+  dim3 grid(a.nsplit, heads_rows);
+  if (D == 128) {
+    if (kv8) hipLaunchKernelGGL((attn_partial_kernel<128, FUSED, true>), grid, dim3(ATT_THREADS), 0, s, a);
+    else hipLaunchKernelGGL((attn_partial_kernel<128, FUSED, false>), grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(heads_rows), dim3(128), 0, s, a);
+  } else {
+    if (kv8) hipLaunchKernelGGL((attn_partial_kernel<64, FUSED, true>), grid, dim3(ATT_THREADS), 0, s, a);
+    else hipLaunchKernelGGL((attn_partial_kernel<64, FUSED, false>), grid, dim3(ATT_THREADS), 0, s, a);
+    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(heads_rows), dim3(64), 0, s, a);
+  }
+}
+
+static int attention_rows(const char* name, const pta_half* q, const void* kv_ring, const int32_t* step, void* workspace,
                           pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
-                          pta_stream_t stream) {
+                          int kv8, int kv_scale, pta_stream_t stream) {
   PTA_REQUIRE(q && kv_ring && step && workspace && out, "%s: null pointer", name);
   PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
   PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
   PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
   PTA_REQUIRE(rows > 0 && rows <= max_len && (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
   PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "%s: q and kv_ring must be 16-byte aligned", name);
+  PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
+  const size_t ring_elems = (size_t)B * Hkv * max_len * D;
   AttnArgs a{};
-  a.q = (const f16*)q; a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
+  a.q = (const f16*)q; a.kring = (const f16*)kv_ring;
+  a.vring = kv8 ? (const f16*)((const uint8_t*)kv_ring + ring_elems) : (const f16*)kv_ring + ring_elems;
   a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B * rows, Hq, max_len); a.rows = rows;
+  a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
-  hipStream_t s = (hipStream_t)stream;
-  dim3 grid(a.nsplit, B * rows * Hq);
-  if (D == 128) {
-    hipLaunchKernelGGL((attn_partial_kernel<128, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * rows * Hq), dim3(128), 0, s, a);
-  } else {
-    hipLaunchKernelGGL((attn_partial_kernel<64, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * rows * Hq), dim3(64), 0, s, a);
-  }
+  launch_attention<false>(a, D, kv8 != 0, B * rows * Hq, (hipStream_t)stream);
   PTA_CHECK_LAUNCH(name);
   return PTA_OK;
 }
@@ -365,44 +429,63 @@ static int attention_rows(const char* name, const pta_half* q, const pta_half* k
 extern "C" int pta_decode_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
                                     pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int use_scale,
                                     pta_stream_t stream) {
-  return attention_rows("pta_decode_attention", q, kv_ring, step, workspace, out, B, 1, Hq, Hkv, D, max_len, use_scale, stream);
+  return attention_rows("pta_decode_attention", q, kv_ring, step, workspace, out, B, 1, Hq, Hkv, D, max_len, use_scale, 0, 0, stream);
 }
 
 extern "C" int pta_prompt_attention(const pta_half* q, const pta_half* kv_ring, const int32_t* step, void* workspace,
                                     pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
                                     pta_stream_t stream) {
-  return attention_rows("pta_prompt_attention", q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale, stream);
+  return attention_rows("pta_prompt_attention", q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale, 0, 0, stream);
+}
+
+extern "C" int pta_prompt_attention_f8(const pta_half* q, const uint8_t* kv_ring, const int32_t* step, void* workspace,
+                                       pta_half* out, int B, int rows, int Hq, int Hkv, int D, int max_len, int use_scale,
+                                       int kv_scale, pta_stream_t stream) {
+  return attention_rows("pta_prompt_attention_f8", q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale, 1,
+                        kv_scale, stream);
+}
+
+static int attention_qkv(const char* name, const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                         int v_stride, void* kv_ring, const int32_t* step, const void* inv_freq, void* workspace,
+                         pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope, int use_scale, int kv8,
+                         int kv_scale, pta_stream_t stream) {
+  PTA_REQUIRE(q && k && v && kv_ring && step && workspace && out, "%s: null pointer", name);
+  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
+  PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
+  PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "%s: unknown rope mode %d", name, rope);
+  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "%s: inv_freq is required for rotary modes", name);
+  PTA_REQUIRE(pta_aligned(kv_ring, 16), "%s: kv_ring must be 16-byte aligned", name);
+  PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
+  const size_t ring_elems = (size_t)B * Hkv * max_len * D;
+  AttnArgs a{};
+  a.kring_w = (f16*)kv_ring;
+  a.vring_w = kv8 ? (f16*)((uint8_t*)kv_ring + ring_elems) : (f16*)kv_ring + ring_elems;
+  a.kring = a.kring_w; a.vring = a.vring_w;
+  a.q_raw = (const f16*)q; a.k_raw = (const f16*)k; a.v_raw = (const f16*)v;
+  a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
+  a.inv_freq = inv_freq; a.rope = rope;
+  a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len); a.rows = 1;
+  a.kv_scale = kv_scale;
+  a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
+  launch_attention<true>(a, D, kv8 != 0, B * Hq, (hipStream_t)stream);
+  PTA_CHECK_LAUNCH(name);
+  return PTA_OK;
 }
 
 extern "C" int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
                                         int v_stride, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
                                         void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
                                         int use_scale, pta_stream_t stream) {
-  PTA_REQUIRE(q && k && v && kv_ring && step && workspace && out, "pta_decode_attention_qkv: null pointer");
-  PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "pta_decode_attention_qkv: bad head counts %d/%d", Hq, Hkv);
-  PTA_REQUIRE(D == 64 || D == 128, "pta_decode_attention_qkv: head size must be 64 or 128, got %d", D);
-  PTA_REQUIRE(max_len > 0, "pta_decode_attention_qkv: max_len = %d", max_len);
-  PTA_REQUIRE(rope == PTA_ROPE_NONE || rope == PTA_ROPE_LLAMA || rope == PTA_ROPE_GLM2, "pta_decode_attention_qkv: unknown rope mode %d", rope);
-  PTA_REQUIRE(rope == PTA_ROPE_NONE || inv_freq, "pta_decode_attention_qkv: inv_freq is required for rotary modes");
-  PTA_REQUIRE(pta_aligned(kv_ring, 16), "pta_decode_attention_qkv: kv_ring must be 16-byte aligned");
-  AttnArgs a{};
-  a.kring = (const f16*)kv_ring; a.vring = (const f16*)kv_ring + (size_t)B * Hkv * max_len * D;
-  a.kring_w = (f16*)kv_ring; a.vring_w = (f16*)kv_ring + (size_t)B * Hkv * max_len * D;
-  a.q_raw = (const f16*)q; a.k_raw = (const f16*)k; a.v_raw = (const f16*)v;
-  a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride;
-  a.inv_freq = inv_freq; a.rope = rope;
-  a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
-  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len); a.rows = 1;
-  a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
-  hipStream_t s = (hipStream_t)stream;
-  dim3 grid(a.nsplit, B * Hq);
-  if (D == 128) {
-    hipLaunchKernelGGL((attn_partial_kernel<128, true>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(B * Hq), dim3(128), 0, s, a);
-  } else {
-    hipLaunchKernelGGL((attn_partial_kernel<64, true>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(B * Hq), dim3(64), 0, s, a);
-  }
-  PTA_CHECK_LAUNCH("pta_decode_attention_qkv");
-  return PTA_OK;
+  return attention_qkv("pta_decode_attention_qkv", q, k, v, q_stride, k_stride, v_stride, kv_ring, step, inv_freq, workspace, out,
+                       B, Hq, Hkv, D, max_len, rope, use_scale, 0, 0, stream);
+}
+
+extern "C" int pta_decode_attention_qkv_f8(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                                           int v_stride, uint8_t* kv_ring, const int32_t* step, const void* inv_freq,
+                                           void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len,
+                                           int rope, int use_scale, int kv_scale, pta_stream_t stream) {
+  return attention_qkv("pta_decode_attention_qkv_f8", q, k, v, q_stride, k_stride, v_stride, kv_ring, step, inv_freq, workspace,
+                       out, B, Hq, Hkv, D, max_len, rope, use_scale, 1, kv_scale, stream);
 }

@@ -37,6 +37,7 @@ class DecoderSpec:
     eos_id: int = -1
     early_stop: bool = False
     topk: int = 1                    # > 1: the next token is one of the top-k, drawn as ops.random_sample does
+    fp8_cache: bool = False          # KV rings hold F143 bytes with metadata scale 1 (KVCacheOp with fp8 = true)
 
     @property
     def norm(self):
@@ -140,7 +141,9 @@ class FusedDecoder:
         self.step = torch.zeros((), dtype=i32, device=device)
         self.keep_going = torch.ones((), dtype=i32, device=device)
         # one ring per layer: keys then values, [2*B*Hkv, max_len, D]
-        self.rings = [buf(2 * B * s.n_kv_head, s.max_len, s.head_dim) for _ in range(s.n_layer)]
+        self.kv_scale = 1 if s.fp8_cache else None        # the constant of custom_ops/kv_cache.cpp:45
+        self.rings = [buf(2 * B * s.n_kv_head, s.max_len, s.head_dim, dtype=torch.uint8 if s.fp8_cache else f16)
+                      for _ in range(s.n_layer)]
         self.attn_ws = K.decode_attention_workspace(B, s.n_head, s.head_dim, s.max_len, device)
         self.graph = None
         self._stream = torch.cuda.Stream()
@@ -161,6 +164,8 @@ class FusedDecoder:
         s, w = self.spec, self.w
         if s.topk != 1:
             raise NotImplementedError("the persistent decode step selects greedily (topk = 1)")
+        if s.fp8_cache:
+            raise NotImplementedError("the persistent decode step keeps its KV cache in fp16")
         if s.family != "llama2" or s.n_kv_head != s.n_head:
             raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
         lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
@@ -245,7 +250,8 @@ class FusedDecoder:
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
             K.decode_attention_qkv(qp, kp, vp, self.rings[li], self.step, w.inv_freq, self.attn_ws, self.ctx, B,
-                                   s.n_head, s.n_kv_head, s.head_dim, s.max_len, s.rope, s.scale_scores, qs, ks, vs)
+                                   s.n_head, s.n_kv_head, s.head_dim, s.max_len, s.rope, s.scale_scores, qs, ks, vs,
+                                   kv_scale=self.kv_scale)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:

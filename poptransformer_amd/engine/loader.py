@@ -59,10 +59,10 @@ def llama2_weights(sd, cfg, device="cuda"):
                         head=linear_from_state_dict(sd, "lm_head", False, device), inv_freq=_dev(inv_freq, device))
 
 
-def llama2_spec(cfg, max_len, batch, pad_id=0, eos_id=2, early_stop=False):
+def llama2_spec(cfg, max_len, batch, pad_id=0, eos_id=2, early_stop=False, fp8_cache=False):
     d, h = cfg["hidden_size"], cfg["num_attention_heads"]
     return DecoderSpec("llama2", cfg["num_hidden_layers"], d, h, h, d // h, cfg["vocab_size"], max_len, batch,
-                       cfg["rms_norm_eps"], pad_id, eos_id, early_stop)
+                       cfg["rms_norm_eps"], pad_id, eos_id, early_stop, fp8_cache=fp8_cache)
 
 
 def gpt2_weights(sd, cfg, device="cuda"):

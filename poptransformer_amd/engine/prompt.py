@@ -86,9 +86,9 @@ class PromptPass(FusedDecoder):
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
             K.prompt_rope_append(qp, kp, vp, self.q_rot, dec.rings[li], self.first, w.inv_freq, B, R, s.n_head,
-                                 s.n_kv_head, s.head_dim, s.max_len, s.rope, qs, ks, vs)
+                                 s.n_kv_head, s.head_dim, s.max_len, s.rope, qs, ks, vs, kv_scale=dec.kv_scale)
             K.prompt_attention(self.q_rot, dec.rings[li], self.first, self.attn_ws, self.ctx, B, R, s.n_head,
-                               s.n_kv_head, s.head_dim, s.max_len, s.scale_scores)
+                               s.n_kv_head, s.head_dim, s.max_len, s.scale_scores, kv_scale=dec.kv_scale)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:

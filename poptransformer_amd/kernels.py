@@ -391,12 +391,25 @@ def decode_attention(q, kv_ring, step, workspace, out, B, Hq, Hkv, D, max_len, u
     return out
 
 
+def _kv_ring_dtype(kv_ring, kv_scale):
+    want = torch.float16 if kv_scale is None else torch.uint8
+    if kv_ring.dtype != want:
+        raise ValueError(f"kv_ring must be {want} ({'fp16' if kv_scale is None else 'FP8'} cache), got {kv_ring.dtype}")
+
+
 def decode_attention_qkv(q, k, v, kv_ring, step, inv_freq, workspace, out, B, Hq, Hkv, D, max_len, rope, use_scale,
-                         q_stride=None, k_stride=None, v_stride=None):
-    """qkv_rope_append + decode_attention in one pass (bit-identical to the two calls)."""
+                         q_stride=None, k_stride=None, v_stride=None, kv_scale=None):
+    """qkv_rope_append + decode_attention in one pass (bit-identical to the two calls).  kv_scale (an int):
+    kv_ring is a uint8 FP8 cache holding F143 bytes of value * 2^-kv_scale."""
     q_stride = Hq * D if q_stride is None else q_stride
     k_stride = Hkv * D if k_stride is None else k_stride
     v_stride = Hkv * D if v_stride is None else v_stride
+    _kv_ring_dtype(kv_ring, kv_scale)
+    if kv_scale is not None:
+        check(_lib.load().pta_decode_attention_qkv_f8(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(kv_ring),
+                                                      _p(step), _p(inv_freq), _p(workspace), _p(out), B, Hq, Hkv, D,
+                                                      max_len, rope, 1 if use_scale else 0, int(kv_scale), _stream()))
+        return out
     check(_lib.load().pta_decode_attention_qkv(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(kv_ring), _p(step),
                                                _p(inv_freq), _p(workspace), _p(out), B, Hq, Hkv, D, max_len, rope,
                                                1 if use_scale else 0, _stream()))
@@ -404,23 +417,35 @@ def decode_attention_qkv(q, k, v, kv_ring, step, inv_freq, workspace, out, B, Hq
 
 
 def prompt_rope_append(q, k, v, q_out, kv_ring, step, inv_freq, B, rows, Hq, Hkv, D, max_len, rope,
-                       q_stride=None, k_stride=None, v_stride=None):
-    """qkv_rope_append over `rows` consecutive positions per sequence (row b*rows + r stands at step + r)."""
+                       q_stride=None, k_stride=None, v_stride=None, kv_scale=None):
+    """qkv_rope_append over `rows` consecutive positions per sequence (row b*rows + r stands at step + r).
+    kv_scale (an int): kv_ring is a uint8 FP8 cache."""
     _need(step, _i32, "step")
     q_stride = Hq * D if q_stride is None else q_stride
     k_stride = Hkv * D if k_stride is None else k_stride
     v_stride = Hkv * D if v_stride is None else v_stride
+    _kv_ring_dtype(kv_ring, kv_scale)
+    if kv_scale is not None:
+        check(_lib.load().pta_prompt_rope_append_f8(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(q_out), _p(kv_ring),
+                                                    _p(step), _p(inv_freq), B, rows, Hq, Hkv, D, max_len, rope,
+                                                    int(kv_scale), _stream()))
+        return
     check(_lib.load().pta_prompt_rope_append(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(q_out), _p(kv_ring),
                                              _p(step), _p(inv_freq), B, rows, Hq, Hkv, D, max_len, rope, _stream()))
 
 
-def prompt_attention(q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale):
+def prompt_attention(q, kv_ring, step, workspace, out, B, rows, Hq, Hkv, D, max_len, use_scale, kv_scale=None):
     """decode_attention over `rows` consecutive positions per sequence; row r attends to positions 0..step+r.
-    workspace: decode_attention_workspace(B * rows, ...)."""
+    workspace: decode_attention_workspace(B * rows, ...).  kv_scale (an int): kv_ring is a uint8 FP8 cache."""
     _need(step, _i32, "step")
     need = _lib.load().pta_decode_attention_workspace_bytes(B * rows, Hq, D, max_len)
     if workspace.numel() * workspace.element_size() < need:
         raise ValueError(f"prompt_attention: the workspace holds {workspace.numel() * workspace.element_size()} bytes, {need} needed")
+    _kv_ring_dtype(kv_ring, kv_scale)
+    if kv_scale is not None:
+        check(_lib.load().pta_prompt_attention_f8(_p(q), _p(kv_ring), _p(step), _p(workspace), _p(out), B, rows, Hq, Hkv, D,
+                                                  max_len, 1 if use_scale else 0, int(kv_scale), _stream()))
+        return out
     check(_lib.load().pta_prompt_attention(_p(q), _p(kv_ring), _p(step), _p(workspace), _p(out), B, rows, Hq, Hkv, D,
                                            max_len, 1 if use_scale else 0, _stream()))
     return out

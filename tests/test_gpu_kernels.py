@@ -473,11 +473,11 @@ def test_kv_cache_pipeline(K):
 
 
 # ---------------------------------------------------------------- attention
-def _attention_reference(family, qs, ks, vs, max_len, D):
+def _attention_reference(family, qs, ks, vs, max_len, D, fp8_cache=False):
     """Runs the oracle chain step by step; returns the context vectors per step."""
     B, Hq = qs[0].shape[0], qs[0].shape[1]
     Hkv = ks[0].shape[1]
-    cache = O.KVCache(max_len, 3, 1)
+    cache = O.KVCache(max_len, 3, 1, fp8=fp8_cache)
     mask = np.full((B, max_len), -10000, np.float16)
     mask[:, 0] = 0
     outs = []
@@ -614,6 +614,72 @@ def test_prompt_rows_equal_the_loop(K, family, B, Hq, Hkv, D, max_len, first, ro
         assert rel_err(got[:, r], loop_out[first + r]) <= 2e-3, f"row {r} against the loop"
     with pytest.raises(ValueError):
         K.prompt_attention(q_rows, rings[1], step, ws, out_rows, B, rows, Hq, Hkv, D, max_len, True)   # workspace of one row
+
+
+@pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 130), ("glm2", 2, 8, 2, 128, 96, 70),
+                                                             ("gpt2", 1, 4, 4, 64, 48, 50)])
+def test_fp8_kv_cache_attention(K, family, B, Hq, Hkv, D, max_len, steps):
+    """KV rings of F143 bytes (metadata scale 1): the stored bytes are bit-exact against the oracle's cast of the
+    rotated keys and the values, the context vectors within 1e-2 of the oracle's attention over the cast-back
+    cache, at every step including those after the ring has wrapped; the pass that prepares its own operands
+    (pta_decode_attention_qkv_f8) gives the same bytes and the same context, bit for bit, as the two calls; and
+    several positions at once (rows > 1) leave the same bytes as the loop."""
+    from poptransformer_amd import _lib
+    rng = np.random.default_rng(B + Hq + D + 1)
+    qs = [(rng.standard_normal((B, Hq, D)) * (0.3 if family == "gpt2" else 1.0)).astype(np.float16) for _ in range(steps)]
+    # GPT-2's chain has no 1/sqrt(D) and an fp16 softmax without max subtraction: keep its scores small
+    ks = [(rng.standard_normal((B, Hkv, D)) * (1.0 if family == "gpt2" else 2.0)).astype(np.float16) for _ in range(steps)]
+    vs = [(rng.standard_normal((B, Hkv, D)) * 150.0).astype(np.float16) for _ in range(steps)]     # some values saturate at 480
+    refs = _attention_reference(family, qs, ks, vs, max_len, D, fp8_cache=True)
+    rope = {"llama": _lib.ROPE_LLAMA, "glm2": _lib.ROPE_GLM2, "gpt2": _lib.ROPE_NONE}[family]
+    inv = None
+    if family == "llama":
+        inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    elif family == "glm2":
+        inv = dev(np.array([1.0 / (10000 ** (i / (D // 2))) for i in range(0, D // 2, 2)]).astype(np.float32))
+    rings = [torch.zeros((2 * B * Hkv, max_len, D), dtype=torch.uint8, device="cuda") for _ in range(3)]
+    ws = K.decode_attention_workspace(B, Hq, D, max_len, "cuda")
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float16, device="cuda")
+    outs = [torch.empty((B, Hq * D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in range(steps):
+        step.fill_(it)
+        q, k, v = dev(qs[it]), dev(ks[it]), dev(vs[it])
+        K.prompt_rope_append(q, k, v, q_rot, rings[0], step, inv, B, 1, Hq, Hkv, D, max_len, rope, kv_scale=1)
+        K.prompt_attention(q_rot, rings[0], step, ws, outs[0], B, 1, Hq, Hkv, D, max_len, family != "gpt2", kv_scale=1)
+        K.decode_attention_qkv(q, k, v, rings[1], step, inv, ws, outs[1], B, Hq, Hkv, D, max_len, rope, family != "gpt2",
+                               kv_scale=1)
+        got = host(outs[0])
+        assert np.isfinite(got).all()
+        assert rel_err(got, refs[it]) <= 1e-2, f"step {it}"
+        assert torch.equal(outs[0], outs[1]), f"step {it}: the fused pass differs"
+    assert torch.equal(rings[0], rings[1])
+    # the bytes of the last max_len positions against the oracle's cast (position p sits in ring row p % max_len)
+    ring = host(rings[0]).reshape(2, B, Hkv, max_len, D)
+    for p_ in range(max(0, steps - max_len), steps):
+        k4 = ks[p_].reshape(B, Hkv, 1, D)
+        if family == "llama":
+            sin, cos = O.llama_sincos(p_, D)
+            k4 = O.llama_rope(k4, sin, cos)
+        elif family == "glm2":
+            cos, sin = O.glm2_sincos(p_, D)
+            k4 = np.swapaxes(O.glm2_rope(np.swapaxes(k4, 1, 2), cos, sin), 1, 2)
+        assert np.array_equal(ring[0, :, :, p_ % max_len], O.f8_encode(k4[:, :, 0], "F143", 1)), f"key bytes of position {p_}"
+        assert np.array_equal(ring[1, :, :, p_ % max_len], O.f8_encode(vs[p_], "F143", 1)), f"value bytes of position {p_}"
+    # the first `rows` positions at once
+    rows = min(32, max_len)
+    stack = lambda xs: dev(np.stack(xs[:rows], axis=1).reshape(B * rows, -1))
+    q_rows = torch.empty((B * rows, Hq, D), dtype=torch.float16, device="cuda")
+    out_rows = torch.empty((B * rows, Hq * D), dtype=torch.float16, device="cuda")
+    ws_rows = K.decode_attention_workspace(B * rows, Hq, D, max_len, "cuda")
+    step.fill_(0)
+    K.prompt_rope_append(stack(qs), stack(ks), stack(vs), q_rows, rings[2], step, inv, B, rows, Hq, Hkv, D, max_len, rope, kv_scale=1)
+    K.prompt_attention(q_rows, rings[2], step, ws_rows, out_rows, B, rows, Hq, Hkv, D, max_len, family != "gpt2", kv_scale=1)
+    got = host(out_rows).reshape(B, rows, Hq * D)
+    for r in range(rows):
+        assert rel_err(got[:, r], refs[r]) <= 1e-2, f"row {r}"
+    with pytest.raises(ValueError):
+        K.prompt_attention(q_rows, rings[2].view(torch.float16), step, ws_rows, out_rows, B, rows, Hq, Hkv, D, max_len, True, kv_scale=1)
 
 
 def test_rope_bit_exact(K):

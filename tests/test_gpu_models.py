@@ -268,3 +268,23 @@ def test_prompt_passes_stop_before_an_end_token_and_check_their_arguments():
     dec.run_steps(32)
     torch.cuda.synchronize()
     assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+
+
+@pytest.mark.parametrize("B", [1, 3])
+def test_llama2_fp8_kv_cache_matches_oracle(B):
+    """INT4 Llama 2 with the KV cache held as F143 bytes: tokens identical to the oracle whose KVCache op casts
+    its input to FP8 and its output back (fp8 = true), logits within 1e-2; the prompt taken in passes gives the
+    same tokens; the cache takes half the bytes."""
+    from poptransformer_amd.engine import fused, loader
+    L, steps, pad, eos = 48, 32, 0, 2
+    sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=1, int4=True)
+    spec = loader.llama2_spec(LLAMA_TINY, L, B, pad, eos, fp8_cache=True)
+    dec = fused.FusedDecoder(spec, loader.llama2_weights(sd, LLAMA_TINY))
+    assert dec.rings[0].dtype == torch.uint8
+    ids = _prompt(np.random.default_rng(7), B, L, 12, LLAMA_TINY["vocab_size"], pad)
+    _compare(dec, OM.Llama2Oracle(sd, LLAMA_TINY, L, B, fp8_cache=True), ids, L, steps, pad, eos)
+    reference = dec.container.cpu().numpy().copy()
+    _prompt_then_loop(dec, ids, steps)
+    assert np.array_equal(dec.container.cpu().numpy(), reference)
+    with pytest.raises(NotImplementedError):
+        dec.enable_persistent()

@@ -144,6 +144,22 @@ def test_kv_cache_step_len_two():
     assert np.array_equal(out[0, :2], b[0]) and np.array_equal(out[0, 2:4], a[0]) and not out[0, 4:].any()
 
 
+def test_kv_cache_fp8_is_the_fp16_cache_on_the_f143_grid():
+    """fp8 = true: every row of the output is the row the fp16 cache holds, cast to F143 with scale 1 and back
+    (the cast is elementwise, so it commutes with the shift); values beyond 240 * 2 saturate at 480, values on
+    the grid come back unchanged, and the rows before step 0 read as zero."""
+    rng = np.random.default_rng(5)
+    plain, cast = O.KVCache(4, 1, 1), O.KVCache(4, 1, 1, fp8=True)
+    for step in range(7):
+        new = (rng.standard_normal((2, 1, 8)) * 300).astype(f16)
+        new[0, 0, :3] = [1000.0, -1000.0, 0.40625]             # saturating, saturating, on the grid (13 * 2^-5)
+        ref = O.f8_decode(O.f8_encode(plain(step, new), "F143", 1), "F143", 1, f16)
+        out = cast(step, new)
+        assert out.dtype == f16 and np.array_equal(out, ref)
+        assert out[0, 0, 0] == 480 and out[0, 0, 1] == -480 and out[0, 0, 2] == np.float16(0.40625)
+    assert not cast(0, new)[:, 1:].any()
+
+
 def test_kv_cache_pipeline_slots():
     op = O.KVCachePipeline(max_len=3, max_bps=2)
     seen = {0: [], 1: []}
