@@ -310,6 +310,8 @@ def main():
                          "of up to 64 rows (--steps passes)")
     ap.add_argument("--fp8-cache", action="store_true",
                     help="decode workload, operators executor: keep the KV cache as F143 bytes (KVCacheOp with fp8 = true)")
+    ap.add_argument("--fuse-norm", choices=["on", "off"], default=None,
+                    help="operators executor: run the norms inside the projections that consume them (default: the decoder's choice)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -348,6 +350,8 @@ def main():
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
     executor = args.executor or ("persistent" if B <= 4 and not args.fp8_cache else "operators")
+    if args.fuse_norm is not None:
+        dec.fuse_norm = args.fuse_norm == "on"
     if executor == "persistent":
         dec.enable_persistent()
     dec.capture()

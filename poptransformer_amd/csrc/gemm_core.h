@@ -444,52 +444,49 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
   // LDS, over the waves; the product pass then normalises every fragment it loads, with the numerics of
   // pta_rmsnorm / pta_layer_norm_ce (rows > 1 variant).
   f16 n_mean = (f16)0.0f, n_r = (f16)1.0f;
-  if constexpr (NORM) {
-    {
-      float s1 = 0.f, s2 = 0.f;
-      for (int kt = wave; kt < KT; kt += WIDE_WAVES)
+  auto norm_statistics = [&]() {
+    float s1 = 0.f, s2 = 0.f;
+    for (int kt = wave; kt < KT; kt += WIDE_WAVES)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int k = kt * 128 + j * 32;
-          if (k + (lane >> 4) * 8 < K) {
-            const f16x8 v = *reinterpret_cast<const f16x8*>(xrow[0] + k);
+      for (int j = 0; j < 4; ++j) {
+        const int k = kt * 128 + j * 32;
+        if (k + (lane >> 4) * 8 < K) {
+          const f16x8 v = *reinterpret_cast<const f16x8*>(xrow[0] + k);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s1 += f; s2 = __builtin_fmaf(f, f, s2); }
-          }
+          for (int e = 0; e < 8; ++e) { const float f = (float)v[e]; s1 += f; s2 = __builtin_fmaf(f, f, s2); }
         }
-      s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
-      s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
-      if (lane < 16) { red[(wave * 16 + lane) * 2] = s1; red[(wave * 16 + lane) * 2 + 1] = s2; }
-      __syncthreads();
-      float sum = 0.f, sq = 0.f;
-#pragma unroll
-      for (int w = 0; w < WIDE_WAVES; ++w) { sum += red[(w * 16 + (lane & 15)) * 2]; sq += red[(w * 16 + (lane & 15)) * 2 + 1]; }
-      __syncthreads();      // the buffer is reused for the partial sums of the product
-      const float inv_n = 1.0f / (float)K;
-      if (a.epi.norm == PTA_NORM_RMS) {
-        n_r = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
-      } else {
-        const float mean = sum * inv_n;
-        n_mean = (f16)mean;
-        float var;
-        if (a.M == 1) var = sq * inv_n - mean * mean + a.epi.norm_eps;          // single-row NormCE
-        else { const float mf = (float)n_mean; var = fmaxf(sq * inv_n - mf * mf, 0.0f) + a.epi.norm_eps; }
-        n_r = (f16)(1.0f / sqrtf(var));
       }
+    s1 += __shfl_xor(s1, 16, 64); s2 += __shfl_xor(s2, 16, 64);
+    s1 += __shfl_xor(s1, 32, 64); s2 += __shfl_xor(s2, 32, 64);
+    if (lane < 16) { red[(wave * 16 + lane) * 2] = s1; red[(wave * 16 + lane) * 2 + 1] = s2; }
+    __syncthreads();
+    float sum = 0.f, sq = 0.f;
+#pragma unroll
+    for (int w = 0; w < WIDE_WAVES; ++w) { sum += red[(w * 16 + (lane & 15)) * 2]; sq += red[(w * 16 + (lane & 15)) * 2 + 1]; }
+    __syncthreads();      // the buffer is reused for the partial sums of the product
+    const float inv_n = 1.0f / (float)K;
+    if (a.epi.norm == PTA_NORM_RMS) {
+      n_r = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
+    } else {
+      const float mean = sum * inv_n;
+      n_mean = (f16)mean;
+      float var;
+      if (a.M == 1) var = sq * inv_n - mean * mean + a.epi.norm_eps;          // single-row NormCE
+      else { const float mf = (float)n_mean; var = fmaxf(sq * inv_n - mf * mf, 0.0f) + a.epi.norm_eps; }
+      n_r = (f16)(1.0f / sqrtf(var));
     }
-  }
+  };
   if constexpr (MT == 1) {
     // UN feature tiles per step, all of their loads requested before the first product (a tile
     // beyond KT repeats the last one with zero activations)
     constexpr int UN = NB * NACC * KV <= 4 ? 2 : 1;
-    for (int kt0 = wave; kt0 < KT; kt0 += WIDE_WAVES * UN) {
-      u32x4 w[UN][NB][NACC][KV];
-      f16x8 xb[UN][4];
+    u32x4 w[UN][NB][NACC][KV];
+    f16x8 xb[UN][4];
+    auto load_w = [&](int kt0) {
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
         const int kt_ = kt0 + u * WIDE_WAVES;
-        const bool there = kt_ < KT;
-        const int kt = there ? kt_ : KT - 1;
+        const int kt = kt_ < KT ? kt_ : KT - 1;
 #pragma unroll
         for (int b = 0; b < NB; ++b)
 #pragma unroll
@@ -497,6 +494,14 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
 #pragma unroll
             for (int v = 0; v < KV; ++v)
               w[u][b][g][v] = __builtin_nontemporal_load(wp[b][g] + ((size_t)kt * KV + v) * 64);
+      }
+    };
+    auto load_x = [&](int kt0) {
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int kt_ = kt0 + u * WIDE_WAVES;
+        const bool there = kt_ < KT;
+        const int kt = there ? kt_ : KT - 1;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int k = kt * 128 + j * 32;
@@ -516,6 +521,8 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
           }
         }
       }
+    };
+    auto products = [&]() {
 #pragma unroll
       for (int u = 0; u < UN; ++u)
 #pragma unroll
@@ -526,6 +533,26 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
             for (int g = 0; g < NACC; ++g)
               acc[b][g][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(w[u][b][g], j, sc[b][g]), xb[u][j],
                                                                     acc[b][g][0], 0, 0, 0);
+    };
+    int kt0 = wave;
+    if constexpr (NORM) {
+      // Fused norm: the first weight tiles are requested before the pass over the activations that gives the
+      // row statistics (lane l holds row l % 16, features (l / 16) * 8 + 0..7 of every 32; the sums meet over
+      // the lane groups and, in LDS, over the waves), so that pass runs while they are on their way.  The
+      // product pass then normalises every fragment it loads, with the numerics of pta_rmsnorm /
+      // pta_layer_norm_ce (rows > 1 variant).
+      if (kt0 < KT) load_w(kt0);
+      norm_statistics();
+      if (kt0 < KT) {
+        load_x(kt0);
+        products();
+        kt0 += WIDE_WAVES * UN;
+      }
+    }
+    for (; kt0 < KT; kt0 += WIDE_WAVES * UN) {
+      load_w(kt0);
+      load_x(kt0);
+      products();
     }
   } else {
     // several row groups: the activation fragments of one 32-feature slice at a time (16 bytes per
