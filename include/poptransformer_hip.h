@@ -81,7 +81,9 @@ int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t st
  * workspace (optional): scratch of pta_linear_workspace_bytes(M, N) bytes, 16-byte aligned.  With it, a
  * single-weight launch of more than 32 rows whose channel count alone cannot fill the machine also
  * splits K across workgroups (fp32 partial sums in the workspace, summed by a second kernel that
- * applies the epilogue).  Calls sharing one workspace must not overlap. */
+ * applies the epilogue).  Calls sharing one workspace must not overlap.
+ * Last of all, with out_fp8_scale: Y = pta_half_to_fp8_grid(Y) - the cast of the next FP8 Linear
+ * (precision_strategy.py:62-66) done where its input is produced; it also applies to the SwiGLU pair. */
 typedef struct pta_fusion {
   const pta_half* bias;        /* [N] or NULL                                   */
   const pta_half* residual;    /* [M, N] or NULL; may alias Y                   */
@@ -94,6 +96,9 @@ typedef struct pta_fusion {
   float norm_eps;
   void* workspace;             /* NULL, or scratch for a K split across workgroups */
   size_t workspace_bytes;
+  const int32_t* out_fp8_scale;/* NULL, or: leave the result on the FP8 grid of this device exponent, as the
+                                  half_to_uint8 of the Linear that consumes it would (pta_half_to_fp8_grid)   */
+  int out_fp8_format;          /* PTA_F143 / PTA_F152                           */
 } pta_fusion;
 
 size_t pta_linear_workspace_bytes(int M, int N);
@@ -142,6 +147,10 @@ int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K
  * r = fp16(1/sqrt(v)); y = fp16(fp16(x*r) * weight).  x, y fp16 [rows, cols]. cols % 8 == 0. */
 int pta_rmsnorm(const pta_half* x, const pta_half* weight, pta_half* y, int rows, int cols, float eps,
                 pta_stream_t stream);
+/* pta_rmsnorm followed by pta_half_to_fp8_grid in one pass: y = grid(rmsnorm(x)) for the FP8 Linear
+ * that consumes the normalised rows (the same two roundings, bit for bit). */
+int pta_rmsnorm_fp8_grid(const pta_half* x, const pta_half* weight, pta_half* y, const int32_t* scale, int format,
+                         int rows, int cols, float eps, pta_stream_t stream);
 
 /* NormCE LayerNorm (ops/customized.py:69-102; custom_ops/NormCE.cpp:534-610).  fp16 in/out,
  * fp32 statistics.  rows == 1 follows calSmallBatchNorm + GetInPlaceNorm (NormCE.cpp:122-200,

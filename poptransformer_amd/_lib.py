@@ -52,7 +52,8 @@ class Fusion(ctypes.Structure):
     _fields_ = [("bias", c_void_p), ("residual", c_void_p), ("act", c_int), ("mul", c_void_p), ("post_scale", c_float),
                 ("norm", c_int),
                 ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float),
-                ("workspace", c_void_p), ("workspace_bytes", c_size_t)]
+                ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+                ("out_fp8_scale", c_void_p), ("out_fp8_format", c_int)]
 
 
 # name -> (restype, argtypes); the order follows include/poptransformer_hip.h
@@ -94,6 +95,7 @@ SIGNATURES = {
     "pta_decode_attention_qkv_f8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                             c_void_p]),
+    "pta_rmsnorm_fp8_grid": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p]),
     "pta_linear_workspace_bytes": (c_size_t, [c_int, c_int]),
     "pta_argmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "pta_topk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),

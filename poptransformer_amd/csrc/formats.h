@@ -73,46 +73,6 @@ struct FmtF16 {
 
 
 // ------------------------------------------------------------------------------------------
-// scalar FP8 codecs (F143 / F152 bytes, see fp8.hip)
-// ------------------------------------------------------------------------------------------
-template <int FMT>  // 0 = F143, 1 = F152
-struct F8 {
-  static constexpr int MB = FMT == 0 ? 3 : 2;
-  static constexpr int BIAS = FMT == 0 ? 8 : 16;
-  static constexpr int EMAX = FMT == 0 ? 15 : 31;
-  static __device__ __forceinline__ float max_value() { return FMT == 0 ? 240.0f : 57344.0f; }
-
-  static __device__ __forceinline__ float decode(uint8_t c) {
-    if (c == 0x80) return __builtin_nanf("");
-    const int e = (c & 0x7F) >> MB, m = c & ((1 << MB) - 1);
-    const float mag = e == 0 ? ldexpf((float)m, 1 - BIAS - MB) : ldexpf((float)((1 << MB) + m), e - BIAS - MB);
-    return (c & 0x80) ? -mag : mag;
-  }
-
-  // round to nearest even on the format's grid, saturating; v is the already descaled value
-  static __device__ __forceinline__ uint8_t encode(float v) {
-    if (v != v) return 0x80;
-    const float mag = fabsf(v);
-    if (mag == 0.0f) return 0;             // no negative zero in these formats
-    if (mag >= max_value()) return (v < 0 ? 0x80 : 0) | 0x7F;
-    int e;
-    (void)frexpf(mag, &e);                 // mag = f * 2^e, f in [0.5, 1)
-    int ef = e - 1 + BIAS;                 // biased exponent of the format
-    if (ef < 1) ef = 1;                    // subnormal range shares the grid of exponent 1
-    const float q = ldexpf(mag, MB - (ef - BIAS));   // value in units of the grid step
-    float r = rintf(q);                    // ties to even
-    int code;
-    if (ef == 1 && r < (float)(1 << MB)) code = (int)r;                    // subnormal (or zero)
-    else {
-      if (r >= (float)(2 << MB)) { r *= 0.5f; ef += 1; }                   // rounded up to the next binade
-      code = (ef << MB) | ((int)r - (1 << MB));
-      if (code > 0x7F) code = 0x7F;
-    }
-    return (uint8_t)((v < 0 && code != 0) ? (code | 0x80) : code);
-  }
-};
-
-// ------------------------------------------------------------------------------------------
 // in-register decode of 4 bytes to 4 fp16 values carrying decode(byte) * 2^-7 (F143) or
 // decode(byte) * 2^-1 ... see the constants below; the missing power of two joins the scale.
 // ------------------------------------------------------------------------------------------

@@ -6,6 +6,7 @@
 // (e.g. models/llama2/model.py:38-46).  Each step therefore rounds to fp16.
 #pragma once
 #include "common.h"
+#include "f8codec.h"
 
 struct GemmEpilogue {
   const f16* bias;
@@ -17,6 +18,8 @@ struct GemmEpilogue {
   const f16* norm_weight;
   const f16* norm_bias;
   float norm_eps;
+  const int32_t* out_fp8_scale;   // when set: the result is left on the FP8 grid of this exponent (unscaled)
+  int out_fp8_format;
 };
 
 __device__ __forceinline__ f16 sigmoid_f16(f16 x) {
@@ -51,11 +54,19 @@ __device__ __forceinline__ f16 apply_epilogue(const GemmEpilogue& e, f16 y, int 
   if (e.mul) y = y * e.mul[(size_t)m * N + n];
   if (e.residual) y = y + e.residual[(size_t)m * N + n];
   if (e.post_scale != 0.0f) y = y * (f16)e.post_scale;
+  if (e.out_fp8_scale) y = f8_grid_value(y, e.out_fp8_scale[0], e.out_fp8_format);
+  return y;
+}
+
+// the SwiGLU pair's result: up * swish(gate), then the optional cast of the epilogue
+__device__ __forceinline__ f16 swiglu_out(const GemmEpilogue& e, f16 gate, f16 up) {
+  f16 y = up * swish_f16(gate);
+  if (e.out_fp8_scale) y = f8_grid_value(y, e.out_fp8_scale[0], e.out_fp8_format);
   return y;
 }
 
 static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const char* name) {
-  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, nullptr, 0.f, PTA_NORM_NONE, nullptr, nullptr, 0.f};
+  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, nullptr, 0.f, PTA_NORM_NONE, nullptr, nullptr, 0.f, nullptr, PTA_F143};
   if (!in) return PTA_OK;
   PTA_REQUIRE(in->act >= PTA_ACT_NONE && in->act <= PTA_ACT_SIGMOID, "%s: unknown activation %d", name, in->act);
   PTA_REQUIRE(in->norm >= PTA_NORM_NONE && in->norm <= PTA_NORM_LAYER, "%s: unknown norm %d", name, in->norm);
@@ -65,6 +76,9 @@ static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const c
   out->mul = (const f16*)in->mul; out->post_scale = in->post_scale;
   out->norm = in->norm; out->norm_weight = (const f16*)in->norm_weight; out->norm_bias = (const f16*)in->norm_bias;
   out->norm_eps = in->norm_eps;
+  PTA_REQUIRE(!in->out_fp8_scale || in->out_fp8_format == PTA_F143 || in->out_fp8_format == PTA_F152,
+              "%s: unsupported fp8 format %d, it must be F143 or F152", name, in->out_fp8_format);
+  out->out_fp8_scale = in->out_fp8_scale; out->out_fp8_format = in->out_fp8_format;
   return PTA_OK;
 }
 
@@ -205,7 +219,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
     if (PAIR) {
       const f16 gate = (f16)sum[0];
       const f16 up = (f16)sum[1];
-      a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
+      a.mat[0].Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
     } else {
       f16 y0 = (f16)sum[0];
       if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
@@ -369,7 +383,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
     if (PAIR) {
       const f16 gate = (f16)sum[0];
       const f16 up = (f16)sum[1];
-      a.mat[0].Y[(size_t)m * N + n] = up * swish_f16(gate);
+      a.mat[0].Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
     } else {
       f16 y0 = (f16)sum[0];
       if (a.mat[mi].bias) y0 = y0 + a.mat[mi].bias[n];
@@ -621,7 +635,7 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_wide_kernel(GemmArgs a, 
       if (PAIR) {
         const f16 gate = (f16)sum[0];
         const f16 up = (f16)sum[1];
-        mat.Y[(size_t)m * N + n] = up * swish_f16(gate);
+        mat.Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
       } else {
         f16 y0 = (f16)sum[0];
         if (mat.bias) y0 = y0 + mat.bias[n];
@@ -823,7 +837,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     if (PAIR) {
       const f16 gate = (f16)sum[0];
       const f16 up = (f16)sum[1];
-      mat.Y[(size_t)m * N + n] = up * swish_f16(gate);
+      mat.Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
     } else {
       f16 y0 = (f16)sum[0];
       if (mat.bias) y0 = y0 + mat.bias[n];

@@ -56,7 +56,8 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
     a.part_bytes = fuse->workspace_bytes;
   }
   PTA_REQUIRE(count == 1 || (!a.epi.bias && !a.epi.residual && !a.epi.mul && a.epi.post_scale == 0.0f && a.epi.act == PTA_ACT_NONE),
-              "pta_linear: with several weights only the norm fields of `fuse` apply (use host_bias for biases)");
+              "pta_linear: with several weights only the norm fields and the output cast of `fuse` apply (use host_bias for biases)");
+  PTA_REQUIRE(!a.epi.out_fp8_scale || count == 1 || swiglu, "pta_linear: the output cast applies to one weight or to a SwiGLU pair");
   hipStream_t s = (hipStream_t)stream;
   switch (kind) {
     case PTA_W_INT4: return run_linear<FmtW4>(a, nb, swiglu, s, "pta_linear");

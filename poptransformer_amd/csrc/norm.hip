@@ -6,6 +6,7 @@
 // the assembly kernel custom_ops/NormCE.S:243-423 (C form NormCECodelets.cpp:181-211) when
 // there are several.  One workgroup normalises one row in a single pass over registers.
 #include "common.h"
+#include "f8codec.h"
 
 constexpr int NORM_THREADS = 256;
 constexpr int NORM_MAX_VEC = 4;  // 8-element vectors per thread: rows up to 8192 columns
@@ -26,7 +27,8 @@ __device__ __forceinline__ float block_sum(float v, float* sh) {
 template <int MODE>
 __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restrict__ x, const f16* __restrict__ gamma,
                                                             const f16* __restrict__ beta, f16* __restrict__ y,
-                                                            int cols, float eps) {
+                                                            int cols, float eps, const int32_t* __restrict__ grid_scale,
+                                                            int grid_format) {
   __shared__ float sh[NORM_THREADS / 64];
   const size_t base = (size_t)blockIdx.x * cols;
   const int nvec = cols >> 3;
@@ -78,6 +80,11 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restric
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = ((v[i][e] - mean16) * r16) * g[e] + b[e];
       }
+      if (grid_scale) {           // the cast of the FP8 Linear that consumes these rows
+        const int gs = grid_scale[0];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = f8_grid_value(o[e], gs, grid_format);
+      }
       *reinterpret_cast<f16x8*>(y + base + (size_t)c * 8) = o;
     }
   }
@@ -98,8 +105,20 @@ extern "C" int pta_rmsnorm(const pta_half* x, const pta_half* weight, pta_half* 
   int rc = check_norm("pta_rmsnorm", x, weight, y, rows, cols);
   if (rc) return rc;
   hipLaunchKernelGGL(norm_kernel<0>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
-                     (const f16*)weight, (const f16*)nullptr, (f16*)y, cols, eps);
+                     (const f16*)weight, (const f16*)nullptr, (f16*)y, cols, eps, (const int32_t*)nullptr, 0);
   PTA_CHECK_LAUNCH("pta_rmsnorm");
+  return PTA_OK;
+}
+
+extern "C" int pta_rmsnorm_fp8_grid(const pta_half* x, const pta_half* weight, pta_half* y, const int32_t* scale,
+                                    int format, int rows, int cols, float eps, pta_stream_t stream) {
+  int rc = check_norm("pta_rmsnorm_fp8_grid", x, weight, y, rows, cols);
+  if (rc) return rc;
+  PTA_REQUIRE(scale, "pta_rmsnorm_fp8_grid: null scale");
+  PTA_REQUIRE(format == PTA_F143 || format == PTA_F152, "pta_rmsnorm_fp8_grid: unsupported fp8 format %d, it must be F143 or F152", format);
+  hipLaunchKernelGGL(norm_kernel<0>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                     (const f16*)weight, (const f16*)nullptr, (f16*)y, cols, eps, scale, format);
+  PTA_CHECK_LAUNCH("pta_rmsnorm_fp8_grid");
   return PTA_OK;
 }
 
@@ -113,10 +132,10 @@ extern "C" int pta_layer_norm_ce(const pta_half* x, const pta_half* gamma, const
   PTA_REQUIRE(cols < 8192, "pta_layer_norm_ce: the normalised size must be below 8192, got %d", cols);
   if (rows == 1)
     hipLaunchKernelGGL(norm_kernel<1>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
-                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps);
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps, (const int32_t*)nullptr, 0);
   else
     hipLaunchKernelGGL(norm_kernel<2>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
-                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps);
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps, (const int32_t*)nullptr, 0);
   PTA_CHECK_LAUNCH("pta_layer_norm_ce");
   return PTA_OK;
 }

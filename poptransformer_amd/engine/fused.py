@@ -155,6 +155,7 @@ class FusedDecoder:
         # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
         self._fp8_buf = {k: buf(B, k) for k in {d, ffn}}
         self._gate, self._up = buf(B, ffn), buf(B, ffn)
+        self._on_grid = {}      # buffer address -> address of the FP8 exponent whose grid its values are on
         self.persistent = None
 
     def enable_persistent(self):
@@ -200,8 +201,33 @@ class FusedDecoder:
         casts its input to FP8 first: the cast needs the normalised values)."""
         if self.fuse_norm and not any(lw.is_fp8 and lw.act_fp8 for lw in consumers):
             return x, K.Norm(gb[0], gb[1], self.spec.eps)
+        grid = self._common_grid(consumers)
+        if grid is not None and self.spec.norm == "rms":
+            # every consumer casts its input to the same FP8 grid: the norm leaves its rows on it
+            buf = self._fp8_buf[x.shape[1]]
+            K.rmsnorm_fp8_grid(x, gb[0], self.spec.eps, grid[0], grid[1], out=buf)
+            self._on_grid[buf.data_ptr()] = self._grid_id(consumers[0])
+            return buf, None
         self._norm(x, gb, self.h)
         return self.h, None
+
+    @staticmethod
+    def _grid_id(lw):
+        """Identifies the FP8 grid an FP8 Linear casts its input to: format and exponent (by value when the
+        loader recorded it, else by the tensor that holds it)."""
+        key = lw.scale_value if lw.scale_value is not None else ("at", lw.w.scale.data_ptr())
+        return (lw.w.format, key)
+
+    @classmethod
+    def _common_grid(cls, consumers):
+        """(scale tensor, format name) when all `consumers` are FP8 Linears that cast their input to one and
+        the same grid, else None."""
+        if not consumers or not all(lw.is_fp8 and lw.act_fp8 for lw in consumers):
+            return None
+        if len({cls._grid_id(lw) for lw in consumers}) != 1:
+            return None
+        first = consumers[0].w
+        return first.scale, ("F143" if first.format == _lib.F143 else "F152")
 
     def _lhs(self, x, lw, norm):
         """Left-hand side for a Linear: FP8 activations are rounded to the FP8 grid first
@@ -210,22 +236,33 @@ class FusedDecoder:
             return x, None, norm
         if norm is not None:                      # the cast needs the normalised values
             raise NotImplementedError("fused norm is not combined with FP8 activations")
+        if self._on_grid.get(x.data_ptr()) == self._grid_id(lw):
+            return x, lw.w.scale, None            # its producer already left x on this Linear's grid
         buf = self._fp8_buf[x.shape[1]]
-        K.half_to_fp8_grid(x, lw.w.scale, "F143", out=buf)
+        self._on_grid.pop(buf.data_ptr(), None)
+        K.half_to_fp8_grid(x, lw.w.scale, "F143" if lw.w.format == _lib.F143 else "F152", out=buf)
         return buf, lw.w.scale, None
 
     def _linear(self, x, lw, out, residual=None, act=_lib.ACT_NONE, norm=None):
         xin, xs, norm = self._lhs(x, lw, norm)
+        self._on_grid.pop(out.data_ptr(), None)
         K.linear(xin, [lw.w], [out], x_scale=xs, bias=lw.bias, residual=residual, act=act, norm=norm,
                  workspace=getattr(self, "_lin_ws", None))
         return out
 
-    def _linear_group(self, x, lws, outs, norm=None, swiglu=False):
-        """Several Linears on the same input: one launch when they are alike, else one each."""
+    def _linear_group(self, x, lws, outs, norm=None, swiglu=False, consumer=None):
+        """Several Linears on the same input: one launch when they are alike, else one each.  `consumer`: the
+        Linear that takes the SwiGLU result; when it casts its input to FP8 the pair's launch does that cast."""
         keys = {lw.group_key() for lw in lws}
+        for o in outs:
+            self._on_grid.pop(o.data_ptr(), None)
         if len(keys) == 1 and (not swiglu or all(lw.bias is None for lw in lws)):
             xin, xs, norm = self._lhs(x, lws[0], norm)
-            K.linear(xin, [lw.w for lw in lws], outs, biases=[lw.bias for lw in lws], x_scale=xs, swiglu=swiglu, norm=norm)
+            grid = self._common_grid([consumer]) if swiglu and consumer is not None else None
+            K.linear(xin, [lw.w for lw in lws], outs, biases=[lw.bias for lw in lws], x_scale=xs, swiglu=swiglu, norm=norm,
+                     out_grid=grid)
+            if grid is not None:
+                self._on_grid[outs[0].data_ptr()] = self._grid_id(consumer)
             return
         if swiglu:                                 # unlike weights: two launches and the elementwise form
             self._linear(x, lws[0], self._gate, norm=norm)
@@ -255,7 +292,7 @@ class FusedDecoder:
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:
-                self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True)
+                self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True, consumer=blk.mlp_out)
             else:
                 self._linear(h, blk.mlp_in[0], self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)

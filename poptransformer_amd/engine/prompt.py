@@ -47,6 +47,7 @@ class PromptPass(FusedDecoder):
         self.attn_ws = K.decode_attention_workspace(M, s.n_head, s.head_dim, s.max_len, self.dev)
         self.fuse_norm = False
         self.persistent = None
+        self._on_grid = {}
         # scratch for the K split of the projections with few output channels (attention output, MLP down)
         self._lin_ws = K.linear_workspace(M, max(d, ffn), self.dev)
 
@@ -92,7 +93,7 @@ class PromptPass(FusedDecoder):
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:
-                self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True)
+                self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True, consumer=blk.mlp_out)
             else:
                 self._linear(h, blk.mlp_in[0], self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)

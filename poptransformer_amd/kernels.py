@@ -49,13 +49,18 @@ def norm_fusable(M, K):
     return M <= 4 and M * (((K + 127) // 128) * 128 + 8) * 2 <= 40 * 1024
 
 
-def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0, workspace=None):
+def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0, workspace=None,
+            out_grid=None):
+    """out_grid: (device int32 exponent, 'F143' | 'F152') - leave the result on that FP8 grid (half_to_fp8_grid)."""
     if (bias is None and residual is None and act == _lib.ACT_NONE and norm is None and mul is None and not post_scale
-            and workspace is None):
+            and workspace is None and out_grid is None):
         return None
+    if out_grid is not None:
+        _need(out_grid[0], _i32, "fp8_scale")
     e = Fusion(_p(bias), _p(residual), act, _p(mul), float(post_scale), norm.kind if norm else _lib.NORM_NONE,
                _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0,
-               _p(workspace), workspace.numel() * workspace.element_size() if workspace is not None else 0)
+               _p(workspace), workspace.numel() * workspace.element_size() if workspace is not None else 0,
+               _p(out_grid[0]) if out_grid is not None else None, _fmt(out_grid[1]) if out_grid is not None else 0)
     return ctypes.byref(e)
 
 
@@ -264,7 +269,7 @@ def _desc(w, x=None, act=_lib.ACT_NONE):
 
 
 def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None, residual=None, act=_lib.ACT_NONE,
-           norm=None, mul=None, post_scale=0.0, xs=None, acts=None, workspace=None):
+           norm=None, mul=None, post_scale=0.0, xs=None, acts=None, workspace=None, out_grid=None):
     """pta_linear: up to four weights of one kind.  They share x, or each takes its own input from
     `xs`.  `biases` / `acts` are per-weight lists (or None); bias / residual / act / mul / post_scale
     apply to the single-weight form only."""
@@ -284,7 +289,7 @@ def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None,
         if w.K != x.shape[1]:
             raise ValueError(f"matmul: contracting dimensions differ ({x.shape[1]} vs {w.K})")
     check(_lib.load().pta_linear(_p(x), _p(x_scale), n, descs, bs, ys, M, 1 if swiglu else 0,
-                                 _fusion(bias, residual, act, norm, mul, post_scale, workspace), _stream()))
+                                 _fusion(bias, residual, act, norm, mul, post_scale, workspace, out_grid), _stream()))
     return outs
 
 
@@ -306,6 +311,20 @@ def rmsnorm(x, weight, eps, out=None):
     if out is None:
         out = torch.empty_like(x)
     check(_lib.load().pta_rmsnorm(_p(x), _p(weight), _p(out), rows, cols, float(eps), _stream()))
+    return out
+
+
+def rmsnorm_fp8_grid(x, weight, eps, scale, fp8_format="F143", out=None):
+    """half_to_fp8_grid(rmsnorm(x)) in one pass."""
+    _need(x, torch.float16, "x")
+    _need(weight, torch.float16, "weight", 1)
+    _need(scale, _i32, "fp8_scale")
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    if out is None:
+        out = torch.empty_like(x)
+    check(_lib.load().pta_rmsnorm_fp8_grid(_p(x), _p(weight), _p(out), _p(scale), _fmt(fp8_format), rows, cols, float(eps),
+                                           _stream()))
     return out
 
 

@@ -349,6 +349,53 @@ def test_fp8_gemm_both_modes(K, M, Kdim, N, fmt):
     assert torch.equal(fw.tiled, fw2.tiled)
 
 
+@pytest.mark.parametrize("fmt,scale", [("F143", -3), ("F143", 2), ("F152", -1)])
+def test_casts_done_by_the_producer_are_bit_identical(K, fmt, scale):
+    """The cast of an FP8 Linear's input done where that input is produced - inside the RMSNorm pass, and in
+    the epilogue of a Linear or of a SwiGLU pair, for 1, 12 and 40 rows (three GEMM kernels) - gives the bits
+    of the separate pta_half_to_fp8_grid pass."""
+    rng = np.random.default_rng(77)
+    sd = dev(np.array([scale], np.int32))
+    for rows in (1, 12, 40):
+        x = (rng.standard_normal((rows, 1024)) * 3).astype(np.float16)
+        g = rng.uniform(0.5, 1.5, 1024).astype(np.float16)
+        fused = K.rmsnorm_fp8_grid(dev(x), dev(g), 1e-5, sd, fmt)
+        two = K.half_to_fp8_grid(K.rmsnorm(dev(x), dev(g), 1e-5), sd, fmt)
+        assert torch.equal(fused, two)
+        assert np.array_equal(host(two), O.f8_decode(O.f8_encode(O.rms_norm(x, g, 1e-5), fmt, scale), fmt, 0, np.float16))
+        N = 8192
+        (pg, sg), (pu, su) = [(rng.integers(-128, 128, size=(N, 512), dtype=np.int8),
+                               rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)) for _ in range(2)]
+        wg, wu = K.W4Weight(dev(pg), dev(sg)), K.W4Weight(dev(pu), dev(su))
+        res = dev(rng.standard_normal((rows, N)).astype(np.float16))
+        y = torch.empty((rows, N), dtype=torch.float16, device="cuda")
+        y2 = torch.empty_like(y)
+        K.linear(dev(x), [wg], [y], residual=res, out_grid=(sd, fmt))
+        K.linear(dev(x), [wg], [y2], residual=res)
+        assert torch.equal(y, K.half_to_fp8_grid(y2, sd, fmt))
+        K.linear(dev(x), [wg, wu], [y, y], swiglu=True, out_grid=(sd, fmt))
+        K.linear(dev(x), [wg, wu], [y2, y2], swiglu=True)
+        assert torch.equal(y, K.half_to_fp8_grid(y2, sd, fmt))
+    with pytest.raises(ValueError):
+        K.linear(dev(x), [wg, wu], [y, y2], out_grid=(sd, fmt))          # two plain weights: no output cast
+    # every fp16 value through the cast of the norm pass (weight 1: x * r with r = 1 exactly needs rows whose
+    # mean square is 1; instead the cast is reached through a Linear with an identity weight and no rounding)
+    allv = np.arange(65536, dtype=np.uint16).view(np.float16).reshape(64, 1024)
+    eye = np.zeros((16, 1024), np.float16)                              # channel c picks feature c
+    eye[np.arange(16), np.arange(16)] = 1
+    picked = allv.reshape(-1, 16)                                       # 4096 groups of 16 values
+    xs = np.zeros((64, 1024), np.float16)
+    w16 = K.F16Weight(dev(eye))
+    for g0 in range(0, 4096, 64):
+        xs[:, :16] = picked[g0:g0 + 64]
+        with np.errstate(invalid="ignore"):
+            safe = np.where(np.isfinite(xs), xs, 0).astype(np.float16)  # a NaN or inf would spread over the row's sums
+        out = torch.empty((64, 16), dtype=torch.float16, device="cuda")
+        K.linear(dev(safe), [w16], [out], out_grid=(sd, fmt))
+        ref = O.f8_decode(O.f8_encode(safe[:, :16], fmt, scale), fmt, 0, np.float16)
+        assert np.array_equal(host(out).view(np.uint16), ref.view(np.uint16)), f"values of group {g0}"
+
+
 def test_fp8_gemm_many_rows_wide_outputs(K):
     rng = np.random.default_rng(22)
     M, Kdim, N = 48, 1024, 8192
