@@ -112,84 +112,35 @@ class ModelWeights:
         return n
 
 
-class FusedDecoder:
-    def __init__(self, spec: DecoderSpec, weights: ModelWeights, device="cuda"):
-        self.spec, self.w, self.dev = spec, weights, device
-        s = spec
-        B, d = s.batch, s.d_model
-        f16, i32 = torch.float16, torch.int32
+class LayerOps:
+    """The per-layer operators over `rows` activation rows: the row buffers and the calls that the decode
+    iteration (rows = batch) and the prompt passes (rows = batch * positions) share."""
+
+    def __init__(self, spec: DecoderSpec, weights: ModelWeights, device, rows):
+        self.spec, self.w, self.dev, self._rows = spec, weights, device, rows
+        s, f16 = spec, torch.float16
 
         def buf(*shape, dtype=f16):
             return torch.zeros(shape, dtype=dtype, device=device)
 
-        self.x, self.h, self.ctx = buf(B, d), buf(B, d), buf(B, d)
-        qkv_n = sum(lw.N for lw in weights.blocks[0].qkv)
-        self.qkv = buf(B, qkv_n)
-        self.q_rot = buf(B, s.n_head, s.head_dim)
-        ffn = weights.blocks[0].mlp_out.K
-        self.act = buf(B, ffn)
-        self.logits = buf(B, s.vocab)
-        self.next_ids = buf(B, dtype=i32)
-        if s.topk > 1:
-            if s.topk > s.vocab:
-                raise ValueError(f"topk = {s.topk} exceeds the vocabulary size {s.vocab}")
-            self._topk_ids, self._topk_vals = buf(B, s.topk, dtype=i32), buf(B, s.topk)
-            self._draws, self._pick = buf(1, s.topk), buf(1, dtype=i32)
-        self.container = buf(B, s.max_len, dtype=i32)
-        self.mask = buf(B, s.max_len)
-        self.stop_mask = buf(B, dtype=i32)
-        self.step = torch.zeros((), dtype=i32, device=device)
-        self.keep_going = torch.ones((), dtype=i32, device=device)
-        # one ring per layer: keys then values, [2*B*Hkv, max_len, D]
-        self.kv_scale = 1 if s.fp8_cache else None        # the constant of custom_ops/kv_cache.cpp:45
-        self.rings = [buf(2 * B * s.n_kv_head, s.max_len, s.head_dim, dtype=torch.uint8 if s.fp8_cache else f16)
-                      for _ in range(s.n_layer)]
-        self.attn_ws = K.decode_attention_workspace(B, s.n_head, s.head_dim, s.max_len, device)
-        self.graph = None
-        self._stream = torch.cuda.Stream()
+        self._buf = buf
+        d, ffn = s.d_model, weights.blocks[0].mlp_out.K
+        self.x, self.h, self.ctx = buf(rows, d), buf(rows, d), buf(rows, d)
+        self.qkv = buf(rows, sum(lw.N for lw in weights.blocks[0].qkv))
+        self.q_rot = buf(rows, s.n_head, s.head_dim)
+        self.act = buf(rows, ffn)
+        self.attn_ws = K.decode_attention_workspace(rows, s.n_head, s.head_dim, s.max_len, device)
         # Measured on MI355X at d = 4096: the norm inside the GEMM costs every workgroup a pass over X and two
-        # barriers: +5 us per launch at batch <= 4 (the stand-alone norm kernel takes 2.4 us) and +5 us per
+        # barriers: +5 us per launch at batch <= 4 (the stand-alone norm kernel takes 2.4 us) and +4 us per
         # launch at batch 16 as well (stand-alone 4.4 us, but two of the three GEMMs that follow a norm each
-        # pay for it), so it stays separate.  The kernels support it (M <= 16); tests cover it.
+        # pay for it), so it stays separate.  The kernels support it (rows <= 16); tests cover it.
         self.fuse_norm = False
         # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
-        self._fp8_buf = {k: buf(B, k) for k in {d, ffn}}
-        self._gate, self._up = buf(B, ffn), buf(B, ffn)
-        self._on_grid = {}      # buffer address -> address of the FP8 exponent whose grid its values are on
-        self.persistent = None
+        self._fp8_buf = {k: buf(rows, k) for k in {d, ffn}}
+        self._gate, self._up = buf(rows, ffn), buf(rows, ffn)
+        self._on_grid = {}      # buffer address -> the FP8 grid (format, exponent) its values are on
+        self._lin_ws = None     # scratch that lets a many-row Linear with few output channels split K
 
-    def enable_persistent(self):
-        """Run each loop iteration as one persistent launch (pta_llama_decode_step) instead of one
-        launch per operator.  Raises NotImplementedError when the model is not an INT4 Llama-2
-        shape the kernel covers; the per-operator path stays available through `persistent = None`."""
-        s, w = self.spec, self.w
-        if s.topk != 1:
-            raise NotImplementedError("the persistent decode step selects greedily (topk = 1)")
-        if s.fp8_cache:
-            raise NotImplementedError("the persistent decode step keeps its KV cache in fp16")
-        if s.family != "llama2" or s.n_kv_head != s.n_head:
-            raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
-        lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
-        if not all(lw.is_int4 and lw.bias is None for lw in lins):
-            raise NotImplementedError("the persistent decode step needs bias-free INT4 Linears")
-        if not isinstance(w.head.w, K.F16Weight) or w.head.bias is not None:
-            raise NotImplementedError("the persistent decode step needs a bias-free fp16 lm_head")
-        layers = []
-        for b, ring in zip(w.blocks, self.rings):
-            q, k, v = b.qkv
-            g, u = b.mlp_in
-            layers.append(dict(wq=q.w.tiled, wk=k.w.tiled, wv=v.w.tiled, wo=b.out.w.tiled, wg=g.w.tiled, wu=u.w.tiled,
-                               wd=b.mlp_out.w.tiled, sq=q.w.scale, sk=k.w.scale, sv=v.w.scale, so=b.out.w.scale,
-                               sg=g.w.scale, su=u.w.scale, sd=b.mlp_out.w.scale, norm1=b.norm1[0], norm2=b.norm2[0],
-                               kv_ring=ring))
-        state = dict(container=self.container, mask=self.mask, stop_mask=self.stop_mask, step=self.step,
-                     keep_going=self.keep_going, next_ids=self.next_ids, logits=self.logits)
-        self.persistent = K.DecodeStep(layers, w.embed, w.final_norm[0], w.head.w.tiled, w.inv_freq, s.batch, s.d_model,
-                                       s.n_head, s.head_dim, w.blocks[0].mlp_out.K, s.vocab, s.max_len, s.eps, s.pad_id,
-                                       s.eos_id, s.early_stop, state)
-        return self
-
-    # ------------------------------------------------------------------ one loop iteration
     def _norm(self, x, gb, out):
         if self.spec.norm == "rms":
             return K.rmsnorm(x, gb[0], self.spec.eps, out)
@@ -247,7 +198,7 @@ class FusedDecoder:
         xin, xs, norm = self._lhs(x, lw, norm)
         self._on_grid.pop(out.data_ptr(), None)
         K.linear(xin, [lw.w], [out], x_scale=xs, bias=lw.bias, residual=residual, act=act, norm=norm,
-                 workspace=getattr(self, "_lin_ws", None))
+                 workspace=self._lin_ws)
         return out
 
     def _linear_group(self, x, lws, outs, norm=None, swiglu=False, consumer=None):
@@ -271,6 +222,82 @@ class FusedDecoder:
             return
         for lw, o in zip(lws, outs):
             self._linear(x, lw, o, norm=norm)
+
+    def _prepare_qkv_views(self, blk):
+        """Output buffers of the projections and the (pointer, row stride) views of q, k, v."""
+        s = self.spec
+        B, Hq, Hkv, D = self._rows, s.n_head, s.n_kv_head, s.head_dim
+        f16 = torch.float16
+        if len(blk.qkv) == 1:           # GPT-2: one row holds q | k | v
+            row = (Hq + 2 * Hkv) * D
+            self._qkv_bufs = [self.qkv]
+            self._qkv_views = (self.qkv, self.qkv[:, Hq * D:], self.qkv[:, (Hq + Hkv) * D:], row, row, row)
+        elif len(blk.qkv) == 3:         # Llama 2: separate q, k, v
+            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
+            q, k, v = self._qkv_bufs
+            self._qkv_views = (q, k, v, Hq * D, Hkv * D, Hkv * D)
+        else:                           # ChatGLM2: query, and key_value holding k | v
+            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
+            q, kv = self._qkv_bufs
+            self._qkv_views = (q, kv, kv[:, Hkv * D:], Hq * D, 2 * Hkv * D, 2 * Hkv * D)
+
+
+class FusedDecoder(LayerOps):
+    def __init__(self, spec: DecoderSpec, weights: ModelWeights, device="cuda"):
+        super().__init__(spec, weights, device, spec.batch)
+        s, buf = spec, self._buf
+        B = s.batch
+        i32 = torch.int32
+        self.logits = buf(B, s.vocab)
+        self.next_ids = buf(B, dtype=i32)
+        if s.topk > 1:
+            if s.topk > s.vocab:
+                raise ValueError(f"topk = {s.topk} exceeds the vocabulary size {s.vocab}")
+            self._topk_ids, self._topk_vals = buf(B, s.topk, dtype=i32), buf(B, s.topk)
+            self._draws, self._pick = buf(1, s.topk), buf(1, dtype=i32)
+        self.container = buf(B, s.max_len, dtype=i32)
+        self.mask = buf(B, s.max_len)
+        self.stop_mask = buf(B, dtype=i32)
+        self.step = torch.zeros((), dtype=i32, device=device)
+        self.keep_going = torch.ones((), dtype=i32, device=device)
+        # one ring per layer: keys then values, [2*B*Hkv, max_len, D]
+        self.kv_scale = 1 if s.fp8_cache else None        # the constant of custom_ops/kv_cache.cpp:45
+        self.rings = [buf(2 * B * s.n_kv_head, s.max_len, s.head_dim, dtype=torch.uint8 if s.fp8_cache else torch.float16)
+                      for _ in range(s.n_layer)]
+        self.graph = None
+        self._stream = torch.cuda.Stream()
+        self.persistent = None
+
+    def enable_persistent(self):
+        """Run each loop iteration as one persistent launch (pta_llama_decode_step) instead of one
+        launch per operator.  Raises NotImplementedError when the model is not an INT4 Llama-2
+        shape the kernel covers; the per-operator path stays available through `persistent = None`."""
+        s, w = self.spec, self.w
+        if s.topk != 1:
+            raise NotImplementedError("the persistent decode step selects greedily (topk = 1)")
+        if s.fp8_cache:
+            raise NotImplementedError("the persistent decode step keeps its KV cache in fp16")
+        if s.family != "llama2" or s.n_kv_head != s.n_head:
+            raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
+        lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
+        if not all(lw.is_int4 and lw.bias is None for lw in lins):
+            raise NotImplementedError("the persistent decode step needs bias-free INT4 Linears")
+        if not isinstance(w.head.w, K.F16Weight) or w.head.bias is not None:
+            raise NotImplementedError("the persistent decode step needs a bias-free fp16 lm_head")
+        layers = []
+        for b, ring in zip(w.blocks, self.rings):
+            q, k, v = b.qkv
+            g, u = b.mlp_in
+            layers.append(dict(wq=q.w.tiled, wk=k.w.tiled, wv=v.w.tiled, wo=b.out.w.tiled, wg=g.w.tiled, wu=u.w.tiled,
+                               wd=b.mlp_out.w.tiled, sq=q.w.scale, sk=k.w.scale, sv=v.w.scale, so=b.out.w.scale,
+                               sg=g.w.scale, su=u.w.scale, sd=b.mlp_out.w.scale, norm1=b.norm1[0], norm2=b.norm2[0],
+                               kv_ring=ring))
+        state = dict(container=self.container, mask=self.mask, stop_mask=self.stop_mask, step=self.step,
+                     keep_going=self.keep_going, next_ids=self.next_ids, logits=self.logits)
+        self.persistent = K.DecodeStep(layers, w.embed, w.final_norm[0], w.head.w.tiled, w.inv_freq, s.batch, s.d_model,
+                                       s.n_head, s.head_dim, w.blocks[0].mlp_out.K, s.vocab, s.max_len, s.eps, s.pad_id,
+                                       s.eos_id, s.early_stop, state)
+        return self
 
     def step_fn(self):
         if self.persistent is not None:
@@ -309,24 +336,6 @@ class FusedDecoder:
             K.take_column(self._topk_ids, self._pick, self.next_ids)
         K.step_update(self.container, self.mask, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
                       s.pad_id, s.eos_id, s.early_stop)
-
-    def _prepare_qkv_views(self, blk):
-        """Output buffers of the projections and the (pointer, row stride) views of q, k, v."""
-        s = self.spec
-        B, Hq, Hkv, D = getattr(self, "_rows", s.batch), s.n_head, s.n_kv_head, s.head_dim
-        f16 = torch.float16
-        if len(blk.qkv) == 1:           # GPT-2: one row holds q | k | v
-            row = (Hq + 2 * Hkv) * D
-            self._qkv_bufs = [self.qkv]
-            self._qkv_views = (self.qkv, self.qkv[:, Hq * D:], self.qkv[:, (Hq + Hkv) * D:], row, row, row)
-        elif len(blk.qkv) == 3:         # Llama 2: separate q, k, v
-            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
-            q, k, v = self._qkv_bufs
-            self._qkv_views = (q, k, v, Hq * D, Hkv * D, Hkv * D)
-        else:                           # ChatGLM2: query, and key_value holding k | v
-            self._qkv_bufs = [torch.zeros((B, lw.N), dtype=f16, device=self.dev) for lw in blk.qkv]
-            q, kv = self._qkv_bufs
-            self._qkv_views = (q, kv, kv[:, Hkv * D:], Hq * D, 2 * Hkv * D, 2 * Hkv * D)
 
     # ------------------------------------------------------------------ loop
     def reset(self, input_ids):

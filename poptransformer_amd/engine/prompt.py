@@ -17,39 +17,21 @@ import torch
 
 from .. import _lib
 from .. import kernels as K
-from .fused import FusedDecoder
+from .fused import LayerOps
 
 
-class PromptPass(FusedDecoder):
-    """Buffers for B*rows rows and one pass over the layers; shares weights and KV rings with `dec`."""
+class PromptPass(LayerOps):
+    """Buffers for B*rows rows and one pass over the layers; shares weights and KV rings with the decoder `dec`."""
 
     def __init__(self, dec, rows):
-        # deliberately not FusedDecoder.__init__: only the row buffers its helper methods use
-        self.spec, self.w, self.dev, self.dec = dec.spec, dec.w, dec.dev, dec
-        s, w = self.spec, self.w
-        self.rows = int(rows)
-        M = self._rows = s.batch * self.rows
-        f16, i32 = torch.float16, torch.int32
-
-        def buf(*shape, dtype=f16):
-            return torch.zeros(shape, dtype=dtype, device=self.dev)
-
-        d, ffn = s.d_model, w.blocks[0].mlp_out.K
-        self.x, self.h, self.ctx = buf(M, d), buf(M, d), buf(M, d)
-        self.qkv = buf(M, sum(lw.N for lw in w.blocks[0].qkv))
-        self.q_rot = buf(M, s.n_head, s.head_dim)
-        self.act = buf(M, ffn)
-        self._fp8_buf = {k: buf(M, k) for k in {d, ffn}}
-        self._gate, self._up = buf(M, ffn), buf(M, ffn)
+        super().__init__(dec.spec, dec.w, dec.dev, dec.spec.batch * int(rows))
+        self.dec, self.rows = dec, int(rows)
+        s, i32 = self.spec, torch.int32
         self.first = torch.zeros((), dtype=i32, device=self.dev)       # position of row 0 of every sequence
         self._offsets = torch.arange(self.rows, dtype=i32, device=self.dev)
         self.graph = None
-        self.attn_ws = K.decode_attention_workspace(M, s.n_head, s.head_dim, s.max_len, self.dev)
-        self.fuse_norm = False
-        self.persistent = None
-        self._on_grid = {}
         # scratch for the K split of the projections with few output channels (attention output, MLP down)
-        self._lin_ws = K.linear_workspace(M, max(d, ffn), self.dev)
+        self._lin_ws = K.linear_workspace(self._rows, max(s.d_model, self.w.blocks[0].mlp_out.K), self.dev)
 
     def run(self, p0):
         """Positions p0 .. p0+rows-1 of every sequence (row b*rows + r is sequence b at p0 + r).  The pass
