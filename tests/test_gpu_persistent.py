@@ -63,6 +63,26 @@ def test_persistent_step_follows_the_per_operator_path(B):
     assert not dec.persistent.failed()
 
 
+def test_prompt_in_passes_then_persistent_steps():
+    """The prompt taken in passes (one launch per operator, several positions at once), then the loop as
+    persistent launches replayed from a graph: container and step equal the oracle's loop."""
+    B, L, steps, pad, eos = 2, 64, 48, 0, 2
+    print("case: prompt passes, then persistent steps", flush=True)
+    sd, _, dec = _decoders(B, L, pad, eos, seed=1)
+    ids = _prompt(np.random.default_rng(13), B, L, 21, LLAMA_TINY["vocab_size"], pad)
+    ids[ids == eos] = eos + 1                # no end token inside the prompt: the passes take all of it
+    ref_container, ref_step = OM.run_decode_loop(OM.Llama2Oracle(sd, LLAMA_TINY, L, B), ids, L, steps, pad, eos)
+    dec.capture()
+    for _ in range(2):                       # the second generation replays the passes' graph as well
+        dec.reset(ids)
+        n = dec.consume_prompt(rows_per_pass=8)
+        assert n == 20
+        dec.run_steps(steps - n)
+        torch.cuda.synchronize()
+        assert not dec.persistent.failed()
+        assert np.array_equal(dec.container.cpu().numpy(), ref_container) and int(dec.step.item()) == ref_step
+
+
 def test_persistent_step_graph_replay_equals_eager():
     B, L, pad, eos = 2, 64, 0, 2
     print("case: persistent step, graph replay vs eager", flush=True)
