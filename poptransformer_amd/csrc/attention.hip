@@ -348,6 +348,10 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       L = __builtin_fmaf(sm_l[i], w, L);
       A = __builtin_fmaf(sm_acc[i][d], w, A);
     }
+    if (a.nsplit == 1) {                     // the only split of this (row, head): the context vector itself
+      a.out[(size_t)bh * D + d] = (f16)((KV8 ? A * kv_mul : A) / L);
+      continue;
+    }
     out[2 + d] = KV8 ? A * kv_mul : A;
     if (d == 0) { out[0] = M; out[1] = L; }
   }
@@ -374,9 +378,11 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
 }
 
 // splits per (sequence, head): about 1024 workgroups in all, never more than one per 64 cache rows
-// (which is what the workspace is sized for)
+// (which is what the workspace is sized for); from 512 (sequence, head) pairs on, one workgroup each, which
+// writes the context vector itself and saves the merging launch
 static int attn_splits(int B, int Hq, int max_len) {
   const int cap = (max_len + 63) / 64;
+  if (B * Hq >= 512) return 1;
   int n = (1024 + B * Hq - 1) / (B * Hq);
   n = n < 1 ? 1 : n;
   return n > cap ? cap : n;
@@ -395,11 +401,11 @@ static void launch_attention(const AttnArgs& a, int D, bool kv8, int heads_rows,
   if (D == 128) {
     if (kv8) hipLaunchKernelGGL((attn_partial_kernel<128, FUSED, true>), grid, dim3(ATT_THREADS), 0, s, a);
     else hipLaunchKernelGGL((attn_partial_kernel<128, FUSED, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(heads_rows), dim3(128), 0, s, a);
+    if (a.nsplit > 1) hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(heads_rows), dim3(128), 0, s, a);
   } else {
     if (kv8) hipLaunchKernelGGL((attn_partial_kernel<64, FUSED, true>), grid, dim3(ATT_THREADS), 0, s, a);
     else hipLaunchKernelGGL((attn_partial_kernel<64, FUSED, false>), grid, dim3(ATT_THREADS), 0, s, a);
-    hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(heads_rows), dim3(64), 0, s, a);
+    if (a.nsplit > 1) hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(heads_rows), dim3(64), 0, s, a);
   }
 }
 
