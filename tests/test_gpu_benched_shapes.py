@@ -1,0 +1,206 @@
+"""Parity at the shapes the benchmark runs, so that every kernel instantiation a profile names is one a test has
+compared with the oracle: the Llama2-7B width (hidden 4096, 32 heads x 128, ffn 11008, vocabulary 32000) with two
+layers through the persistent decode step at batch 1 and 4 and through the per-operator path at batch 16, the single
+INT4 operator X[M,4096] . W[4096,11008] for M in {1, 4, 16, 64}, and launches of 5..16 rows over 688 channel
+blocks (a count that is no multiple of the three blocks a workgroup takes)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import models as OM
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+LLAMA_7B_WIDTH = dict(vocab_size=32000, hidden_size=4096, rms_norm_eps=1e-5, num_attention_heads=32,
+                      intermediate_size=11008, num_hidden_layers=2)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rel_err(got, ref):
+    return np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() / np.abs(ref.astype(np.float64)).max()
+
+
+class _Linear32:
+    """O.matmul with the fp16 -> fp32 conversion of the weight done once instead of per call (the conversion is
+    exact, the product and its rounding are O.matmul's): the oracle takes 0.2 s per token instead of 1 s."""
+
+    def __init__(self, lin):
+        assert lin.b is None and lin.w.dtype == np.float16
+        self.w32 = lin.w.astype(np.float32)
+
+    def __call__(self, x):
+        assert x.dtype == np.float16
+        return np.matmul(x.astype(np.float32), self.w32).astype(np.float16)
+
+
+def _fast(oracle):
+    for lay in oracle.layers:
+        for k in ("q", "k", "v", "o", "gate", "up", "down"):
+            lay[k] = _Linear32(lay[k])
+    oracle.head = _Linear32(oracle.head)
+    return oracle
+
+
+@pytest.fixture(scope="module")
+def wide():
+    """(state dict, oracle with its Linears prepared); the tests take copies of the oracle with caches of their own."""
+    sd = OM.make_llama2_state_dict(LLAMA_7B_WIDTH, seed=21, int4=True)
+    # the conversion check of _Linear32 against O.matmul itself, once, on the real weights
+    lin = OM._Linear(sd, "model.layers.0.self_attn.q_proj", False)
+    x = np.random.default_rng(0).standard_normal((3, 4096)).astype(np.float16)
+    assert np.array_equal(_Linear32(lin)(x), O.matmul(x, lin.w))
+    return sd, _fast(OM.Llama2Oracle(sd, LLAMA_7B_WIDTH, 8, 1))
+
+
+def _oracle(template, L, B):
+    o = copy.copy(template)
+    o.L, o.B = L, B
+    o.layers = [dict(lay, cache=O.KVCache(L, 3, 1)) for lay in template.layers]
+    return o
+
+
+def _prompt(rng, B, L, n, vocab, pad):
+    ids = np.full((B, L), pad, np.int32)
+    ids[:, :n] = rng.integers(3, vocab, size=(B, n))
+    return ids
+
+
+def _follow(dec, oracle, ids, L, steps, pad, eos, tol=1e-2):
+    """Runs `steps` loop iterations on both sides.  Every iteration: fp16 logits within `tol` (max relative
+    error), the selected ids equal wherever the oracle's two best logits are further apart than 0.3 % of the
+    largest logit.  At a nearer tie either candidate is a correct greedy choice; when the decoder took the other
+    one its container entry is set to the oracle's, so that the two generations stay comparable.  Returns the
+    number of such ties."""
+    trace = []
+    ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos, trace=trace)
+    dec.reset(ids)
+    worst, ties = 0.0, 0
+    for it in range(steps):
+        dec.step_fn()
+        torch.cuda.synchronize()
+        ref_ids, ref_logits = trace[it]
+        got = dec.logits.cpu().numpy().astype(np.float64)
+        ref = ref_logits.astype(np.float64)
+        worst = max(worst, np.abs(got - ref).max() / np.abs(ref).max())
+        got_ids = dec.next_ids.cpu().numpy()
+        top2 = np.sort(ref, axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 3e-3 * np.abs(ref).max()
+        assert np.array_equal(got_ids[clear], ref_ids[clear]), f"token ids differ at step {it} without a near tie"
+        for b in np.nonzero(got_ids != ref_ids)[0]:
+            ties += 1
+            order = np.argsort(ref[b])
+            assert got_ids[b] in order[-2:], f"step {it}: the decoder's token is not one of the two tied candidates"
+            if it + 1 < L and ids[b, it + 1] == pad:
+                dec.container[b, it + 1] = int(ref_ids[b])
+    assert worst <= tol, f"logits max rel err {worst}"
+    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+    assert int(dec.step.item()) == ref_step
+    return ties
+
+
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("B,plen", [(1, 136), (4, 136)])
+def test_persistent_step_at_7b_width_matches_oracle(wide, B, plen):
+    """decode_step_kernel<2,6,3,1> (batch 1) and <2,6,3,4> (batch 4): the prompt is taken token by token by the
+    kernel itself, then 32 tokens are generated; by then three (batch 1) or two (batch 4) attention splits of
+    every head hold rows, so the merge of split partials is part of what is compared."""
+    from poptransformer_amd.engine import fused, loader
+    L, pad, eos = 176, 0, 2
+    steps = plen - 1 + 32
+    print(f"case: persistent step at the 7B width, batch {B}, {steps} iterations", flush=True)
+    sd, template = wide
+    oracle = _oracle(template, L, B)
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_7B_WIDTH, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_7B_WIDTH))
+    dec.enable_persistent()
+    ids = _prompt(np.random.default_rng(31 + B), B, L, plen, LLAMA_7B_WIDTH["vocab_size"], pad)
+    ties = _follow(dec, oracle, ids, L, steps, pad, eos)
+    assert not dec.persistent.failed()
+    assert ties <= 8, "near ties should be rare"
+
+
+@pytest.mark.timeout(600)
+def test_per_operator_path_at_7b_width_batch_16_matches_oracle(wide):
+    """Batch 16 on the per-operator path: gemv_wide_kernel with three channel blocks per workgroup (q/k/v in one
+    launch, gate/up + SwiGLU, and the lm_head), one attention workgroup per (sequence, head)."""
+    from poptransformer_amd.engine import fused, loader
+    B, L, pad, eos, plen = 16, 48, 0, 2, 8
+    steps = plen - 1 + 32
+    print("case: per-operator path at the 7B width, batch 16", flush=True)
+    sd, template = wide
+    oracle = _oracle(template, L, B)
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_7B_WIDTH, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_7B_WIDTH))
+    ids = _prompt(np.random.default_rng(77), B, L, plen, LLAMA_7B_WIDTH["vocab_size"], pad)
+    ties = _follow(dec, oracle, ids, L, steps, pad, eos)
+    assert ties <= 40
+
+
+# ---------------------------------------------------------------- the single INT4 operator at its own shape
+def _w4_case(seed, M, Kdim, N):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    packed = rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8)
+    scale = rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)
+    return x, packed, scale
+
+
+@pytest.fixture(scope="module")
+def c2():
+    """X[M,4096] . W[4096,11008]: packed nibbles uniform, scale U(0.005, 0.02), the float64 product of the
+    unpacked matrix kept for the accuracy bound."""
+    _, packed, scale = _w4_case(4096 + 11008, 1, 4096, 11008)
+    w16 = O.int4_to_half(packed, scale, 1)
+    return packed, scale, w16
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 64])
+def test_w4a16_gemm_at_the_single_operator_shape(c2, M):
+    from poptransformer_amd import kernels as K
+    packed, scale, w16 = c2
+    x = np.random.default_rng(100 + M).standard_normal((M, 4096)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    got = host(K.w4a16_gemm(dev(x), w))
+    ref = O.matmul(x, w16)
+    assert got.shape == (M, 11008)
+    assert rel_err(got, ref) <= 1e-2
+    ref64 = x.astype(np.float64) @ w16.astype(np.float64)
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
+
+
+@pytest.mark.parametrize("M", [5, 12, 16])
+def test_w4a16_5_to_16_rows_over_688_channel_blocks(c2, M):
+    """5..16 rows and more channel blocks than twice the compute units: a workgroup takes three blocks, and 688
+    is no multiple of three, so the last workgroup's spare block is a clamped duplicate.  Plain launch with bias
+    and residual, three matrices in one launch, and the SwiGLU pair."""
+    from poptransformer_amd import kernels as K
+    packed, scale, w16 = c2
+    N, Kdim = 11008, 4096
+    rng = np.random.default_rng(200 + M)
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    y = O.matmul(x, w16)
+    got = host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res)))
+    assert rel_err(got, ((y + bias).astype(np.float16) + res).astype(np.float16)) <= 1e-2
+    # a second and third matrix of other widths in the same launch (q | k | v of the decode step are one launch)
+    _, p2, s2 = _w4_case(300 + M, 1, Kdim, 4096)
+    _, p3, s3 = _w4_case(400 + M, 1, Kdim, 2064)               # 129 blocks
+    outs = K.w4a16_gemm_multi(dev(x), [w, K.W4Weight(dev(p2), dev(s2)), K.W4Weight(dev(p3), dev(s3))])
+    assert rel_err(host(outs[0]), y) <= 1e-2
+    assert rel_err(host(outs[1]), O.w4a16_matmul(x, p2, s2)) <= 1e-2
+    assert rel_err(host(outs[2]), O.w4a16_matmul(x, p3, s3)) <= 1e-2
+    _, pu, su = _w4_case(500 + M, 1, Kdim, N)
+    got = host(K.w4a16_gemm_swiglu(dev(x), w, K.W4Weight(dev(pu), dev(su))))
+    ref = (O.w4a16_matmul(x, pu, su) * O.swish(y)).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
