@@ -13,7 +13,9 @@ tables, closed forms, brute force on tiny inputs and library routines (see ``tes
 Functions whose exact numerics live in a third-party dependency of the reference that is not
 part of its tree are PARITY UNPINNED; they implement the documented format and say so:
   * ``f8_encode`` / ``f8_decode``  (poprt 1.1.0 ``convert_float_to_uint8``; Poplar SDK 3.2
-    ``popops::cast`` to QUARTER)
+    ``popops::cast`` to QUARTER).  Inside each format's range they are checked against torch's
+    fnuz casts; that values beyond the range saturate at the largest finite code is an
+    assumption that nothing checks
   * ``gelu`` (PopART ``aiGraphcore.gelu``), ``swish`` (``aiGraphcore.swish``)
   * accumulation order of every MatMul (poplin), tie-breaking of ``popnn::topK``
 """

@@ -1,7 +1,9 @@
 #!/usr/bin/env python3
 """Writes the fixtures of this directory from sources that are independent of the oracle and of the kernels:
 torch's float8 fnuz casts, scipy, torch.nn.functional and Hugging Face model classes built from local
-configs (nothing is downloaded).  The reference repository holds no test vectors of its own; these stand in
+configs (nothing is downloaded).  The FP8 fixtures hold values inside each format's range only: what the
+Graphcore cast does beyond it (taken here to saturate at the largest finite value, where torch's fnuz cast
+gives NaN) is an assumption that no fixture pins.  The reference repository holds no test vectors of its own; these stand in
 for them.  Run from the repository root: `python tests/golden/make_vectors.py`.
 
 Model weights are not stored: `seeded_state_dict` regenerates them from a numpy seed, in the key order of
@@ -9,6 +11,7 @@ the Hugging Face state dict, and the script loads exactly those values into the 
 it computes the expected logits.
 """
 import os
+import sys
 
 import numpy as np
 import torch
@@ -45,7 +48,81 @@ def llama_shapes(cfg):
     return shapes
 
 
+GLM_GOLDEN = dict(padded_vocab_size=256, hidden_size=256, layernorm_epsilon=1e-5, multi_query_group_num=2,
+                  num_attention_heads=4, ffn_hidden_size=352, num_layers=2, kv_channels=64)
+
+
+def chatglm2_shapes(cfg):
+    """Keys and shapes of a ChatGLM2 checkpoint as the reference holds it after the split of `query_key_value`
+    into `query` / `key_value` and of `dense_h_to_4h` into `_1` (gate) / `_2` (up)
+    (poptransformer/models/chatglm2/model.py:256-274)."""
+    d, f, v = cfg["hidden_size"], cfg["ffn_hidden_size"], cfg["padded_vocab_size"]
+    kv = 2 * cfg["multi_query_group_num"] * cfg["kv_channels"]
+    shapes = [("transformer.embedding.word_embeddings.weight", (v, d))]
+    for i in range(cfg["num_layers"]):
+        p = f"transformer.encoder.layers.{i}."
+        shapes += [(p + "input_layernorm.weight", (d,)), (p + "self_attention.query.weight", (d, d)),
+                   (p + "self_attention.query.bias", (d,)), (p + "self_attention.key_value.weight", (kv, d)),
+                   (p + "self_attention.key_value.bias", (kv,)), (p + "self_attention.dense.weight", (d, d)),
+                   (p + "post_attention_layernorm.weight", (d,)), (p + "mlp.dense_h_to_4h_1.weight", (f, d)),
+                   (p + "mlp.dense_h_to_4h_2.weight", (f, d)), (p + "mlp.dense_4h_to_h.weight", (d, f))]
+    shapes += [("transformer.encoder.final_layernorm.weight", (d,)), ("transformer.output_layer.weight", (v, d))]
+    return shapes
+
+
+def glm_hf_state_dict(sd, cfg):
+    """The ChatGLM2 checkpoint `sd` under the parameter names of Hugging Face's GlmForCausalLM, the same block
+    (RMSNorm, q/k/v with bias over grouped KV heads, rotary embedding on interleaved pairs of the first half of
+    each head, fused gate | up SwiGLU): `key_value` rows are k then v, `gate_up_proj` rows are gate then up."""
+    half = cfg["multi_query_group_num"] * cfg["kv_channels"]
+    out = {"model.embed_tokens.weight": sd["transformer.embedding.word_embeddings.weight"],
+           "model.norm.weight": sd["transformer.encoder.final_layernorm.weight"],
+           "lm_head.weight": sd["transformer.output_layer.weight"]}
+    for i in range(cfg["num_layers"]):
+        p, h = f"transformer.encoder.layers.{i}.", f"model.layers.{i}."
+        out[h + "input_layernorm.weight"] = sd[p + "input_layernorm.weight"]
+        out[h + "post_attention_layernorm.weight"] = sd[p + "post_attention_layernorm.weight"]
+        out[h + "self_attn.q_proj.weight"] = sd[p + "self_attention.query.weight"]
+        out[h + "self_attn.q_proj.bias"] = sd[p + "self_attention.query.bias"]
+        out[h + "self_attn.k_proj.weight"] = sd[p + "self_attention.key_value.weight"][:half]
+        out[h + "self_attn.k_proj.bias"] = sd[p + "self_attention.key_value.bias"][:half]
+        out[h + "self_attn.v_proj.weight"] = sd[p + "self_attention.key_value.weight"][half:]
+        out[h + "self_attn.v_proj.bias"] = sd[p + "self_attention.key_value.bias"][half:]
+        out[h + "self_attn.o_proj.weight"] = sd[p + "self_attention.dense.weight"]
+        out[h + "mlp.gate_up_proj.weight"] = np.concatenate([sd[p + "mlp.dense_h_to_4h_1.weight"],
+                                                             sd[p + "mlp.dense_h_to_4h_2.weight"]], axis=0)
+        out[h + "mlp.down_proj.weight"] = sd[p + "mlp.dense_4h_to_h.weight"]
+    return out
+
+
+def glm_logits():
+    """ChatGLM2 block pinned end to end: Hugging Face GlmForCausalLM (built from a local config, nothing is
+    downloaded) holding the seeded fp16 weights in fp32, logits of every position of two sequences."""
+    from transformers import GlmConfig, GlmForCausalLM
+    cfg = GLM_GOLDEN
+    hf = GlmForCausalLM(GlmConfig(
+        vocab_size=cfg["padded_vocab_size"], hidden_size=cfg["hidden_size"], intermediate_size=cfg["ffn_hidden_size"],
+        num_hidden_layers=cfg["num_layers"], num_attention_heads=cfg["num_attention_heads"],
+        num_key_value_heads=cfg["multi_query_group_num"], head_dim=cfg["kv_channels"], hidden_act="silu",
+        rms_norm_eps=cfg["layernorm_epsilon"], max_position_embeddings=64, tie_word_embeddings=False,
+        rope_parameters={"rope_type": "default", "rope_theta": 10000.0, "partial_rotary_factor": 0.5},
+        attention_bias=True, pad_token_id=0)).eval()
+    sd = seeded_state_dict(chatglm2_shapes(cfg), seed=2025)
+    mapped = glm_hf_state_dict(sd, cfg)
+    missing = hf.load_state_dict({k: torch.from_numpy(np.ascontiguousarray(v).astype(np.float32)) for k, v in mapped.items()},
+                                 strict=False)
+    assert not missing.unexpected_keys and all("rotary" in k for k in missing.missing_keys), missing
+    toks = np.random.default_rng(6).integers(1, cfg["padded_vocab_size"], size=(2, 24)).astype(np.int32)
+    with torch.no_grad():
+        logits = hf(torch.from_numpy(toks.astype(np.int64))).logits.numpy()
+    np.savez_compressed(os.path.join(HERE, "glm_hf.npz"), tokens=toks, logits=logits.astype(np.float32), seed=np.int64(2025))
+
+
 def main():
+    if len(sys.argv) > 1 and sys.argv[1] == "glm":      # only the fixture added last; the others stay byte-identical
+        glm_logits()
+        print("glm_hf.npz", os.path.getsize(os.path.join(HERE, "glm_hf.npz")))
+        return
     # FP8: the fnuz formats of torch (e4m3fnuz = 1-4-3 bias 8, e5m2fnuz = 1-5-2 bias 16, NaN 0x80)
     codes = torch.arange(256, dtype=torch.uint8)
     rng = np.random.default_rng(12)
@@ -108,6 +185,7 @@ def main():
     with torch.no_grad():
         logits = hf(torch.from_numpy(toks.astype(np.int64))).logits.numpy()
     np.savez_compressed(os.path.join(HERE, "llama_hf.npz"), tokens=toks, logits=logits.astype(np.float32), seed=np.int64(2024))
+    glm_logits()
     for f in sorted(os.listdir(HERE)):
         print(f, os.path.getsize(os.path.join(HERE, f)))
 

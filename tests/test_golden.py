@@ -8,7 +8,7 @@ import pytest
 
 from oracle import models as OM
 from oracle import ops as O
-from tests.golden.make_vectors import LLAMA_GOLDEN, llama_shapes, seeded_state_dict
+from tests.golden.make_vectors import GLM_GOLDEN, LLAMA_GOLDEN, chatglm2_shapes, llama_shapes, seeded_state_dict
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 f16, f32 = np.float16, np.float32
@@ -67,6 +67,22 @@ def test_oracle_llama_logits():
         assert rel(logits, g["logits"][:, step]) < 2e-2, f"step {step}"
 
 
+def test_oracle_chatglm2_logits():
+    """ChatGLM2Oracle end to end (fp16) against Hugging Face's GlmForCausalLM - the same block: RMSNorm, q/k/v
+    with bias over two KV heads, rotary embedding on interleaved pairs of the first half of each head, fused
+    gate | up SwiGLU - holding the same seeded weights, position by position."""
+    g = load("glm_hf.npz")
+    sd = seeded_state_dict(chatglm2_shapes(GLM_GOLDEN), int(g["seed"]))
+    toks = g["tokens"]
+    B, L = toks.shape
+    model = OM.ChatGLM2Oracle(sd, GLM_GOLDEN, L, B, "fp16")
+    mask = np.full((B, L), -10000, f16)
+    for step in range(L):
+        mask[:, step] = 0
+        _, logits = model.step(toks[:, step].reshape(B, 1), step, mask)
+        assert rel(logits, g["logits"][:, step]) < 2e-2, f"step {step}"
+
+
 # ------------------------------------------------------------------ kernels against the fixtures (GPU)
 @pytest.mark.gpu
 @pytest.mark.parametrize("fmt", ["F143", "F152"])
@@ -117,6 +133,27 @@ def test_kernel_llama_logits_against_hugging_face():
     toks = g["tokens"]
     B, L = toks.shape
     dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_GOLDEN, L + 1, B, pad_id=0, eos_id=-1), loader.llama2_weights(sd, LLAMA_GOLDEN))
+    ids = np.zeros((B, L + 1), np.int32)
+    ids[:, :L] = toks
+    dec.reset(ids)
+    for step in range(L):
+        dec.step_fn()
+        torch.cuda.synchronize()
+        assert rel(dec.logits.cpu().numpy(), g["logits"][:, step]) < 2e-2, f"step {step}"
+
+
+@pytest.mark.gpu
+def test_kernel_chatglm2_logits_against_hugging_face():
+    """The ChatGLM2 decoder on the GPU (fp16 weights, one launch per operator) against the logits of Hugging
+    Face's GlmForCausalLM for the same weights and tokens, position by position."""
+    import torch
+    from poptransformer_amd.engine import fused, loader
+    g = load("glm_hf.npz")
+    sd = seeded_state_dict(chatglm2_shapes(GLM_GOLDEN), int(g["seed"]))
+    toks = g["tokens"]
+    B, L = toks.shape
+    dec = fused.FusedDecoder(loader.chatglm2_spec(GLM_GOLDEN, L + 1, B, pad_id=0, eos_id=-1),
+                             loader.chatglm2_weights(sd, GLM_GOLDEN, "fp16"))
     ids = np.zeros((B, L + 1), np.int32)
     ids[:, :L] = toks
     dec.reset(ids)

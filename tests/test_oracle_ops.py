@@ -376,10 +376,11 @@ def test_f8_encode_matches_fnuz_cast_and_roundtrips(fmt, tdt):
     got = O.f8_encode(x, fmt, 0)
     ref = torch.from_numpy(x.astype(f32)).to(tdt).view(torch.uint8).numpy()
     assert np.array_equal(got, ref)
-    # every representable value encodes to its own code; values beyond the range saturate
+    # every representable value encodes to its own code
     codes = np.array([c for c in range(256) if c not in (0x80,)], np.uint8)
     assert np.array_equal(O.f8_encode(O.f8_decode(codes, fmt, 0, np.float32), fmt, 0), codes)
-    assert O.f8_encode(np.array([1e9, -1e9], f32), fmt, 0).tolist() == [0x7F, 0xFF]
+    # Beyond the largest finite value nothing here is a pin: torch's fnuz cast gives NaN there, the oracle
+    # saturates (its header and the fixture generator record that as an assumption about the Graphcore cast).
     # scale: encode(x, s) stores x * 2^-s
     assert np.array_equal(O.f8_encode(x, fmt, -1), O.f8_encode((x.astype(f32) * 2), fmt, 0))
 
