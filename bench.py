@@ -4,8 +4,11 @@
 A "step" is one iteration of the decode loop (one new token per sequence): embedding, 32
 transformer blocks (RMSNorm, INT4 q/k/v/o and SwiGLU projections, rotary embedding, KV append,
 attention over the cache, residuals), final norm, fp16 lm_head, greedy selection and the loop
-bookkeeping.  The default run follows the headline configuration: batch 1, a 128-token prompt
-consumed token by token (the untimed warm-up), then 256 timed new tokens, KV cache length 2048.
+bookkeeping.  The default run follows the headline configuration: batch 1, a 128-token prompt, then
+256 timed new tokens (contexts 128..383), KV cache length 2048.  The prompt's 128 loop iterations are
+always run untimed first (in passes of up to 64 rows; ``--prompt-loop``: one iteration per position, as
+the reference's loop does), then ``--warmup`` further untimed iterations, then ``--steps`` timed ones: the
+timed iterations generate new tokens whatever the flags are.
 
 By default the iteration runs as one persistent launch (pta_llama_decode_step, batch <= 4);
 ``--executor operators`` runs it as one launch per operator instead.
@@ -35,6 +38,7 @@ import numpy as np
 LLAMA2_7B = dict(vocab_size=32000, hidden_size=4096, rms_norm_eps=1e-5, num_attention_heads=32,
                  intermediate_size=11008, num_hidden_layers=32)
 MAX_LEN = 2048
+PROMPT = 128            # prompt positions of the headline configuration; always consumed untimed
 HBM_PEAK_GBS = 8000.0
 
 
@@ -197,12 +201,15 @@ RWKV4_7B = dict(num_hidden_layers=32, hidden_size=4096, attention_hidden_size=40
 
 def other_model_workload(args):
     """ChatGLM2-6B-shape FP8 decode (F143 weights and activations, fp16 KV cache of length 4096) or
-    RWKV-4-7B-shape INT4 recurrent decode, one launch per operator replayed from a HIP graph.  The prompt is
-    consumed token by token in the untimed warm-up.  Reported like the headline, without a kernel leg."""
+    RWKV-4-7B-shape INT4 recurrent decode, one launch per operator replayed from a HIP graph.  The prompt of
+    the configuration (512 / 64 positions) is consumed untimed, then --warmup further untimed iterations.
+    Reported like the headline, without a kernel leg."""
     import torch
     from poptransformer_amd.engine import fused, loader, rwkv, synthetic
     B = args.batch
     rng = np.random.Generator(np.random.PCG64(1234))
+    prompt = 512 if args.workload == "chatglm2" else 64          # of the respective benchmark configuration
+    first = prompt + args.warmup                                  # first timed loop iteration
     if args.workload == "chatglm2":
         cfg, max_len = CHATGLM2_6B, 4096
         weights = synthetic.chatglm2_synthetic_weights(cfg, "fp8", seed=0)
@@ -216,7 +223,7 @@ def other_model_workload(args):
         def step_bytes(t):
             return wbytes + per_pos * (t + 1) + B * cfg["hidden_size"] * 2
     else:
-        cfg, max_len = RWKV4_7B, args.warmup + args.steps + 2
+        cfg, max_len = RWKV4_7B, first + args.steps + 2
         weights = synthetic.rwkv_synthetic_weights(cfg, seed=0)
         dec = rwkv.RWKVDecoder(loader.rwkv_spec(cfg, max_len, B, pad_id=0, eos_id=-1), weights)
         wbytes, vocab = weights.nbytes(), cfg["vocab_size"]
@@ -226,26 +233,28 @@ def other_model_workload(args):
 
         def step_bytes(t):
             return wbytes + state + B * cfg["hidden_size"] * 2
-    if args.warmup + args.steps + 1 > max_len:
-        print(f"warmup + steps must stay below the sequence length {max_len}", file=sys.stderr)
+    if first + args.steps + 1 > max_len:
+        print(f"prompt ({prompt}) + warmup + steps must stay below the sequence length {max_len}", file=sys.stderr)
         sys.exit(2)
     dec.capture()
     ids = np.zeros((B, max_len), np.int32)
-    ids[:, :args.warmup] = rng.integers(3, vocab, size=(B, args.warmup))
+    ids[:, :prompt] = rng.integers(3, vocab, size=(B, prompt))
     dec.reset(ids)
-    dec.run_steps(args.warmup)
+    done = dec.consume_prompt(dec.prompt_positions()) if hasattr(dec, "consume_prompt") and not args.prompt_loop else 0
+    dec.run_steps(first - done)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     dec.run_steps(args.steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    mean_bytes = float(np.mean([step_bytes(t) for t in range(args.warmup, args.warmup + args.steps)]))
+    mean_bytes = float(np.mean([step_bytes(t) for t in range(first, first + args.steps)]))
     print(json.dumps({
         "metric": "decode tokens/s + % of HBM roofline", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": f"{name}, batch {B}, prompt {args.warmup} consumed token by token, "
-                               f"{args.steps} new tokens", "batch": B, "executor": "operators"},
+        "config": {"workload": f"{name}, batch {B}, prompt {prompt} consumed "
+                               f"{'in passes of up to 64 rows' if done else 'token by token'} (untimed), timed context "
+                               f"{first}..{first + args.steps - 1}", "batch": B, "executor": "operators"},
         "step_algorithmic_bytes": mean_bytes,
         "step_roofline_frac": mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9),
     }))
@@ -302,7 +311,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
-    ap.add_argument("--warmup", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=0,
+                    help="decode workload: untimed loop iterations AFTER the 128-token prompt (which is always consumed "
+                         "untimed); other workloads: untimed steps")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
                     help="default: persistent when the batch fits it (<= 4), else operators")
@@ -315,9 +326,9 @@ def main():
                     help="decode workload, operators executor: keep the KV cache as F143 bytes (KVCacheOp with fp8 = true)")
     ap.add_argument("--fuse-norm", choices=["on", "off"], default=None,
                     help="operators executor: run the norms inside the projections that consume them (default: the decoder's choice)")
-    ap.add_argument("--prompt-passes", action="store_true",
-                    help="decode workload: take the prompt's positions of the untimed warm-up in passes of up to 64 rows "
-                         "(FusedDecoder.consume_prompt) instead of one loop iteration per position")
+    ap.add_argument("--prompt-loop", action="store_true",
+                    help="decode workload: consume the (untimed) prompt one loop iteration per position, as the reference's "
+                         "loop does, instead of in passes of up to 64 rows (FusedDecoder.consume_prompt)")
     ap.add_argument("--no-batch16", action="store_true",
                     help="default run only: skip the second, batch-16 measurement that is reported beside the headline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -334,8 +345,8 @@ def main():
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
-    if args.workload == "decode" and args.warmup + args.steps + 1 > MAX_LEN:
-        print(f"warmup + steps must stay below the KV cache length {MAX_LEN}", file=sys.stderr)
+    if args.workload == "decode" and PROMPT + args.warmup + args.steps + 1 > MAX_LEN:
+        print(f"prompt ({PROMPT}) + warmup + steps must stay below the KV cache length {MAX_LEN}", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -365,16 +376,22 @@ def main():
     dec.capture()
 
     rng = np.random.Generator(np.random.PCG64(1234))
-    prompt = 128
+    prompt = PROMPT
     ids = np.zeros((B, MAX_LEN), np.int32)                       # pad id 0 after the prompt
     ids[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B, prompt))
-    dec.reset(ids)
 
-    in_passes = 0
-    if args.prompt_passes:
-        in_passes = dec.consume_prompt(min(args.warmup, dec.prompt_positions()))
-    dec.run_steps(args.warmup - in_passes)
-    torch.cuda.synchronize()
+    def to_first_timed_context(d, ids):
+        """Untimed: the prompt's 128 loop iterations (contexts 0..127; in passes of up to 64 rows unless
+        --prompt-loop), then --warmup further iterations.  Whatever --warmup is, the timed iterations start at
+        context 128 + warmup: they are iterations that generate new tokens."""
+        d.reset(ids)
+        done = 0 if args.prompt_loop else d.consume_prompt(d.prompt_positions())
+        d.run_steps(prompt - done + args.warmup)
+        torch.cuda.synchronize()
+        return done
+
+    in_passes = to_first_timed_context(dec, ids)
+    t_first = prompt + args.warmup
     t0 = time.perf_counter()
     dec.run_steps(args.steps)
     torch.cuda.synchronize()
@@ -382,7 +399,7 @@ def main():
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = B * args.steps / dt
     kvb = 1 if args.fp8_cache else 2
-    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t, kvb) for t in range(args.warmup, args.warmup + args.steps)])
+    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t, kvb) for t in range(t_first, t_first + args.steps)])
     step_frac = mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9)
 
     stream = torch.cuda.Stream()
@@ -391,10 +408,10 @@ def main():
             print("the persistent decode step reported a failure", file=sys.stderr)
             sys.exit(1)
         # Dominant kernel: the decode-step kernel itself, one launch per step.  Timed with events on the
-        # stream it is launched on, continuing the generation (so the context keeps growing as it does in
-        # the timed region above); its algorithmic bytes are the step's.
-        reps = min(64, MAX_LEN - 2 - args.warmup - args.steps)
-        t_first = args.warmup + args.steps
+        # stream it is launched on, over the SAME contexts as the timed region above: the loop's step counter is
+        # set back (the container keeps the tokens generated above, so the iterations repeat exactly).
+        reps = args.steps
+        dec.step.fill_(t_first)
         with torch.cuda.stream(stream):
             stream.wait_stream(torch.cuda.current_stream())
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -440,15 +457,18 @@ def main():
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
-        "config": {"workload": f"Llama2-7B-shape INT4 greedy decode, batch {B}, prompt {prompt} consumed "
-                               f"{'in passes of up to 64 rows' if in_passes else 'token by token'}, "
-                               f"context {args.warmup}..{args.warmup + args.steps - 1}, {'FP8 (F143)' if args.fp8_cache else 'fp16'} KV cache "
-                               f"length {MAX_LEN}",
+        "config": {"workload": f"Llama2-7B INT4 greedy decode, batch {B}, timed context {t_first}..{t_first + args.steps - 1} "
+                               f"after the {prompt}-token prompt (untimed, "
+                               f"{'passes of <= 64 rows' if in_passes else 'token by token'}), "
+                               f"{'F143' if args.fp8_cache else 'fp16'} KV cache of {MAX_LEN}",
                    "batch": B, "kv_cache_len": MAX_LEN, "executor": executor},
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": recorded_traffic() if executor == "persistent" and B == 1 else None,
+                     "traffic_source": ("recorded, not measured in this run: hardware counters of an earlier profiled "
+                                        "run, profiles/" + os.path.basename(PMC_SUMMARY))
+                     if executor == "persistent" and B == 1 else None,
                      "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }
     if B == 1 and not args.no_batch16 and not args.copy_calibration:
@@ -461,16 +481,15 @@ def main():
         dec16.capture()
         ids16 = np.zeros((B16, MAX_LEN), np.int32)
         ids16[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B16, prompt))
-        dec16.reset(ids16)
-        dec16.run_steps(args.warmup)
-        torch.cuda.synchronize()
+        to_first_timed_context(dec16, ids16)
         t0 = time.perf_counter()
         dec16.run_steps(args.steps)
         torch.cuda.synchronize()
         dt16 = time.perf_counter() - t0
-        bytes16 = float(np.mean([algorithmic_step_bytes(cfg, B16, t) for t in range(args.warmup, args.warmup + args.steps)]))
+        bytes16 = float(np.mean([algorithmic_step_bytes(cfg, B16, t) for t in range(t_first, t_first + args.steps)]))
         out["batch16"] = {"value": B16 * args.steps / dt16, "unit": "tokens/s", "ms_per_step": dt16 / args.steps * 1e3,
-                          "executor": "operators", "step_algorithmic_bytes": bytes16,
+                          "executor": "operators", "timed_context": [t_first, t_first + args.steps - 1],
+                          "step_algorithmic_bytes": bytes16,
                           "step_roofline_frac": bytes16 / (dt16 / args.steps) / (HBM_PEAK_GBS * 1e9)}
     if args.copy_calibration:
         src = torch.empty(1 << 29, dtype=torch.float16, device="cuda").normal_()
