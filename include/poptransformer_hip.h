@@ -439,6 +439,19 @@ int pta_llama_decode_step(const pta_decode_model* model, const pta_decode_state*
 /* Copies the failure word of the workspace to *failed (synchronises with `stream`). */
 int pta_decode_step_failed(const void* workspace, int* failed, pta_stream_t stream);
 
+/* pta_llama_decode_step for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * workspace is an array built into the library, 16 MiB of device memory that every GPU the library runs on
+ * holds until the process ends; a model whose workspace (pta_decode_step_workspace_bytes) is larger is
+ * refused with PTA_EINVAL.  The call allocates and frees nothing.  Its first call on a device looks up
+ * the array's address there: make that call outside any capture.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls in stream order do not, also when
+ * they serve different models.  There is no workspace pointer to hand to pta_decode_step_failed: a launch
+ * that gave up leaves `*state->step` as it was, which is how the caller sees it, and every later launch does
+ * nothing until one is made with clear_failure != 0 (a one-thread kernel clears the failure word first). */
+int pta_llama_decode_step_static(const pta_decode_model* model, const pta_decode_state* state, int clear_failure,
+                                 pta_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,8 @@
 // and phase at the 7B shape) instead of being issued where registers first become free.  Every
 // tile has a fixed place in one register array for the whole layer loop, so that no requested tile
 // is ever moved between registers (a move waits for the load and for the burst around it).
+#include <mutex>
+
 #include "common.h"
 #include "formats.h"
 
@@ -1142,8 +1144,7 @@ extern "C" size_t pta_decode_step_workspace_bytes(const pta_decode_model* model)
   return layout_for(model, cus).total;
 }
 
-extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
-                                     pta_stream_t stream) {
+static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace, pta_stream_t stream) {
   PTA_REQUIRE(mdl && st && workspace, "pta_llama_decode_step: null pointer");
   PTA_REQUIRE(mdl->layers && mdl->n_layer > 0 && mdl->embed && mdl->final_norm && mdl->head && mdl->inv_freq,
               "pta_llama_decode_step: incomplete model");
@@ -1215,6 +1216,71 @@ extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_deco
   hipLaunchKernelGGL(var->kern, dim3(cus), dim3(DS_THREADS), lds, (hipStream_t)stream, a);
   PTA_CHECK_LAUNCH("pta_llama_decode_step");
   return PTA_OK;
+}
+
+extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
+                                     pta_stream_t stream) {
+  return decode_step_launch(mdl, st, workspace, stream);
+}
+
+// ------------------------------------------------------------------------------------------ the same step without a workspace argument
+// The workspace of pta_llama_decode_step (result slots, attention partials, synchronisation words) in a
+// file-scope device array, for callers that cannot allocate.  Every device holds its own copy of the
+// array at its own address; the name `scratch` is only a host-side handle, so the address is looked up
+// once per device with hipGetSymbolAddress and kept.  The array starts zeroed (epoch 0, no failure), which
+// is the state the kernel expects of a fresh workspace; later launches continue the epoch of the one before,
+// whatever model they serve, because the synchronisation words sit at the same offsets for every shape.
+namespace {
+constexpr size_t DS_STATIC_BYTES = (size_t)16 << 20;
+constexpr int DS_MAX_DEVICES = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[DS_STATIC_BYTES];
+
+namespace {
+std::mutex g_static_mutex;
+void* g_static_ptr[DS_MAX_DEVICES] = {};
+
+__global__ void clear_failure_kernel(unsigned* sync) {
+  if (threadIdx.x == 0 && blockIdx.x == 0)
+    __hip_atomic_store((DS_GLOBAL unsigned*)(sync + 1), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+}  // namespace
+
+extern "C" int pta_llama_decode_step_static(const pta_decode_model* mdl, const pta_decode_state* st, int clear_failure,
+                                            pta_stream_t stream) {
+  PTA_REQUIRE(mdl && st, "pta_llama_decode_step_static: null pointer");
+  int dev = 0;
+  PTA_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < DS_MAX_DEVICES,
+              "pta_llama_decode_step_static: cannot identify the current device");
+  int cus = 0;
+  PTA_REQUIRE(device_cus(&cus) == 0, "pta_llama_decode_step_static: cannot read the compute-unit count of the current device");
+  if (!shape_ok(mdl)) {
+    pta_set_error("pta_llama_decode_step_static: unsupported shape (see pta_llama_decode_step)");
+    return PTA_EUNSUPPORTED;
+  }
+  const size_t need = layout_for(mdl, cus).total;
+  PTA_REQUIRE(need <= DS_STATIC_BYTES,
+              "pta_llama_decode_step_static: this model needs %zu bytes of workspace, the built-in array holds %zu; use "
+              "pta_llama_decode_step with a workspace of its own", need, (size_t)DS_STATIC_BYTES);
+  void* ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+      void* p = nullptr;
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !p) {
+        pta_set_error("pta_llama_decode_step_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        return PTA_EHIP;
+      }
+      g_static_ptr[dev] = p;
+    }
+    ws = g_static_ptr[dev];
+  }
+  if (clear_failure) {
+    hipLaunchKernelGGL(clear_failure_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned*)ws);
+    PTA_CHECK_LAUNCH("pta_llama_decode_step_static");
+  }
+  return decode_step_launch(mdl, st, ws, stream);
 }
 
 extern "C" int pta_decode_step_failed(const void* workspace, int* failed, pta_stream_t stream) {

@@ -578,6 +578,12 @@ class DecodeStep:
         check(_lib.load().pta_llama_decode_step(ctypes.byref(self.model), ctypes.byref(self.state), _p(self.workspace),
                                                 _stream()))
 
+    def launch_static(self, clear_failure=False):
+        """The same iteration through the entry point that allocates nothing: its workspace is the array built
+        into the library, not `self.workspace` (pta_llama_decode_step_static)."""
+        check(_lib.load().pta_llama_decode_step_static(ctypes.byref(self.model), ctypes.byref(self.state),
+                                                       1 if clear_failure else 0, _stream()))
+
     def failed(self):
         flag = ctypes.c_int(0)
         check(_lib.load().pta_decode_step_failed(_p(self.workspace), ctypes.byref(flag), _stream()))
