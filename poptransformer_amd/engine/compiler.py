@@ -5,10 +5,12 @@ this package knows - GPT-2, Llama 2, ChatGLM2, RWKV as the models build them thr
 API - is additionally mapped onto the fused executor for its family: the family is read off the
 state-dict keys the layers registered as initializer names, the shapes off a one-iteration probe of
 the interpreter, and the weights off the initializers.  The fused executor is then VALIDATED: it
-must generate the same token ids as the interpreter on a probe prompt, otherwise the graph stays
-on the interpreter.  A fused executor therefore never changes what a graph computes; it only
-changes how fast.
+must generate the same token ids as the interpreter on a probe prompt (for a sampling graph: the same top-k candidates), otherwise
+the graph stays on the interpreter - or, for a strict session, compilation fails.  An INT4 Llama-2
+graph at batch <= 4 is further mapped onto the one-launch-per-iteration persistent step, validated
+the same way, and prompts are taken in passes over several positions.
 """
+import dataclasses
 import logging
 
 import numpy as np
@@ -89,13 +91,20 @@ def _dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+def _need(facts, key):
+    """An initializer the family's graph must hold; a graph without it is not that family's graph."""
+    if key not in facts.init:
+        raise ValueError(f"initializer {key} is missing")
+    return facts.init[key]
+
+
 def _linear(facts, ctx, bias, precision):
     """A Linear as the layer bound it (layers/linear.py + utils/param_handler.py): fp16 [in, out];
     packed INT4 int8 [out, in/2] with `<key>_scale` fp16 [out]; F143 bytes [in, out] with an int32
     `<key>_scale` exponent."""
     key = f"{ctx}.weight"
-    w = facts.init[key]
-    b = _dev(facts.init[f"{ctx}.bias"].astype(np.float16)) if bias else None
+    w = _need(facts, key)
+    b = _dev(_need(facts, f"{ctx}.bias").astype(np.float16)) if bias else None
     scale = facts.init.get(key + "_scale")
     if w.dtype == np.int8:
         if scale is None:
@@ -111,7 +120,7 @@ def _linear(facts, ctx, bias, precision):
 
 
 def _vec(facts, key):
-    return _dev(facts.init[key].astype(np.float16).reshape(-1))
+    return _dev(_need(facts, key).astype(np.float16).reshape(-1))
 
 
 def _precision(facts, probe_ops):
@@ -137,7 +146,7 @@ def _eps_from_normce(facts):
 
 
 # ----------------------------------------------------------------------------------- families
-def _build_transformer(facts, shapes, family):
+def _build_transformer(facts, shapes, family, topk=1, fp8_cache=False):
     kv = shapes["custom.KVCache"][0][1]              # updater [2, B, Hkv, 1, D]
     sm = shapes["custom.SoftmaxV3"][0][0]            # scores  [B, Hq, 1, L]
     Hkv, D, Hq = kv[2], kv[4], sm[1]
@@ -154,7 +163,7 @@ def _build_transformer(facts, shapes, family):
                 out=_linear(facts, p + "self_attn.o_proj", False, prec),
                 mlp_in=[_linear(facts, p + "mlp." + n, False, prec) for n in ("gate_proj", "up_proj")],
                 mlp_out=_linear(facts, p + "mlp.down_proj", False, prec)))
-        embed = facts.init["model.embed_tokens.weight"]
+        embed = _need(facts, "model.embed_tokens.weight")
         inv = np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16)
         w = ModelWeights(_dev(embed.astype(np.float16)), None, blocks, (_vec(facts, "model.norm.weight"), None),
                          _linear(facts, "lm_head", False, prec), _dev(inv))
@@ -173,7 +182,7 @@ def _build_transformer(facts, shapes, family):
                 out=_linear(facts, p + "self_attention.dense", False, prec),
                 mlp_in=[_linear(facts, p + "mlp.dense_h_to_4h_1", False, prec), _linear(facts, p + "mlp.dense_h_to_4h_2", False, prec)],
                 mlp_out=_linear(facts, p + "mlp.dense_4h_to_h", False, prec)))
-        embed = facts.init["transformer.embedding.word_embeddings.weight"]
+        embed = _need(facts, "transformer.embedding.word_embeddings.weight")
         rot = D // 2
         inv = np.array([1.0 / (10000 ** (i / rot)) for i in range(0, rot, 2)]).astype(np.float32)
         w = ModelWeights(_dev(embed.astype(np.float16)), None, blocks,
@@ -192,8 +201,8 @@ def _build_transformer(facts, shapes, family):
                 out=_linear(facts, p + "attn.c_proj", True, prec),
                 mlp_in=[_linear(facts, p + "mlp.c_fc", True, prec)],
                 mlp_out=_linear(facts, p + "mlp.c_proj", True, prec)))
-        wte = _dev(facts.init["transformer.wte.weight"].astype(np.float16))
-        w = ModelWeights(wte, _dev(facts.init["transformer.wpe.weight"].astype(np.float16)), blocks,
+        wte = _dev(_need(facts, "transformer.wte.weight").astype(np.float16))
+        w = ModelWeights(wte, _dev(_need(facts, "transformer.wpe.weight").astype(np.float16)), blocks,
                          (_vec(facts, "transformer.ln_f.weight"), _vec(facts, "transformer.ln_f.bias")),
                          LinearWeights(K.F16Weight(wte)), None)
         eps = _eps_from_normce(facts)
@@ -201,11 +210,11 @@ def _build_transformer(facts, shapes, family):
         raise ValueError("layer count does not match the KV caches in the graph")
     d_model = w.embed.shape[1]
     spec = DecoderSpec(family, n_layer, d_model, Hq, Hkv, D, w.head.N, facts.max_len, facts.batch, eps, facts.pad_id,
-                       facts.eos_id, facts.early_stop)
-    return fused.FusedDecoder(spec, w)
+                       facts.eos_id, facts.early_stop, topk=topk, fp8_cache=fp8_cache)
+    return spec, w
 
 
-def _build_rwkv(facts, shapes):
+def _build_rwkv(facts, shapes, topk=1):
     from .rwkv import RWKVBlockWeights, RWKVDecoder, RWKVSpec, RWKVWeights
     n_layer = facts.count_layers("rwkv.blocks.{}.ln1.weight")
     prec = _precision(facts, facts.ops)
@@ -229,7 +238,7 @@ def _build_rwkv(facts, shapes):
             ffn_receptance=_linear(facts, p + "feed_forward.receptance", False, prec),
             ffn_value=_linear(facts, p + "feed_forward.value", False, prec),
             ffn_mix=[_vec(facts, p + f"feed_forward.time_mix_{n}") for n in ("key", "receptance")]))
-    w = RWKVWeights(_dev(facts.init["rwkv.embeddings.weight"].astype(np.float16)), blocks, ln("rwkv.ln_out"),
+    w = RWKVWeights(_dev(_need(facts, "rwkv.embeddings.weight").astype(np.float16)), blocks, ln("rwkv.ln_out"),
                     _linear(facts, "head", False, prec))
     d = w.embed.shape[1]
     # every `rescale_every` blocks the hidden state is halved by a Div node
@@ -237,7 +246,7 @@ def _build_rwkv(facts, shapes):
                 and float(_const_value(facts.body, n.inputs[1])) == 2.0)
     rescale = n_layer // n_div if n_div else 0
     spec = RWKVSpec(n_layer, d, blocks[0].att_key.N, blocks[0].ffn_key.N, w.head.N, facts.max_len, facts.batch,
-                    _eps_from_normce(facts), rescale, facts.pad_id, facts.eos_id, facts.early_stop)
+                    _eps_from_normce(facts), rescale, facts.pad_id, facts.eos_id, facts.early_stop, topk=topk)
     return RWKVDecoder(spec, w)
 
 
@@ -255,11 +264,14 @@ def _family(facts):
 
 # ----------------------------------------------------------------------------------- programs
 class FusedProgram:
-    def __init__(self, decoder, facts, anchors, batches_per_step, kind):
+    fallback_reason = None
+
+    def __init__(self, decoder, facts, anchors, batches_per_step, kind, prompt_passes=False):
         self.decoder, self.facts, self.anchors, self.bps, self.kind = decoder, facts, list(anchors), batches_per_step, kind
+        self.prompt_passes = prompt_passes
 
     def _run_once(self, ids):
-        container, step = self.decoder.run(ids, self.facts.max_loop)
+        container, step = self.decoder.run(ids, self.facts.max_loop, prompt_passes=self.prompt_passes)
         out = {}
         if len(self.anchors) > 0:
             out[self.anchors[0]] = container
@@ -281,7 +293,7 @@ class FusedProgram:
         return {a: np.zeros(lead + s, t) for a, (s, t) in zip(self.anchors, shapes)}
 
 
-def _probe_ids(facts, seed):
+def _probe_ids(facts, seed, n=3):
     rng = np.random.default_rng(seed)
     vocab_guess = 64
     for key, arr in facts.init.items():
@@ -289,7 +301,7 @@ def _probe_ids(facts, seed):
             vocab_guess = arr.shape[0]
             break
     ids = np.full((facts.batch, facts.max_len), facts.pad_id, np.int32)
-    n = min(3, facts.max_len)
+    n = min(n, facts.max_len)
     p = rng.integers(0, vocab_guess, size=(facts.batch, n))
     p[p == facts.pad_id] = (facts.pad_id + 1) % vocab_guess
     p[p == facts.eos_id] = (facts.eos_id + 1) % vocab_guess if facts.eos_id >= 0 else p[p == facts.eos_id]
@@ -297,14 +309,80 @@ def _probe_ids(facts, seed):
     return ids
 
 
-def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True):
-    """Returns an executor with `run(feeds) -> {anchor: array}` and `anchor_arrays()`; its `kind`
-    attribute says which one it is ('interpreter' or 'fused:<family>')."""
+def _sampling_k(facts):
+    """k of LMHead's selection, read off the loop body: 1 for the top-1 graph, k for ops.random_sample
+    (aiOnnx.topk with k > 1 whose pick is the argmax of aiOnnx.randomnormal draws, ops/popart.py:25-29)."""
+    ks = []
+    for n in facts.body.nodes:
+        if n.op == "aiOnnx.topk":
+            k = _const_value(facts.body, n.inputs[1])
+            if k is None:
+                raise ValueError("aiOnnx.topk with a k that is not a constant")
+            ks.append(int(np.asarray(k).reshape(-1)[0]))
+    random = facts.ops.get("aiOnnx.randomnormal", 0)
+    if not random:
+        if ks != [1]:
+            raise ValueError(f"expected one top-1 selection in the loop body, found topk with k = {ks}")
+        return 1
+    if random != 1 or len(ks) != 1 or ks[0] < 2:
+        raise ValueError(f"random draws in the loop body that are not one ops.random_sample (topk k = {ks})")
+    return ks[0]
+
+
+def _fp8_cache_of(facts, requested):
+    """Whether the KV caches hold F143 bytes: the session option, or the `fp8` attribute of the graph's KVCache
+    nodes (the reference's ops.kv_cache always records False, ops/customized.py:32)."""
+    flags = {bool(n.attrs.get("fp8")) for n in facts.body.nodes if n.op == "custom.KVCache"}
+    if len(flags) > 1:
+        raise ValueError("KVCache nodes with and without fp8 storage in one graph")
+    return bool(requested) or (flags == {True})
+
+
+def _validate_greedy(decoder, prog, facts, ids, steps, prompt_passes, what):
+    want = prog._run_once({facts.ids_name: ids})[prog.interp_outputs[0]]
+    got, _ = decoder.run(ids, steps, prompt_passes=prompt_passes)
+    if not np.array_equal(got, want):
+        raise ValueError(f"{what} does not reproduce the graph's tokens on the probe")
+
+
+def _validate_sampling(decoder, prog, facts, ids, steps, k):
+    """A sampling graph draws from its own generator, so tokens are not comparable; the candidates are.  The probe
+    holds a token at every position it reaches (nothing that is drawn feeds back), and the top-k ids of every
+    iteration must equal those of the interpreter, in order."""
+    interp = prog.interp
+    interp.value_trace = {"aiOnnx.topk": []}
+    try:
+        prog._run_once({facts.ids_name: ids})
+        want = [np.asarray(o[1]).reshape(facts.batch, k) for o in interp.value_trace["aiOnnx.topk"]]
+    finally:
+        interp.value_trace = None
+    if len(want) != steps:
+        raise ValueError("the probe did not run the expected number of iterations")
+    decoder.reset(ids)
+    for it in range(steps):
+        decoder.step_fn()
+        torch.cuda.synchronize()
+        if not np.array_equal(decoder.select.ids.cpu().numpy(), want[it]):
+            raise ValueError(f"the fused executor's top-{k} candidates differ from the graph's at probe iteration {it}")
+
+
+def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True, strict=False, fp8_cache=False,
+                  persistent=True, prompt_passes=True):
+    """Returns an executor with `run(feeds) -> {anchor: array}` and `anchor_arrays()`; its `kind` attribute says
+    which one it is: 'interpreter', 'fused:<family>' (one launch per operator, replayed from a HIP graph) or
+    'fused:llama2:persistent' (one launch per loop iteration).  A graph the fused executors do not cover stays on
+    the interpreter, with the reason in `fallback_reason`; with `strict` that is an error instead.
+    persistent: use the one-launch iteration where the model allows it (INT4 Llama 2, batch <= 4, top-1; it needs
+    the whole device for itself while it runs).  prompt_passes: the leading iterations that only read the prompt
+    run as passes over several positions.  fp8_cache: KV caches hold F143 bytes (KVCache with fp8 = true)."""
     from .. import _lib
     _lib.load()                                   # no HIP library, no executor: there is no CPU path
     prog = InterpretedProgram(graph, anchors, batches_per_step)
     if not allow_fused:
+        if strict:
+            raise ValueError("strict: the session asks for a fused executor but allow_fused is off")
         return prog
+    interp = prog.interp
     try:
         facts = GraphFacts(graph)
         family = _family(facts)
@@ -312,30 +390,71 @@ def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True):
             raise ValueError("no known model family among the initializer names")
         if len(anchors) > 2 or list(anchors) != list(graph.outputs)[:len(anchors)]:
             raise ValueError("anchors other than the loop outputs")
-        # one-iteration probe: operand shapes of the native operators, and the reference output
-        interp = prog.interp
+        prog.interp_outputs = list(graph.outputs)
+        k = _sampling_k(facts)
+        use_fp8_cache = _fp8_cache_of(facts, fp8_cache)
+        if use_fp8_cache and family == "rwkv":
+            raise ValueError("fp8_cache: a recurrent model has no KV cache")
+        steps = min(PROBE_STEPS, facts.max_loop)
+        # one-iteration probe: operand shapes of the native operators
         interp.shape_trace = {}
         interp.max_trips = 1
-        ids = _probe_ids(facts, 0)
+        ids = _probe_ids(facts, 0, n=3 if k == 1 else steps + 1)
         prog._run_once({facts.ids_name: ids})
         shapes, interp.shape_trace = interp.shape_trace, None
-        decoder = _build_rwkv(facts, shapes) if family == "rwkv" else _build_transformer(facts, shapes, family)
-        # validation: identical ids after a few iterations, eager and replayed
-        steps = min(PROBE_STEPS, facts.max_loop)
+        if family == "rwkv":
+            decoder = _build_rwkv(facts, shapes, k)
+        else:
+            spec, weights = _build_transformer(facts, shapes, family, k, use_fp8_cache)
+            decoder = fused.FusedDecoder(spec, weights)
+        passes = prompt_passes and hasattr(decoder, "consume_prompt")
         interp.max_trips = steps
-        want = prog._run_once({facts.ids_name: ids})[graph.outputs[0]]
-        got, _ = decoder.run(ids, steps)
-        if not np.array_equal(got, want):
-            raise ValueError("the fused executor does not reproduce the graph's tokens on the probe")
-        decoder.capture()
-        got, _ = decoder.run(ids, steps)
-        if not np.array_equal(got, want):
-            raise ValueError("the captured HIP graph does not reproduce the graph's tokens on the probe")
+        if k > 1:
+            _validate_sampling(decoder, prog, facts, ids, steps, k)
+            decoder.capture()
+            kind = f"fused:{family}"
+        elif use_fp8_cache and not any(n.attrs.get("fp8") for n in facts.body.nodes if n.op == "custom.KVCache"):
+            # the option changes what the graph computes (its caches are fp16): nothing to compare the tokens with;
+            # the executor is checked against the graph with fp16 caches first, then switched
+            plain = fused.FusedDecoder(dataclasses.replace(spec, fp8_cache=False), weights)
+            _validate_greedy(plain, prog, facts, ids, steps, passes, "the fused executor")
+            del plain
+            decoder.capture()
+            kind = f"fused:{family}"
+        else:
+            # validation: identical ids after a few iterations, eager and replayed
+            _validate_greedy(decoder, prog, facts, ids, steps, passes, "the fused executor")
+            decoder.capture()
+            _validate_greedy(decoder, prog, facts, ids, steps, passes, "the captured HIP graph")
+            kind = f"fused:{family}"
+            if persistent and hasattr(decoder, "enable_persistent"):
+                try:
+                    decoder.enable_persistent()
+                except NotImplementedError as e:
+                    prog.persistent_reason = str(e)
+                else:
+                    decoder.capture()
+                    try:
+                        _validate_greedy(decoder, prog, facts, ids, steps, passes, "the persistent decode step")
+                        kind += ":persistent"
+                    except (ValueError, RuntimeError) as e:
+                        if strict:
+                            raise
+                        log.warning("the persistent decode step is not used: %s", e)
+                        prog.persistent_reason = str(e)
+                        decoder.persistent = None
+                        decoder.capture()
         interp.max_trips = None
-        return FusedProgram(decoder, facts, anchors, batches_per_step, f"fused:{family}")
-    except Exception as e:  # noqa: BLE001 - any failure keeps the graph on the interpreter
-        prog.interp.max_trips = None
-        prog.interp.shape_trace = None
+        out = FusedProgram(decoder, facts, anchors, batches_per_step, kind, passes)
+        out.persistent_reason = getattr(prog, "persistent_reason", None)
+        return out
+    except (ValueError, NotImplementedError) as e:
+        # the expected ways a graph is outside what the fused executors cover; anything else is a bug and propagates
+        interp.max_trips = None
+        interp.shape_trace = None
+        interp.value_trace = None
+        if strict:
+            raise
         log.warning("graph stays on the op-by-op interpreter: %s", e)
         prog.fallback_reason = str(e)
         return prog

@@ -242,6 +242,32 @@ class LayerOps:
             self._qkv_views = (q, kv, kv[:, Hkv * D:], Hq * D, 2 * Hkv * D, 2 * Hkv * D)
 
 
+class NextToken:
+    """LMHead's selection (layers/lm_head.py:52-56) over the logits of one iteration: top-1, or with topk > 1
+    ops.random_sample (ops/popart.py:25-29): the top-k ids, then the column chosen by the argmax of k normal
+    draws, one draw per iteration for the whole batch."""
+
+    def __init__(self, batch, vocab, topk, device):
+        if topk < 1 or topk > vocab:
+            raise ValueError(f"topk = {topk} outside [1, vocabulary size {vocab}]")
+        self.topk = topk
+        if topk > 1:
+            i32, f16 = torch.int32, torch.float16
+            self.ids = torch.zeros((batch, topk), dtype=i32, device=device)
+            self.vals = torch.zeros((batch, topk), dtype=f16, device=device)
+            self.draws = torch.zeros((1, topk), dtype=f16, device=device)
+            self.pick = torch.zeros((1,), dtype=i32, device=device)
+
+    def __call__(self, logits, next_ids):
+        if self.topk == 1:
+            K.argmax(logits, next_ids)
+            return
+        K.topk(logits, self.topk, self.ids, self.vals)
+        self.draws.normal_()
+        K.argmax(self.draws, self.pick)
+        K.take_column(self.ids, self.pick, next_ids)
+
+
 class FusedDecoder(LayerOps):
     def __init__(self, spec: DecoderSpec, weights: ModelWeights, device="cuda"):
         super().__init__(spec, weights, device, spec.batch)
@@ -250,11 +276,7 @@ class FusedDecoder(LayerOps):
         i32 = torch.int32
         self.logits = buf(B, s.vocab)
         self.next_ids = buf(B, dtype=i32)
-        if s.topk > 1:
-            if s.topk > s.vocab:
-                raise ValueError(f"topk = {s.topk} exceeds the vocabulary size {s.vocab}")
-            self._topk_ids, self._topk_vals = buf(B, s.topk, dtype=i32), buf(B, s.topk)
-            self._draws, self._pick = buf(1, s.topk), buf(1, dtype=i32)
+        self.select = NextToken(B, s.vocab, s.topk, device)
         self.container = buf(B, s.max_len, dtype=i32)
         self.mask = buf(B, s.max_len)
         self.stop_mask = buf(B, dtype=i32)
@@ -325,15 +347,7 @@ class FusedDecoder(LayerOps):
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)
         h, nrm = self._normed(self.x, w.final_norm, [w.head])
         self._linear(h, w.head, self.logits, norm=nrm)
-        if s.topk == 1:
-            K.argmax(self.logits, self.next_ids)
-        else:
-            # layers/lm_head.py:52-53 -> ops.random_sample (ops/popart.py:25-29): the top-k ids, then the column
-            # chosen by the argmax of k normal draws, one draw per step for the whole batch
-            K.topk(self.logits, s.topk, self._topk_ids, self._topk_vals)
-            self._draws.normal_()
-            K.argmax(self._draws, self._pick)
-            K.take_column(self._topk_ids, self._pick, self.next_ids)
+        self.select(self.logits, self.next_ids)
         K.step_update(self.container, self.mask, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
                       s.pad_id, s.eos_id, s.early_stop)
 
@@ -421,11 +435,16 @@ class FusedDecoder(LayerOps):
             for _ in range(n):
                 self.graph.replay()
 
-    def run(self, input_ids, max_loop, check_every=16):
+    def run(self, input_ids, max_loop, check_every=16, prompt_passes=False):
         """The whole generation (one `session.run` of the reference, poptransformer/sessions.py:47-49).
-        Returns (container, step) like the anchors 'Loop:0' and 'Loop:1'."""
+        Returns (container, step) like the anchors 'Loop:0' and 'Loop:1'.  prompt_passes: the leading
+        iterations that only read the prompt run as passes over several positions (consume_prompt)."""
         self.reset(input_ids)
         done = 0
+        if prompt_passes:
+            n = min(self.prompt_positions(), max_loop)
+            if n > 0:
+                done = self.consume_prompt(n)
         while done < max_loop:
             n = min(check_every, max_loop - done) if self.spec.early_stop else max_loop - done
             self.run_steps(n)
@@ -434,6 +453,7 @@ class FusedDecoder(LayerOps):
                 break
         torch.cuda.synchronize()
         if self.persistent is not None and self.persistent.failed():
-            raise RuntimeError("persistent decode step: a workgroup never reached the grid barrier (the kernel needs "
-                               "every compute unit of the device while it runs); the loop state was not advanced")
+            raise RuntimeError("persistent decode step: a workgroup gave up waiting (the kernel needs every compute unit "
+                               "of the device for itself while it runs); the loop state was not advanced past the failing "
+                               "iteration.  The failure word is sticky: persistent.clear_failure() re-arms the decoder")
         return self.container.cpu().numpy(), int(self.step.item())

@@ -91,6 +91,9 @@ class Interpreter:
         if self.shape_trace is not None and op.startswith("custom."):
             self.shape_trace.setdefault(op, []).append([tuple(t.shape) for t in ins])
         out = fn(n, env, *ins)
+        if self.value_trace is not None and op in self.value_trace:
+            vals = out if isinstance(out, (list, tuple)) else [out]
+            self.value_trace[op].append([v.detach().cpu().numpy() for v in vals])
         if isinstance(out, (list, tuple)):
             for t, v in zip(n.outputs, out):
                 env[t] = v
@@ -265,6 +268,7 @@ class Interpreter:
     loop_checks_condition = True
     max_trips = None            # cap on loop iterations (shape discovery, validation probes)
     shape_trace = None          # when a dict: operand shapes of the native operators, per op name
+    value_trace = None          # when a dict {op name: []}: the outputs of every execution of those ops (host copies)
 
     def _aiGraphcore_call(self, n, env, *ins):
         body = n.subgraph
@@ -345,6 +349,7 @@ class InterpretedProgram:
         self.graph, self.anchors, self.bps = graph, list(anchors), batches_per_step
         self.interp = Interpreter(graph)
         self.kind = "interpreter"
+        self.fallback_reason = None
         self._shapes = None
 
     def _run_once(self, feeds):

@@ -13,7 +13,7 @@ import torch
 
 from .. import _lib
 from .. import kernels as K
-from .fused import LinearWeights
+from .fused import LinearWeights, NextToken
 
 
 @dataclass
@@ -30,6 +30,7 @@ class RWKVSpec:
     pad_id: int = 0
     eos_id: int = -1
     early_stop: bool = False
+    topk: int = 1                    # > 1: ops.random_sample among the top-k (layers/lm_head.py:52-53)
 
 
 @dataclass
@@ -83,6 +84,7 @@ class RWKVDecoder:
         self.fk, self.fr = buf(B, f), buf(B, d)
         self.logits = buf(B, s.vocab)
         self.next_ids = buf(B, dtype=i32)
+        self.select = NextToken(B, s.vocab, s.topk, device)
         self.container = buf(B, s.max_len, dtype=i32)
         self.stop_mask = buf(B, dtype=i32)
         self.step = torch.zeros((), dtype=i32, device=device)
@@ -128,7 +130,7 @@ class RWKVDecoder:
             K.linear(self.fk, [blk.ffn_value.w], [x], mul=self.fr, residual=x, post_scale=0.5 if halve else 0.0)
         K.layer_norm_ce(x, w.ln_out[0], w.ln_out[1], s.eps, self.h)
         K.linear(self.h, [w.head.w], [self.logits])
-        K.argmax(self.logits, self.next_ids)
+        self.select(self.logits, self.next_ids)
         K.step_update(self.container, None, self.stop_mask, self.step, self.next_ids, None, self.keep_going,
                       s.pad_id, s.eos_id, s.early_stop)
 
@@ -164,7 +166,9 @@ class RWKVDecoder:
             else:
                 self.graph.replay()
 
-    def run(self, input_ids, max_loop, check_every=16):
+    def run(self, input_ids, max_loop, check_every=16, prompt_passes=False):
+        """prompt_passes is accepted for symmetry with the transformer executor; a recurrent model reads its
+        prompt one position per iteration."""
         self.reset(input_ids)
         done = 0
         while done < max_loop:

@@ -584,6 +584,12 @@ class DecodeStep:
         check(_lib.load().pta_llama_decode_step_static(ctypes.byref(self.model), ctypes.byref(self.state),
                                                        1 if clear_failure else 0, _stream()))
 
+    def clear_failure(self):
+        """Re-arms a workspace whose failure word a launch has set (the word is sticky: until it is cleared every
+        launch returns at once)."""
+        torch.cuda.synchronize()
+        self.workspace.view(torch.int32)[1] = 0
+
     def failed(self):
         flag = ctypes.c_int(0)
         check(_lib.load().pta_decode_step_failed(_p(self.workspace), ctypes.byref(flag), _stream()))

@@ -362,7 +362,7 @@ class InferenceSession:
     def prepareDevice(self, **kwargs):
         from ..engine import compiler
         self.executor = compiler.compile_graph(self.graph, list(self.data_flow.anchors), self.data_flow.batches_per_step,
-                                               getattr(self, "allow_fused", True))
+                                               getattr(self, "allow_fused", True), **getattr(self, "executor_options", {}))
 
     def weightsFromHost(self):
         if self.executor is None:

@@ -16,7 +16,15 @@ class Session:
         self.constant_folding_of_multiple_consumers = kwargs.get("constant_folding_of_multiple_consumers", False)
         self.use_loop_candidate_creator = kwargs.get("use_loop_candidate_creator", True)
         self.profile_name = kwargs.get("profile_name", None)
+        # executor choices of this build (the reference has one executor, PopART's):
+        #   allow_fused   map a known decoder loop onto the fused executors (else: op by op)
+        #   strict        fail compilation instead of falling back to the op-by-op interpreter
+        #   persistent    one launch per loop iteration where the model allows it (INT4 Llama 2, batch <= 4); that
+        #                 kernel occupies every compute unit while it runs: nothing else may run on the device beside it
+        #   prompt_passes take the prompt's positions in passes of up to 64 rows instead of one per iteration
+        #   fp8_cache     KV caches hold F143 bytes, as the KVCache op does with fp8 = true
         self.allow_fused = kwargs.get("allow_fused", True)
+        self.executor_options = {k: kwargs[k] for k in ("strict", "persistent", "prompt_passes", "fp8_cache") if k in kwargs}
         self.enable_pipeline = REGISTRY.get("enable_pipeline")
         self.batch_per_step = REGISTRY.get("batch_per_step")
 
@@ -31,6 +39,7 @@ class Session:
         self.session = popart.InferenceSession(fnModel=model.model_proto, deviceInfo=self.device_info,
                                                dataFlow=self.data_flow, userOptions=self.options)
         self.session.allow_fused = self.allow_fused
+        self.session.executor_options = self.executor_options
         self.session.prepareDevice()
         self.session.weightsFromHost()
         self._anchor_arrays = self.session.initAnchorArrays()
@@ -57,4 +66,10 @@ class Session:
 
     @property
     def executor_kind(self):
+        """'interpreter', 'fused:<family>' or 'fused:llama2:persistent'."""
         return self.session.executor.kind
+
+    @property
+    def fallback_reason(self):
+        """Why the graph runs on the op-by-op interpreter although fused executors were allowed (else None)."""
+        return getattr(self.session.executor, "fallback_reason", None)

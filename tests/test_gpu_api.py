@@ -49,21 +49,25 @@ def _robust_reference(make_oracle, make_ids, L, steps, pad, eos, seeds=range(6),
     return best
 
 
-def _session(model_cls, precision, B, model_kwargs, allow_fused):
+def _session(model_cls, precision, B, model_kwargs, allow_fused, **session_kwargs):
     from poptransformer_amd.sessions import Session
     from poptransformer_amd.utils import prepare_model_session
-    cfg = {"global_args": {"batch_size": B, "precision": precision}, "model": model_kwargs, "session": {"allow_fused": allow_fused}}
+    cfg = {"global_args": {"batch_size": B, "precision": precision}, "model": model_kwargs,
+           "session": dict(session_kwargs, allow_fused=allow_fused)}
     return prepare_model_session(cfg, model_cls, Session)
 
 
-def _check(model_cls, precision, B, L, steps, pad, eos, sd, hf_config, oracle, make_ids, extra=None):
+def _check(model_cls, precision, B, L, steps, pad, eos, sd, hf_config, oracle, make_ids, extra=None, kind=None,
+           session_kwargs=None):
     ids, ref_c, ref_s, cols = _robust_reference(oracle, make_ids, L, steps, pad, eos)
     for allow_fused in (False, True):
         kw = dict(hf_config=hf_config, state_dict=sd, pad_token_id=pad, eos_token_id=eos, max_length=L, max_loop=steps)
         kw.update(extra or {})
-        session, model = _session(model_cls, precision, B, kw, allow_fused)
+        session, model = _session(model_cls, precision, B, kw, allow_fused, **(session_kwargs or {}) if allow_fused else {})
         if allow_fused:
-            assert session.executor_kind.startswith("fused:"), getattr(session.session.executor, "fallback_reason", "")
+            assert session.executor_kind.startswith("fused:"), session.fallback_reason
+            if kind is not None:
+                assert session.executor_kind == kind, getattr(session.session.executor, "persistent_reason", None)
         else:
             assert session.executor_kind == "interpreter"
         session.run(model.build_input_dict(input_ids=[list(r[r != pad]) for r in ids]))
@@ -81,7 +85,69 @@ def test_llama2_int4_through_the_operator_api():
     B, L, steps, pad, eos = 2, 32, 20, 0, 2
     sd = OM.make_llama2_state_dict(LLAMA, seed=21, int4=True)
     ids = lambda seed: _ids(np.random.default_rng(100 + seed), B, L, 5, 512, pad)
-    _check(LLAMA2DecModel, "int4", B, L, steps, pad, eos, sd, LLAMA, lambda: OM.Llama2Oracle(sd, LLAMA, L, B), ids)
+    # Session.compile alone reaches the one-launch-per-iteration step, and Session.run takes the prompt in passes
+    _check(LLAMA2DecModel, "int4", B, L, steps, pad, eos, sd, LLAMA, lambda: OM.Llama2Oracle(sd, LLAMA, L, B), ids,
+           kind="fused:llama2:persistent", session_kwargs={"strict": True})
+
+
+def test_llama2_session_options_choose_the_executor():
+    """persistent = False keeps one launch per operator; fp8_cache = True makes the KV caches F143 bytes (the
+    KVCache op with fp8 = true), which the persistent step does not cover: per-operator executor, tokens equal to
+    the oracle's with an FP8 cache."""
+    from poptransformer_amd.models.llama2 import LLAMA2DecModel
+    B, L, steps, pad, eos = 2, 32, 20, 0, 2
+    sd = OM.make_llama2_state_dict(LLAMA, seed=21, int4=True)
+    ids = lambda seed: _ids(np.random.default_rng(100 + seed), B, L, 5, 512, pad)
+    kw = dict(hf_config=LLAMA, state_dict=sd, pad_token_id=pad, eos_token_id=eos, max_length=L, max_loop=steps)
+    session, model = _session(LLAMA2DecModel, "int4", B, kw, True, persistent=False, strict=True)
+    assert session.executor_kind == "fused:llama2" and session.session.executor.decoder.persistent is None
+    session, model = _session(LLAMA2DecModel, "int4", B, kw, True, fp8_cache=True, strict=True)
+    assert session.executor_kind == "fused:llama2" and session.session.executor.decoder.spec.fp8_cache
+    probe, ref_c, ref_s, cols = _robust_reference(lambda: OM.Llama2Oracle(sd, LLAMA, L, B, fp8_cache=True), ids, L, steps, pad, eos)
+    session.run(model.build_input_dict(input_ids=[list(r[r != pad]) for r in probe]))
+    got = session.anchor_arrays["Loop:0"]
+    for r in range(B):
+        assert np.array_equal(got[r, :cols[r]], ref_c[r, :cols[r]])
+
+
+def test_sampling_graph_is_compiled_as_a_sampling_executor():
+    """A model built with topk = 3 records ops.random_sample; the compiler must read k off the graph (a greedy
+    executor would be a different program) and validate the candidates, not the drawn tokens.  Every generated
+    token is then one of the three best of the oracle's logits for the same history."""
+    from poptransformer_amd.models.llama2 import LLAMA2DecModel
+    B, L, steps, pad, eos, k = 2, 32, 20, 0, -1, 3
+    sd = OM.make_llama2_state_dict(LLAMA, seed=26, int4=True)
+    kw = dict(hf_config=LLAMA, state_dict=sd, pad_token_id=pad, eos_token_id=eos, max_length=L, max_loop=steps, topk=k)
+    session, model = _session(LLAMA2DecModel, "int4", B, kw, True, strict=True)
+    assert session.executor_kind == "fused:llama2"                 # the persistent step selects greedily: not used
+    assert session.session.executor.decoder.spec.topk == k
+    ids = _ids(np.random.default_rng(8), B, L, 4, 512, pad)
+    session.run({"input_ids": ids})
+    got = session.anchor_arrays["Loop:0"]
+    assert np.array_equal(got[:, :4], ids[:, :4]) and (got[:, 4:steps + 1] != pad).all()
+    # the oracle, fed the session's own tokens: each one must be among its top k at the position before
+    forced = got.copy()
+    trace = []
+    OM.run_decode_loop(OM.Llama2Oracle(sd, LLAMA, L, B), forced, L, steps, pad, eos, trace=trace)
+    for t in range(3, steps):
+        logits = trace[t][1].astype(np.float32)
+        for b in range(B):
+            # candidates within fp16 rounding of the k-th best count as well
+            kth = np.sort(logits[b])[-k]
+            assert logits[b, got[b, t + 1]] >= kth - 4e-3 * np.abs(logits[b]).max(), f"position {t + 1}, row {b}"
+
+
+def test_strict_session_refuses_to_fall_back():
+    """A graph the fused executors do not cover (fp32 weights) runs op by op, with the reason on record; a strict
+    session fails to compile instead."""
+    from poptransformer_amd.models.llama2 import LLAMA2DecModel
+    B, L, pad, eos = 1, 16, 0, 2
+    sd = {k: v.astype(np.float32) for k, v in OM.make_llama2_state_dict(LLAMA, seed=27, int4=False).items()}
+    kw = dict(hf_config=LLAMA, state_dict=sd, pad_token_id=pad, eos_token_id=eos, max_length=L, max_loop=4)
+    session, _ = _session(LLAMA2DecModel, "fp32", B, kw, True)
+    assert session.executor_kind == "interpreter" and "fp16, INT4 or FP8" in session.fallback_reason
+    with pytest.raises(ValueError):
+        _session(LLAMA2DecModel, "fp32", B, kw, True, strict=True)
 
 
 def test_gpt2_fp16_through_the_operator_api():
