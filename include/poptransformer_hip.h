@@ -198,6 +198,15 @@ int pta_kv_cache_append(void* cache, const void* updater, const int32_t* step, i
 int pta_kv_cache_read(const void* cache, void* out, const int32_t* step, int outer, int max_len, int inner,
                       int elem_bytes, int max_bps, pta_stream_t stream);
 
+/* KVCachePipeline with transpose = 1, literal (custom_ops/kv_cache_pipeline.cpp:397-451; codelet
+ * custom_ops/kv_cache_codelet.cpp:170-212): the max_bps persistent registers `caches`
+ * [max_bps, outer, inner, max_len] keep the sequence as their last axis; all are zeroed when *step == 0;
+ * register *step % max_bps is shifted by one element along that axis in place, with the new row
+ * `updater` [outer, 1, inner] at index 0; `out` [outer, max_len, inner] receives that register in the
+ * input's layout (the op's output).  step_len is 1, as the op itself requires (pipeline.cpp:410). */
+int pta_kv_cache_pipeline_seq_last(void* caches, void* out, const void* updater, const int32_t* step, int outer,
+                                   int max_len, int inner, int elem_bytes, int max_bps, pta_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * Attention for one new position per sequence
  * ---------------------------------------------------------------------------------- */
@@ -283,6 +292,24 @@ int pta_topk(const pta_half* logits, int32_t* ids, pta_half* values, int rows, i
 /* The slice of ops.random_sample (ops/popart.py:25-29): out[r] = candidates[r, *pick] for candidates
  * int32 [rows, k] and a device index `pick` (clamped into [0, k)), the same column for every row. */
 int pta_take_column(const int32_t* candidates, const int32_t* pick, int32_t* out, int rows, int k, pta_stream_t stream);
+
+/* Bytes of the workspace of pta_beam_search_step (the per-beam candidates); 0 for beam_size outside [1, 64]. */
+size_t pta_beam_search_workspace_bytes(int batch, int beam);
+
+/* One call of the BeamSearch op (custom_ops/beam_search_custom_op.cpp:333-478; shape guards :103-177).
+ * logits [batch, beam, vocab] and prob_container [batch, beam] of `dtype` (PTA_F16 / PTA_F32), hyp_container
+ * int32 [batch, max_len, beam], `step` a device int32.  Per beam the `beam` best scores over the vocabulary;
+ *   *step == 0: next_id = global_best_id = the ids of beam 0, hyp_container[:, 0] = next_id, prob_container =
+ *     the scores of beam 0;
+ *   otherwise: candidate (i, j) = prob_container[i] + score j of beam i (added in `dtype`); the `beam` best
+ *     of the beam * beam candidates give global_best_id (flat index i * beam + j), next_id (their ids) and
+ *     prob_container; every row of hyp_container is re-gathered from the parent hypotheses i and row *step
+ *     (if inside the container) takes next_id.
+ * Equal scores are taken in ascending order of index.  The containers are updated in place; next_id and
+ * global_best_id are int32 [batch, beam]. */
+int pta_beam_search_step(const void* logits, int dtype, int32_t* hyp_container, void* prob_container, const int32_t* step,
+                         int32_t* next_id, int32_t* global_best_id, void* workspace, int batch, int beam, int vocab,
+                         int max_len, pta_stream_t stream);
 
 /* Embedding rows (layers/embedding.py:34-36); with pos_table also GPT-2's wte[id] + wpe[*pos]
  * (models/gpt2/embedding.py:31-36).  out [rows, cols].  Row b uses

@@ -153,15 +153,29 @@ class KVCachePipeline:
     custom_ops/kv_cache_codelet.cpp:18-131: max_bps independent caches; bpsIdx = step % max_bps
     (codelet:27-35); every cache zeroed when step == 0 (:46-64); only cache bpsIdx shifts in the
     new rows and is returned (pipeline.cpp:422-439).  The sequence axis must be rank - 2
-    (custom_ops/kv_cache_pipeline.hpp:80-88)."""
+    (custom_ops/kv_cache_pipeline.hpp:80-88).
+    transpose (pipeline.cpp:397-401,445-449; codelet:170-212): the op swaps the last two axes of its input, keeps
+    the persistent caches with the sequence as the LAST axis, shifts cache bpsIdx by one element along it in place
+    (new element at index 0; step_len must be 1, pipeline.cpp:410) and swaps the axes of its output back: the
+    output equals that of transpose = 0, the stored layout (`stored()`) differs."""
 
-    def __init__(self, max_len, max_bps, step_len=1):
-        self.max_len, self.max_bps, self.step_len = max_len, max_bps, step_len
+    def __init__(self, max_len, max_bps, step_len=1, transpose=False):
+        if transpose and step_len != 1:
+            raise ValueError("transpose = 1 takes one new row per call")
+        self.max_len, self.max_bps, self.step_len, self.transpose = max_len, max_bps, step_len, transpose
         self.caches = None
+
+    def stored(self):
+        """The persistent tensors as the op holds them: [.., D, max_len] each when transpose, else [.., max_len, D]."""
+        return [c.copy() for c in self.caches]
 
     def __call__(self, step, updater):
         updater = np.asarray(updater)
-        axis = updater.ndim - 2
+        if self.transpose:
+            updater = np.swapaxes(updater, -1, -2)            # pipeline.cpp:397-401: the sequence becomes the last axis
+            axis = updater.ndim - 1
+        else:
+            axis = updater.ndim - 2
         if self.caches is None:
             shape = list(updater.shape)
             shape[axis] = self.max_len
@@ -171,7 +185,7 @@ class KVCachePipeline:
         i = int(step) % self.max_bps
         keep = np.take(self.caches[i], range(0, self.max_len - self.step_len), axis=axis)
         self.caches[i] = np.concatenate([updater, keep], axis=axis)
-        return self.caches[i]
+        return np.swapaxes(self.caches[i], -1, -2) if self.transpose else self.caches[i]
 
 
 # --------------------------------------------------------------------------------------
@@ -303,6 +317,60 @@ def sigmoid(x):
     x = np.asarray(x)
     with np.errstate(over="ignore"):
         return (f32(1.0) / (f32(1.0) + np.exp(-x.astype(f32)))).astype(x.dtype)
+
+
+# --------------------------------------------------------------------------------------
+# BeamSearch (custom_ops/beam_search_custom_op.cpp)
+# --------------------------------------------------------------------------------------
+def _topk_desc(x, k):
+    """Values and indices of the k largest entries along the last axis, largest first, equal values in
+    ascending order of index (popnn::topK with sorted = true; its tie order is not pinned by the reference tree)."""
+    order = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k]
+    return np.take_along_axis(x, order, axis=-1), order.astype(np.int32)
+
+
+def beam_search_step(logits, hyp_container, prob_container, step, beam_size):
+    """BeamSearchOpx::grow (custom_ops/beam_search_custom_op.cpp:333-478), one call of the op.
+    logits [B, beam, V] (fp16 or fp32: the scores that add along a hypothesis), hyp_container int32
+    [B, max_len, beam], prob_container [B, beam] of the logits' dtype, step int.  Returns (next_id [B, beam],
+    global_best_id [B, beam], hyp_container, prob_container); the containers are new arrays.
+    Shape guards: BeamSearchOp::setup (:103-177).
+      every step: per beam the `beam` best scores and ids over the vocabulary (:347-354);
+      step == 0 (:371-385): next_id = global_best_id = the ids of beam 0; hyp_container[:, 0] = next_id;
+        prob_container = the scores of beam 0;
+      step != 0 (:387-466): candidate (i, j) = prob_container[i] + score j of beam i, added in the containers'
+        dtype (:400-401); row `step` of the beam-by-beam expanded hypotheses takes the candidate ids (:403-417;
+        a step beyond the container writes nothing); the `beam` best candidates over the beam * beam (:424-432)
+        give global_best_id (flat index i * beam + j), next_id (their ids, :438-446), every row of hyp_container
+        re-gathered from the parent beam i (:452-463) and prob_container (:465-466)."""
+    logits = np.asarray(logits)
+    hyp = np.asarray(hyp_container)
+    prob = np.asarray(prob_container)
+    if logits.ndim != 3:
+        raise ValueError(f"[Beam Search] The rank of logits should be 3. But now it is {logits.ndim}.")
+    B, nb, V = logits.shape
+    if beam_size > V:
+        raise ValueError("[Beam Search] The parameter 'beam_size' should not be greater than the vocab_size")
+    if hyp.ndim != 3 or prob.ndim != 2:
+        raise ValueError("[Beam Search] hyp_container must have rank 3 and prob_container rank 2")
+    if hyp.shape[0] != B or prob.shape[0] != B or nb != beam_size or hyp.shape[2] != beam_size or prob.shape[1] != beam_size:
+        raise ValueError("[Beam Search] batch or beam sizes of logits, hyp_container and prob_container differ")
+    dt = prob.dtype
+    best_v, best_i = _topk_desc(logits, beam_size)                      # [B, beam, beam]
+    if int(step) == 0:
+        next_id = best_i[:, 0, :].copy()
+        out_h = hyp.copy()
+        out_h[:, 0, :] = next_id
+        return next_id, next_id.copy(), out_h, best_v[:, 0, :].astype(dt)
+    cand = (best_v.astype(dt) + prob[:, :, None]).astype(dt).reshape(B, beam_size * beam_size)
+    ids = best_i.reshape(B, beam_size * beam_size)
+    temp = np.repeat(hyp, beam_size, axis=2)                            # [B, max_len, beam * beam]: entry i * beam + j = hyp[.., i]
+    if 0 <= int(step) < hyp.shape[1]:
+        temp[:, int(step), :] = ids
+    g_v, g_i = _topk_desc(cand, beam_size)                              # [B, beam]
+    next_id = np.take_along_axis(ids, g_i, axis=1)
+    out_h = np.take_along_axis(temp, np.broadcast_to(g_i[:, None, :], (B, hyp.shape[1], beam_size)), axis=2)
+    return next_id.astype(np.int32), g_i.astype(np.int32), out_h.astype(np.int32), g_v.astype(dt)
 
 
 # --------------------------------------------------------------------------------------

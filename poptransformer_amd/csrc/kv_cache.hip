@@ -153,3 +153,79 @@ extern "C" int pta_kv_cache_read(const void* cache, void* out, const int32_t* st
   PTA_CHECK_LAUNCH("pta_kv_cache_read");
   return PTA_OK;
 }
+
+// KVCachePipeline with transpose = 1 (custom_ops/kv_cache_pipeline.cpp:397-451, codelet
+// custom_ops/kv_cache_codelet.cpp:170-212): the max_bps persistent caches keep the sequence as their LAST axis,
+// [outer, inner, max_len]; register step % max_bps is shifted by one element along that axis IN PLACE (there
+// is no clone), the new row goes to index 0, and the op's output is that register in the input's own layout
+// [outer, max_len, inner].  All registers are zeroed when step == 0 (codelet:46-64).  step_len is 1: the op
+// copies the input into output[..., 0:1] (pipeline.cpp:410).
+// One workgroup owns KT_D features of one `outer` row of one register and walks the sequence in chunks from the
+// end to the start: a chunk's sources (element l - 1 for element l) lie in the chunk itself or at the end of
+// the next lower one, which is still untouched, and inside a chunk every load is done before the first store.
+constexpr int KT_D = 32, KT_L = 64;
+
+template <typename E>
+__global__ __launch_bounds__(256) void kv_seq_last_kernel(E* __restrict__ caches, E* __restrict__ out,
+                                                          const E* __restrict__ upd, const int32_t* __restrict__ step_p,
+                                                          int outer, int max_len, int inner, int max_bps) {
+  __shared__ E tile[KT_D][KT_L + 1];
+  const int st = *step_p;
+  const int reg = blockIdx.z, sel = ((st % max_bps) + max_bps) % max_bps;
+  if (reg != sel && st != 0) return;             // other registers are only touched by the zeroing at step 0
+  const int o = blockIdx.y, d0 = blockIdx.x * KT_D;
+  E* cache = caches + ((size_t)reg * outer + o) * inner * max_len;
+  const int nd = inner - d0 < KT_D ? inner - d0 : KT_D;
+  const int chunks = (max_len + KT_L - 1) / KT_L;
+  for (int c = chunks - 1; c >= 0; --c) {
+    const int l0 = c * KT_L;
+    const int nl = max_len - l0 < KT_L ? max_len - l0 : KT_L;
+    // tile[d][j] = the value element l0 + j will hold
+    for (int t = threadIdx.x; t < KT_D * KT_L; t += 256) {
+      const int d = t / KT_L, j = t % KT_L;
+      if (d < nd && j < nl) {
+        const int l = l0 + j;
+        E v = (E)0;
+        if (reg == sel) {
+          if (l == 0) v = upd[(size_t)o * inner + d0 + d];
+          else if (st != 0) v = cache[(size_t)(d0 + d) * max_len + l - 1];
+        }
+        tile[d][j] = v;
+      }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < KT_D * KT_L; t += 256) {
+      const int d = t / KT_L, j = t % KT_L;
+      if (d < nd && j < nl) cache[(size_t)(d0 + d) * max_len + l0 + j] = tile[d][j];
+    }
+    if (reg == sel) {
+      for (int t = threadIdx.x; t < KT_D * KT_L; t += 256) {
+        const int j = t / KT_D, d = t % KT_D;
+        if (d < nd && j < nl) out[((size_t)o * max_len + l0 + j) * inner + d0 + d] = tile[d][j];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+extern "C" int pta_kv_cache_pipeline_seq_last(void* caches, void* out, const void* updater, const int32_t* step, int outer,
+                                              int max_len, int inner, int elem_bytes, int max_bps, pta_stream_t stream) {
+  int rc = check_kv("pta_kv_cache_pipeline_seq_last", outer, max_len, 1, inner, elem_bytes);
+  if (rc) return rc;
+  PTA_REQUIRE(caches && out && updater && step, "pta_kv_cache_pipeline_seq_last: null pointer");
+  PTA_REQUIRE(max_bps >= 1 && max_bps <= 65535 && outer <= 65535,
+              "pta_kv_cache_pipeline_seq_last: max_bps and outer must lie in [1, 65535]");
+  const dim3 grid((unsigned)((inner + KT_D - 1) / KT_D), (unsigned)outer, (unsigned)max_bps);
+  hipStream_t s = (hipStream_t)stream;
+  if (elem_bytes == 1)
+    hipLaunchKernelGGL(kv_seq_last_kernel<uint8_t>, grid, dim3(256), 0, s, (uint8_t*)caches, (uint8_t*)out,
+                       (const uint8_t*)updater, step, outer, max_len, inner, max_bps);
+  else if (elem_bytes == 2)
+    hipLaunchKernelGGL(kv_seq_last_kernel<uint16_t>, grid, dim3(256), 0, s, (uint16_t*)caches, (uint16_t*)out,
+                       (const uint16_t*)updater, step, outer, max_len, inner, max_bps);
+  else
+    hipLaunchKernelGGL(kv_seq_last_kernel<uint32_t>, grid, dim3(256), 0, s, (uint32_t*)caches, (uint32_t*)out,
+                       (const uint32_t*)updater, step, outer, max_len, inner, max_bps);
+  PTA_CHECK_LAUNCH("pta_kv_cache_pipeline_seq_last");
+  return PTA_OK;
+}

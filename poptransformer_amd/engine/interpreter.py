@@ -300,6 +300,42 @@ class Interpreter:
         K.kv_cache_update(cache, clone, upd.contiguous(), step.reshape(()).to(torch.int32).contiguous(), axis)
         return cache
 
+    def _custom_KVCachePipeline(self, n, env, step, upd):
+        a = n.attrs
+        if a.get("fp8"):
+            raise NotImplementedError("KVCachePipeline with fp8 storage")
+        max_len, max_bps, step_len = a["max_len"], a["max_bps"], a.get("step_len", 1)
+        axis = a.get("sequence_axis", -2)
+        axis = axis + upd.dim() if axis < 0 else axis
+        if axis != upd.dim() - 2:
+            raise popart_exception(f"[KVCachePipeline] Only support axis = {upd.dim() - 2}(or -2),but now it is {axis}.")
+        if step_len != 1 or upd.shape[axis] != 1:
+            raise NotImplementedError("KVCachePipeline: one new row per call (step_len = 1)")
+        outer, inner = int(np.prod(upd.shape[:axis])), upd.shape[-1]
+        st = step.reshape(()).to(torch.int32).contiguous()
+        key = n.outputs[0]
+        shape = list(upd.shape)
+        shape[axis] = max_len
+        out = torch.empty(shape, dtype=upd.dtype, device=upd.device)
+        if a.get("transpose"):
+            if key not in self.state:
+                self.state[key] = torch.zeros((max_bps, outer, inner, max_len), dtype=upd.dtype, device=upd.device)
+            return K.kv_cache_pipeline_seq_last(self.state[key], out, upd.contiguous(), st, outer, max_len, inner, max_bps)
+        if key not in self.state:
+            self.state[key] = torch.zeros((max_bps, outer, max_len, inner), dtype=upd.dtype, device=upd.device)
+        # the ring addresses rows by step / max_bps: the calls must come with step = 0, 1, 2, ... as a loop issues them
+        K.kv_cache_append(self.state[key], upd.contiguous(), st, outer, max_len, inner, max_bps)
+        return K.kv_cache_read(self.state[key], out, st, outer, max_len, inner, max_bps)
+
+    def _custom_BeamSearch(self, n, env, logits, hyp, prob, step):
+        beam = int(n.attrs["beam_size"])
+        if logits.dim() == 3 and logits.shape[1] != beam:
+            raise popart_exception(f"[Beam Search] logits.shape[1]({logits.shape[1]}) should beequal to parameter "
+                                   f"'beam_size'({beam}).")
+        hyp, prob = hyp.to(torch.int32).contiguous().clone(), prob.contiguous().clone()
+        next_id, best = K.beam_search_step(logits, hyp, prob, step.reshape(()).to(torch.int32).contiguous())
+        return [next_id, best, hyp, prob]
+
     def _custom_SoftmaxV3(self, n, env, x):
         axis = n.attrs["axis"]
         if x.dim() < 2:

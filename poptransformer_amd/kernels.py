@@ -389,6 +389,40 @@ def kv_cache_read(ring, out, step, outer, max_len, inner, max_bps=1):
     return out
 
 
+def kv_cache_pipeline_seq_last(caches, out, updater, step, outer, max_len, inner, max_bps):
+    """KVCachePipeline with transpose = 1: `caches` [max_bps, outer, inner, max_len] updated in place, `out`
+    [outer, max_len, inner] the op's output."""
+    _need(step, _i32, "step")
+    check(_lib.load().pta_kv_cache_pipeline_seq_last(_p(caches), _p(out), _p(updater), _p(step), outer, max_len, inner,
+                                                     caches.element_size(), max_bps, _stream()))
+    return out
+
+
+def beam_search_step(logits, hyp_container, prob_container, step, workspace=None):
+    """One call of the BeamSearch op; the containers are updated in place.  Returns (next_id, global_best_id)."""
+    if logits.dim() != 3:
+        raise ValueError(f"[Beam Search] The rank of logits should be 3. But now it is {logits.dim()}.")
+    if hyp_container.dim() != 3 or prob_container.dim() != 2:
+        raise ValueError("[Beam Search] hyp_container must have rank 3 and prob_container rank 2")
+    B, beam, V = logits.shape
+    if tuple(prob_container.shape) != (B, beam) or hyp_container.shape[0] != B or hyp_container.shape[2] != beam:
+        raise ValueError("[Beam Search] batch or beam sizes of logits, hyp_container and prob_container differ")
+    if logits.dtype not in (torch.float16, torch.float32) or prob_container.dtype != logits.dtype:
+        raise ValueError("[Beam Search] logits and prob_container must both be float16 or float32")
+    _need(hyp_container, _i32, "hyp_container")
+    _need(step, _i32, "step")
+    lib = _lib.load()
+    if workspace is None:
+        workspace = torch.empty(max(lib.pta_beam_search_workspace_bytes(B, beam), 256), dtype=torch.uint8, device=logits.device)
+    next_id = torch.empty((B, beam), dtype=_i32, device=logits.device)
+    best = torch.empty((B, beam), dtype=_i32, device=logits.device)
+    logits = logits.contiguous()
+    check(lib.pta_beam_search_step(_p(logits), _lib.F16 if logits.dtype == torch.float16 else _lib.F32,
+                                   _p(hyp_container), _p(prob_container), _p(step), _p(next_id), _p(best), _p(workspace),
+                                   B, beam, V, hyp_container.shape[1], _stream()))
+    return next_id, best
+
+
 # ------------------------------------------------------------------ attention ------------
 def qkv_rope_append(q, k, v, q_out, kv_ring, step, inv_freq, B, Hq, Hkv, D, max_len, rope,
                     q_stride=None, k_stride=None, v_stride=None):

@@ -257,6 +257,24 @@ def kv_cache(graph, step, updater, max_len, sequence_axis=1, step_len=1):
                    {"max_len": max_len, "step_len": step_len, "sequence_axis": sequence_axis, "fp8": False})
 
 
+def kv_cache_pipeline(graph, step, updater, max_len, max_bps, step_len=1, sequence_axis=-2, fp8=False, transpose=0):
+    """The KVCachePipeline custom op (custom_ops/kv_cache_pipeline.hpp:104-145: attributes max_len, max_bps,
+    step_len, sequence_axis, fp8, transpose).  The reference registers the op but has no Python wrapper for it;
+    this one follows the wrapper of KVCache (customized.py:21-35)."""
+    return _custom(graph, "KVCachePipeline", [step, updater],
+                   {"max_len": max_len, "max_bps": max_bps, "step_len": step_len, "sequence_axis": sequence_axis,
+                    "fp8": fp8, "transpose": transpose, "debug_str": "kv_cache_pipeline"})
+
+
+def beam_search(graph, logits, hyp_container, prob_container, step, beam_size):
+    """The BeamSearch custom op (custom_ops/beam_search_custom_op.cpp:53-214: inputs logits, hyp_container,
+    prob_container, step; attribute beam_size; outputs next_id, global_best_id, hyp_container, prob_container).
+    The reference registers the op but has no Python wrapper for it.  Returns the four output ids."""
+    return graph.customOp(opName="BeamSearch", domain=_DOMAIN, opVersion=1,
+                          inputs=[logits, hyp_container, prob_container, step],
+                          attributes={"beam_size": beam_size}, numOutputs=4)
+
+
 def remap_tensor(graph, x, fwd_after_matmul=0, name="remap"):
     """customized.py:38-54: an IPU tile-layout hint; the values are unchanged."""
     return _custom(graph, "Remap", [x], {"fwd_grain_size": 8, "bwd_grain_size": 8, "fwd_clone_layout": 0,

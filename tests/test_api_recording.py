@@ -57,6 +57,15 @@ def test_ops_record_reference_custom_ops(fresh):
         ops.layer_norm_ce(g, x, w, w, 1e-5, 2, 1, 8192)          # customized.py:81-82
     ops.int4_to_half(g, x, w, x)
     assert g.nodes[-1].attrs == {"axis": 1, "remap": 1}
+    # the two registered ops the reference has no Python wrapper for: attribute names of their OpCreators
+    ops.kv_cache_pipeline(g, step, x, 16, 3, transpose=1)
+    n = g.nodes[-1]
+    assert n.op == "custom.KVCachePipeline" and n.inputs == [step, x]
+    assert {k: n.attrs[k] for k in ("max_len", "max_bps", "step_len", "sequence_axis", "fp8", "transpose")} == \
+        {"max_len": 16, "max_bps": 3, "step_len": 1, "sequence_axis": -2, "fp8": False, "transpose": 1}
+    outs = ops.beam_search(g, x, x, x, step, 4)
+    n = g.nodes[-1]
+    assert n.op == "custom.BeamSearch" and len(outs) == 4 and n.outputs == outs and n.attrs == {"beam_size": 4}
     ops.half_to_uint8(g, x, w)
     assert g.nodes[-1].op == "custom.CastToUint8WithoutShapeInfer" and g.nodes[-1].attrs == {"fp8Format": "F143"}
     ops.fp8_matmul(g, x, x, w, w)

@@ -194,3 +194,45 @@ def test_early_stop_and_unknown_graphs_stay_on_the_interpreter():
         session.run({"input_ids": ids})
         assert np.array_equal(session.anchor_arrays["Loop:0"], ref_c)
         assert int(np.asarray(session.anchor_arrays["Loop:1"]).reshape(-1)[0]) == ref_s
+
+
+def test_beam_search_and_pipeline_cache_through_the_operator_api():
+    """A graph of the two registered custom ops the reference's models never call - BeamSearch and KVCachePipeline
+    (transpose 0 and 1) - run op by op, against the oracle, one run of the graph per step with host-fed inputs
+    (the caches are op state and persist between the runs)."""
+    import torch
+    from oracle import ops as O
+    from poptransformer_amd import ops, popart
+    from poptransformer_amd.engine.interpreter import Interpreter
+    from poptransformer_amd.utils import REGISTRY, register_global_args
+    REGISTRY.reset()
+    register_global_args({"batch_size": 2, "precision": "fp16"})
+    g = REGISTRY.get("main_graph")
+    B, beam, V, L, max_len, max_bps = 2, 3, 50, 6, 5, 2
+    logits = g.addInputTensor(popart.TensorInfo("FLOAT16", [B, beam, V]), "logits")
+    hyp = g.addInputTensor(popart.TensorInfo("INT32", [B, L, beam]), "hyp")
+    prob = g.addInputTensor(popart.TensorInfo("FLOAT16", [B, beam]), "prob")
+    step = g.addInputTensor(popart.TensorInfo("INT32", []), "step")
+    row = g.addInputTensor(popart.TensorInfo("FLOAT16", [B, 2, 1, 8]), "row")
+    outs = ops.beam_search(g, logits, hyp, prob, step, beam)
+    c0 = ops.kv_cache_pipeline(g, step, row, max_len, max_bps)
+    c1 = ops.kv_cache_pipeline(g, step, row, max_len, max_bps, transpose=1)
+    interp = Interpreter(g)
+    interp.reset()
+    rng = np.random.default_rng(44)
+    hyp_v, prob_v = np.zeros((B, L, beam), np.int32), np.zeros((B, beam), np.float16)
+    caches = O.KVCachePipeline(max_len, max_bps)
+    for it in range(2 * max_len + 2):
+        lg = np.log(rng.dirichlet(np.full(V, 0.5), size=(B, beam))).astype(np.float16)
+        rw = rng.standard_normal((B, 2, 1, 8)).astype(np.float16)
+        ref = O.beam_search_step(lg, hyp_v, prob_v, it, beam)
+        ref_cache = caches(it, rw)
+        feeds = {logits: lg, hyp: hyp_v, prob: prob_v, step: np.array(it, np.int32), row: rw}
+        env = {k: torch.from_numpy(np.ascontiguousarray(v)).cuda() for k, v in feeds.items()}
+        interp.run_graph(g, env)
+        torch.cuda.synchronize()
+        got = [interp._get(env, t).cpu().numpy() for t in outs + [c0, c1]]
+        for a, b in zip(got[:4], ref):
+            assert np.array_equal(a, b), f"beam search output differs at step {it}"
+        assert np.array_equal(got[4], ref_cache) and np.array_equal(got[5], ref_cache), f"pipeline cache differs at step {it}"
+        hyp_v, prob_v = ref[2], ref[3]

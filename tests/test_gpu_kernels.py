@@ -871,3 +871,64 @@ def test_topk_guards_and_take_column(K):
     for pick, col in ((0, 0), (3, 3), (7, 3), (-2, 0)):     # out-of-range picks are clamped
         got = host(K.take_column(cand, dev(np.array([pick], np.int32))))
         assert np.array_equal(got, np.arange(12).reshape(3, 4)[:, col])
+
+
+# ---------------------------------------------------------------- BeamSearch, KVCachePipeline transpose
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("B,beam,V,L", [(2, 4, 1000, 12), (1, 1, 37, 5), (3, 8, 32000, 20), (2, 64, 80, 9)])
+def test_beam_search_step_bit_exact(K, dtype, B, beam, V, L):
+    """Ids, flat candidate indices, both containers bit for bit over more steps than the container has rows
+    (the steps beyond it only re-gather), fp16 logits with many equal scores included."""
+    rng = np.random.default_rng(B * 1000 + beam + V)
+    tdt = torch.float16 if dtype == np.float16 else torch.float32
+    hyp_ref = rng.integers(-5, 5, size=(B, L, beam)).astype(np.int32)      # whatever the caller left there
+    prob_ref = rng.standard_normal((B, beam)).astype(dtype)
+    hyp, prob = dev(hyp_ref), dev(prob_ref)
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    ws = torch.empty(K._lib.load().pta_beam_search_workspace_bytes(B, beam), dtype=torch.uint8, device="cuda")
+    for it in range(L + 2):
+        # log-probabilities of a peaked distribution; in fp16 many of them coincide
+        logits = np.log(rng.dirichlet(np.full(V, 0.3), size=(B, beam)) + 1e-9).astype(dtype)
+        nxt_ref, best_ref, hyp_ref, prob_ref = O.beam_search_step(logits, hyp_ref, prob_ref, it, beam)
+        step.fill_(it)
+        nxt, best = K.beam_search_step(dev(logits).to(tdt), hyp, prob, step, ws)
+        assert np.array_equal(host(nxt), nxt_ref), f"next_id differs at step {it}"
+        assert np.array_equal(host(best), best_ref), f"global_best_id differs at step {it}"
+        assert np.array_equal(host(hyp), hyp_ref), f"hyp_container differs at step {it}"
+        assert np.array_equal(host(prob).view(np.uint8), prob_ref.view(np.uint8)), f"prob_container differs at step {it}"
+
+
+def test_beam_search_guards(K):
+    z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        K.beam_search_step(z(2, 5), z(1, 4, 2, dt=torch.int32), z(1, 2), step)            # rank of logits
+    with pytest.raises(ValueError):
+        K.beam_search_step(z(1, 2, 5), z(1, 4, 3, dt=torch.int32), z(1, 2), step)         # beam sizes differ
+    with pytest.raises(ValueError):
+        K.beam_search_step(z(1, 6, 5), z(1, 4, 6, dt=torch.int32), z(1, 6), step)         # beam > vocabulary
+    with pytest.raises(ValueError):
+        K.beam_search_step(z(1, 2, 5), z(1, 4, 2, dt=torch.int32), z(1, 2, dt=torch.float32), step)
+
+
+@pytest.mark.parametrize("shape,max_len,max_bps,dtype", [((2, 2, 1, 16), 4, 3, np.float16), ((3, 1, 40), 130, 2, np.float16),
+                                                           ((2, 1, 1, 128), 70, 1, np.uint8), ((1, 5, 1, 33), 65, 2, np.float32)])
+def test_kv_cache_pipeline_seq_last(K, shape, max_len, max_bps, dtype):
+    """transpose = 1: the registers keep the sequence as their last axis and shift in place; output and stored
+    registers against the oracle bit for bit, over more steps than the registers hold, then a second generation
+    from step 0 (which zeroes every register)."""
+    rng = np.random.default_rng(max_len + max_bps)
+    ref_op = O.KVCachePipeline(max_len, max_bps, transpose=True)
+    outer, inner = int(np.prod(shape[:-2])), shape[-1]
+    tdt = {np.float16: torch.float16, np.uint8: torch.uint8, np.float32: torch.float32}[dtype]
+    caches = torch.full((max_bps, outer, inner, max_len), 5, dtype=tdt, device="cuda")     # stale contents before step 0
+    out = torch.empty(shape[:-2] + (max_len, inner), dtype=tdt, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for it in list(range(max_bps * (max_len + 2))) + [0, 1, 2, 3]:
+        upd = rng.integers(0, 255, size=shape).astype(np.uint8) if dtype == np.uint8 else rng.standard_normal(shape).astype(dtype)
+        ref = ref_op(it, upd)
+        step.fill_(it)
+        K.kv_cache_pipeline_seq_last(caches, out, dev(upd), step, outer, max_len, inner, max_bps)
+        assert np.array_equal(host(out), ref), f"output differs at step {it}"
+        stored = np.stack([c.reshape(outer, inner, max_len) for c in ref_op.stored()])
+        assert np.array_equal(host(caches), stored), f"stored registers differ at step {it}"

@@ -403,3 +403,95 @@ def test_fp8_matmul_modes():
         O.fp8_matmul(x.astype(f32), w8, s, s)
     with pytest.raises(ValueError):
         O.f8_encode(x, "F999", 0)
+
+
+# ---------------------------------------------------------------- BeamSearch, KVCachePipeline transpose
+def _beam_brute_force(logits, hyps, scores, beam):
+    """Textbook beam step on explicit hypotheses: every (hypothesis, token) extension scored by
+    score + logit, the `beam` best kept (ties: lower hypothesis, then lower token).  No top-k per beam, no flat
+    candidate index, no container: an independent formulation of what the op computes for one sequence."""
+    ext = []
+    for i, (h, s) in enumerate(zip(hyps, scores)):
+        for v in range(logits.shape[1]):
+            ext.append((-(float(s) + float(logits[i, v])), i, v, h + [v]))
+    ext.sort(key=lambda e: (e[0], e[1], e[2]))
+    best = ext[:beam]
+    return [e[3] for e in best], [-e[0] for e in best], [e[1] for e in best], [e[2] for e in best]
+
+
+@pytest.mark.parametrize("beam,V", [(2, 7), (3, 11), (4, 6)])
+def test_beam_search_step_equals_brute_force(beam, V):
+    """fp32 scores drawn from a grid whose sums are exact and distinct, so the op's two-stage selection (top-k
+    per beam, then top-k of beam * beam) must keep exactly the brute-force best extensions: tokens, parent
+    hypotheses, scores and the whole hypothesis container, over several steps and two sequences."""
+    rng = np.random.default_rng(beam * 100 + V)
+    B, L, steps = 2, 6, 5
+    hyp = np.full((B, L, beam), -7, np.int32)
+    prob = np.zeros((B, beam), f32)
+    explicit = [None] * B
+    for step in range(steps):
+        # distinct values k / 1024 per sequence: sums of up to six of them stay exact in fp32
+        logits = np.stack([rng.permutation(beam * V * 40)[:beam * V].reshape(beam, V) for _ in range(B)]).astype(f32) / 1024
+        nxt, gbest, hyp, prob = O.beam_search_step(logits, hyp, prob, step, beam)
+        for b in range(B):
+            if step == 0:
+                order = np.argsort(-logits[b, 0], kind="stable")[:beam]
+                explicit[b] = ([[int(v)] for v in order], [float(logits[b, 0, v]) for v in order])
+                assert np.array_equal(nxt[b], order) and np.array_equal(gbest[b], order)
+            else:
+                hyps, scores, parents, toks = _beam_brute_force(logits[b], *explicit[b], beam)
+                explicit[b] = (hyps, scores)
+                assert np.array_equal(nxt[b], toks)
+                assert np.array_equal(gbest[b] // beam, parents)
+                # the flat index names the parent and the rank of the token among the parent's candidates
+                for r in range(beam):
+                    rank = int(np.argsort(-logits[b, parents[r]], kind="stable").tolist().index(toks[r]))
+                    assert gbest[b, r] == parents[r] * beam + rank
+            assert np.array_equal(prob[b], np.array(explicit[b][1], f32))
+            assert np.array_equal(hyp[b, :step + 1].T, np.array(explicit[b][0], np.int32))
+            assert (hyp[b, step + 1:] == -7).all()          # rows beyond the step are only permuted
+
+
+def test_beam_search_step_guards_dtype_and_ties():
+    logits = np.zeros((1, 2, 5), f16)
+    with pytest.raises(ValueError):
+        O.beam_search_step(logits[0], np.zeros((1, 4, 2), np.int32), np.zeros((1, 2), f16), 0, 2)
+    with pytest.raises(ValueError):
+        O.beam_search_step(logits, np.zeros((1, 4, 3), np.int32), np.zeros((1, 2), f16), 0, 2)
+    with pytest.raises(ValueError):
+        O.beam_search_step(logits, np.zeros((1, 4, 2), np.int32), np.zeros((1, 2), f16), 0, 6)
+    # equal scores come in ascending order of index, and the sum is rounded in the containers' type
+    nxt, gbest, hyp, prob = O.beam_search_step(logits, np.zeros((1, 4, 2), np.int32), np.zeros((1, 2), f16), 0, 2)
+    assert nxt.tolist() == [[0, 1]] and prob.dtype == f16
+    big = np.full((1, 2, 5), 2048.0, f16)
+    big[0, :, 1] = 1.0
+    _, gbest, _, prob = O.beam_search_step(big, hyp, np.array([[1.0, 0.0]], f16), 1, 2)
+    assert prob.tolist() == [[2048.0, 2048.0]] and gbest.tolist() == [[0, 1]]       # fp16(2048 + 1) = 2048: a tie
+    # a step beyond the container writes no row
+    _, _, h2, _ = O.beam_search_step(big, hyp, np.array([[1.0, 0.0]], f16), 9, 2)
+    assert np.array_equal(np.sort(h2, axis=2), np.sort(hyp[:, :, [0, 0]], axis=2))
+
+
+def test_kv_cache_pipeline_transposed_storage():
+    """transpose = 1: the output is that of transpose = 0, the stored registers are its transposes, and one call
+    moves every stored element one place along the last axis - the element loop of the codelet
+    (custom_ops/kv_cache_codelet.cpp:180-211) written out for a single feature row."""
+    rng = np.random.default_rng(31)
+    max_len, max_bps = 6, 2
+    plain, seq_last = O.KVCachePipeline(max_len, max_bps), O.KVCachePipeline(max_len, max_bps, transpose=True)
+    row = np.zeros(max_len, f16)                          # feature 3 of outer index (1, 0) in register 1
+    for step in list(range(9)) + [0, 1, 2]:               # a second generation restarts at step 0
+        upd = rng.standard_normal((2, 2, 1, 4)).astype(f16)
+        a, b = plain(step, upd), seq_last(step, upd)
+        assert np.array_equal(a, b)
+        for p, q in zip(plain.stored(), seq_last.stored()):
+            assert q.shape == (2, 2, 4, max_len) and np.array_equal(np.swapaxes(p, -1, -2), q)
+        if step == 0:
+            row[:] = 0
+        if step % max_bps == 1:
+            for j in range(max_len - 1, 0, -1):
+                row[j] = row[j - 1]
+            row[0] = upd[1, 0, 0, 3]
+        assert np.array_equal(seq_last.stored()[1][1, 0, 3], row)
+    with pytest.raises(ValueError):
+        O.KVCachePipeline(4, 2, step_len=2, transpose=True)
