@@ -100,16 +100,46 @@ __global__ __launch_bounds__(256) void f8_tile_kernel(const uint8_t* __restrict_
   tiled[vi] = o;
 }
 
-extern "C" size_t pta_fp8_tiled_bytes(int N, int K) { return gemv_tiled_bytes(N, K, 2); }
+// One flag byte per tile behind the tiles: nonzero when the tile holds one of the three codes whose F143 value is not
+// half of the OCP e4m3 value of the same bits (0x7F, 0xFF: +-240 against NaN; 0x80: NaN against -0).  The kernels that
+// feed the bytes to the FP8 matrix instruction multiply such a tile the exact way instead (gemm_f8n.h).
+__global__ __launch_bounds__(64) void f8_tile_flags_kernel(const u32x4* __restrict__ tiled, uint8_t* __restrict__ flags,
+                                                           size_t tiles) {
+  const size_t tile = blockIdx.x;
+  if (tile >= tiles) return;
+  bool special = false;
+#pragma unroll
+  for (int v = 0; v < 2; ++v) {
+    const u32x4 w = tiled[(tile * 2 + v) * 64 + threadIdx.x];
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t b = (w[d] >> (8 * i)) & 0xFFu;
+        special = special || b == 0x7Fu || b == 0xFFu || b == 0x80u;
+      }
+  }
+  const bool any = __any(special);
+  if (threadIdx.x == 0) flags[tile] = any ? 1 : 0;
+}
+
+extern "C" size_t pta_fp8_tiled_bytes(int N, int K) {
+  const size_t tiles = gemv_tiled_bytes(N, K, 2);
+  if (tiles == 0) return 0;
+  return tiles + ((tiles / 2048 + 15) & ~(size_t)15);
+}
 
 extern "C" int pta_fp8_tile(const uint8_t* w, void* tiled, int N, int K, int w_is_kn, pta_stream_t stream) {
   PTA_REQUIRE(w && tiled, "pta_fp8_tile: null pointer");
   PTA_REQUIRE(N > 0 && K > 0, "pta_fp8_tile: need N > 0 and K > 0, got N=%d K=%d", N, K);
   PTA_REQUIRE(pta_aligned(tiled, 16), "pta_fp8_tile: tiled buffer must be 16-byte aligned");
   const int KT = (K + 127) / 128;
-  const size_t total = pta_fp8_tiled_bytes(N, K) / 16;
+  const size_t tile_bytes = gemv_tiled_bytes(N, K, 2);
+  const size_t total = tile_bytes / 16;
   hipLaunchKernelGGL(f8_tile_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, w,
                      (u32x4*)tiled, N, K, KT, w_is_kn, total);
+  hipLaunchKernelGGL(f8_tile_flags_kernel, dim3((unsigned)(tile_bytes / 2048)), dim3(64), 0, (hipStream_t)stream,
+                     (const u32x4*)tiled, (uint8_t*)tiled + tile_bytes, tile_bytes / 2048);
   PTA_CHECK_LAUNCH("pta_fp8_tile");
   return PTA_OK;
 }

@@ -6,6 +6,7 @@
 // fp8: CastToUint8 + FP8MatMul; fp8_weight: FP8MatMul on fp16 activations; fp16: MatMul).
 #include "common.h"
 #include "formats.h"
+#include "gemm_f8n.h"
 
 int f8_decode_unscaled_launch(const uint8_t* in, f16* out, size_t n, int format, hipStream_t s);
 
@@ -15,9 +16,20 @@ static int run_linear(GemmArgs& a, int total_nb, int swiglu, hipStream_t s, cons
   return dispatch_gemv<Fmt, false>(a, total_nb, s, name);
 }
 
-extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_weight* host_w,
-                          const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
-                          const pta_fusion* fuse, pta_stream_t stream) {
+// PTA_FP8_NATIVE=0 in the environment keeps FP8 x FP8 products on the fp16 instruction (decode of both operands),
+// for comparisons; read once.
+static bool fp8_native_enabled() {
+  static const bool on = [] {
+    const char* v = getenv("PTA_FP8_NATIVE");
+    return !(v && v[0] == '0');
+  }();
+  return on;
+}
+
+// x_bytes: X holds F143 bytes [M, K] instead of fp16 values (FP8 weights of format F143 only)
+static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int count, const pta_weight* host_w,
+                       const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
+                       const pta_fusion* fuse, pta_stream_t stream) {
   PTA_REQUIRE(host_w && host_Y, "pta_linear: null pointer");
   PTA_REQUIRE(count >= 1 && count <= 4, "pta_linear: count must be in [1, 4], got %d", count);
   PTA_REQUIRE(!swiglu || count == 2, "pta_linear: a SwiGLU pair is exactly two weights (gate, up)");
@@ -59,12 +71,24 @@ extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, 
               "pta_linear: with several weights only the norm fields and the output cast of `fuse` apply (use host_bias for biases)");
   PTA_REQUIRE(!a.epi.out_fp8_scale || count == 1 || swiglu, "pta_linear: the output cast applies to one weight or to a SwiGLU pair");
   hipStream_t s = (hipStream_t)stream;
+  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || fp8_native_enabled())) {
+    // both operands F143: the FP8 matrix instruction (an uint8 left-hand side has no other path)
+    if (x_bytes) return swiglu ? dispatch_gemv_f8n<true, true>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, true>(a, nb, s, "pta_linear");
+    return swiglu ? dispatch_gemv_f8n<true, false>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, false>(a, nb, s, "pta_linear");
+  }
+  PTA_REQUIRE(!x_bytes, "pta_linear: an uint8 left-hand side needs F143 weights, M <= 16 and K >= 1024");
   switch (kind) {
     case PTA_W_INT4: return run_linear<FmtW4>(a, nb, swiglu, s, "pta_linear");
     case PTA_W_F16: return run_linear<FmtF16>(a, nb, swiglu, s, "pta_linear");
     case PTA_W_F143: return run_linear<FmtF8<0>>(a, nb, swiglu, s, "pta_linear");
     default: return run_linear<FmtF8<1>>(a, nb, swiglu, s, "pta_linear");
   }
+}
+
+extern "C" int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_weight* host_w,
+                          const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
+                          const pta_fusion* fuse, pta_stream_t stream) {
+  return linear_impl(X, x_scale, 0, count, host_w, host_bias, host_Y, M, swiglu, fuse, stream);
 }
 
 extern "C" size_t pta_linear_workspace_bytes(int M, int N) {
@@ -123,6 +147,12 @@ extern "C" int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_r
     PTA_REQUIRE(format_lhs == PTA_F143 || format_lhs == PTA_F152, "pta_fp8_gemm: unsupported fp8 format %d, it must be F143 or F152", format_lhs);
     PTA_REQUIRE(scale_lhs && workspace && pta_aligned(workspace, 16), "pta_fp8_gemm: an fp8 left-hand side needs its scale and a 16-byte aligned workspace");
     PTA_REQUIRE(M >= 1 && K >= 1, "pta_fp8_gemm: empty left-hand side");
+    if (format_lhs == PTA_F143 && format_rhs == PTA_F143 && M <= 16 && K >= 1024 && K % 8 == 0 && pta_aligned(lhs, 8) &&
+        fp8_native_enabled() && !(fuse && fuse->norm != PTA_NORM_NONE)) {
+      // the bytes go to the FP8 matrix instruction as they are
+      pta_weight w8{PTA_W_F143, tiled_rhs, scale_rhs, N, K, nullptr, PTA_ACT_NONE};
+      return linear_impl(lhs, scale_lhs, 1, 1, &w8, nullptr, &Y, M, 0, fuse, stream);
+    }
     f8_decode_unscaled_launch((const uint8_t*)lhs, (f16*)workspace, (size_t)M * K, format_lhs, (hipStream_t)stream);
     X = (const f16*)workspace;
     xs = scale_lhs;

@@ -212,7 +212,7 @@ class F8Weight:
         self.N, self.K = (w.shape[1], w.shape[0]) if kn else w.shape
         self.scale = scale
         lib = _lib.load()
-        self.tiled = torch.empty(lib.pta_fp8_tiled_bytes(self.N, self.K), dtype=torch.uint8, device=w.device)
+        self.tiled = torch.zeros(lib.pta_fp8_tiled_bytes(self.N, self.K), dtype=torch.uint8, device=w.device)
         check(lib.pta_fp8_tile(_p(w), _p(self.tiled), self.N, self.K, 1 if kn else 0, _stream()))
 
     @property

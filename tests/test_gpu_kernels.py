@@ -932,3 +932,70 @@ def test_kv_cache_pipeline_seq_last(K, shape, max_len, max_bps, dtype):
         assert np.array_equal(host(out), ref), f"output differs at step {it}"
         stored = np.stack([c.reshape(outer, inner, max_len) for c in ref_op.stored()])
         assert np.array_equal(host(caches), stored), f"stored registers differ at step {it}"
+
+
+# ---------------------------------------------------------------- FP8 x FP8 on the FP8 matrix instruction
+def _f143_case(rng, M, Kdim, N, scale, specials):
+    """Random F143 bytes for both operands; with `specials`, the three codes whose value is not half of the OCP
+    value of the same bits (+240, -240 and, optionally, NaN) are placed in weights and activations."""
+    x8 = O.f8_encode(rng.standard_normal((M, Kdim)).astype(np.float16), "F143", scale)
+    w8 = O.f8_encode((rng.standard_normal((Kdim, N)) * 0.02).astype(np.float32), "F143", scale)
+    if specials:
+        w8[3, 0], w8[Kdim - 1, N - 1], w8[130, min(17, N - 1)] = 0x7F, 0xFF, 0x7F
+        x8[0, 5], x8[M - 1, Kdim - 2] = 0x7F, 0xFF
+        w8[7, 1], x8[0, 200] = 0x01, 0x81                   # the smallest subnormals
+    return x8, w8
+
+
+@pytest.mark.parametrize("M,Kdim,N", [(1, 4096, 48), (8, 4096, 8192), (16, 1160, 13696), (5, 13696, 4096)])
+@pytest.mark.parametrize("specials", [False, True])
+def test_fp8_products_on_the_fp8_matrix_instruction(K, M, Kdim, N, specials):
+    """Both operands F143, up to 16 rows: the bytes go to the FP8 instruction as they are.  Left-hand side as bytes
+    and as fp16 values on the grid; one, two and three channel blocks per workgroup; a ragged last feature tile;
+    +-240 and subnormals in both operands (steps holding +-240 are multiplied through exact fp16 decodes)."""
+    rng = np.random.default_rng(M + Kdim + N)
+    scale = -1
+    x8, w8 = _f143_case(rng, M, Kdim, N, scale, specials)
+    sd = dev(np.array([scale], np.int32))
+    fw = K.F8Weight(dev(w8), sd, "F143", kn=True)
+    ref = O.fp8_matmul(x8, w8, [scale], [scale], "F143", "F143")
+    tol = 2.0 ** -10 * np.abs(ref.astype(np.float64)).max()                    # one fp16 rounding of the largest output
+    got = host(K.fp8_gemm(dev(x8), fw, K.fp8_gemm_workspace(M, Kdim, "cuda"), x_scale=sd, x_format="F143"))
+    assert np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() <= tol
+    xg = dev(O.f8_decode(x8, "F143", 0, np.float16))                           # the same activations as grid values
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    K.linear(xg, [fw], [out], x_scale=sd)
+    assert np.abs(host(out).astype(np.float64) - ref.astype(np.float64)).max() <= tol
+
+
+def test_fp8_products_pair_multi_and_nan(K):
+    rng = np.random.default_rng(77)
+    M, Kdim, N, scale = 8, 4096, 13696, -2
+    sd = dev(np.array([scale], np.int32))
+    x8, wg8 = _f143_case(rng, M, Kdim, N, scale, True)
+    _, wu8 = _f143_case(rng, M, Kdim, N, scale, True)
+    xg = dev(O.f8_decode(x8, "F143", 0, np.float16))
+    g, u = K.F8Weight(dev(wg8), sd, "F143", kn=True), K.F8Weight(dev(wu8), sd, "F143", kn=True)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    K.linear(xg, [g, u], [out, out], x_scale=sd, swiglu=True)
+    rg, ru = (O.fp8_matmul(x8, w, [scale], [scale]) for w in (wg8, wu8))
+    ref = (ru * O.swish(rg)).astype(np.float16)
+    assert rel_err(host(out), ref) <= 1e-2
+    # two matrices of different widths in one launch, each with a bias
+    _, w2 = _f143_case(rng, M, Kdim, 512, scale, True)
+    b1, b2 = rng.standard_normal(N).astype(np.float16), rng.standard_normal(512).astype(np.float16)
+    o1, o2 = torch.empty((M, N), dtype=torch.float16, device="cuda"), torch.empty((M, 512), dtype=torch.float16, device="cuda")
+    K.linear(xg, [g, K.F8Weight(dev(w2), sd, "F143", kn=True)], [o1, o2], biases=[dev(b1), dev(b2)], x_scale=sd)
+    assert rel_err(host(o1), (rg + b1).astype(np.float16)) <= 1e-2
+    assert rel_err(host(o2), (O.fp8_matmul(x8, w2, [scale], [scale]) + b2).astype(np.float16)) <= 1e-2
+    # the NaN code: as a weight it poisons its output channel, as an activation its row - and nothing else
+    wn, xn = wg8.copy(), x8.copy()
+    wn[900, 33] = 0x80
+    xn[2, 1000] = 0x80
+    got = host(K.fp8_gemm(dev(xn), K.F8Weight(dev(wn), sd, "F143", kn=True), K.fp8_gemm_workspace(M, Kdim, "cuda"),
+                          x_scale=sd, x_format="F143"))
+    with np.errstate(invalid="ignore"):
+        ref = O.fp8_matmul(xn, wn, [scale], [scale])
+    assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.isnan(ref[2]).all() and np.isnan(ref[:, 33]).all()
+    ok = ~np.isnan(ref)
+    assert np.abs(got[ok].astype(np.float64) - ref[ok].astype(np.float64)).max() <= 2.0 ** -10 * np.abs(ref[ok].astype(np.float64)).max()
