@@ -9,7 +9,10 @@
 // holds one of the three codes is multiplied the other way instead: both operands decoded exactly to fp16 (every
 // F143 value is an fp16 value) into the fp16 instruction, with a second accumulator.  Which weight tiles hold such
 // a code is recorded once, when the weights are tiled (one flag byte per tile behind the tiles); the activations
-// are checked as they are loaded.
+// are checked as they are loaded.  Activations of +-240 are what a saturating cast leaves, so they can be frequent;
+// they stay on the FP8 instruction: 240 = 224 + 16, both F143 values with OCP bytes, so the step is multiplied twice,
+// once with 224 and once with 16 in the places of the 240s (zero elsewhere), which is exact.  Only a NaN activation
+// sends a step the slow way.
 //
 // Activations arrive either as F143 bytes [M, K] (an uint8 left-hand side, as the reference's FP8MatMul takes it)
 // or as fp16 values on the F143 grid without their scale (what pta_half_to_fp8_grid and the producers' output
@@ -26,8 +29,8 @@ __host__ __device__ inline size_t f8_tile_flags_offset(int N, int K) {
   return (size_t)((N + 15) / 16) * (size_t)((K + 127) / 128) * 2048;
 }
 
-// 8 fp16 values on the F143 grid (|v| <= 240 or NaN) -> their 8 F143 bytes, and whether any of them is 240, -240 or
-// NaN.  v * 2^-7 is exact (an F143 subnormal becomes an fp16 subnormal) and carries the byte's exponent and
+// 8 fp16 values on the F143 grid (|v| <= 240 or NaN) -> their 8 F143 bytes (+-240 -> 0x7F / 0xFF), and whether any of
+// them is beyond 240 (NaN).  v * 2^-7 is exact (an F143 subnormal becomes an fp16 subnormal) and carries the byte's exponent and
 // mantissa in bits 13..7 of each half.
 __device__ __forceinline__ u32x2 f143_bytes_of_grid(f16x8 v, bool& special) {
   const u32x4 d = bitcast<u32x4>(v);
@@ -45,25 +48,37 @@ __device__ __forceinline__ u32x2 f143_bytes_of_grid(f16x8 v, bool& special) {
     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(b) : "v"(t >> 7), "s"(0x007F007Fu), "v"(sign));
     p[i] = b;      // byte of the low half in bits 7..0, of the high half in bits 23..16
   }
-  special = big >= 0x5B80u;      // fp16 240.0 and everything above it, NaN included
+  special = big > 0x5B80u;       // above fp16 240.0: NaN (a grid value is never larger)
   u32x2 r;
   r[0] = __builtin_amdgcn_perm(p[1], p[0], 0x06040200u);
   r[1] = __builtin_amdgcn_perm(p[3], p[2], 0x06040200u);
   return r;
 }
 
-// whether any of the 8 bytes is 0x7F, 0xFF or 0x80
-__device__ __forceinline__ bool f143_has_special(u32x2 q) {
+// whether any of the 8 bytes is 0x80 (NaN)
+__device__ __forceinline__ bool f143_has_nan(u32x2 q) {
   bool s = false;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const uint32_t t = q[i] & 0x7F7F7F7Fu;
-    const uint32_t is7f = (t + 0x01010101u) & 0x80808080u;                 // low seven bits all ones
-    const uint32_t nonzero = (t + 0x7F7F7F7Fu) & 0x80808080u;              // low seven bits not all zero
-    const uint32_t is80 = q[i] & ~nonzero & 0x80808080u;
-    s = s || (is7f | is80) != 0;
+    const uint32_t nonzero = ((q[i] & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) & 0x80808080u;      // low seven bits not all zero
+    s = s || (q[i] & ~nonzero & 0x80808080u) != 0;
   }
   return s;
+}
+
+// Splits the bytes 0x7F / 0xFF (+-240) of q into +-224 (0x7E / 0xFE, left in q) and +-16 (0x60 / 0xE0, returned; zero
+// bytes elsewhere).  Returns whether there was any.
+__device__ __forceinline__ bool f143_split_240(u32x2& q, u32x2& extra) {
+  bool any = false;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint32_t is7f = ((q[i] & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u;         // 0x80 where the low seven bits are all ones
+    const uint32_t one = is7f >> 7;
+    extra[i] = one * 0x60u | (q[i] & is7f);
+    q[i] -= one;
+    any = any || is7f != 0;
+  }
+  return any;
 }
 
 // exact decode of 8 bytes, NaN for 0x80 (the slow path takes no shortcuts; kept out of line: it is rare)
@@ -133,42 +148,48 @@ __global__ __launch_bounds__(WIDE_WAVES * 64) void gemv_f8n_kernel(GemmArgs a, i
         for (int v = 0; v < 2; ++v) w[b][g][v] = __builtin_nontemporal_load(wp[b][g] + ((size_t)kt * 2 + v) * 64);
         fl[b][g] = flags[b][g][kt];
       }
-    u32x2 xq[4];
-    unsigned xspecial = 0;      // bit j: step j of this tile holds a special activation (same in every lane)
+    u32x2 xq[4], xe[4];
+    unsigned xnan = 0, xsplit = 0;   // bit j: step j holds a NaN activation / activations of +-240 (same in every lane)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k = kt * 128 + j * 32;
       const bool in = k + (lane >> 4) * 8 < K;
-      bool sp = false;
+      bool nan = false;
       if constexpr (XBYTES) {
         xq[j] = in ? *reinterpret_cast<const u32x2*>(xq8 + k) : u32x2{0, 0};
-        sp = f143_has_special(xq[j]);
+        nan = f143_has_nan(xq[j]);
       } else {
         const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        xq[j] = f143_bytes_of_grid(in ? *reinterpret_cast<const f16x8*>(xh + k) : z, sp);
+        xq[j] = f143_bytes_of_grid(in ? *reinterpret_cast<const f16x8*>(xh + k) : z, nan);
       }
-      if (__any(sp)) xspecial |= 1u << j;
+      if (__any(nan)) xnan |= 1u << j;
+      if (__any(f143_split_240(xq[j], xe[j]))) xsplit |= 1u << j;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const long xb = bitcast<long>(xq[j]);
+      const long xb = bitcast<long>(xq[j]), xb2 = bitcast<long>(xe[j]);
+      const bool split = (xsplit >> j) & 1u;
 #pragma unroll
       for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int g = 0; g < NACC; ++g) {
           const uint32_t lo = w[b][g][j >> 1][(j & 1) * 2], hi = w[b][g][j >> 1][(j & 1) * 2 + 1];
-          const bool slow = __builtin_amdgcn_readfirstlane(fl[b][g]) != 0 || ((xspecial >> j) & 1u);
+          const bool slow = __builtin_amdgcn_readfirstlane(fl[b][g]) != 0 || ((xnan >> j) & 1u);
           if (!slow) {
-            acc[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(bitcast<long>(u32x2{lo, hi}), xb, acc[b][g], 0, 0, 0);
+            const long wb = bitcast<long>(u32x2{lo, hi});
+            acc[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wb, xb, acc[b][g], 0, 0, 0);
+            if (split) acc[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(wb, xb2, acc[b][g], 0, 0, 0);
           } else {
-            const int k = kt * 128 + j * 32;
-            f16x8 xe;
-            if constexpr (XBYTES) xe = f143_decode8_exact(xq[j][0], xq[j][1]);
+            // both operands decoded exactly; the activation bytes are put together again first (224 + 16 -> 240)
+            const u32x2 whole = {xq[j][0] + ((xe[j][0] >> 6) & 0x01010101u), xq[j][1] + ((xe[j][1] >> 6) & 0x01010101u)};
+            f16x8 xv;
+            if constexpr (XBYTES) xv = f143_decode8_exact(whole[0], whole[1]);
             else {
+              const int k = kt * 128 + j * 32;
               const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-              xe = k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xh + k) : z;
+              xv = k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xh + k) : z;
             }
-            accx[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f143_decode8_exact(lo, hi), xe, accx[b][g], 0, 0, 0);
+            accx[b][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f143_decode8_exact(lo, hi), xv, accx[b][g], 0, 0, 0);
           }
         }
     }

@@ -71,8 +71,14 @@ static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int c
               "pta_linear: with several weights only the norm fields and the output cast of `fuse` apply (use host_bias for biases)");
   PTA_REQUIRE(!a.epi.out_fp8_scale || count == 1 || swiglu, "pta_linear: the output cast applies to one weight or to a SwiGLU pair");
   hipStream_t s = (hipStream_t)stream;
-  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || fp8_native_enabled())) {
-    // both operands F143: the FP8 matrix instruction (an uint8 left-hand side has no other path)
+  // Both operands F143: the FP8 matrix instruction.  fp16 grid values are turned into bytes by every workgroup that
+  // reads them (about 60 vector instructions per 32-feature step), which pays only when the bytes feed several
+  // products.  Measured at the ChatGLM2-6B shape, 8 rows, saturating activations (every step multiplied twice, 224
+  // and 16): the SwiGLU pair 31.2 against 32.5 us on the fp16 instruction with decoded weights; one channel block per
+  // workgroup (4096 x 4096) 16.2 against 11.5 us, q | kv and the lm_head slower as well.  So fp16 grid values take
+  // this path for the SwiGLU pair only; an uint8 left-hand side always comes here.
+  const bool several = swiglu != 0;
+  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || (fp8_native_enabled() && several))) {
     if (x_bytes) return swiglu ? dispatch_gemv_f8n<true, true>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, true>(a, nb, s, "pta_linear");
     return swiglu ? dispatch_gemv_f8n<true, false>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, false>(a, nb, s, "pta_linear");
   }
