@@ -263,16 +263,17 @@ def other_model_workload(args):
 
 def prompt_workload(args):
     """The prompt of the Llama2-7B-shape INT4 model in passes (FusedDecoder.consume_prompt): a step is one pass of
-    64 // batch consecutive positions of every sequence through the 32 blocks (no head: the loop discards the
+    --rows-per-pass // batch consecutive positions of every sequence through the 32 blocks (no head: the loop discards the
     tokens of these positions).  --steps passes are timed after one untimed run of the same prompt; the number of
     passes is capped by the KV cache length."""
     import torch
     from poptransformer_amd.engine import fused, loader, synthetic
     B, cfg = args.batch, LLAMA2_7B
-    if B > 64:
-        print("the prompt passes take at most 64 rows: batch <= 64", file=sys.stderr)
+    rows = args.rows_per_pass
+    if B > rows or rows > 256:
+        print("the prompt passes take at most 256 rows: batch <= --rows-per-pass <= 256", file=sys.stderr)
         sys.exit(2)
-    R = 64 // B
+    R = rows // B
     passes = max(1, min(args.steps, (MAX_LEN - 2) // R))
     n = passes * R
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
@@ -281,11 +282,13 @@ def prompt_workload(args):
     ids = np.zeros((B, MAX_LEN), np.int32)
     ids[:, :n + 1] = rng.integers(3, cfg["vocab_size"], size=(B, n + 1))
     dec.reset(ids)
-    dec.consume_prompt(n)                      # untimed: allocates the row buffers, warms every code path
+    dec.consume_prompt(n, rows_per_pass=R)     # untimed: allocates the row buffers, warms every code path
+    dec.reset(ids)
+    dec.consume_prompt(n, rows_per_pass=R)     # untimed: records the pass into a HIP graph
     dec.reset(ids)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    dec.consume_prompt(n)
+    dec.consume_prompt(n, rows_per_pass=R)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     d, f, nl = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
@@ -322,6 +325,8 @@ def main():
                          "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
                          "rwkv: RWKV-4-7B-shape INT4 recurrent decode; prompt: the headline model's prompt in passes "
                          "of up to 64 rows (--steps passes)")
+    ap.add_argument("--rows-per-pass", type=int, default=64,
+                    help="prompt workload: rows (batch x positions) per pass, up to 256")
     ap.add_argument("--fp8-cache", action="store_true",
                     help="decode workload, operators executor: keep the KV cache as F143 bytes (KVCacheOp with fp8 = true)")
     ap.add_argument("--fuse-norm", choices=["on", "off"], default=None,

@@ -119,6 +119,7 @@ struct GemmArgs {
   int ksplit;          // 0 or 1: no split
 };
 constexpr int GEMM_MAX_KSPLIT = 4;
+constexpr int GEMM_MAX_ROWS = 256;
 
 template <class Fmt, int MT, int NW, bool PAIR>
 __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
@@ -776,14 +777,25 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     if (kt < KT) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        f16x8 xb[MT];
+        if constexpr (MT <= 4) {
+          f16x8 xb[MT];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xb[mt] = *reinterpret_cast<const f16x8*>(cur + mt * 16 * TILE_XSTRIDE + m * 32);
+          for (int mt = 0; mt < MT; ++mt) xb[mt] = *reinterpret_cast<const f16x8*>(cur + mt * 16 * TILE_XSTRIDE + m * 32);
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          const f16x8 av = Fmt::a_operand(w_cur[st], m, sc[st]);
+          for (int st = 0; st < 2; ++st) {
+            const f16x8 av = Fmt::a_operand(w_cur[st], m, sc[st]);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[st][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[mt], acc[st][mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt) acc[st][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[mt], acc[st][mt], 0, 0, 0);
+          }
+        } else {
+          // many row groups: both weight fragments decoded once, then one activation fragment at a time feeds both
+          const f16x8 av0 = Fmt::a_operand(w_cur[0], m, sc[0]), av1 = Fmt::a_operand(w_cur[1], m, sc[1]);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const f16x8 xb = *reinterpret_cast<const f16x8*>(cur + mt * 16 * TILE_XSTRIDE + m * 32);
+            acc[0][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av0, xb, acc[0][mt], 0, 0, 0);
+            acc[1][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av1, xb, acc[1][mt], 0, 0, 0);
+          }
         }
       }
     }
@@ -797,6 +809,38 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     __syncthreads();
   }
 
+  if constexpr (KQ == 1) {
+    // one K group: every wave holds finished sums.  Lane l has channels (l / 16) * 4 + r, r = 0..3, of row l % 16 of
+    // each row group, for both of its streams.
+    const GemmMat& mat = a.mat[PAIR ? 0 : mi];
+    const int N = mat.N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + (lane & 15);
+      if (m >= M) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (PAIR) {
+          const int n = nb[0] * 16 + (lane >> 4) * 4 + r;
+          if (n >= N) continue;
+          const f16 gate = (f16)Fmt::finish(acc[0][mt][r], sc[0]), up = (f16)Fmt::finish(acc[1][mt][r], sc[1]);
+          mat.Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
+        } else {
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            const int n = nb[st] * 16 + (lane >> 4) * 4 + r;
+            if (n >= N) continue;
+            if (nsl > 1) { a.part[((size_t)blockIdx.y * M + m) * N + n] = acc[st][mt][r]; continue; }
+            f16 y0 = (f16)Fmt::finish(acc[st][mt][r], sc[st]);
+            if (mat.bias) y0 = y0 + mat.bias[n];
+            y0 = apply_act(mat.act, y0);
+            mat.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
+          }
+        }
+      }
+    }
+    return;
+  }
   // partial sums of the K groups meet in LDS (the staging area is free after the last barrier)
 #pragma unroll
   for (int st = 0; st < 2; ++st)
@@ -870,7 +914,7 @@ static int launch_gemm_tile(const GemmArgs& a, int total_nb, hipStream_t s, cons
   static bool ready = false;
   constexpr int WPG = TILE_WAVES / KQ;
   const size_t stage = (size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2;
-  const size_t redb = (size_t)TILE_WAVES * 2 * MT * 256 * 4;
+  const size_t redb = KQ == 1 ? 0 : (size_t)TILE_WAVES * 2 * MT * 256 * 4;      // one K group: no meeting in LDS
   const size_t smem = stage > redb ? stage : redb;
   static_assert((size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2 <= 160 * 1024, "staging beyond the LDS of a compute unit");
   if (!ready) {
@@ -936,7 +980,51 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 }
 
 template <class Fmt, bool PAIR>
+static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name);
+
+// 65..256 rows.  Up to 128 rows, where the channel blocks divide into workgroup tiles: the staged kernel with 8 row
+// groups (2 K groups of 4 waves; 8 channel blocks or 4 SwiGLU pairs per workgroup), every weight tile decoded once for
+// all rows; a single matrix with few channels also splits K when a workspace is at hand.  Otherwise, and beyond 128
+// rows, the rows go through the smaller paths in turn, 128 or 64 at a time.  (A variant with 16 row groups per wave
+// was measured: it needs more registers than a wave has - 41..53 spilled - and ran 10 times slower.)
+template <class Fmt, bool PAIR>
+static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  const int cus = device_compute_units();
+  const int per_wg = PAIR ? 4 : 8;
+  const bool tiles = a.epi.norm == PTA_NORM_NONE && tile_fits(a, per_wg, 2, PAIR);
+  if (tiles && a.M <= 128) {
+    GemmArgs b = a;
+    const int wgs = total_nb / per_wg;
+    int nsl = wgs > 0 ? cus / wgs : 1;
+    nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
+    while (nsl > 1 && a.KT < nsl * 8) --nsl;
+    if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
+    const int rc = launch_gemm_tile<Fmt, 8, 2, PAIR>(b, total_nb, s, name);
+    if (rc) return rc;
+    PTA_CHECK_LAUNCH(name);
+    return PTA_OK;
+  }
+  const int chunk = tiles ? 128 : 64;
+  for (int m0 = 0; m0 < a.M; m0 += chunk) {
+    GemmArgs b = a;
+    b.M = a.M - m0 < chunk ? a.M - m0 : chunk;
+    if (b.X) b.X += (size_t)m0 * a.K;
+    for (int i = 0; i < a.count; ++i) {
+      if (b.mat[i].X) b.mat[i].X += (size_t)m0 * a.K;
+      if (!PAIR || i == 0) b.mat[i].Y += (size_t)m0 * a.mat[i].N;
+    }
+    if (PAIR) b.mat[1].Y = b.mat[0].Y;
+    if (b.epi.residual) b.epi.residual += (size_t)m0 * a.mat[0].N;
+    if (b.epi.mul) b.epi.mul += (size_t)m0 * a.mat[0].N;
+    const int rc = dispatch_gemv<Fmt, PAIR>(b, total_nb, s, name);
+    if (rc) return rc;
+  }
+  return PTA_OK;
+}
+
+template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  if (a.M > 64) return dispatch_many_rows<Fmt, PAIR>(a, total_nb, s, name);
   const size_t xbytes = (size_t)a.M * (a.KT * 128 + 8) * 2;
   bool all_shared_x = true;
   for (int i = 0; i < a.count; ++i) all_shared_x = all_shared_x && a.mat[i].X == nullptr;
@@ -994,7 +1082,7 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
 
 static inline int check_gemv_common(const char* name, const void* X, int M, int K) {
   PTA_REQUIRE(X, "%s: null X", name);
-  PTA_REQUIRE(M >= 1 && M <= 64, "%s: M must be in [1, 64], got %d", name, M);
+  PTA_REQUIRE(M >= 1 && M <= GEMM_MAX_ROWS, "%s: M must be in [1, %d], got %d", name, GEMM_MAX_ROWS, M);
   PTA_REQUIRE(K > 0 && (K % 8) == 0, "%s: K must be a positive multiple of 8, got %d", name, K);
   PTA_REQUIRE(pta_aligned(X, 16), "%s: X must be 16-byte aligned", name);
   return PTA_OK;

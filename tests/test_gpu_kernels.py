@@ -263,7 +263,7 @@ def test_w4a16_guards(K):
     with pytest.raises(ValueError):
         K.w4a16_gemm(dev(np.zeros((1, 64), np.float16)), w)
     with pytest.raises(ValueError):
-        K.w4a16_gemm(dev(np.zeros((65, 128), np.float16)), w)
+        K.w4a16_gemm(dev(np.zeros((257, 128), np.float16)), w)
 
 
 # ---------------------------------------------------------------- FP16 GEMM
@@ -999,3 +999,52 @@ def test_fp8_products_pair_multi_and_nan(K):
     assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.isnan(ref[2]).all() and np.isnan(ref[:, 33]).all()
     ok = ~np.isnan(ref)
     assert np.abs(got[ok].astype(np.float64) - ref[ok].astype(np.float64)).max() <= 2.0 ** -10 * np.abs(ref[ok].astype(np.float64)).max()
+
+
+# ---------------------------------------------------------------- 65..256 rows
+@pytest.mark.parametrize("M", [65, 128, 200, 256])
+@pytest.mark.parametrize("Kdim,N", [(4096, 4096), (1160, 8192), (11008, 4096), (512, 100)])
+def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
+    """More than 64 rows: the staged kernel with 8 or 16 row groups (with and without the K split that a workspace
+    allows; 1160 features = a ragged last tile), and for channel counts that do not divide into its workgroup tiles
+    (100) the 64-row paths over the rows in turn.  Bias, and a residual that aliases the output."""
+    x, packed, scale = _w4_case(M + Kdim + N, M, Kdim, N)
+    rng = np.random.default_rng(M * N)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    ref = ((O.w4a16_matmul(x, packed, scale) + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res))), ref) <= 1e-2
+    ws = K.linear_workspace(M, N, "cuda")
+    ws.fill_(0xFF)
+    y = dev(res.copy())
+    K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=y, out=y, workspace=ws)
+    assert rel_err(host(y), ref) <= 1e-2
+
+
+def test_gemm_up_to_256_rows_exact_integers_pair_and_other_formats(K):
+    rng = np.random.default_rng(61)
+    for M in (96, 256):
+        Kdim, N = 1024, 8192
+        x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
+        q = rng.integers(-8, 8, size=(N, Kdim))
+        w = K.W4Weight(dev(O.pack_int4(q)), dev(np.ones(N, np.float16)))
+        assert np.array_equal(host(K.w4a16_gemm(dev(x), w)).astype(np.int64), x.astype(np.int64) @ q.T.astype(np.int64))
+        # SwiGLU pair, three matrices in one launch
+        xr = rng.standard_normal((M, Kdim)).astype(np.float16)
+        mats = [(rng.integers(-128, 128, size=(n, Kdim // 2), dtype=np.int8), rng.uniform(0.005, 0.02, size=(n,)).astype(np.float16))
+                for n in (11008, 11008, 4096, 2048)]
+        ws = [K.W4Weight(dev(p), dev(s_)) for p, s_ in mats]
+        got = host(K.w4a16_gemm_swiglu(dev(xr), ws[0], ws[1]))
+        ref = (O.w4a16_matmul(xr, *mats[1]) * O.swish(O.w4a16_matmul(xr, *mats[0]))).astype(np.float16)
+        assert rel_err(got, ref) <= 1e-2
+        for (p, s_), o in zip(mats[1:], K.w4a16_gemm_multi(dev(xr), ws[1:])):
+            assert rel_err(host(o), O.w4a16_matmul(xr, p, s_)) <= 1e-2
+        # fp16 and FP8 weights
+        wf = (rng.standard_normal((768, Kdim)) * 0.05).astype(np.float16)
+        assert rel_err(host(K.f16_gemm(dev(xr), K.F16Weight(dev(wf)))), O.matmul(xr, wf.T.copy())) <= 1e-2
+        w8 = O.f8_encode((rng.standard_normal((Kdim, 4096)) * 0.02).astype(np.float32), "F143", -1)
+        fw = K.F8Weight(dev(w8), dev(np.array([-1], np.int32)), "F143", kn=True)
+        assert rel_err(host(K.fp8_gemm(dev(xr), fw, K.fp8_gemm_workspace(M, Kdim, "cuda"))), O.fp8_matmul(xr, w8, [-1], [-1])) <= 1e-2
+    with pytest.raises(ValueError):
+        K.w4a16_gemm(dev(rng.standard_normal((257, 1024)).astype(np.float16)), w)
