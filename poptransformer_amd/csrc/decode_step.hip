@@ -303,12 +303,13 @@ struct NoScales {};
 // SCALED: the sums are over stored codes q + 8; 8 * sum(x) (xsum: per-wave partial sums of the staged
 // activations) comes off and the channel's scale (SC[scbase + r] of the finishing lane, whose
 // channel is lane % 16) is applied before the rounding to fp16.
-template <int NRB, int EPI, bool SCALED = false, class Scales = NoScales>
+template <int NRB, int EPI, bool SCALED = false, class Scales = NoScales, int MB = DS_MAXB, int RED = DS_RED>
 __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (&out)[NRB], int ostride, f16 res, int u,
                                            int N, int M, float* red, int& red_buf, const float* xsum = nullptr,
                                            const Scales& SC = Scales{}, int scbase = 0) {
+  constexpr int DS_MAXB = MB;      // rows a reduction buffer has room for (shadows the narrow kernel's constant)
   const int wave = wave_id(), lane = lane_id();
-  float* rb = red + red_buf * DS_RED;
+  float* rb = red + red_buf * RED;
   if ((lane & 15) < M) {
 #pragma unroll
     for (int r = 0; r < NRB; ++r)
@@ -1087,15 +1088,388 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------ 5..16 sequences
+// The same iteration for up to 16 sequences.  Sixteen activation rows no longer fit in LDS next to the reduction
+// buffers (16 x 4096 halves are 128 KiB, 16 x 11008 are 344), so nothing is staged: a wave multiplies K tiles
+// wave, wave + 16, ... and therefore needs, of every activation row, exactly the features of ITS tiles - it loads
+// them itself, as the B operands of its products (lane l: row l % 16, features (l / 16) * 8 + 0..7 of each 32-feature
+// step), straight from the producer's slot, polling until no element is the filler.  Every element of a slot is read
+// by exactly one wave of the workgroup.  RMS statistics and the sums of the rows (for the offset of the stored INT4
+// codes) are partial per wave and meet in LDS.
+constexpr int DW_MAXB = 16;
+constexpr int DW_RED = DS_WAVES * 3 * 256;                  // floats of one reduction buffer: up to three matrices
+constexpr int DW_TAIL_FLOATS = 2 * DS_WAVES * DW_MAXB + 64 + 4;   // norm sums | row sums | selection scratch | flags
+
+struct XTile {
+  f16x8 v[4];      // the four 32-feature steps of one K tile
+};
+
+// This wave's fragments of K tile kt of X (fp16 [M, K], a producer's slot): loaded until none of their elements is the
+// filler.  Returns false when the wait was given up.  Features beyond K read as zero.
+__device__ __forceinline__ bool fetch_xtile(const f16* X, int M, int K, int kt, XTile& t, Waiter& w) {
+  const int lane = lane_id();
+  int row = lane & 15;
+  row = row < M ? row : M - 1;                // padding rows repeat the last one; their products are never stored
+  u32x4 v[4];
+  bool need[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v[j] = u32x4{0, 0, 0, 0};
+    need[j] = kt * 128 + j * 32 + (lane >> 4) * 8 < K;
+  }
+  for (;;) {
+    bool pending = false;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (need[j]) v[j] = get16(X, (size_t)M * K * 2, ((size_t)row * K + kt * 128 + j * 32 + (lane >> 4) * 8) * 2);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (need[j]) {
+        if (has_empty16(v[j])) pending = true;
+        else need[j] = false;
+      }
+    if (!__any(pending) || w.give_up()) break;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) t.v[j] = bitcast<f16x8>(v[j]);
+  return *w.lds_dead == 0;
+}
+
+// sums over the lane groups that share a row: afterwards lanes 0..15 (and their images) hold the row's total of the wave
+__device__ __forceinline__ float rows_of_wave(float v) {
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// RMSNorm of the rows whose fragments the waves hold (layers/rms_layer_norm.py:26-36, as pta_rmsnorm): the sums of
+// squares meet in LDS, every lane then scales its own fragments.  NT tiles per wave; tiles beyond KT hold zeros.
+template <int NT>
+__device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* norm_w, int K, int KT, float eps, float* sums) {
+  const int lane = lane_id(), wave = wave_id();
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const float f = (float)t[i].v[j][e]; sq = __builtin_fmaf(f, f, sq); }
+  sq = rows_of_wave(sq);
+  if (lane < 16) sums[wave * DW_MAXB + lane] = sq;
+  wg_sync();
+  float tot = 0.f;
+#pragma unroll
+  for (int ww = 0; ww < DS_WAVES; ++ww) tot += sums[ww * DW_MAXB + (lane & 15)];
+  const f16 r16 = (f16)(1.0f / sqrtf(tot * (1.0f / (float)K) + eps));
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int kt = wave + i * DS_WAVES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = kt * 128 + j * 32 + (lane >> 4) * 8;
+      if (kt < KT && k < K) {
+        const f16x8 gm = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(norm_w) + k);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[i].v[j][e] = (t[i].v[j][e] * r16) * gm[e];
+      }
+    }
+  }
+}
+
+// The rows' sums over this wave's fragments go to LDS (the INT4 products multiply by the stored codes q + 8 and take
+// 8 * sum(x) off at the end); `first`: the first contribution of the phase replaces what the slot held.
+template <int NT>
+__device__ __forceinline__ float xtiles_rowsum(const XTile (&t)[NT]) {
+  float s1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s1 += (float)t[i].v[j][e];
+  return rows_of_wave(s1);
+}
+
+// acc[r][0 / 1] += the products of tile `i` of unit u's NRB matrices (places BASE + r * TPW + i) with the fragments x
+template <int NRB, int TPW, int BASE, int NSLOT>
+__device__ __forceinline__ void wide_tile_product(const u32x4 (&S)[NSLOT], f32x4 (&acc)[NRB][2], int i, const XTile& x) {
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+#pragma unroll
+    for (int r = 0; r < NRB; ++r) {
+      const u32x4 wv = S[BASE + r * TPW + i];
+      u32x4 c;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) c[d] = (m >= 2 ? wv[d] >> 8 : wv[d]) & ((m & 1) ? 0x00f000f0u : 0x000f000fu);
+      acc[r][m & 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bitcast<f16x8>(c), x.v[m], acc[r][m & 1], 0, 0, 0);
+    }
+  }
+}
+
+// out = fp16(scale * sum) of unit u, from the tiles in places [BASE, BASE + NRB * TPW) and the fragments xt (tile i of
+// this wave in xt[i]); see gemv_slots for the numerics.
+template <int NRB, int TPW, int EPI, int BASE, int SCBASE, int NSLOT, int NSC>
+__device__ __forceinline__ f16 wide_unit(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB], int ostride,
+                                         f16 res, int u, int n_units, int N, int KT, int M, const XTile (&xt)[TPW], float* red,
+                                         int& red_buf, const float* xsum) {
+  if (u >= n_units) return res;
+  const int wave = wave_id();
+  f32x4 acc[NRB][2];
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) acc[r][0] = acc[r][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < TPW; ++i)
+    if (wave + i * DS_WAVES < KT) wide_tile_product<NRB, TPW, BASE>(S, acc, i, xt[i]);
+  f32x4 sum[NRB];
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) sum[r] = acc[r][0] * 16777216.0f + acc[r][1] * 1048576.0f;
+  return finish_unit<NRB, EPI, true, f16x2[NSC], DW_MAXB, DW_RED>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+}
+
+template <int TPW_D, int TPW_F, int U_F>
+__global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  if (*a.keep_going == 0) return;
+  if (__hip_atomic_load((DS_GLOBAL unsigned*)(a.sync + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
+  const int KT_D = (a.d + 127) / 128, KT_F = (a.ffn + 127) / 128;
+  float* att_lds = reinterpret_cast<float*>(smem);
+  float* red = reinterpret_cast<float*>(smem + a.region0);
+  float* scratch = red + 2 * DW_RED;                               // [16 waves][16 rows] sums of squares
+  float* xsum = scratch + DS_WAVES * DW_MAXB;                      // [16 waves][16 rows] sums of the rows
+  float* sel = xsum + DS_WAVES * DW_MAXB;                          // selection scratch (64 floats), then flags
+  int* lds_dead = reinterpret_cast<int*>(sel + 64);
+  f16* cs = reinterpret_cast<f16*>(scratch + DW_TAIL_FLOATS);      // [D]: cos, sin of this step's angles
+  uint32_t* lds_layers = reinterpret_cast<uint32_t*>(cs + DS_D);   // [n_layer] descriptors
+
+  const int M = a.B;
+  const int step = *a.step;
+  const int nb_d = (a.d + 15) / 16, nb_f = (a.ffn + 15) / 16, nb_v = (a.vocab + 15) / 16;
+  const int G = gridDim.x, wg = blockIdx.x;
+  const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+  Waiter w{a.sync + 1, lds_dead, 0};
+  int red_buf = 0;
+  const size_t xslot = (size_t)M * a.d;
+
+  // ---- set-up: as in decode_step_kernel
+  {
+    const int tid = thread_id();
+    if (tid == 0) *lds_dead = 0;
+    const u32x4 filler = {DS_EMPTY32, DS_EMPTY32, DS_EMPTY32, DS_EMPTY32};
+    char* fill = reinterpret_cast<char*>(a.xres + xslot);
+    for (size_t off = ((size_t)wg * DS_THREADS + tid) * 16; off < a.fill_bytes; off += (size_t)G * DS_THREADS * 16) {
+      const size_t win = off & ~(((size_t)1 << 30) - 1);
+      put16(fill + win, a.fill_bytes - win < ((size_t)1 << 31) ? a.fill_bytes - win : ((size_t)1 << 31), off - win, filler);
+    }
+    for (size_t i = ((size_t)wg * DS_THREADS + tid) * 8; i < (size_t)M * a.vocab; i += (size_t)G * DS_THREADS * 8)
+      put16(a.logits, (size_t)M * a.vocab * 2, i * 2, filler);
+    for (int i = tid; i < a.n_layer * DS_LAYER_WORDS; i += DS_THREADS) lds_layers[i] = a.layers[i];
+    if (tid < DS_D / 2) {
+      const f16 ang = (f16)((float)(f16)(float)step * (float)a.inv_freq[tid]);
+      cs[tid] = (f16)cosf((float)ang);
+      cs[DS_D / 2 + tid] = (f16)sinf((float)ang);
+    }
+    const int col = step < a.max_len ? step : a.max_len - 1;
+    for (int i = wg * DS_THREADS + tid; i < M * a.d; i += G * DS_THREADS) {
+      const int b = i / a.d, c = i % a.d;
+      int id = a.container[(size_t)b * a.max_len + col];
+      id = id < 0 ? 0 : (id >= a.vocab ? a.vocab - 1 : id);
+      put(a.xres + i, a.embed[(size_t)id * a.d + c]);
+    }
+  }
+  wg_sync();
+
+  // places of the units in the tile array: as in decode_step_kernel
+  constexpr int T = TPW_D;
+  constexpr int NSLOT = 8 * T;
+  constexpr int S_QKV = 0, S_O = 3 * T, S_GU0 = 4 * T, S_GU1 = 6 * T, S_GU2 = 0, S_D = 3 * T;
+  constexpr int NSC = 9;
+  constexpr int C_QKV = 0, C_O = 3, C_GU0 = 4, C_GU1 = 6, C_GU2 = 0, C_D = 8;
+  constexpr int D_EARLY = TPW_F < T ? TPW_F : T;
+  static_assert(U_F <= 3 && TPW_F <= 3 * T, "see decode_step_kernel");
+  u32x4 S[NSLOT];
+  f16x2 SC[NSC];
+  {
+    const LayerPtrs L0 = layer_ptrs(lds_layers, 0);
+    const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
+    load_slots<3, T, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
+  }
+  grid_barrier(a.sync, epoch, G, wg, w);
+  bool alive = *lds_dead == 0;
+
+  // the residual element of this thread's output (epilogue mapping of finish_unit: row tid / 16, channel tid % 16)
+  f16 res = (f16)0.0f;
+  if (alive) {
+    const int tid = thread_id();
+    const int m_ = tid >> 4, n = wg * 16 + (tid & 15);
+    const bool on = m_ < M && n < a.d;
+    res = wait_value(a.xres + (on ? (size_t)m_ * a.d + n : 0), on, w);
+  }
+  const int wave = wave_id(), lane = lane_id();
+
+  for (int li = 0; li < a.n_layer && alive; ++li) {
+    const LayerPtrs L = layer_ptrs(lds_layers, li);
+    const bool more = li + 1 < a.n_layer;
+    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);
+    const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
+    const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
+    const Mat m3n[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
+    f16* const x_in = a.xres + (size_t)(2 * li) * xslot;
+    f16* const x_mid = x_in + xslot;
+    f16* const x_out = x_mid + xslot;
+    XTile xt[T];
+    // ---- RMSNorm + q/k/v
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      xt[i] = XTile{};
+      if (wave + i * DS_WAVES < KT_D) fetch_xtile(x_in, M, a.d, wave + i * DS_WAVES, xt[i], w);
+    }
+    {
+      const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
+      load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
+      load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+    }
+    norm_xtiles<T>(xt, L.get<const f16>(P_N1), a.d, KT_D, a.eps, scratch);
+    alive = *lds_dead == 0;      // behind the barrier of the norm: the same answer in every wave
+    if (!alive) break;
+    {
+      const float s1 = xtiles_rowsum<T>(xt);
+      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      f16* q = a.qkv + (size_t)li * M * 3 * a.d;
+      f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
+      wide_unit<3, T, EPI_STORE, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
+    }
+    load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+    // ---- rotary + KV append + attention
+    {
+      f16* kring = L.get<f16>(P_KV);
+      const int units = M * a.H * a.nsplit;
+      for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
+      if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
+    }
+    // ---- o_proj + residual
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      xt[i] = XTile{};
+      if (wave + i * DS_WAVES < KT_D) fetch_xtile(a.ctx + (size_t)li * xslot, M, a.d, wave + i * DS_WAVES, xt[i], w);
+    }
+    if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
+    wg_sync();      // the row sums of the previous phase have been read; every wave knows whether one gave up
+    alive = *lds_dead == 0;
+    if (!alive) break;
+    {
+      const float s1 = xtiles_rowsum<T>(xt);
+      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      f16* const o1[1] = {x_mid};
+      res = wide_unit<1, T, EPI_RESIDUAL, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
+    }
+    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    // ---- RMSNorm + gate/up + SwiGLU, one unit after the other
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      xt[i] = XTile{};
+      if (wave + i * DS_WAVES < KT_D) fetch_xtile(x_mid, M, a.d, wave + i * DS_WAVES, xt[i], w);
+    }
+    norm_xtiles<T>(xt, L.get<const f16>(P_N2), a.d, KT_D, a.eps, scratch);
+    alive = *lds_dead == 0;
+    if (!alive) break;
+    {
+      const float s1 = xtiles_rowsum<T>(xt);
+      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      f16* act = a.act + (size_t)li * M * a.ffn;
+      f16* const o2[2] = {act, act};
+      wide_unit<2, T, EPI_SWIGLU, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
+      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+      if constexpr (U_F > 1)
+        wide_unit<2, T, EPI_SWIGLU, S_GU1, C_GU1>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
+      if constexpr (U_F > 2)
+        wide_unit<2, T, EPI_SWIGLU, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
+    }
+    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    // ---- down + residual: the fragments of one K tile at a time
+    {
+      f32x4 acc[1][2];
+      acc[0][0] = acc[0][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+      float s1 = 0.f;
+      const f16* actx = a.act + (size_t)li * M * a.ffn;
+#pragma unroll
+      for (int i = 0; i < TPW_F; ++i) {
+        if (wave + i * DS_WAVES < KT_F) {
+          XTile x1;
+          fetch_xtile(actx, M, a.ffn, wave + i * DS_WAVES, x1, w);
+          const XTile one[1] = {x1};
+          s1 += xtiles_rowsum<1>(one);
+          wide_tile_product<1, TPW_F, S_D>(S, acc, i, x1);
+        }
+      }
+      wg_sync();      // the row sums of the previous phase have been read; every wave knows whether one gave up
+      alive = *lds_dead == 0;
+      if (!alive) break;
+      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+      f32x4 sum[1];
+      sum[0] = acc[0][0] * 16777216.0f + acc[0][1] * 1048576.0f;
+      f16* const o1[1] = {x_out};
+      if (wg < nb_d)
+        res = finish_unit<1, EPI_RESIDUAL, true, f16x2[NSC], DW_MAXB, DW_RED>(sum, o1, a.d, res, wg, a.d, M, red, red_buf, xsum, SC, C_D);
+    }
+  }
+  // ---- final RMSNorm + lm_head, streamed unit by unit with the next unit's tiles in flight
+  if (alive) {
+    XTile xt[T];
+#pragma unroll
+    for (int i = 0; i < T; ++i) {
+      xt[i] = XTile{};
+      if (wave + i * DS_WAVES < KT_D)
+        fetch_xtile(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, wave + i * DS_WAVES, xt[i], w);
+    }
+    wg_sync();
+    alive = *lds_dead == 0;
+    if (alive) {
+      norm_xtiles<T>(xt, a.final_norm, a.d, KT_D, a.eps, scratch);
+      const Mat m1[1] = {{a.head, nullptr}};
+      f16* const o1[1] = {a.logits};
+      Unit<FmtF16, 1, T> even, odd;
+      auto head_unit = [&](const Unit<FmtF16, 1, T>& t, int u) {
+        if (u >= nb_v) return;
+        f32x4 acc[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+          if (wave + i * DS_WAVES < KT_D) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(FmtF16::a_operand(t.w[0][i], j, t.sc[0]), xt[i].v[j], acc[0], 0, 0, 0);
+          }
+        finish_unit<1, EPI_STORE, false, NoScales, DW_MAXB, DW_RED>(acc, o1, a.vocab, (f16)0.0f, u, a.vocab, M, red, red_buf);
+      };
+      load_unit(even, m1, wg, nb_v, a.vocab, KT_D);
+      for (int u = wg; u < nb_v; u += 2 * G) {
+        load_unit(odd, m1, u + G, nb_v, a.vocab, KT_D);
+        head_unit(even, u);
+        load_unit(even, m1, u + 2 * G, nb_v, a.vocab, KT_D);
+        head_unit(odd, u + G);
+      }
+    }
+  }
+  // ---- selection and bookkeeping
+  if (wg == 0) {
+    if (alive) select_and_advance(a, sel, w);
+    if (thread_id() == 0)
+      __hip_atomic_store((DS_GLOBAL unsigned*)a.sync, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 struct Variant {
-  int tpw_d, tpw_f, u_f, maxb;
+  int tpw_d, tpw_f, u_f, minb, maxb;
   void (*kern)(DsArgs);
   bool ready;
 };
 Variant g_variants[] = {
-    {1, 1, 1, 4, decode_step_kernel<1, 1, 1, 4>, false},   // small test shapes
-    {2, 6, 3, 1, decode_step_kernel<2, 6, 3, 1>, false},   // 7B: hidden 4096, ffn 11008, batch 1
-    {2, 6, 3, 4, decode_step_kernel<2, 6, 3, 4>, false},   // 7B, batch 2..4
+    {1, 1, 1, 1, 4, decode_step_kernel<1, 1, 1, 4>, false},        // small test shapes
+    {2, 6, 3, 1, 1, decode_step_kernel<2, 6, 3, 1>, false},        // 7B: hidden 4096, ffn 11008, batch 1
+    {2, 6, 3, 2, 4, decode_step_kernel<2, 6, 3, 4>, false},        // 7B, batch 2..4
+    {1, 1, 1, 5, 16, decode_step_wide_kernel<1, 1, 1>, false},     // small test shapes, batch 5..16
+    {2, 6, 3, 5, 16, decode_step_wide_kernel<2, 6, 3>, false},     // 7B, batch 5..16
 };
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -1131,7 +1505,7 @@ Layout layout_for(const pta_decode_model* m, int cus) {
 }
 
 bool shape_ok(const pta_decode_model* m) {
-  return m && m->batch >= 1 && m->batch <= DS_MAXB && m->hidden > 0 && m->n_head > 0 && m->ffn > 0 && m->vocab > 0 &&
+  return m && m->batch >= 1 && m->batch <= DW_MAXB && m->hidden > 0 && m->n_head > 0 && m->ffn > 0 && m->vocab > 0 &&
          m->max_len > 0 && m->n_layer > 0 && m->head_dim == DS_D && m->hidden == m->n_head * DS_D && m->ffn % 8 == 0 &&
          m->vocab % 8 == 0;
 }
@@ -1163,12 +1537,12 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   const int u_f = (nb_f + cus - 1) / cus;
   Variant* var = nullptr;
   for (Variant& v : g_variants)
-    if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B <= v.maxb && !var) var = &v;
+    if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B >= v.minb && B <= v.maxb && !var) var = &v;
   if (!shape_ok(mdl) || nb_d > cus || !var) {
     pta_set_error("pta_llama_decode_step: supports batch <= %d, head size %d, hidden = heads * head size <= %d, ffn "
                   "and vocabulary sizes that are multiples of 8, and the (hidden, ffn) of the 7B model or small test "
                   "shapes (got batch %d, head size %d, hidden %d, heads %d, ffn %d, vocabulary %d)",
-                  DS_MAXB, DS_D, 16 * cus, B, mdl->head_dim, d, H, ffn, mdl->vocab);
+                  DW_MAXB, DS_D, 16 * cus, B, mdl->head_dim, d, H, ffn, mdl->vocab);
     return PTA_EUNSUPPORTED;
   }
 
@@ -1193,13 +1567,15 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.trace = (unsigned long long*)(ws + lay.trace);
   a.fill_bytes = lay.trace - (lay.xres + (size_t)B * d * 2);   // everything after the first residual slot
   a.nsplit = splits_for(cus, B, H);
+  const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
-  size_t region0 = (size_t)B * xstride * 2;
+  size_t region0 = wide ? 0 : (size_t)B * xstride * 2;
   if (region0 < (size_t)DS_ATT_FLOATS * 4) region0 = (size_t)DS_ATT_FLOATS * 4;
   region0 = (region0 + 15) & ~(size_t)15;
   a.region0 = (int)region0;
-  const size_t lds = region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
-                     (size_t)mdl->n_layer * sizeof(pta_decode_layer);
+  const size_t lds = wide ? region0 + (size_t)(2 * DW_RED + DW_TAIL_FLOATS) * 4 + DS_D * 2 + (size_t)mdl->n_layer * sizeof(pta_decode_layer)
+                          : region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
+                                (size_t)mdl->n_layer * sizeof(pta_decode_layer);
   PTA_REQUIRE(lds <= 160 * 1024, "pta_llama_decode_step: %zu bytes of LDS exceed a compute unit's 160 KiB", lds);
 
   if (!var->ready) {

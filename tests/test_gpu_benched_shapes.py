@@ -145,6 +145,24 @@ def test_per_operator_path_at_7b_width_batch_16_matches_oracle(wide):
     assert ties <= 40
 
 
+@pytest.mark.timeout(600)
+def test_persistent_step_at_7b_width_batch_16_matches_oracle(wide):
+    """decode_step_wide_kernel<2,6,3> (batch 5..16: every wave loads the activation fragments of its own K tiles):
+    a prompt long enough that a cache chunk boundary is crossed, then 32 generated tokens."""
+    from poptransformer_amd.engine import fused, loader
+    B, L, pad, eos, plen = 16, 112, 0, 2, 72
+    steps = plen - 1 + 32
+    print("case: persistent step at the 7B width, batch 16", flush=True)
+    sd, template = wide
+    oracle = _oracle(template, L, B)
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_7B_WIDTH, L, B, pad, eos), loader.llama2_weights(sd, LLAMA_7B_WIDTH))
+    dec.enable_persistent()
+    ids = _prompt(np.random.default_rng(78), B, L, plen, LLAMA_7B_WIDTH["vocab_size"], pad)
+    ties = _follow(dec, oracle, ids, L, steps, pad, eos)
+    assert not dec.persistent.failed()
+    assert ties <= 40
+
+
 # ---------------------------------------------------------------- the single INT4 operator at its own shape
 def _w4_case(seed, M, Kdim, N):
     rng = np.random.default_rng(seed)

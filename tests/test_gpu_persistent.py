@@ -19,7 +19,7 @@ def _decoders(B, L, pad, eos, seed, early_stop=False):
     return sd, fused.FusedDecoder(spec, w), fused.FusedDecoder(spec, w).enable_persistent()
 
 
-@pytest.mark.parametrize("B", [1, 3])
+@pytest.mark.parametrize("B", [1, 3, 5, 8, 16])
 def test_persistent_step_matches_oracle(B):
     """Greedy ids identical over the first 32 steps, fp16 logits within 1e-2 (max relative error)."""
     L, steps, pad, eos = 48, 32, 0, 2
@@ -31,12 +31,13 @@ def test_persistent_step_matches_oracle(B):
     assert not dec.persistent.failed()
 
 
-@pytest.mark.parametrize("B", [1, 4])
+@pytest.mark.parametrize("B", [1, 4, 7, 16])
 def test_persistent_step_follows_the_per_operator_path(B):
     """Step by step over a long generation: logits agree to 2e-3 of their largest magnitude (the two
     paths merge attention partial sums in different orders) and the selected ids are equal wherever
     the per-operator logits separate the best two candidates by more than that; the comparison ends
-    at the first step where a near tie sends the two generations apart."""
+    at the first step where a near tie sends the two generations apart (with more than 4 sequences, where
+    near ties are frequent, the persistent decoder is then given the reference's token and goes on)."""
     L, pad, eos = 200, 0, 2
     print("case: persistent step vs per-operator path, batch", B, flush=True)
     _, ref, dec = _decoders(B, L, pad, eos, seed=5)
@@ -51,14 +52,18 @@ def test_persistent_step_follows_the_per_operator_path(B):
         a = ref.logits.float().cpu().numpy()
         b = dec.logits.float().cpu().numpy()
         scale = np.abs(a).max()
-        assert np.abs(a - b).max() <= 2e-3 * scale, f"logits differ at step {it}"
+        # beyond 4 sequences the per-operator path runs other kernels (exact INT4 decode, other summation orders)
+        tol = 2e-3 if B <= 4 else 4e-3
+        assert np.abs(a - b).max() <= tol * scale, f"logits differ at step {it}"
         top2 = np.sort(a, axis=1)[:, -2:]
-        clear = (top2[:, 1] - top2[:, 0]) > 4e-3 * scale
+        clear = (top2[:, 1] - top2[:, 0]) > 2 * tol * scale
         ia, ib = ref.next_ids.cpu().numpy(), dec.next_ids.cpu().numpy()
         assert np.array_equal(ia[clear], ib[clear]), f"ids differ at step {it} without a near tie"
         compared += 1
         if not np.array_equal(ref.container.cpu().numpy(), dec.container.cpu().numpy()):
-            break
+            if B <= 4:
+                break
+            dec.container.copy_(ref.container)      # a near tie (asserted above): follow the reference's choice
     assert compared >= 32
     assert not dec.persistent.failed()
 
@@ -142,6 +147,6 @@ def test_persistent_step_rejects_unsupported_models():
     with pytest.raises(NotImplementedError):
         dec.enable_persistent()
     sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=1, int4=True)
-    spec = loader.llama2_spec(LLAMA_TINY, 48, 5, 0, 2)           # batch 5 > 4
+    spec = loader.llama2_spec(LLAMA_TINY, 48, 17, 0, 2)          # batch 17 > 16
     with pytest.raises(NotImplementedError):
         fused.FusedDecoder(spec, loader.llama2_weights(sd, LLAMA_TINY)).enable_persistent()
