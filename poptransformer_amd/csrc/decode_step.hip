@@ -51,7 +51,7 @@ constexpr int DS_D = 128;                                   // head size
 constexpr int DS_MAX_SPLIT = 16;
 constexpr int DS_PART = DS_D + 2;                           // floats of one attention partial
 constexpr int DS_RED = DS_WAVES * 6 * 16 * DS_MAXB;         // floats in one reduction buffer (up to six matrices)
-constexpr int DS_ATT_FLOATS = 3 * DS_D / 2 + 2 * DS_WAVES + DS_WAVES * DS_D;
+constexpr int DS_ATT_FLOATS = 3 * DS_D + 2 * DS_WAVES + DS_WAVES * DS_D;     // q | k | v of two units, per-wave softmax states
 constexpr int DS_XSUM = DS_WAVES * DS_MAXB + 64 + 4;        // offset of the per-wave sums of the staged activations
 constexpr int DS_TAIL_FLOATS = DS_XSUM + DS_WAVES * DS_MAXB; // norm sums | selection scratch | flags | activation sums
 constexpr int DS_LAYER_WORDS = sizeof(pta_decode_layer) / 4;
@@ -81,6 +81,8 @@ struct DsArgs {
   f16* act;              // [n_layer][B, ffn]
   float* part;           // [n_layer][B*H, nsplit, DS_PART]
   size_t fill_bytes;     // qkv .. end of part, contiguous from xres + B*d (the first residual is not filled)
+  unsigned* flags;       // [4 n_layer + 1][DW_REPLICAS][flag_words] arrival words of decode_step_wide_kernel, behind part
+  int flag_words;        // words of one row: the workgroups, rounded up to a KiB
   unsigned* sync;
   int nsplit;
   int region0;           // bytes of the activation / attention area at the start of LDS
@@ -805,6 +807,113 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
   wg_sync();
 }
 
+// Two (sequence, head) units at a time, eight waves each, for launches without splits (nsplit == 1: at least as many
+// units as workgroups): the same arithmetic as attention_unit per unit - the online-softmax state of a row group
+// depends on the rows it visits, so the outputs differ from a sixteen-wave pass in the last bits, as they do between
+// split counts.  bh1 < 0: the second half of the workgroup has no unit.
+__device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* kring_base, int bh0, int bh1, int step, float* lds,
+                                              const f16* cs, Waiter& w) {
+  constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2, WPU = DS_WAVES / 2;
+  const int wave = wave_id(), lane = lane_id();
+  const int half = wave / WPU, wv = wave % WPU;
+  const int bh = half ? bh1 : bh0;
+  const bool active = bh >= 0;
+  const int b = active ? bh / a.H : 0, h = active ? bh % a.H : 0;
+  const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
+  const int pos = step % a.max_len;
+  f16* q_s = reinterpret_cast<f16*>(lds) + half * 3 * D;      // [D] rotated q | [D] rotated new k | [D] new v, per unit
+  f16* k_s = q_s + D;
+  f16* v_s = k_s + D;
+  float* sm_m = lds + 3 * D;                                   // [DS_WAVES]
+  float* sm_l = sm_m + DS_WAVES;
+  float* sm_acc = sm_l + DS_WAVES;                             // [DS_WAVES][D]
+  const f16* qrow = a.qkv + ((size_t)li * a.B + b) * 3 * a.d + h * D;
+  f16* kring = kring_base + ((size_t)b * a.H + h) * a.max_len * D;
+  f16* vring = kring + (size_t)a.B * a.H * a.max_len * D;
+  {
+    const int t = thread_id() - half * WPU * 64;
+    const int which = t / D, d_ = t % D;
+    const bool on = active && t < 3 * D;
+    const f16* row = qrow + (size_t)(which < 3 ? which : 0) * a.d;
+    f16 x0, x1;
+    wait_pair(row + d_, on, row + (d_ < HALF ? d_ + HALF : d_ - HALF), on && which < 2, x0, x1, w);
+    if (on) {
+      f16 y = x0;
+      if (which < 2) {
+        const int i = d_ < HALF ? d_ : d_ - HALF;
+        const f16 rot = d_ < HALF ? -x1 : x1;
+        y = x0 * cs[i] + rot * cs[HALF + i];
+      }
+      q_s[which * D + d_] = y;
+      if (which == 1) as_global(kring)[(size_t)pos * D + d_] = y;
+      if (which == 2) as_global(vring)[(size_t)pos * D + d_] = y;
+    }
+  }
+  wg_sync();
+  if (active) {
+    const int grp = lane / LPP, sub = lane % LPP, d0 = sub * 8;
+    float qf[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qf[e] = (float)q_s[d0 + e];
+    const f16 scale = (f16)0.08838834764831845f;   // fp16(1/sqrt(128))
+    float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    for (int p0 = wv * PPW; p0 < valid; p0 += WPU * PPW) {
+      const int p = p0 + grp;
+      const bool on = p < valid;
+      const int pc = on ? p : valid - 1;
+      f16x8 k8, v8;
+      if (pc == pos) {      // this step's row: taken from LDS, its global copy is being written
+        k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
+        v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
+      } else {
+        k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)pc * D + d0);
+        v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)pc * D + d0);
+      }
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
+#pragma unroll
+      for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      f16 s16 = (f16)s;          // fp16 output of the q.K^T MatMul
+      s16 = s16 * scale;         // fp16 multiply by fp16(1/sqrt(D))
+      const float x = on ? (float)s16 : -INFINITY;
+      const float mn = fmaxf(m, x);
+      const float corr = m == -INFINITY ? 0.f : __expf(m - mn);
+      const float pe = on ? __expf(x - mn) : 0.f;
+      l = l * corr + pe;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
+      m = mn;
+    }
+    merge_lanes(m, l, acc, 16);
+    merge_lanes(m, l, acc, 32);
+    if (lane == 0) { sm_m[wave] = m; sm_l[wave] = l; }
+    if (lane < LPP) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sm_acc[wave * D + d0 + e] = acc[e];
+    }
+  }
+  wg_sync();
+  {
+    const int d_ = thread_id() - half * WPU * 64;
+    if (active && d_ < D) {      // the first two waves of each half
+      float Mx = -INFINITY, Ls = 0.f, As = 0.f;
+#pragma unroll
+      for (int i = 0; i < WPU; ++i) Mx = fmaxf(Mx, sm_m[half * WPU + i]);
+#pragma unroll
+      for (int i = 0; i < WPU; ++i) {
+        const float wgt = sm_m[half * WPU + i] == -INFINITY ? 0.f : __expf(sm_m[half * WPU + i] - Mx);
+        Ls = __builtin_fmaf(sm_l[half * WPU + i], wgt, Ls);
+        As = __builtin_fmaf(sm_acc[(half * WPU + i) * D + d_], wgt, As);
+      }
+      put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
+    }
+  }
+  wg_sync();
+}
+
 // ------------------------------------------------------------------------------------------ selection and bookkeeping
 // Top-1 per sequence (lowest index among equals), then the container / mask / stop-mask update of
 // models/base_model.py:313-355 exactly as step_update_kernel in select.hip; workgroup 0 only.
@@ -1098,41 +1207,62 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
 // codes) are partial per wave and meet in LDS.
 constexpr int DW_MAXB = 16;
 constexpr int DW_RED = DS_WAVES * 3 * 256;                  // floats of one reduction buffer: up to three matrices
-constexpr int DW_TAIL_FLOATS = 2 * DS_WAVES * DW_MAXB + 64 + 4;   // norm sums | row sums | selection scratch | flags
+constexpr int DW_SCL = 6 * 16;                                // channel scales of one phase: up to three gate / up pairs
+constexpr int DW_TAIL_FLOATS = 2 * DS_WAVES * DW_MAXB + 64 + 4 + 2 * DW_SCL;   // norm sums | row sums | selection scratch | flags | scales
 
 struct XTile {
   f16x8 v[4];      // the four 32-feature steps of one K tile
 };
 
-// This wave's fragments of K tile kt of X (fp16 [M, K], a producer's slot): loaded until none of their elements is the
-// filler.  Returns false when the wait was given up.  Features beyond K read as zero.
-__device__ __forceinline__ bool fetch_xtile(const f16* X, int M, int K, int kt, XTile& t, Waiter& w) {
+// Arrival words.  Workgroup g sets word g of a phase's row once everything it stored for the phase has reached
+// memory: its stores are agent-scope, written through, and a wave's memory counter reaching zero says that wave's have
+// arrived; the storing waves wait for that, the workgroup meets, the first wave writes the word.  A row exists in
+// DW_REPLICAS copies, 1 KiB or more apart, and a consumer polls copy (its index % DW_REPLICAS): 256 compute units
+// polling one KiB would all queue at one memory channel.  The launch cleared the rows before its grid barrier.  Only
+// the first wave of a consumer polls, at agent scope; the workgroup meets, and only then are the phase's values read -
+// with ordinary loads.
+constexpr int DW_REPLICAS = 16;
+__device__ __forceinline__ void announce(unsigned* rows, int row_words, int wg, bool stored) {
+  if (stored) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  wg_sync();
+  if (wave_id() == 0 && lane_id() < DW_REPLICAS)
+    __hip_atomic_store((DS_GLOBAL unsigned*)(rows + (size_t)lane_id() * row_words + wg), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// false when the wait was given up (by this or an earlier wait of the workgroup)
+__device__ __forceinline__ bool await_row(const unsigned* rows, int row_words, int G, int wg, Waiter& w) {
+  if (wave_id() == 0) {
+    const unsigned* row = rows + (size_t)(wg % DW_REPLICAS) * row_words;
+    const int lane = lane_id();
+    for (;;) {
+      bool ok = true;
+      for (int o = lane * 4; o < G; o += 256) {
+        const u32x4 v = get16(row, (size_t)G * 4, (size_t)o * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ok = ok && (o + i >= G || v[i] == 1u);
+      }
+      if (__all(ok) || w.give_up()) break;
+    }
+  }
+  wg_sync();
+  asm volatile("" ::: "memory");      // the values are requested after the row has been seen complete
+  return *w.lds_dead == 0;
+}
+
+// This wave's fragments of K tile kt of X (fp16 [M, K], a slot whose arrival row has been seen complete), through the
+// caches: the 256 workgroups read the same values, and all but the first read of a line in each L2 stay out of the
+// fabric.  Nothing of a slot is in a cache before its arrival: the launch starts with an agent-scope acquire (no
+// line of the previous launch survives), no slot of this protocol is written with the filler, and every address is
+// written once per launch.  Features beyond K read as zero.
+__device__ __forceinline__ void load_xtile(const f16* X, int M, int K, int kt, XTile& t) {
   const int lane = lane_id();
   int row = lane & 15;
   row = row < M ? row : M - 1;                // padding rows repeat the last one; their products are never stored
-  u32x4 v[4];
-  bool need[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    v[j] = u32x4{0, 0, 0, 0};
-    need[j] = kt * 128 + j * 32 + (lane >> 4) * 8 < K;
+    const int k = kt * 128 + j * 32 + (lane >> 4) * 8;
+    t.v[j] = f16x8{};
+    if (k < K) t.v[j] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(X) + (size_t)row * K + k);
   }
-  for (;;) {
-    bool pending = false;
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (need[j]) v[j] = get16(X, (size_t)M * K * 2, ((size_t)row * K + kt * 128 + j * 32 + (lane >> 4) * 8) * 2);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (need[j]) {
-        if (has_empty16(v[j])) pending = true;
-        else need[j] = false;
-      }
-    if (!__any(pending) || w.give_up()) break;
-  }
-#pragma unroll
-  for (int j = 0; j < 4; ++j) t.v[j] = bitcast<f16x8>(v[j]);
-  return *w.lds_dead == 0;
 }
 
 // sums over the lane groups that share a row: afterwards lanes 0..15 (and their images) hold the row's total of the wave
@@ -1143,9 +1273,10 @@ __device__ __forceinline__ float rows_of_wave(float v) {
 }
 
 // RMSNorm of the rows whose fragments the waves hold (layers/rms_layer_norm.py:26-36, as pta_rmsnorm): the sums of
-// squares meet in LDS, every lane then scales its own fragments.  NT tiles per wave; tiles beyond KT hold zeros.
+// squares meet in LDS, every lane then scales its own fragments by the weights normw_fetch brought to LDS.  NT tiles
+// per wave; tiles beyond KT hold zeros.
 template <int NT>
-__device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* norm_w, int K, int KT, float eps, float* sums) {
+__device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* lds_w, int K, int KT, float eps, float* sums) {
   const int lane = lane_id(), wave = wave_id();
   float sq = 0.f;
 #pragma unroll
@@ -1168,7 +1299,7 @@ __device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* norm_w, i
     for (int j = 0; j < 4; ++j) {
       const int k = kt * 128 + j * 32 + (lane >> 4) * 8;
       if (kt < KT && k < K) {
-        const f16x8 gm = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(norm_w) + k);
+        const f16x8 gm = *reinterpret_cast<const f16x8*>(lds_w + k);
 #pragma unroll
         for (int e = 0; e < 8; ++e) t[i].v[j][e] = (t[i].v[j][e] * r16) * gm[e];
       }
@@ -1190,14 +1321,15 @@ __device__ __forceinline__ float xtiles_rowsum(const XTile (&t)[NT]) {
   return rows_of_wave(s1);
 }
 
-// acc[r][0 / 1] += the products of tile `i` of unit u's NRB matrices (places BASE + r * TPW + i) with the fragments x
-template <int NRB, int TPW, int BASE, int NSLOT>
-__device__ __forceinline__ void wide_tile_product(const u32x4 (&S)[NSLOT], f32x4 (&acc)[NRB][2], int i, const XTile& x) {
+// acc[r][0 / 1] += the products of tile `i` of unit u's NRB matrices (places base + r * TPW + i; constants once the
+// callers' loops are unrolled) with the fragments x
+template <int NRB, int TPW, int NSLOT>
+__device__ __forceinline__ void wide_tile_product(const u32x4 (&S)[NSLOT], f32x4 (&acc)[NRB][2], int base, int i, const XTile& x) {
 #pragma unroll
   for (int m = 0; m < 4; ++m) {
 #pragma unroll
     for (int r = 0; r < NRB; ++r) {
-      const u32x4 wv = S[BASE + r * TPW + i];
+      const u32x4 wv = S[base + r * TPW + i];
       u32x4 c;
 #pragma unroll
       for (int d = 0; d < 4; ++d) c[d] = (m >= 2 ? wv[d] >> 8 : wv[d]) & ((m & 1) ? 0x00f000f0u : 0x000f000fu);
@@ -1206,24 +1338,116 @@ __device__ __forceinline__ void wide_tile_product(const u32x4 (&S)[NSLOT], f32x4
   }
 }
 
+// Requests tiles [FIRST, FIRST + COUNT) of unit u's NRB matrices into places BASE + t (tile t = r * TPW + i is tile i of
+// this wave of matrix r), as load_slots does, without the scales.
+template <int NRB, int TPW, int BASE, int FIRST = 0, int COUNT = NRB * TPW, int NSLOT>
+__device__ __forceinline__ void load_tiles(u32x4 (&S)[NSLOT], const Mat (&m)[NRB], int u, int n_units, int KT) {
+  static_assert(BASE + NRB * TPW <= NSLOT, "unit outside the register array");
+  static_assert(FIRST >= 0 && COUNT >= 0 && FIRST + COUNT <= NRB * TPW, "tiles outside the unit");
+  const int wave = wave_id(), lane = lane_id();
+  u = u < n_units ? u : n_units - 1;
+#pragma unroll
+  for (int t = FIRST; t < FIRST + COUNT; ++t) {
+    const int r = t / TPW, i = t % TPW;
+    int kt = wave + i * DS_WAVES;
+    kt = kt < KT ? kt : KT - 1;
+    S[BASE + t] = __builtin_nontemporal_load(as_global(m[r].tiled) + ((size_t)u * KT + kt) * 64 + lane);
+  }
+}
+
+// The scales of unit u's channels (channel lane % 16) of NRB matrices: requested by the first wave before it requests
+// its activation fragments and written to LDS once those have arrived (a wave's loads complete in order), so that no
+// wave waits for a load of its own in the epilogue, behind the tiles requested ahead.
+template <int NRB>
+__device__ __forceinline__ void request_scales(const Mat (&m)[NRB], int u, int n_units, int N, f16 (&v)[NRB]) {
+  u = u < n_units ? u : n_units - 1;
+  int row = u * 16 + (lane_id() & 15);
+  row = row < N ? row : N - 1;
+#pragma unroll
+  for (int r = 0; r < NRB; ++r) v[r] = as_global(m[r].scale)[row];
+}
+template <int NRB>
+__device__ __forceinline__ void keep_scales(const f16 (&v)[NRB], float* scl) {
+  const int lane = lane_id();
+  if (lane < 16) {
+#pragma unroll
+    for (int r = 0; r < NRB; ++r) scl[r * 16 + lane] = (float)v[r];
+  }
+}
+
+// This wave's partial sums of matrix r of a unit (accumulator layout: lane l holds channels (l / 16) * 4 + 0..3 of
+// row l % 16) go to the reduction buffer: [wave][r][lane] vectors of four channels.
+template <int NRB>
+__device__ __forceinline__ void wide_stash(const f32x4& sum, int r, float* rb) {
+  const int wave = wave_id(), lane = lane_id();
+  *reinterpret_cast<f32x4*>(rb + ((wave * NRB + r) * 64 + lane) * 4) = sum;
+}
+
+// The partial sums of all waves meet: thread (r * 16 + m) * 16 + ch finishes channel ch of row m of matrix r
+// (EPI_SWIGLU: of the gate / up pair).  xsum: the waves' sums of the rows (8 * sum(x) comes off, the stored codes are
+// q + 8); scl[r * 16 + ch]: the channels' scales.  Returns the value stored (the thread's residual element in the next
+// residual phase).
+template <int NRB, int EPI>
+__device__ __forceinline__ f16 wide_finish(f16* const (&out)[NRB], int ostride, f16 res, int u, int N, int M, const float* rb,
+                                           const float* xsum, const float* scl) {
+  wg_sync();
+  f16 y = res;
+  const int tid = thread_id();
+  constexpr int MATS = EPI == EPI_SWIGLU ? 1 : NRB;
+  if (tid < MATS * 256) {
+    const int r = tid >> 8, m_ = (tid >> 4) & 15, ch = tid & 15;
+    const int n = u * 16 + ch;
+    if (m_ < M && n < N) {
+      float off = 0.f;
+#pragma unroll 8
+      for (int w = 0; w < DS_WAVES; ++w) off += xsum[w * DW_MAXB + m_];
+      off *= 8.0f;
+      const int at = ((ch >> 2) * 16 + m_) * 4 + (ch & 3);
+      if (EPI == EPI_SWIGLU) {
+        float sg = 0.f, su = 0.f;
+#pragma unroll 4
+        for (int w = 0; w < DS_WAVES; ++w) {
+          sg += rb[(w * NRB + 0) * 256 + at];
+          su += rb[(w * NRB + (NRB > 1 ? 1 : 0)) * 256 + at];
+        }
+        sg = (sg - off) * scl[ch];
+        su = (su - off) * scl[(NRB > 1 ? 16 : 0) + ch];
+        put(out[0] + (size_t)m_ * ostride + n, (f16)su * swish_f16((f16)sg));
+      } else {
+        float s = 0.f;
+#pragma unroll 8
+        for (int w = 0; w < DS_WAVES; ++w) s += rb[(w * NRB + r) * 256 + at];
+        s = (s - off) * scl[r * 16 + ch];
+        y = (f16)s;
+        if (EPI == EPI_RESIDUAL) y = y + res;
+        put(out[r] + (size_t)m_ * ostride + n, y);
+      }
+    }
+  }
+  return y;
+}
+
 // out = fp16(scale * sum) of unit u, from the tiles in places [BASE, BASE + NRB * TPW) and the fragments xt (tile i of
-// this wave in xt[i]); see gemv_slots for the numerics.
-template <int NRB, int TPW, int EPI, int BASE, int SCBASE, int NSLOT, int NSC>
-__device__ __forceinline__ f16 wide_unit(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB], int ostride,
+// this wave in xt[i]); see gemv_slots for the numerics.  One matrix at a time: its accumulators are stored before the
+// next one's are started.
+template <int NRB, int TPW, int EPI, int BASE, int NSLOT>
+__device__ __forceinline__ f16 wide_unit(const u32x4 (&S)[NSLOT], const float* scl, f16* const (&out)[NRB], int ostride,
                                          f16 res, int u, int n_units, int N, int KT, int M, const XTile (&xt)[TPW], float* red,
                                          int& red_buf, const float* xsum) {
   if (u >= n_units) return res;
   const int wave = wave_id();
-  f32x4 acc[NRB][2];
+  float* rb = red + red_buf * DW_RED;
 #pragma unroll
-  for (int r = 0; r < NRB; ++r) acc[r][0] = acc[r][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < NRB; ++r) {
+    f32x4 acc[1][2];
+    acc[0][0] = acc[0][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int i = 0; i < TPW; ++i)
-    if (wave + i * DS_WAVES < KT) wide_tile_product<NRB, TPW, BASE>(S, acc, i, xt[i]);
-  f32x4 sum[NRB];
-#pragma unroll
-  for (int r = 0; r < NRB; ++r) sum[r] = acc[r][0] * 16777216.0f + acc[r][1] * 1048576.0f;
-  return finish_unit<NRB, EPI, true, f16x2[NSC], DW_MAXB, DW_RED>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+    for (int i = 0; i < TPW; ++i)
+      if (wave + i * DS_WAVES < KT) wide_tile_product<1, TPW>(S, acc, BASE + r * TPW, i, xt[i]);
+    wide_stash<NRB>(acc[0][0] * 16777216.0f + acc[0][1] * 1048576.0f, r, rb);
+  }
+  red_buf ^= 1;
+  return wide_finish<NRB, EPI>(out, ostride, res, u, N, M, rb, xsum, scl);
 }
 
 template <int TPW_D, int TPW_F, int U_F>
@@ -1238,28 +1462,37 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
   float* xsum = scratch + DS_WAVES * DW_MAXB;                      // [16 waves][16 rows] sums of the rows
   float* sel = xsum + DS_WAVES * DW_MAXB;                          // selection scratch (64 floats), then flags
   int* lds_dead = reinterpret_cast<int*>(sel + 64);
-  f16* cs = reinterpret_cast<f16*>(scratch + DW_TAIL_FLOATS);      // [D]: cos, sin of this step's angles
+  float* scl = sel + 64 + 4;                                       // [2][6][16] channel scales, the phases in turn
+  f16* normw = reinterpret_cast<f16*>(scratch + DW_TAIL_FLOATS);   // [d rounded up to 512]: normw_fetch writes whole KiB
+  f16* cs = normw + ((a.d + 511) & ~511);                          // [D]: cos, sin of this step's angles
   uint32_t* lds_layers = reinterpret_cast<uint32_t*>(cs + DS_D);   // [n_layer] descriptors
 
   const int M = a.B;
   const int step = *a.step;
   const int nb_d = (a.d + 15) / 16, nb_f = (a.ffn + 15) / 16, nb_v = (a.vocab + 15) / 16;
   const int G = gridDim.x, wg = blockIdx.x;
+  struct { int wg; } g{wg};       // for TRACE
+  (void)g;
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
   Waiter w{a.sync + 1, lds_dead, 0};
   int red_buf = 0;
   const size_t xslot = (size_t)M * a.d;
 
-  // ---- set-up: as in decode_step_kernel
+  // ---- set-up: as in decode_step_kernel, except that only the slots the attention phase and the selection poll
+  //      (q/k/v, attention partials, logits) are filled; the arrival rows are cleared
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");      // no cache holds a line of an earlier launch
   {
     const int tid = thread_id();
     if (tid == 0) *lds_dead = 0;
     const u32x4 filler = {DS_EMPTY32, DS_EMPTY32, DS_EMPTY32, DS_EMPTY32};
-    char* fill = reinterpret_cast<char*>(a.xres + xslot);
-    for (size_t off = ((size_t)wg * DS_THREADS + tid) * 16; off < a.fill_bytes; off += (size_t)G * DS_THREADS * 16) {
-      const size_t win = off & ~(((size_t)1 << 30) - 1);
-      put16(fill + win, a.fill_bytes - win < ((size_t)1 << 31) ? a.fill_bytes - win : ((size_t)1 << 31), off - win, filler);
-    }
+    const u32x4 zero = {0, 0, 0, 0};
+    const size_t first = ((size_t)wg * DS_THREADS + tid) * 16, stride = (size_t)G * DS_THREADS * 16;
+    const size_t qkv_bytes = (size_t)a.n_layer * M * 3 * a.d * 2;
+    const size_t part_bytes = (size_t)(reinterpret_cast<unsigned char*>(a.flags) - reinterpret_cast<unsigned char*>(a.part));
+    const size_t flag_bytes = (size_t)(4 * a.n_layer + 1) * DW_REPLICAS * a.flag_words * 4;
+    for (size_t off = first; off < qkv_bytes; off += stride) put16(a.qkv, qkv_bytes, off, filler);
+    for (size_t off = first; off < part_bytes; off += stride) put16(a.part, part_bytes, off, filler);
+    for (size_t off = first; off < flag_bytes; off += stride) put16(a.flags, flag_bytes, off, zero);
     for (size_t i = ((size_t)wg * DS_THREADS + tid) * 8; i < (size_t)M * a.vocab; i += (size_t)G * DS_THREADS * 8)
       put16(a.logits, (size_t)M * a.vocab * 2, i * 2, filler);
     for (int i = tid; i < a.n_layer * DS_LAYER_WORDS; i += DS_THREADS) lds_layers[i] = a.layers[i];
@@ -1278,25 +1511,25 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
   }
   wg_sync();
 
-  // places of the units in the tile array: as in decode_step_kernel
+  // Places of the units in the tile array: as in decode_step_kernel.  The tiles are requested later than there, so
+  // that at most 12 places hold tiles at any time: activation fragments and tiles share the 128 registers of a wave,
+  // and a value that does not fit is reloaded from scratch memory behind every tile requested ahead.
   constexpr int T = TPW_D;
   constexpr int NSLOT = 8 * T;
   constexpr int S_QKV = 0, S_O = 3 * T, S_GU0 = 4 * T, S_GU1 = 6 * T, S_GU2 = 0, S_D = 3 * T;
-  constexpr int NSC = 9;
-  constexpr int C_QKV = 0, C_O = 3, C_GU0 = 4, C_GU1 = 6, C_GU2 = 0, C_D = 8;
   constexpr int D_EARLY = TPW_F < T ? TPW_F : T;
   static_assert(U_F <= 3 && TPW_F <= 3 * T, "see decode_step_kernel");
   u32x4 S[NSLOT];
-  f16x2 SC[NSC];
   {
     const LayerPtrs L0 = layer_ptrs(lds_layers, 0);
+    normw_fetch(L0.get<const f16>(P_N1), normw, a.d);
     const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
-    load_slots<3, T, S_QKV, C_QKV>(S, SC, m3, wg, nb_d, a.d, KT_D);
+    load_tiles<3, T, S_QKV>(S, m3, wg, nb_d, KT_D);
   }
   grid_barrier(a.sync, epoch, G, wg, w);
   bool alive = *lds_dead == 0;
 
-  // the residual element of this thread's output (epilogue mapping of finish_unit: row tid / 16, channel tid % 16)
+  // the residual element of this thread's output (epilogue mapping of wide_finish: row tid / 16, channel tid % 16)
   f16 res = (f16)0.0f;
   if (alive) {
     const int tid = thread_id();
@@ -1304,129 +1537,189 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     const bool on = m_ < M && n < a.d;
     res = wait_value(a.xres + (on ? (size_t)m_ * a.d + n : 0), on, w);
   }
-  const int wave = wave_id(), lane = lane_id();
+  const int wave = wave_id();
+  auto phase_rows = [&](int phase) { return a.flags + (size_t)phase * DW_REPLICAS * a.flag_words; };
 
   for (int li = 0; li < a.n_layer && alive; ++li) {
     const LayerPtrs L = layer_ptrs(lds_layers, li);
     const bool more = li + 1 < a.n_layer;
     const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);
-    const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
-    const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
-    const Mat m3n[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
+    // the matrices' pointers are rebuilt from the descriptor words where they are used (a few lane reads each): held
+    // across the layer they would not fit the scalar registers
+#define M3 {layer_mat(L, P_WQ, P_SQ), layer_mat(L, P_WK, P_SK), layer_mat(L, P_WV, P_SV)}
+#define MO {layer_mat(L, P_WO, P_SO)}
+#define MGU {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)}
+#define MD {layer_mat(L, P_WD, P_SD)}
+#define M3N {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)}
     f16* const x_in = a.xres + (size_t)(2 * li) * xslot;
     f16* const x_mid = x_in + xslot;
     f16* const x_out = x_mid + xslot;
     XTile xt[T];
-    // ---- RMSNorm + q/k/v
-#pragma unroll
-    for (int i = 0; i < T; ++i) {
-      xt[i] = XTile{};
-      if (wave + i * DS_WAVES < KT_D) fetch_xtile(x_in, M, a.d, wave + i * DS_WAVES, xt[i], w);
-    }
+    // ---- RMSNorm + q/k/v (scales in the first of the two LDS places, which the phases take in turn)
+    TRACE(0);
     {
-      const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
-      load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
-      load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+      f16 sv[3] = {};
+      if (wave == 0) { const Mat mm[3] = M3; request_scales<3>(mm, wg, nb_d, a.d, sv); }
+      // the first layer's input is the embedding rows, complete since the grid barrier
+      if (li > 0) await_row(phase_rows(4 * li), a.flag_words, G, wg, w);
+#pragma unroll
+      for (int i = 0; i < T; ++i) {
+        xt[i] = XTile{};
+        if (wave + i * DS_WAVES < KT_D) load_xtile(x_in, M, a.d, wave + i * DS_WAVES, xt[i]);
+      }
+      if (wave == 0) keep_scales<3>(sv, scl);
     }
-    norm_xtiles<T>(xt, L.get<const f16>(P_N1), a.d, KT_D, a.eps, scratch);
+    { const Mat mm[1] = MO; load_tiles<1, T, S_O>(S, mm, wg, nb_d, KT_D); }
+    { const Mat mm[2] = MGU; load_tiles<2, T, S_GU0, 0, T>(S, mm, wg, nb_f, KT_D); }
+    TRACE(1);
+    norm_xtiles<T>(xt, normw, a.d, KT_D, a.eps, scratch);
     alive = *lds_dead == 0;      // behind the barrier of the norm: the same answer in every wave
     if (!alive) break;
     {
       const float s1 = xtiles_rowsum<T>(xt);
-      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      if (lane_id() < 16) xsum[wave * DW_MAXB + lane_id()] = s1;
       f16* q = a.qkv + (size_t)li * M * 3 * a.d;
       f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
-      wide_unit<3, T, EPI_STORE, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
+      wide_unit<3, T, EPI_STORE, S_QKV>(S, scl, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
     }
-    load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+    { const Mat mm[2] = MGU; load_tiles<2, T, S_GU0, T, T>(S, mm, wg, nb_f, KT_D); }
+    TRACE(2);
     // ---- rotary + KV append + attention
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
-      for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
-      if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
+      if (a.nsplit == 1) {
+        for (int u = wg; u < units; u += 2 * G) attention_two(a, li, kring, u, u + G < units ? u + G : -1, step, att_lds, cs, w);
+      } else {
+        for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
+      }
+      // the head outputs are stored by waves 0, 1 and (second unit of attention_two) 8, 9
+      announce(phase_rows(4 * li + 1), a.flag_words, wg, wave < 2 || wave == 8 || wave == 9);
+      if constexpr (U_F > 1) { const Mat mm[2] = MGU; load_tiles<2, T, S_GU1>(S, mm, wg + G, nb_f, KT_D); }
     }
+    TRACE(3);
     // ---- o_proj + residual
+    {
+      f16 sv[1] = {};
+      if (wave == 0) { const Mat mm[1] = MO; request_scales<1>(mm, wg, nb_d, a.d, sv); }
+      await_row(phase_rows(4 * li + 1), a.flag_words, G, wg, w);
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
-      xt[i] = XTile{};
-      if (wave + i * DS_WAVES < KT_D) fetch_xtile(a.ctx + (size_t)li * xslot, M, a.d, wave + i * DS_WAVES, xt[i], w);
+      for (int i = 0; i < T; ++i) {
+        xt[i] = XTile{};
+        if (wave + i * DS_WAVES < KT_D) load_xtile(a.ctx + (size_t)li * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
+      }
+      if (wave == 0) keep_scales<1>(sv, scl + DW_SCL);
     }
-    if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     wg_sync();      // the row sums of the previous phase have been read; every wave knows whether one gave up
     alive = *lds_dead == 0;
     if (!alive) break;
+    TRACE(4);
     {
       const float s1 = xtiles_rowsum<T>(xt);
-      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      if (lane_id() < 16) xsum[wave * DW_MAXB + lane_id()] = s1;
       f16* const o1[1] = {x_mid};
-      res = wide_unit<1, T, EPI_RESIDUAL, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
+      res = wide_unit<1, T, EPI_RESIDUAL, S_O>(S, scl + DW_SCL, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xt, red, red_buf, xsum);
     }
-    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    announce(phase_rows(4 * li + 2), a.flag_words, wg, wave < 4);
+    if constexpr (U_F > 2) { const Mat mm[2] = MGU; load_tiles<2, T, S_GU2>(S, mm, wg + 2 * G, nb_f, KT_D); }
+    normw_fetch(L.get<const f16>(P_N2), normw, a.d);
+    TRACE(5);
     // ---- RMSNorm + gate/up + SwiGLU, one unit after the other
+    {
+      f16 sv[U_F][2] = {};
+      if (wave == 0) {
 #pragma unroll
-    for (int i = 0; i < T; ++i) {
-      xt[i] = XTile{};
-      if (wave + i * DS_WAVES < KT_D) fetch_xtile(x_mid, M, a.d, wave + i * DS_WAVES, xt[i], w);
+        for (int k = 0; k < U_F; ++k) { const Mat mm[2] = MGU; request_scales<2>(mm, wg + k * G, nb_f, a.ffn, sv[k]); }
+      }
+      await_row(phase_rows(4 * li + 2), a.flag_words, G, wg, w);
+#pragma unroll
+      for (int i = 0; i < T; ++i) {
+        xt[i] = XTile{};
+        if (wave + i * DS_WAVES < KT_D) load_xtile(x_mid, M, a.d, wave + i * DS_WAVES, xt[i]);
+      }
+      if (wave == 0) {
+#pragma unroll
+        for (int k = 0; k < U_F; ++k) keep_scales<2>(sv[k], scl + k * 32);
+      }
     }
-    norm_xtiles<T>(xt, L.get<const f16>(P_N2), a.d, KT_D, a.eps, scratch);
+    TRACE(6);
+    norm_xtiles<T>(xt, normw, a.d, KT_D, a.eps, scratch);
     alive = *lds_dead == 0;
     if (!alive) break;
     {
       const float s1 = xtiles_rowsum<T>(xt);
-      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
+      if (lane_id() < 16) xsum[wave * DW_MAXB + lane_id()] = s1;
       f16* act = a.act + (size_t)li * M * a.ffn;
       f16* const o2[2] = {act, act};
-      wide_unit<2, T, EPI_SWIGLU, S_GU0, C_GU0>(S, SC, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
-      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+      wide_unit<2, T, EPI_SWIGLU, S_GU0>(S, scl, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
       if constexpr (U_F > 1)
-        wide_unit<2, T, EPI_SWIGLU, S_GU1, C_GU1>(S, SC, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
+        wide_unit<2, T, EPI_SWIGLU, S_GU1>(S, scl + 32, o2, a.ffn, (f16)0.0f, wg + G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
       if constexpr (U_F > 2)
-        wide_unit<2, T, EPI_SWIGLU, S_GU2, C_GU2>(S, SC, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
+        wide_unit<2, T, EPI_SWIGLU, S_GU2>(S, scl + 64, o2, a.ffn, (f16)0.0f, wg + 2 * G, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
     }
-    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-    // ---- down + residual: the fragments of one K tile at a time
+    announce(phase_rows(4 * li + 3), a.flag_words, wg, wave < 4);
+    { const Mat mm[1] = MD; load_tiles<1, TPW_F, S_D>(S, mm, wg, nb_d, KT_F); }
+    TRACE(7);
+    // ---- down + residual: the fragments of one K tile at a time, the next tile's requested before the wait
     {
       f32x4 acc[1][2];
       acc[0][0] = acc[0][1] = f32x4{0.f, 0.f, 0.f, 0.f};
       float s1 = 0.f;
       const f16* actx = a.act + (size_t)li * M * a.ffn;
+      f16 sv[1] = {};
+      if (wave == 0) { const Mat mm[1] = MD; request_scales<1>(mm, wg, nb_d, a.d, sv); }
+      await_row(phase_rows(4 * li + 3), a.flag_words, G, wg, w);
+      XTile ahead;
+      load_xtile(actx, M, a.ffn, wave, ahead);
+      if (wave == 0) keep_scales<1>(sv, scl + DW_SCL);      // requested before the arrival row: here by now
+      { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 2 * T, T>(S, mm, wg, nb_d, KT_D); }      // the next layer's v and q
+      { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 0, T>(S, mm, wg, nb_d, KT_D); }
 #pragma unroll
       for (int i = 0; i < TPW_F; ++i) {
         if (wave + i * DS_WAVES < KT_F) {
-          XTile x1;
-          fetch_xtile(actx, M, a.ffn, wave + i * DS_WAVES, x1, w);
+          const XTile x1 = ahead;
+          if (i + 1 < TPW_F && wave + (i + 1) * DS_WAVES < KT_F) load_xtile(actx, M, a.ffn, wave + (i + 1) * DS_WAVES, ahead);
           const XTile one[1] = {x1};
           s1 += xtiles_rowsum<1>(one);
-          wide_tile_product<1, TPW_F, S_D>(S, acc, i, x1);
+          wide_tile_product<1, TPW_F>(S, acc, S_D, i, x1);
         }
       }
       wg_sync();      // the row sums of the previous phase have been read; every wave knows whether one gave up
       alive = *lds_dead == 0;
       if (!alive) break;
-      if (lane < 16) xsum[wave * DW_MAXB + lane] = s1;
-      load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-      f32x4 sum[1];
-      sum[0] = acc[0][0] * 16777216.0f + acc[0][1] * 1048576.0f;
+      TRACE(8);
+      if (lane_id() < 16) xsum[wave * DW_MAXB + lane_id()] = s1;
       f16* const o1[1] = {x_out};
-      if (wg < nb_d)
-        res = finish_unit<1, EPI_RESIDUAL, true, f16x2[NSC], DW_MAXB, DW_RED>(sum, o1, a.d, res, wg, a.d, M, red, red_buf, xsum, SC, C_D);
+      if (wg < nb_d) {
+        float* rb = red + red_buf * DW_RED;
+        wide_stash<1>(acc[0][0] * 16777216.0f + acc[0][1] * 1048576.0f, 0, rb);
+        red_buf ^= 1;
+        res = wide_finish<1, EPI_RESIDUAL>(o1, a.d, res, wg, a.d, M, rb, xsum, scl + DW_SCL);
+      }
+      announce(phase_rows(4 * li + 4), a.flag_words, wg, wave < 4);
+      { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, T, T>(S, mm, wg, nb_d, KT_D); }
+      normw_fetch(more ? Ln.get<const f16>(P_N1) : a.final_norm, normw, a.d);
+      TRACE(9);
     }
   }
+#undef M3
+#undef MO
+#undef MGU
+#undef MD
+#undef M3N
   // ---- final RMSNorm + lm_head, streamed unit by unit with the next unit's tiles in flight
   if (alive) {
     XTile xt[T];
+    alive = await_row(phase_rows(4 * a.n_layer), a.flag_words, G, wg, w);
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       xt[i] = XTile{};
-      if (wave + i * DS_WAVES < KT_D)
-        fetch_xtile(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, wave + i * DS_WAVES, xt[i], w);
+      if (wave + i * DS_WAVES < KT_D) load_xtile(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
     }
     wg_sync();
     alive = *lds_dead == 0;
     if (alive) {
-      norm_xtiles<T>(xt, a.final_norm, a.d, KT_D, a.eps, scratch);
+      norm_xtiles<T>(xt, normw, a.d, KT_D, a.eps, scratch);
       const Mat m1[1] = {{a.head, nullptr}};
       f16* const o1[1] = {a.logits};
       Unit<FmtF16, 1, T> even, odd;
@@ -1486,9 +1779,11 @@ int splits_for(int cus, int B, int H) {
   return n < 1 ? 1 : (n > DS_MAX_SPLIT ? DS_MAX_SPLIT : n);
 }
 
+size_t flag_words_for(int cus) { return ((size_t)cus + 255) & ~(size_t)255; }
+
 // byte offsets of the workspace parts
 struct Layout {
-  size_t sync, xres, qkv, ctx, act, part, trace, total;
+  size_t sync, xres, qkv, ctx, act, part, flags, trace, total;
 };
 Layout layout_for(const pta_decode_model* m, int cus) {
   const size_t B = m->batch, d = m->hidden, L = m->n_layer, f = m->ffn, H = m->n_head;
@@ -1499,7 +1794,8 @@ Layout layout_for(const pta_decode_model* m, int cus) {
   l.ctx = l.qkv + align256(L * B * 3 * d * 2);
   l.act = l.ctx + align256(L * B * d * 2);
   l.part = l.act + align256(L * B * f * 2);
-  l.trace = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
+  l.flags = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
+  l.trace = l.flags + align256((4 * L + 1) * 16 /* DW_REPLICAS */ * flag_words_for(cus) * 4);
   l.total = l.trace + (size_t)cus * 256;
   return l;
 }
@@ -1565,7 +1861,9 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.act = (f16*)(ws + lay.act);
   a.part = (float*)(ws + lay.part);
   a.trace = (unsigned long long*)(ws + lay.trace);
-  a.fill_bytes = lay.trace - (lay.xres + (size_t)B * d * 2);   // everything after the first residual slot
+  a.fill_bytes = lay.flags - (lay.xres + (size_t)B * d * 2);   // everything after the first residual slot, up to the flags
+  a.flags = (unsigned*)(ws + lay.flags);
+  a.flag_words = (int)flag_words_for(cus);
   a.nsplit = splits_for(cus, B, H);
   const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
@@ -1573,7 +1871,8 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   if (region0 < (size_t)DS_ATT_FLOATS * 4) region0 = (size_t)DS_ATT_FLOATS * 4;
   region0 = (region0 + 15) & ~(size_t)15;
   a.region0 = (int)region0;
-  const size_t lds = wide ? region0 + (size_t)(2 * DW_RED + DW_TAIL_FLOATS) * 4 + DS_D * 2 + (size_t)mdl->n_layer * sizeof(pta_decode_layer)
+  const size_t lds = wide ? region0 + (size_t)(2 * DW_RED + DW_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
+                                (size_t)mdl->n_layer * sizeof(pta_decode_layer)
                           : region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
                                 (size_t)mdl->n_layer * sizeof(pta_decode_layer);
   PTA_REQUIRE(lds <= 160 * 1024, "pta_llama_decode_step: %zu bytes of LDS exceed a compute unit's 160 KiB", lds);
