@@ -650,6 +650,12 @@ __device__ __forceinline__ void normw_fetch(const f16* w, f16* lds_w, int d) {
 }
 
 // ------------------------------------------------------------------------------------------ attention phase
+// Element (row m, feature n) of an activation slot of decode_step_wide_kernel, in halves: the slot is
+// [features / 8][16 rows][8 features], so that the 64 lanes of a wave (lane = 16 * (eight-feature group
+// % 4) + row) read one contiguous KiB per 32-feature step - whole cache lines, which the memory pipeline
+// delivers at twice the rate of sixteen 64-byte pieces of sixteen rows.
+__device__ __forceinline__ size_t grouped_at(int m, int n) { return (size_t)(n >> 3) * 128 + m * 8 + (n & 7); }
+
 // merges the online-softmax state of the lane `o` lanes away into this lane's
 __device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8], int o) {
   const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
@@ -667,6 +673,7 @@ __device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8],
 // angles), append of the new K/V row to the ring by the split whose range holds it, online-softmax
 // attention over this split's rows.  Split 0 of a head collects the partials of the other splits
 // that have rows and writes the head's output.
+template <bool GROUPED = false>
 __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kring_base, int unit, int step, float* lds,
                                                const f16* cs, Waiter& w) {
   constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2;
@@ -801,7 +808,8 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
         As = As * ca + as * cb;
         Mx = mn;
       }
-      put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
+      if constexpr (GROUPED) put(a.ctx + (size_t)li * 16 * a.d + grouped_at(b, h * D + d_), (f16)(As / Ls));
+      else put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
     }
   }
   wg_sync();
@@ -908,7 +916,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
         Ls = __builtin_fmaf(sm_l[half * WPU + i], wgt, Ls);
         As = __builtin_fmaf(sm_acc[(half * WPU + i) * D + d_], wgt, As);
       }
-      put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
+      put(a.ctx + (size_t)li * 16 * a.d + grouped_at(b, h * D + d_), (f16)(As / Ls));      // the layout of decode_step_wide_kernel
     }
   }
   wg_sync();
@@ -1252,16 +1260,15 @@ __device__ __forceinline__ bool await_row(const unsigned* rows, int row_words, i
 // caches: the 256 workgroups read the same values, and all but the first read of a line in each L2 stay out of the
 // fabric.  Nothing of a slot is in a cache before its arrival: the launch starts with an agent-scope acquire (no
 // line of the previous launch survives), no slot of this protocol is written with the filler, and every address is
-// written once per launch.  Features beyond K read as zero.
+// written once per launch.  The slot is laid out for this read (grouped_at): a wave's 64 loads of a step are one
+// contiguous KiB.  Features beyond K and rows beyond M read as zero.
 __device__ __forceinline__ void load_xtile(const f16* X, int M, int K, int kt, XTile& t) {
   const int lane = lane_id();
-  int row = lane & 15;
-  row = row < M ? row : M - 1;                // padding rows repeat the last one; their products are never stored
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int k = kt * 128 + j * 32 + (lane >> 4) * 8;
     t.v[j] = f16x8{};
-    if (k < K) t.v[j] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(X) + (size_t)row * K + k);
+    if ((lane & 15) < M && kt * 128 + j * 32 + (lane >> 4) * 8 < K)      // rows beyond M are never written
+      t.v[j] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(X) + ((size_t)(kt * 4 + j) * 64 + lane) * 8);
   }
 }
 
@@ -1272,19 +1279,28 @@ __device__ __forceinline__ float rows_of_wave(float v) {
   return v;
 }
 
+// sum over the eight elements of v of v[e] * u[e], added to s in fp32: four two-element dot products
+__device__ __forceinline__ float dot8(f16x8 v, f16x8 u, float s) {
+  s = __builtin_amdgcn_fdot2(__builtin_shufflevector(v, v, 0, 1), __builtin_shufflevector(u, u, 0, 1), s, false);
+  s = __builtin_amdgcn_fdot2(__builtin_shufflevector(v, v, 2, 3), __builtin_shufflevector(u, u, 2, 3), s, false);
+  s = __builtin_amdgcn_fdot2(__builtin_shufflevector(v, v, 4, 5), __builtin_shufflevector(u, u, 4, 5), s, false);
+  s = __builtin_amdgcn_fdot2(__builtin_shufflevector(v, v, 6, 7), __builtin_shufflevector(u, u, 6, 7), s, false);
+  return s;
+}
+
 // RMSNorm of the rows whose fragments the waves hold (layers/rms_layer_norm.py:26-36, as pta_rmsnorm): the sums of
 // squares meet in LDS, every lane then scales its own fragments by the weights normw_fetch brought to LDS.  NT tiles
 // per wave; tiles beyond KT hold zeros.
 template <int NT>
 __device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* lds_w, int K, int KT, float eps, float* sums) {
   const int lane = lane_id(), wave = wave_id();
+  // sixteen rows of K features are 6 lane operations per element when done one element at a time - microseconds
+  // per phase on the four SIMDs; two-element dot products and packed fp16 multiplies take a third of that
   float sq = 0.f;
 #pragma unroll
   for (int i = 0; i < NT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) { const float f = (float)t[i].v[j][e]; sq = __builtin_fmaf(f, f, sq); }
+    for (int j = 0; j < 4; ++j) sq = dot8(t[i].v[j], t[i].v[j], sq);
   sq = rows_of_wave(sq);
   if (lane < 16) sums[wave * DW_MAXB + lane] = sq;
   wg_sync();
@@ -1292,6 +1308,7 @@ __device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* lds_w, in
 #pragma unroll
   for (int ww = 0; ww < DS_WAVES; ++ww) tot += sums[ww * DW_MAXB + (lane & 15)];
   const f16 r16 = (f16)(1.0f / sqrtf(tot * (1.0f / (float)K) + eps));
+  const f16x8 r8 = {r16, r16, r16, r16, r16, r16, r16, r16};
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
     const int kt = wave + i * DS_WAVES;
@@ -1300,24 +1317,23 @@ __device__ __forceinline__ void norm_xtiles(XTile (&t)[NT], const f16* lds_w, in
       const int k = kt * 128 + j * 32 + (lane >> 4) * 8;
       if (kt < KT && k < K) {
         const f16x8 gm = *reinterpret_cast<const f16x8*>(lds_w + k);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) t[i].v[j][e] = (t[i].v[j][e] * r16) * gm[e];
+        t[i].v[j] = (t[i].v[j] * r8) * gm;      // fp16(fp16(x * r) * g), element by element
       }
     }
   }
 }
 
-// The rows' sums over this wave's fragments go to LDS (the INT4 products multiply by the stored codes q + 8 and take
-// 8 * sum(x) off at the end); `first`: the first contribution of the phase replaces what the slot held.
+// The rows' sums over this wave's fragments (the INT4 products multiply by the stored codes q + 8 and take
+// 8 * sum(x) off at the end), in fp32.
 template <int NT>
 __device__ __forceinline__ float xtiles_rowsum(const XTile (&t)[NT]) {
+  const f16 one = (f16)1.0f;
+  const f16x8 ones = {one, one, one, one, one, one, one, one};
   float s1 = 0.f;
 #pragma unroll
   for (int i = 0; i < NT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s1 += (float)t[i].v[j][e];
+    for (int j = 0; j < 4; ++j) s1 = dot8(t[i].v[j], ones, s1);
   return rows_of_wave(s1);
 }
 
@@ -1385,7 +1401,8 @@ __device__ __forceinline__ void wide_stash(const f32x4& sum, int r, float* rb) {
 
 // The partial sums of all waves meet: thread (r * 16 + m) * 16 + ch finishes channel ch of row m of matrix r
 // (EPI_SWIGLU: of the gate / up pair).  xsum: the waves' sums of the rows (8 * sum(x) comes off, the stored codes are
-// q + 8); scl[r * 16 + ch]: the channels' scales.  Returns the value stored (the thread's residual element in the next
+// q + 8); scl[r * 16 + ch]: the channels' scales.  EPI_STORE writes row-major outputs (q/k/v, read by the attention
+// phase), the others activation slots in the layout of grouped_at.  Returns the value stored (the thread's residual element in the next
 // residual phase).
 template <int NRB, int EPI>
 __device__ __forceinline__ f16 wide_finish(f16* const (&out)[NRB], int ostride, f16 res, int u, int N, int M, const float* rb,
@@ -1412,15 +1429,19 @@ __device__ __forceinline__ f16 wide_finish(f16* const (&out)[NRB], int ostride, 
         }
         sg = (sg - off) * scl[ch];
         su = (su - off) * scl[(NRB > 1 ? 16 : 0) + ch];
-        put(out[0] + (size_t)m_ * ostride + n, (f16)su * swish_f16((f16)sg));
+        put(out[0] + grouped_at(m_, n), (f16)su * swish_f16((f16)sg));
       } else {
         float s = 0.f;
 #pragma unroll 8
         for (int w = 0; w < DS_WAVES; ++w) s += rb[(w * NRB + r) * 256 + at];
         s = (s - off) * scl[r * 16 + ch];
         y = (f16)s;
-        if (EPI == EPI_RESIDUAL) y = y + res;
-        put(out[r] + (size_t)m_ * ostride + n, y);
+        if (EPI == EPI_RESIDUAL) {
+          y = y + res;
+          put(out[r] + grouped_at(m_, n), y);
+        } else {
+          put(out[r] + (size_t)m_ * ostride + n, y);
+        }
       }
     }
   }
@@ -1476,7 +1497,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
   Waiter w{a.sync + 1, lds_dead, 0};
   int red_buf = 0;
-  const size_t xslot = (size_t)M * a.d;
+  const size_t xslot = (size_t)DW_MAXB * a.d;      // halves of one residual-stream slot: always sixteen rows
 
   // ---- set-up: as in decode_step_kernel, except that only the slots the attention phase and the selection poll
   //      (q/k/v, attention partials, logits) are filled; the arrival rows are cleared
@@ -1506,7 +1527,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       const int b = i / a.d, c = i % a.d;
       int id = a.container[(size_t)b * a.max_len + col];
       id = id < 0 ? 0 : (id >= a.vocab ? a.vocab - 1 : id);
-      put(a.xres + i, a.embed[(size_t)id * a.d + c]);
+      put(a.xres + grouped_at(b, c), a.embed[(size_t)id * a.d + c]);
     }
   }
   wg_sync();
@@ -1535,7 +1556,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     const int tid = thread_id();
     const int m_ = tid >> 4, n = wg * 16 + (tid & 15);
     const bool on = m_ < M && n < a.d;
-    res = wait_value(a.xres + (on ? (size_t)m_ * a.d + n : 0), on, w);
+    res = wait_value(a.xres + (on ? grouped_at(m_, n) : 0), on, w);
   }
   const int wave = wave_id();
   auto phase_rows = [&](int phase) { return a.flags + (size_t)phase * DW_REPLICAS * a.flag_words; };
@@ -1591,7 +1612,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       if (a.nsplit == 1) {
         for (int u = wg; u < units; u += 2 * G) attention_two(a, li, kring, u, u + G < units ? u + G : -1, step, att_lds, cs, w);
       } else {
-        for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
+        for (int u = wg; u < units; u += G) attention_unit<true>(a, li, kring, u, step, att_lds, cs, w);
       }
       // the head outputs are stored by waves 0, 1 and (second unit of attention_two) 8, 9
       announce(phase_rows(4 * li + 1), a.flag_words, wg, wave < 2 || wave == 8 || wave == 9);
@@ -1649,7 +1670,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     {
       const float s1 = xtiles_rowsum<T>(xt);
       if (lane_id() < 16) xsum[wave * DW_MAXB + lane_id()] = s1;
-      f16* act = a.act + (size_t)li * M * a.ffn;
+      f16* act = a.act + (size_t)li * DW_MAXB * a.ffn;
       f16* const o2[2] = {act, act};
       wide_unit<2, T, EPI_SWIGLU, S_GU0>(S, scl, o2, a.ffn, (f16)0.0f, wg, nb_f, a.ffn, KT_D, M, xt, red, red_buf, xsum);
       if constexpr (U_F > 1)
@@ -1665,7 +1686,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       f32x4 acc[1][2];
       acc[0][0] = acc[0][1] = f32x4{0.f, 0.f, 0.f, 0.f};
       float s1 = 0.f;
-      const f16* actx = a.act + (size_t)li * M * a.ffn;
+      const f16* actx = a.act + (size_t)li * DW_MAXB * a.ffn;
       f16 sv[1] = {};
       if (wave == 0) { const Mat mm[1] = MD; request_scales<1>(mm, wg, nb_d, a.d, sv); }
       await_row(phase_rows(4 * li + 3), a.flag_words, G, wg, w);
@@ -1787,13 +1808,14 @@ struct Layout {
 };
 Layout layout_for(const pta_decode_model* m, int cus) {
   const size_t B = m->batch, d = m->hidden, L = m->n_layer, f = m->ffn, H = m->n_head;
+  const size_t R = B > DS_MAXB ? DW_MAXB : B;      // rows of an activation slot: decode_step_wide_kernel's hold sixteen
   Layout l;
   l.sync = 0;
   l.xres = align256((size_t)(16 + cus) * 4);
-  l.qkv = l.xres + align256((2 * L + 1) * B * d * 2);
+  l.qkv = l.xres + align256((2 * L + 1) * R * d * 2);
   l.ctx = l.qkv + align256(L * B * 3 * d * 2);
-  l.act = l.ctx + align256(L * B * d * 2);
-  l.part = l.act + align256(L * B * f * 2);
+  l.act = l.ctx + align256(L * R * d * 2);
+  l.part = l.act + align256(L * R * f * 2);
   l.flags = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
   l.trace = l.flags + align256((4 * L + 1) * 16 /* DW_REPLICAS */ * flag_words_for(cus) * 4);
   l.total = l.trace + (size_t)cus * 256;
