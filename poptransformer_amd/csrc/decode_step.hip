@@ -46,6 +46,7 @@ namespace {
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
+constexpr int DS_REPLICAS = 16;                             // copies of a row of arrival words, see grid_barrier
 constexpr int DS_MAXB = 4;
 constexpr int DS_D = 128;                                   // head size
 constexpr int DS_MAX_SPLIT = 16;
@@ -83,6 +84,7 @@ struct DsArgs {
   size_t fill_bytes;     // qkv .. end of part, contiguous from xres + B*d (the first residual is not filled)
   unsigned* flags;       // [4 n_layer + 1][DW_REPLICAS][flag_words] arrival words of decode_step_wide_kernel, behind part
   int flag_words;        // words of one row: the workgroups, rounded up to a KiB
+  uint32_t* best;        // [workgroups][16 rows][2]: value bits and index of each workgroup's largest logit per row (wide kernel)
   unsigned* sync;
   int nsplit;
   int region0;           // bytes of the activation / attention area at the start of LDS
@@ -91,8 +93,10 @@ struct DsArgs {
 
 #ifdef DS_TRACE
 #define TRACE(i) do { if (li == 1 && thread_id() == 0) a.trace[g.wg * 32 + (i)] = wall_clock64(); } while (0)
+#define TRACE_STEP(i) do { if (thread_id() == 0) a.trace[g.wg * 32 + (i)] = wall_clock64(); } while (0)
 #else
 #define TRACE(i) do {} while (0)
+#define TRACE_STEP(i) do {} while (0)
 #endif
 
 // The asm statements make the thread index opaque at each use, so that what a phase derives from
@@ -216,18 +220,21 @@ __device__ __forceinline__ void wait_triple(const float* p0, const float* p1, co
 }
 
 // The one grid barrier of a launch (after the slots have been filled).  sync[0] holds the epoch
-// base, sync[1] the error word, sync[16 + g] the arrival word of workgroup g.
+// base, sync[1] the error word, sync[16 + r * G + g] copy r of the arrival word of workgroup g: the
+// words of one copy share a memory channel, and G workgroups polling one copy queue there for
+// microseconds, so every workgroup writes DS_REPLICAS copies and polls copy g % DS_REPLICAS.
 __device__ __forceinline__ void grid_barrier(unsigned* sync, unsigned epoch, int G, int wg, Waiter& w) {
   const int wave = wave_id(), lane = lane_id();
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's agent-scope stores have completed
   wg_sync();
-  if (thread_id() == 0)
-    __hip_atomic_store((DS_GLOBAL unsigned*)(sync + 16 + wg), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (wave == 0) {
+    if (lane < DS_REPLICAS)
+      __hip_atomic_store((DS_GLOBAL unsigned*)(sync + 16 + lane * G + wg), epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned* mine = sync + 16 + (wg % DS_REPLICAS) * G;
     for (;;) {
       bool ok = true;
       for (int i = lane; i < G; i += 64) {
-        const unsigned v = __hip_atomic_load((DS_GLOBAL unsigned*)(sync + 16 + i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned v = __hip_atomic_load((DS_GLOBAL unsigned*)(mine + i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         ok = ok && ((int)(v - epoch) >= 0);
       }
       if (__all(ok) || w.give_up()) break;
@@ -923,55 +930,16 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
 }
 
 // ------------------------------------------------------------------------------------------ selection and bookkeeping
-// Top-1 per sequence (lowest index among equals), then the container / mask / stop-mask update of
-// models/base_model.py:313-355 exactly as step_update_kernel in select.hip; workgroup 0 only.
-// Returns false when the wait for the logits was given up (nothing is updated then).
-__device__ __forceinline__ bool select_and_advance(const DsArgs& a, float* lds, Waiter& w) {
-  float* sv = lds;
-  int* si = reinterpret_cast<int*>(lds + DS_WAVES);
-  int* ids = si + DS_WAVES;
-  const int lane = lane_id(), wave = wave_id();
-  for (int b = 0; b < a.B; ++b) {
-    const f16* xr = a.logits + (size_t)b * a.vocab;
-    float best = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i0 = thread_id() * 8; __any(i0 < a.vocab); i0 += DS_THREADS * 8) {
-      const bool on = i0 < a.vocab;      // vocab is a multiple of 8
-      u32x4 v = {0, 0, 0, 0};
-      for (;;) {
-        if (on) v = get16(xr, (size_t)a.vocab * 2, (size_t)i0 * 2);
-        if (!__any(on && has_empty16(v)) || w.give_up()) break;
-      }
-      if (on) {
-        const f16x8 h = bitcast<f16x8>(v);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float f = (float)h[e];
-          if (f > best) { best = f; bi = i0 + e; }
-        }
-      }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-    }
-    if (lane == 0) { sv[wave] = best; si[wave] = bi; }
-    wg_sync();
-    if (thread_id() == 0) {
-      for (int ww = 1; ww < DS_WAVES; ++ww)
-        if (sv[ww] > best || (sv[ww] == best && si[ww] < bi)) { best = sv[ww]; bi = si[ww]; }
-      ids[b] = bi == 0x7fffffff ? 0 : bi;
-    }
-    wg_sync();
-  }
-  if (*w.lds_dead != 0) return false;
-  if (thread_id() == 0) {
+// The container / mask / stop-mask update of models/base_model.py:313-355 exactly as step_update_kernel in
+// select.hip, from the rows' picks in ids (LDS); the first wave, one lane per row.
+__device__ __forceinline__ void advance_rows(const DsArgs& a, const int* ids) {
+  if (wave_id() == 0) {      // lane b takes row b: the rows' loads travel together
+    const int b = lane_id();
+    const bool on = b < a.B;
     const int ns = *a.step + 1;
-    int stopped_before = 0;
-    for (int b = 0; b < a.B; ++b) {
-      if (a.stop_mask[b]) ++stopped_before;
+    const bool stopped = on && a.stop_mask[on ? b : 0] != 0;
+    const int stopped_before = __popcll(__ballot(stopped));
+    if (on) {
       int id = ids[b];
       a.next_ids[b] = id;
       if (ns < a.max_len) {
@@ -980,11 +948,84 @@ __device__ __forceinline__ bool select_and_advance(const DsArgs& a, float* lds, 
         id = slot == a.pad_id ? id : slot;
         a.container[(size_t)b * a.max_len + ns] = id;
       }
-      a.stop_mask[b] |= (id == a.eos_id) ? 1 : 0;
+      if (id == a.eos_id) a.stop_mask[b] |= 1;
     }
-    *a.keep_going = a.early_stop ? (stopped_before < a.B ? 1 : 0) : 1;
-    *a.step = ns;
+    if (b == 0) {
+      *a.keep_going = a.early_stop ? (stopped_before < a.B ? 1 : 0) : 1;
+      *a.step = ns;
+    }
   }
+}
+
+// Top-1 per sequence (lowest index among equals) over the logits, then advance_rows; workgroup 0 only.
+// Returns false when the wait for the logits was given up (nothing is updated then).
+__device__ __forceinline__ bool select_and_advance(const DsArgs& a, float* lds, Waiter& w) {
+  float* sv = lds;
+  int* si = reinterpret_cast<int*>(lds + DS_WAVES);
+  int* ids = si + DS_WAVES;
+  const int lane = lane_id(), wave = wave_id();
+  // All rows at once: 16, 8, 4, 2 or 1 waves per row for up to 1, 2, 4, 8, 16 rows.  A wave takes the 512-element
+  // pieces part, part + wpr, ... of its row, eight pieces per round trip.
+  constexpr int U = 8;
+  const int wpr = a.B <= 1 ? 16 : a.B <= 2 ? 8 : a.B <= 4 ? 4 : a.B <= 8 ? 2 : 1;
+  const int row = wave / wpr, part = wave % wpr;
+  const bool active = row < a.B;
+  const f16* xr = a.logits + (size_t)(active ? row : 0) * a.vocab;
+  float best = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int c = part * 512; c < a.vocab; c += wpr * 512 * U) {
+    u32x4 v[U];
+    bool need[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      v[u] = u32x4{0, 0, 0, 0};
+      need[u] = active && c + u * wpr * 512 + lane * 8 < a.vocab;      // vocab is a multiple of 8
+    }
+    for (;;) {
+      bool pending = false;
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (need[u]) v[u] = get16(xr, (size_t)a.vocab * 2, (size_t)(c + u * wpr * 512 + lane * 8) * 2);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (need[u]) {
+          if (has_empty16(v[u])) pending = true;
+          else need[u] = false;
+        }
+      if (!__any(pending) || w.give_up()) break;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i0 = c + u * wpr * 512 + lane * 8;
+      if (active && i0 < a.vocab) {
+        const f16x8 h = bitcast<f16x8>(v[u]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float f = (float)h[e];
+          if (f > best) { best = f; bi = i0 + e; }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+  }
+  if (lane == 0) { sv[wave] = best; si[wave] = bi; }
+  wg_sync();
+  if (thread_id() < a.B) {
+    const int b = thread_id();
+    best = sv[b * wpr];
+    bi = si[b * wpr];
+    for (int ww = 1; ww < wpr; ++ww)
+      if (sv[b * wpr + ww] > best || (sv[b * wpr + ww] == best && si[b * wpr + ww] < bi)) { best = sv[b * wpr + ww]; bi = si[b * wpr + ww]; }
+    ids[b] = bi == 0x7fffffff ? 0 : bi;
+  }
+  wg_sync();
+  if (*w.lds_dead != 0) return false;
+  advance_rows(a, ids);
   return true;
 }
 
@@ -1229,7 +1270,7 @@ struct XTile {
 // polling one KiB would all queue at one memory channel.  The launch cleared the rows before its grid barrier.  Only
 // the first wave of a consumer polls, at agent scope; the workgroup meets, and only then are the phase's values read -
 // with ordinary loads.
-constexpr int DW_REPLICAS = 16;
+constexpr int DW_REPLICAS = DS_REPLICAS;
 __device__ __forceinline__ void announce(unsigned* rows, int row_words, int wg, bool stored) {
   if (stored) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   wg_sync();
@@ -1501,7 +1542,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 
   // ---- set-up: as in decode_step_kernel, except that only the slots the attention phase and the selection poll
   //      (q/k/v, attention partials, logits) are filled; the arrival rows are cleared
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");      // no cache holds a line of an earlier launch
+  TRACE_STEP(26);
+  if (wave_id() == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");      // no cache holds a line of an earlier launch
+  TRACE_STEP(25);
   {
     const int tid = thread_id();
     if (tid == 0) *lds_dead = 0;
@@ -1514,6 +1557,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     for (size_t off = first; off < qkv_bytes; off += stride) put16(a.qkv, qkv_bytes, off, filler);
     for (size_t off = first; off < part_bytes; off += stride) put16(a.part, part_bytes, off, filler);
     for (size_t off = first; off < flag_bytes; off += stride) put16(a.flags, flag_bytes, off, zero);
+    for (size_t off = first; off < (size_t)G * 128; off += stride) put16(a.best, (size_t)G * 128, off, filler);
     for (size_t i = ((size_t)wg * DS_THREADS + tid) * 8; i < (size_t)M * a.vocab; i += (size_t)G * DS_THREADS * 8)
       put16(a.logits, (size_t)M * a.vocab * 2, i * 2, filler);
     for (int i = tid; i < a.n_layer * DS_LAYER_WORDS; i += DS_THREADS) lds_layers[i] = a.layers[i];
@@ -1547,8 +1591,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     const Mat m3[3] = {layer_mat(L0, P_WQ, P_SQ), layer_mat(L0, P_WK, P_SK), layer_mat(L0, P_WV, P_SV)};
     load_tiles<3, T, S_QKV>(S, m3, wg, nb_d, KT_D);
   }
+  TRACE_STEP(27);
   grid_barrier(a.sync, epoch, G, wg, w);
   bool alive = *lds_dead == 0;
+  TRACE_STEP(28);
 
   // the residual element of this thread's output (epilogue mapping of wide_finish: row tid / 16, channel tid % 16)
   f16 res = (f16)0.0f;
@@ -1723,6 +1769,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       TRACE(9);
     }
   }
+  TRACE_STEP(29);
 #undef M3
 #undef MO
 #undef MGU
@@ -1744,6 +1791,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       const Mat m1[1] = {{a.head, nullptr}};
       f16* const o1[1] = {a.logits};
       Unit<FmtF16, 1, T> even, odd;
+      // thread 16 m + ch finishes channel ch of row m of every unit and keeps the row's largest logit among them (the
+      // lowest index among equals: the units come in ascending order, NaN is never larger)
+      float top = -INFINITY;
+      int top_at = 0x7fffffff;
       auto head_unit = [&](const Unit<FmtF16, 1, T>& t, int u) {
         if (u >= nb_v) return;
         f32x4 acc[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
@@ -1754,7 +1805,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
             for (int j = 0; j < 4; ++j)
               acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(FmtF16::a_operand(t.w[0][i], j, t.sc[0]), xt[i].v[j], acc[0], 0, 0, 0);
           }
-        finish_unit<1, EPI_STORE, false, NoScales, DW_MAXB, DW_RED>(acc, o1, a.vocab, (f16)0.0f, u, a.vocab, M, red, red_buf);
+        const f16 y = finish_unit<1, EPI_STORE, false, NoScales, DW_MAXB, DW_RED>(acc, o1, a.vocab, (f16)0.0f, u, a.vocab, M, red, red_buf);
+        const int tid = thread_id(), n = u * 16 + (tid & 15);
+        if (tid < 16 * M && n < a.vocab && (float)y > top) { top = (float)y; top_at = n; }
       };
       load_unit(even, m1, wg, nb_v, a.vocab, KT_D);
       for (int u = wg; u < nb_v; u += 2 * G) {
@@ -1763,14 +1816,67 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
         load_unit(even, m1, u + 2 * G, nb_v, a.vocab, KT_D);
         head_unit(odd, u + G);
       }
+      // the sixteen channels of a row meet; the row's pair goes to this workgroup's place
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(top, o, 64);
+        const int oi = __shfl_xor(top_at, o, 64);
+        if (ov > top || (ov == top && oi < top_at)) { top = ov; top_at = oi; }
+      }
+      const int tid = thread_id();
+      if (tid < 16 * M && (tid & 15) == 0) {
+        uint32_t* mine = a.best + ((size_t)wg * 16 + (tid >> 4)) * 2;
+        __hip_atomic_store((DS_GLOBAL uint32_t*)mine, bitcast<uint32_t>(top), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store((DS_GLOBAL uint32_t*)(mine + 1), (uint32_t)top_at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   }
+  TRACE_STEP(30);
   // ---- selection and bookkeeping
   if (wg == 0) {
-    if (alive) select_and_advance(a, sel, w);
+    if (alive) {
+      // wave r gathers row r's pairs of all workgroups (neither word of a pair is ever the filler)
+      int* ids = reinterpret_cast<int*>(sel);
+      const int lane = lane_id();
+      float top = -INFINITY;
+      int top_at = 0x7fffffff;
+      if (wave < M) {
+        for (int g0 = 0; g0 < G; g0 += 256) {      // four pairs per lane travel together
+          uint32_t vb[4], ib[4];
+          for (;;) {
+            bool pending = false;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int gg = g0 + k * 64 + lane;
+              const uint32_t* p = a.best + ((size_t)(gg < G ? gg : G - 1) * 16 + wave) * 2;
+              vb[k] = get_bits(reinterpret_cast<const float*>(p));
+              ib[k] = get_bits(reinterpret_cast<const float*>(p + 1));
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) pending = pending || vb[k] == DS_EMPTY32 || ib[k] == DS_EMPTY32;
+            if (!__any(pending) || w.give_up()) break;
+          }
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const float v = bitcast<float>(vb[k]);
+            if (g0 + k * 64 + lane < G && (v > top || (v == top && (int)ib[k] < top_at))) { top = v; top_at = (int)ib[k]; }
+          }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+          const float ov = __shfl_xor(top, o, 64);
+          const int oi = __shfl_xor(top_at, o, 64);
+          if (ov > top || (ov == top && oi < top_at)) { top = ov; top_at = oi; }
+        }
+        if (lane == 0) ids[wave] = top_at == 0x7fffffff ? 0 : top_at;
+      }
+      wg_sync();
+      if (*lds_dead == 0) advance_rows(a, ids);
+    }
     if (thread_id() == 0)
       __hip_atomic_store((DS_GLOBAL unsigned*)a.sync, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  TRACE_STEP(31);
 }
 
 struct Variant {
@@ -1804,20 +1910,21 @@ size_t flag_words_for(int cus) { return ((size_t)cus + 255) & ~(size_t)255; }
 
 // byte offsets of the workspace parts
 struct Layout {
-  size_t sync, xres, qkv, ctx, act, part, flags, trace, total;
+  size_t sync, xres, qkv, ctx, act, part, flags, best, trace, total;
 };
 Layout layout_for(const pta_decode_model* m, int cus) {
   const size_t B = m->batch, d = m->hidden, L = m->n_layer, f = m->ffn, H = m->n_head;
   const size_t R = B > DS_MAXB ? DW_MAXB : B;      // rows of an activation slot: decode_step_wide_kernel's hold sixteen
   Layout l;
   l.sync = 0;
-  l.xres = align256((size_t)(16 + cus) * 4);
+  l.xres = align256((size_t)(16 + DS_REPLICAS * cus) * 4);
   l.qkv = l.xres + align256((2 * L + 1) * R * d * 2);
   l.ctx = l.qkv + align256(L * B * 3 * d * 2);
   l.act = l.ctx + align256(L * R * d * 2);
   l.part = l.act + align256(L * R * f * 2);
   l.flags = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
-  l.trace = l.flags + align256((4 * L + 1) * 16 /* DW_REPLICAS */ * flag_words_for(cus) * 4);
+  l.best = l.flags + align256((4 * L + 1) * DS_REPLICAS * flag_words_for(cus) * 4);
+  l.trace = l.best + align256((size_t)cus * 16 * 2 * 4);
   l.total = l.trace + (size_t)cus * 256;
   return l;
 }
@@ -1886,6 +1993,7 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.fill_bytes = lay.flags - (lay.xres + (size_t)B * d * 2);   // everything after the first residual slot, up to the flags
   a.flags = (unsigned*)(ws + lay.flags);
   a.flag_words = (int)flag_words_for(cus);
+  a.best = (uint32_t*)(ws + lay.best);
   a.nsplit = splits_for(cus, B, H);
   const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
