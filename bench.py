@@ -10,11 +10,11 @@ always run untimed first (in passes of up to 64 rows; ``--prompt-loop``: one ite
 the reference's loop does), then ``--warmup`` further untimed iterations, then ``--steps`` timed ones: the
 timed iterations generate new tokens whatever the flags are.
 
-By default the iteration runs as one persistent launch (pta_llama_decode_step, batch <= 4);
+By default the iteration runs as one persistent launch (pta_llama_decode_step, batch <= 16);
 ``--executor operators`` runs it as one launch per operator instead.
 
-The default run also measures batch 16 (same model and step counts, one launch per operator) and reports it
-under "batch16" beside the batch-1 headline.
+The default run also measures batch 16 (same model, step counts and executor) and reports it under "batch16"
+beside the batch-1 headline.
 
 Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel measured with events
 on the stream it runs on (the persistent decode-step kernel: one launch moves the whole step's
@@ -319,7 +319,7 @@ def main():
                          "untimed); other workloads: untimed steps")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--executor", choices=["persistent", "operators"], default=None,
-                    help="default: persistent when the batch fits it (<= 4), else operators")
+                    help="default: persistent when the batch fits it (<= 16, fp16 cache), else operators")
     ap.add_argument("--workload", choices=["decode", "gemm", "chatglm2", "rwkv", "prompt"], default="decode",
                     help="decode: the Llama2-7B-shape INT4 decode loop (the headline); gemm: the single INT4 "
                          "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
@@ -373,7 +373,7 @@ def main():
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
-    executor = args.executor or ("persistent" if B <= 4 and not args.fp8_cache else "operators")
+    executor = args.executor or ("persistent" if B <= 16 and not args.fp8_cache else "operators")
     if args.fuse_norm is not None:
         dec.fuse_norm = args.fuse_norm == "on"
     if executor == "persistent":
@@ -427,7 +427,8 @@ def main():
         torch.cuda.synchronize()
         kernel_s = e0.elapsed_time(e1) * 1e-3 / reps
         kernel_bytes = float(np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(t_first, t_first + reps)]))
-        kernel_name = "decode_step_kernel<2, 6, 3, %d> (whole decode step)" % (1 if B == 1 else 4)
+        kernel_name = ("decode_step_kernel<2, 6, 3, %d>" % (1 if B == 1 else 4) if B <= 4 else
+                       "decode_step_wide_kernel<2, 6, 3>") + " (whole decode step)"
     else:
         # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
         # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
@@ -477,12 +478,14 @@ def main():
                      "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }
     if B == 1 and not args.no_batch16 and not args.copy_calibration:
-        # the metric names batch 1 and batch 16: the same model, prompt and step counts at batch 16 (one launch per
-        # operator from a HIP graph), reported beside the headline; `value` stays the batch-1 figure
+        # the metric names batch 1 and batch 16: the same model, prompt, step counts and executor at batch 16,
+        # reported beside the headline; `value` stays the batch-1 figure
         del dec
         torch.cuda.empty_cache()
         B16 = 16
         dec16 = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B16, pad_id=0, eos_id=2), weights)
+        if executor == "persistent":
+            dec16.enable_persistent()
         dec16.capture()
         ids16 = np.zeros((B16, MAX_LEN), np.int32)
         ids16[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B16, prompt))
@@ -491,9 +494,12 @@ def main():
         dec16.run_steps(args.steps)
         torch.cuda.synchronize()
         dt16 = time.perf_counter() - t0
+        if executor == "persistent" and dec16.persistent.failed():
+            print("the persistent decode step reported a failure at batch 16", file=sys.stderr)
+            sys.exit(1)
         bytes16 = float(np.mean([algorithmic_step_bytes(cfg, B16, t) for t in range(t_first, t_first + args.steps)]))
         out["batch16"] = {"value": B16 * args.steps / dt16, "unit": "tokens/s", "ms_per_step": dt16 / args.steps * 1e3,
-                          "executor": "operators", "timed_context": [t_first, t_first + args.steps - 1],
+                          "executor": executor, "timed_context": [t_first, t_first + args.steps - 1],
                           "step_algorithmic_bytes": bytes16,
                           "step_roofline_frac": bytes16 / (dt16 / args.steps) / (HBM_PEAK_GBS * 1e9)}
     if args.copy_calibration:

@@ -411,8 +411,9 @@ int pta_rwkv_wkv(const pta_half* k, const pta_half* v, const pta_half* r, const 
  * models/llama2/model.py:162-197: embedding, every decoder layer, final RMSNorm, lm_head,
  * top-1, container / mask / stop-mask update).  The reference compiles this loop body into one
  * Poplar program; this entry is its counterpart for INT4 Llama-2 shapes: a single persistent
- * kernel, one workgroup per compute unit, phases separated by a grid-wide barrier, the weights of
- * later phases requested early.  Results equal those of the per-operator entry points above run in the
+ * kernel, one workgroup per compute unit; a phase hands its results to the next through slots of the
+ * workspace that the consumers poll (no grid-wide barrier between phases), the weights of later phases
+ * are requested early.  Results equal those of the per-operator entry points above run in the
  * reference's order, up to the order in which attention partial sums are merged.
  * ---------------------------------------------------------------------------------- */
 
@@ -451,8 +452,10 @@ typedef struct pta_decode_state {
  * few synchronisation words.  The caller zeroes it once after allocating it (256-byte aligned). */
 size_t pta_decode_step_workspace_bytes(const pta_decode_model* model);
 
-/* Enqueues one loop iteration.  Supports batch <= 4, head_dim 128, hidden = n_head * 128 with
- * (hidden, ffn) of the 7B model or a small test shape; PTA_EUNSUPPORTED otherwise.
+/* Enqueues one loop iteration.  Supports batch <= 16, head_dim 128, hidden = n_head * 128 with
+ * (hidden, ffn) of the 7B model or a small test shape; PTA_EUNSUPPORTED otherwise.  Batches of 5..16
+ * run a second kernel of the same structure (activations as matrix-instruction fragments in registers
+ * instead of staged in LDS).
  * Needs every compute unit of the device for itself while it runs: workgroups wait for each
  * other's results, every wait is bounded, and if one gives up it sets word 1 of the workspace
  * (sticky), the loop state is left untouched and the kernel ends; pta_decode_step_failed reports it.

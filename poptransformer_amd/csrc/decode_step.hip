@@ -845,6 +845,24 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
   const f16* qrow = a.qkv + ((size_t)li * a.B + b) * 3 * a.d + h * D;
   f16* kring = kring_base + ((size_t)b * a.H + h) * a.max_len * D;
   f16* vring = kring + (size_t)a.B * a.H * a.max_len * D;
+  // The cache rows of the first NPRE rounds (a round: four rows per wave) are requested before q, k and v are waited
+  // for: the rows are known, and they travel while the producers' values do.  (More rounds, or a window that is
+  // requested again as it is visited, do not fit the registers next to the weight tiles in flight.)
+  constexpr int NPRE = 4;
+  f16x8 kp[NPRE], vp[NPRE];
+  {
+    const int grp = lane / LPP, d0 = (lane % LPP) * 8;
+#pragma unroll
+    for (int it = 0; it < NPRE; ++it) {
+      const int p = wv * PPW + grp + it * WPU * PPW;
+      kp[it] = f16x8{};
+      vp[it] = f16x8{};
+      if (active && p < valid && p != pos) {
+        kp[it] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)p * D + d0);
+        vp[it] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)p * D + d0);
+      }
+    }
+  }
   {
     const int t = thread_id() - half * WPU * 64;
     const int which = t / D, d_ = t % D;
@@ -874,18 +892,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (int p0 = wv * PPW; p0 < valid; p0 += WPU * PPW) {
-      const int p = p0 + grp;
-      const bool on = p < valid;
-      const int pc = on ? p : valid - 1;
-      f16x8 k8, v8;
-      if (pc == pos) {      // this step's row: taken from LDS, its global copy is being written
-        k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
-        v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
-      } else {
-        k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)pc * D + d0);
-        v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)pc * D + d0);
-      }
+    auto visit = [&](f16x8 k8, f16x8 v8, bool on) {
       float s = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
@@ -901,6 +908,34 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
       m = mn;
+    };
+#pragma unroll
+    for (int it = 0; it < NPRE; ++it) {
+      const int p0 = wv * PPW + it * WPU * PPW;
+      if (p0 < valid) {
+        const int p = p0 + grp;
+        const bool on = p < valid;
+        f16x8 k8 = kp[it], v8 = vp[it];
+        if ((on ? p : valid - 1) == pos) {      // this step's row: taken from LDS, its global copy is being written
+          k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
+          v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
+        }
+        visit(k8, v8, on);
+      }
+    }
+    for (int p0 = wv * PPW + NPRE * WPU * PPW; p0 < valid; p0 += WPU * PPW) {
+      const int p = p0 + grp;
+      const bool on = p < valid;
+      const int pc = on ? p : valid - 1;
+      f16x8 k8, v8;
+      if (pc == pos) {
+        k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
+        v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
+      } else {
+        k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)pc * D + d0);
+        v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)pc * D + d0);
+      }
+      visit(k8, v8, on);
     }
     merge_lanes(m, l, acc, 16);
     merge_lanes(m, l, acc, 32);

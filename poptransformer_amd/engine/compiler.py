@@ -7,7 +7,7 @@ state-dict keys the layers registered as initializer names, the shapes off a one
 the interpreter, and the weights off the initializers.  The fused executor is then VALIDATED: it
 must generate the same token ids as the interpreter on a probe prompt (for a sampling graph: the same top-k candidates), otherwise
 the graph stays on the interpreter - or, for a strict session, compilation fails.  An INT4 Llama-2
-graph at batch <= 4 is further mapped onto the one-launch-per-iteration persistent step, validated
+graph at batch <= 16 is further mapped onto the one-launch-per-iteration persistent step, validated
 the same way, and prompts are taken in passes over several positions.
 """
 import dataclasses
@@ -372,7 +372,7 @@ def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True, strict=F
     which one it is: 'interpreter', 'fused:<family>' (one launch per operator, replayed from a HIP graph) or
     'fused:llama2:persistent' (one launch per loop iteration).  A graph the fused executors do not cover stays on
     the interpreter, with the reason in `fallback_reason`; with `strict` that is an error instead.
-    persistent: use the one-launch iteration where the model allows it (INT4 Llama 2, batch <= 4, top-1; it needs
+    persistent: use the one-launch iteration where the model allows it (INT4 Llama 2, batch <= 16, top-1; it needs
     the whole device for itself while it runs).  prompt_passes: the leading iterations that only read the prompt
     run as passes over several positions.  fp8_cache: KV caches hold F143 bytes (KVCache with fp8 = true)."""
     from .. import _lib

@@ -19,7 +19,7 @@ class Session:
         # executor choices of this build (the reference has one executor, PopART's):
         #   allow_fused   map a known decoder loop onto the fused executors (else: op by op)
         #   strict        fail compilation instead of falling back to the op-by-op interpreter
-        #   persistent    one launch per loop iteration where the model allows it (INT4 Llama 2, batch <= 4); that
+        #   persistent    one launch per loop iteration where the model allows it (INT4 Llama 2, batch <= 16); that
         #                 kernel occupies every compute unit while it runs: nothing else may run on the device beside it
         #   prompt_passes take the prompt's positions in passes of up to 64 rows instead of one per iteration
         #   fp8_cache     KV caches hold F143 bytes, as the KVCache op does with fp8 = true
