@@ -338,11 +338,46 @@ def _fp8_cache_of(facts, requested):
     return bool(requested) or (flags == {True})
 
 
-def _validate_greedy(decoder, prog, facts, ids, steps, prompt_passes, what):
+def _validate_greedy_up_to_a_tie(decoder, prog, facts, steps, prompt_passes, what, seeds=(0, 1, 2, 3, 4, 5), least=3):
+    """The fused executors' arithmetic is not bit for bit the graph's (projections that the graph runs one by one
+    share a launch with another summation order; the one-launch iteration applies an INT4 scale to the fp32 sum,
+    the graph to every weight): greedy tokens are comparable only up to the first iteration
+    whose two largest logits, in any row, are closer than 0.5 % of the largest magnitude (5 % where the graph casts
+    activations to FP8: one code of an activation is an eighth of its value) - there a last-bit difference may
+    legitimately pick the other token, and everything after it differs.  Probes (a fixed list of
+    seeds) are tried until one has `least` comparable generated tokens; all of those must be equal.  A probe whose
+    tokens are all equal is accepted as it is."""
+    interp = prog.interp
+    margin = 0.05 if any("CastToUint8" in n.op for n in facts.body.nodes) else 0.005
+    # first the plain check: every token of one probe equal (it holds whenever no near tie decides, and always
+    # for an executor that repeats the graph's arithmetic)
+    ids = _probe_ids(facts, seeds[0], n=3)
     want = prog._run_once({facts.ids_name: ids})[prog.interp_outputs[0]]
     got, _ = decoder.run(ids, steps, prompt_passes=prompt_passes)
-    if not np.array_equal(got, want):
-        raise ValueError(f"{what} does not reproduce the graph's tokens on the probe")
+    if np.array_equal(got, want):
+        return
+    for seed in seeds:
+        ids = _probe_ids(facts, seed, n=3)
+        interp.input_trace = {"aiOnnx.topk": []}
+        try:
+            want = prog._run_once({facts.ids_name: ids})[prog.interp_outputs[0]]
+            logits = [np.asarray(i[0], np.float32).reshape(facts.batch, -1) for i in interp.input_trace["aiOnnx.topk"]]
+        finally:
+            interp.input_trace = None
+        first_tie = len(logits)
+        for t, lg in enumerate(logits):
+            top2 = np.sort(lg, axis=1)[:, -2:]
+            if (top2[:, 1] - top2[:, 0] < margin * np.abs(lg).max()).any():
+                first_tie = t
+                break
+        cols = min(first_tie + 1, want.shape[1])          # the token chosen at iteration t lands in column t + 1
+        if cols - 3 < least:
+            continue
+        got, _ = decoder.run(ids, steps, prompt_passes=prompt_passes)
+        if not np.array_equal(got[:, :cols], want[:, :cols]):
+            raise ValueError(f"{what} does not reproduce the graph's tokens on the probe (seed {seed}, {cols} columns)")
+        return
+    raise ValueError(f"{what}: no probe among the seeds has {least} generated tokens before a near tie")
 
 
 def _validate_sampling(decoder, prog, facts, ids, steps, k):
@@ -417,15 +452,15 @@ def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True, strict=F
             # the option changes what the graph computes (its caches are fp16): nothing to compare the tokens with;
             # the executor is checked against the graph with fp16 caches first, then switched
             plain = fused.FusedDecoder(dataclasses.replace(spec, fp8_cache=False), weights)
-            _validate_greedy(plain, prog, facts, ids, steps, passes, "the fused executor")
+            _validate_greedy_up_to_a_tie(plain, prog, facts, steps, passes, "the fused executor")
             del plain
             decoder.capture()
             kind = f"fused:{family}"
         else:
-            # validation: identical ids after a few iterations, eager and replayed
-            _validate_greedy(decoder, prog, facts, ids, steps, passes, "the fused executor")
+            # validation: identical ids over a few iterations (up to a near tie), eager and replayed
+            _validate_greedy_up_to_a_tie(decoder, prog, facts, steps, passes, "the fused executor")
             decoder.capture()
-            _validate_greedy(decoder, prog, facts, ids, steps, passes, "the captured HIP graph")
+            _validate_greedy_up_to_a_tie(decoder, prog, facts, steps, passes, "the captured HIP graph")
             kind = f"fused:{family}"
             if persistent and hasattr(decoder, "enable_persistent"):
                 try:
@@ -435,7 +470,7 @@ def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True, strict=F
                 else:
                     decoder.capture()
                     try:
-                        _validate_greedy(decoder, prog, facts, ids, steps, passes, "the persistent decode step")
+                        _validate_greedy_up_to_a_tie(decoder, prog, facts, steps, passes, "the persistent decode step")
                         kind += ":persistent"
                     except (ValueError, RuntimeError) as e:
                         if strict:

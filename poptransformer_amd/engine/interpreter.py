@@ -90,6 +90,8 @@ class Interpreter:
             raise NotImplementedError(f"operator {op} is not implemented")
         if self.shape_trace is not None and op.startswith("custom."):
             self.shape_trace.setdefault(op, []).append([tuple(t.shape) for t in ins])
+        if self.input_trace is not None and op in self.input_trace:
+            self.input_trace[op].append([v.detach().cpu().numpy() if torch.is_tensor(v) else v for v in ins])
         out = fn(n, env, *ins)
         if self.value_trace is not None and op in self.value_trace:
             vals = out if isinstance(out, (list, tuple)) else [out]
@@ -269,6 +271,7 @@ class Interpreter:
     max_trips = None            # cap on loop iterations (shape discovery, validation probes)
     shape_trace = None          # when a dict: operand shapes of the native operators, per op name
     value_trace = None          # when a dict {op name: []}: the outputs of every execution of those ops (host copies)
+    input_trace = None          # the same for their inputs
 
     def _aiGraphcore_call(self, n, env, *ins):
         body = n.subgraph

@@ -90,6 +90,16 @@ def test_llama2_int4_through_the_operator_api():
            kind="fused:llama2:persistent", session_kwargs={"strict": True})
 
 
+def test_llama2_int4_batch_6_through_the_operator_api():
+    """Batches of 5..16 reach the one-launch iteration as well (its sixteen-row kernel)."""
+    from poptransformer_amd.models.llama2 import LLAMA2DecModel
+    B, L, steps, pad, eos = 6, 32, 20, 0, 2
+    sd = OM.make_llama2_state_dict(LLAMA, seed=21, int4=True)
+    ids = lambda seed: _ids(np.random.default_rng(300 + seed), B, L, 5, 512, pad)
+    _check(LLAMA2DecModel, "int4", B, L, steps, pad, eos, sd, LLAMA, lambda: OM.Llama2Oracle(sd, LLAMA, L, B), ids,
+           kind="fused:llama2:persistent", session_kwargs={"strict": True})
+
+
 def test_llama2_session_options_choose_the_executor():
     """persistent = False keeps one launch per operator; fp8_cache = True makes the KV caches F143 bytes (the
     KVCache op with fp8 = true), which the persistent step does not cover: per-operator executor, tokens equal to
