@@ -98,7 +98,9 @@ def cpu_baseline(seconds_budget=20.0):
                       f"layer time scaled x{LLAMA2_7B['num_hidden_layers'] // layers}"}
 
 
-PMC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "llama2_7b_int4_b1_decode_step_pmc.txt")
+def pmc_summary_path(B):
+    """The committed hardware-counter summary of the decode-step kernel at batch B (1 and 16 are recorded)."""
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", f"llama2_7b_int4_b{B}_decode_step_pmc.txt")
 
 
 def summarize_pmc(fetch_csv, write_csv):
@@ -116,7 +118,7 @@ def summarize_pmc(fetch_csv, write_csv):
     out = {}
     for counter, path in (("FETCH_SIZE", fetch_csv), ("WRITE_SIZE", write_csv)):
         vals = per_kernel(path, counter)
-        step = [v for k, v in vals.items() if "decode_step_kernel" in k]
+        step = [v for k, v in vals.items() if "decode_step_kernel" in k or "decode_step_wide_kernel" in k]
         cal = [v for k, v in vals.items() if "neg_kernel" in k or "NegFunctor" in k or "neg" in k.lower()]
         if not step or not cal:
             raise SystemExit(f"{path}: decode-step or calibration kernel not found")
@@ -125,16 +127,16 @@ def summarize_pmc(fetch_csv, write_csv):
         factor = (1 << 20) / cal_kib                      # the calibration kernel moves 1 GiB = 2^20 KiB each way
         mean_kib = sum(step) / len(step)
         out[counter] = mean_kib * factor * 1024
-        print(f"{counter}: decode_step_kernel mean {mean_kib:.1f} KiB over {len(step)} launches "
+        print(f"{counter}: decode-step kernel mean {mean_kib:.1f} KiB over {len(step)} launches "
               f"(min {min(step):.1f}, max {max(step):.1f}); calibration kernel reads {cal_kib:.1f} KiB for 2^20 KiB "
               f"-> factor {factor:.4f} -> {out[counter]:.0f} bytes per launch")
     print(f"traffic_bytes_per_launch = {out['FETCH_SIZE'] + out['WRITE_SIZE']:.0f}")
 
 
-def recorded_traffic():
+def recorded_traffic(B):
     """HBM bytes per launch of the decode-step kernel from the committed counter summary, or None."""
     try:
-        for line in open(PMC_SUMMARY):
+        for line in open(pmc_summary_path(B)):
             if line.startswith("traffic_bytes_per_launch"):
                 return float(line.split("=")[1])
     except OSError:
@@ -471,10 +473,10 @@ def main():
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": recorded_traffic() if executor == "persistent" and B == 1 else None,
+                     "traffic": recorded_traffic(B) if executor == "persistent" else None,
                      "traffic_source": ("recorded, not measured in this run: hardware counters of an earlier profiled "
-                                        "run, profiles/" + os.path.basename(PMC_SUMMARY))
-                     if executor == "persistent" and B == 1 else None,
+                                        "run, profiles/" + os.path.basename(pmc_summary_path(B)))
+                     if executor == "persistent" and recorded_traffic(B) is not None else None,
                      "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }
     if B == 1 and not args.no_batch16 and not args.copy_calibration:

@@ -244,6 +244,14 @@ int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, const pta_hal
                              void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
                              int use_scale, pta_stream_t stream);
 
+/* pta_decode_attention_qkv whose context vector is left on an FP8 grid: out = pta_half_to_fp8_grid(context,
+ * out_fp8_scale, out_fp8_format), bit for bit - the cast with which the next FP8 Linear starts
+ * (half_to_uint8, utils/param_handler/precision_strategy.py:62-66), done where the value is produced. */
+int pta_decode_attention_qkv_grid(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                                  int v_stride, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                                  void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope,
+                                  int use_scale, const int32_t* out_fp8_scale, int out_fp8_format, pta_stream_t stream);
+
 /* The same two operators over `rows` consecutive positions of every sequence at once - the prompt.
  * The reference feeds a prompt through its loop one token per iteration (the container keeps the
  * prompt's ids, models/base_model.py:313-318); its two-stage ChatGLM graphs run the same layers with

@@ -11,6 +11,7 @@
 // fp16 rounding of the context vector.
 #include "common.h"
 #include "formats.h"
+#include "f8codec.h"
 
 // ------------------------------------------------------------------------------------------
 // q/k rotary embedding + KV ring append.
@@ -184,7 +185,15 @@ struct AttnArgs {
   f16* kring_w; f16* vring_w;
   const void* inv_freq;
   int rope;
+  // when set: the context vector is left on the FP8 grid of this device exponent (the cast of the next Linear)
+  const int32_t* out_fp8_scale;
+  int out_fp8_format;
 };
+
+// the value stored for a context element: as computed, or rounded to the FP8 grid its consumer casts to
+__device__ __forceinline__ f16 attn_result(const AttnArgs& a, f16 y) {
+  return a.out_fp8_scale ? f8_grid_value(y, a.out_fp8_scale[0], a.out_fp8_format) : y;
+}
 
 __device__ __forceinline__ int attn_chunk(int valid, int nsplit) {
   int c = (valid + nsplit - 1) / nsplit;
@@ -349,7 +358,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       A = __builtin_fmaf(sm_acc[i][d], w, A);
     }
     if (a.nsplit == 1) {                     // the only split of this (row, head): the context vector itself
-      a.out[(size_t)bh * D + d] = (f16)((KV8 ? A * kv_mul : A) / L);
+      a.out[(size_t)bh * D + d] = attn_result(a, (f16)((KV8 ? A * kv_mul : A) / L));
       continue;
     }
     out[2 + d] = KV8 ? A * kv_mul : A;
@@ -374,7 +383,7 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
     L = __builtin_fmaf(ps[1], w, L);
     A = __builtin_fmaf(ps[2 + d], w, A);
   }
-  a.out[(size_t)bh * D + d] = (f16)(A / L);
+  a.out[(size_t)bh * D + d] = attn_result(a, (f16)(A / L));
 }
 
 // splits per (sequence, head): about 1024 workgroups in all, never more than one per 64 cache rows
@@ -454,8 +463,10 @@ extern "C" int pta_prompt_attention_f8(const pta_half* q, const uint8_t* kv_ring
 static int attention_qkv(const char* name, const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
                          int v_stride, void* kv_ring, const int32_t* step, const void* inv_freq, void* workspace,
                          pta_half* out, int B, int Hq, int Hkv, int D, int max_len, int rope, int use_scale, int kv8,
-                         int kv_scale, pta_stream_t stream) {
+                         int kv_scale, pta_stream_t stream, const int32_t* out_fp8_scale = nullptr, int out_fp8_format = 0) {
   PTA_REQUIRE(q && k && v && kv_ring && step && workspace && out, "%s: null pointer", name);
+  PTA_REQUIRE(!out_fp8_scale || out_fp8_format == PTA_F143 || out_fp8_format == PTA_F152,
+              "%s: unsupported fp8 format %d, it must be F143 or F152", name, out_fp8_format);
   PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
   PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
   PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
@@ -474,6 +485,7 @@ static int attention_qkv(const char* name, const pta_half* q, const pta_half* k,
   a.step = step; a.part = (float*)workspace; a.out = (f16*)out;
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B, Hq, max_len); a.rows = 1;
   a.kv_scale = kv_scale;
+  a.out_fp8_scale = out_fp8_scale; a.out_fp8_format = out_fp8_format;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   launch_attention<true>(a, D, kv8 != 0, B * Hq, (hipStream_t)stream);
   PTA_CHECK_LAUNCH(name);
@@ -486,6 +498,16 @@ extern "C" int pta_decode_attention_qkv(const pta_half* q, const pta_half* k, co
                                         int use_scale, pta_stream_t stream) {
   return attention_qkv("pta_decode_attention_qkv", q, k, v, q_stride, k_stride, v_stride, kv_ring, step, inv_freq, workspace, out,
                        B, Hq, Hkv, D, max_len, rope, use_scale, 0, 0, stream);
+}
+
+extern "C" int pta_decode_attention_qkv_grid(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,
+                                             int v_stride, pta_half* kv_ring, const int32_t* step, const void* inv_freq,
+                                             void* workspace, pta_half* out, int B, int Hq, int Hkv, int D, int max_len,
+                                             int rope, int use_scale, const int32_t* out_fp8_scale, int out_fp8_format,
+                                             pta_stream_t stream) {
+  PTA_REQUIRE(out_fp8_scale, "pta_decode_attention_qkv_grid: null pointer");
+  return attention_qkv("pta_decode_attention_qkv_grid", q, k, v, q_stride, k_stride, v_stride, kv_ring, step, inv_freq, workspace,
+                       out, B, Hq, Hkv, D, max_len, rope, use_scale, 0, 0, stream, out_fp8_scale, out_fp8_format);
 }
 
 extern "C" int pta_decode_attention_qkv_f8(const pta_half* q, const pta_half* k, const pta_half* v, int q_stride, int k_stride,

@@ -335,9 +335,14 @@ class FusedDecoder(LayerOps):
             h, nrm = self._normed(self.x, blk.norm1, blk.qkv)
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
             qp, kp, vp, qs, ks, vs = self._qkv_views
+            # the output projection's cast of its input to FP8 is done by the attention where it stores the context
+            grid = self._common_grid([blk.out]) if self.kv_scale is None else None
+            self._on_grid.pop(self.ctx.data_ptr(), None)
             K.decode_attention_qkv(qp, kp, vp, self.rings[li], self.step, w.inv_freq, self.attn_ws, self.ctx, B,
                                    s.n_head, s.n_kv_head, s.head_dim, s.max_len, s.rope, s.scale_scores, qs, ks, vs,
-                                   kv_scale=self.kv_scale)
+                                   kv_scale=self.kv_scale, out_grid=grid)
+            if grid is not None:
+                self._on_grid[self.ctx.data_ptr()] = self._grid_id(blk.out)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:

@@ -451,13 +451,23 @@ def _kv_ring_dtype(kv_ring, kv_scale):
 
 
 def decode_attention_qkv(q, k, v, kv_ring, step, inv_freq, workspace, out, B, Hq, Hkv, D, max_len, rope, use_scale,
-                         q_stride=None, k_stride=None, v_stride=None, kv_scale=None):
+                         q_stride=None, k_stride=None, v_stride=None, kv_scale=None, out_grid=None):
     """qkv_rope_append + decode_attention in one pass (bit-identical to the two calls).  kv_scale (an int):
-    kv_ring is a uint8 FP8 cache holding F143 bytes of value * 2^-kv_scale."""
+    kv_ring is a uint8 FP8 cache holding F143 bytes of value * 2^-kv_scale.  out_grid: (device int32 exponent,
+    'F143' | 'F152') - the context vector is left on that FP8 grid (half_to_fp8_grid); fp16 caches only."""
     q_stride = Hq * D if q_stride is None else q_stride
     k_stride = Hkv * D if k_stride is None else k_stride
     v_stride = Hkv * D if v_stride is None else v_stride
     _kv_ring_dtype(kv_ring, kv_scale)
+    if out_grid is not None:
+        if kv_scale is not None:
+            raise NotImplementedError("decode_attention_qkv: out_grid with an FP8 cache")
+        _need(out_grid[0], _i32, "fp8_scale")
+        check(_lib.load().pta_decode_attention_qkv_grid(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(kv_ring),
+                                                        _p(step), _p(inv_freq), _p(workspace), _p(out), B, Hq, Hkv, D,
+                                                        max_len, rope, 1 if use_scale else 0, _p(out_grid[0]),
+                                                        _fmt(out_grid[1]), _stream()))
+        return out
     if kv_scale is not None:
         check(_lib.load().pta_decode_attention_qkv_f8(_p(q), _p(k), _p(v), q_stride, k_stride, v_stride, _p(kv_ring),
                                                       _p(step), _p(inv_freq), _p(workspace), _p(out), B, Hq, Hkv, D,

@@ -612,6 +612,15 @@ def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, H
                                family != "gpt2", row, row, row)
         assert torch.equal(outs[0], outs[1]), f"context differs at step {it}"
     assert torch.equal(rings[0], rings[1])
+    # the same pass leaving its context vectors on an FP8 grid: the bits of the separate cast (the ring already holds
+    # this step's row: the append writes the same values again)
+    for fmt, scale in (("F143", -1), ("F152", 2)):
+        sd = dev(np.array([scale], np.int32))
+        on_grid = torch.empty_like(outs[1])
+        K.decode_attention_qkv(q, k, v, rings[1], step, inv, wss[1], on_grid, B, Hq, Hkv, D, max_len, rope,
+                               family != "gpt2", row, row, row, out_grid=(sd, fmt))
+        assert torch.equal(on_grid, K.half_to_fp8_grid(outs[1], sd, fmt))
+    assert torch.equal(rings[0], rings[1])
 
 
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,first,rows", [("llama", 2, 4, 4, 128, 160, 0, 32), ("llama", 1, 4, 4, 128, 160, 70, 64),
