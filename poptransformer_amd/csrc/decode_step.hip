@@ -1958,8 +1958,9 @@ Layout layout_for(const pta_decode_model* m, int cus) {
   l.act = l.ctx + align256(L * R * d * 2);
   l.part = l.act + align256(L * R * f * 2);
   l.flags = l.part + align256(L * B * H * splits_for(cus, (int)B, (int)H) * DS_PART * 4);
-  l.best = l.flags + align256((4 * L + 1) * DS_REPLICAS * flag_words_for(cus) * 4);
-  l.trace = l.best + align256((size_t)cus * 16 * 2 * 4);
+  // arrival words and per-workgroup best logits: decode_step_wide_kernel only
+  l.best = l.flags + (B > DS_MAXB ? align256((4 * L + 1) * DS_REPLICAS * flag_words_for(cus) * 4) : 0);
+  l.trace = l.best + (B > DS_MAXB ? align256((size_t)cus * 16 * 2 * 4) : 0);
   l.total = l.trace + (size_t)cus * 256;
   return l;
 }
