@@ -272,8 +272,8 @@ def prompt_workload(args):
     from poptransformer_amd.engine import fused, loader, synthetic
     B, cfg = args.batch, LLAMA2_7B
     rows = args.rows_per_pass
-    if B > rows or rows > 256:
-        print("the prompt passes take at most 256 rows: batch <= --rows-per-pass <= 256", file=sys.stderr)
+    if B > rows or rows > 2048:
+        print("the prompt passes take at most 2048 rows: batch <= --rows-per-pass <= 2048", file=sys.stderr)
         sys.exit(2)
     R = rows // B
     passes = max(1, min(args.steps, (MAX_LEN - 2) // R))
@@ -328,7 +328,7 @@ def main():
                          "rwkv: RWKV-4-7B-shape INT4 recurrent decode; prompt: the headline model's prompt in passes "
                          "of up to 64 rows (--steps passes)")
     ap.add_argument("--rows-per-pass", type=int, default=64,
-                    help="prompt workload: rows (batch x positions) per pass, up to 256")
+                    help="prompt workload: rows (batch x positions) per pass, up to 2048")
     ap.add_argument("--fp8-cache", action="store_true",
                     help="decode workload, operators executor: keep the KV cache as F143 bytes (KVCacheOp with fp8 = true)")
     ap.add_argument("--fuse-norm", choices=["on", "off"], default=None,

@@ -109,7 +109,7 @@ enum { PTA_ACT_NONE = 0, PTA_ACT_GELU_TANH = 1, PTA_ACT_RELU_SQUARE = 2, PTA_ACT
 /* Fused Int4ToHalf(axis=1) + MatMul (utils/param_handler/precision_strategy.py:56-60,74-75):
  * Y[M,N] = fp16( X[M,K] @ W ), W[k,n] = fp16(nibble(k,n) * scale[n]) exactly as
  * pta_int4_to_half(axis=1) would produce, fp32 accumulation, never materialised.
- * `tiled` comes from pta_w4_tile.  1 <= M <= 256.  `fuse` may be NULL. */
+ * `tiled` comes from pta_w4_tile.  1 <= M <= 4096.  `fuse` may be NULL. */
 int pta_w4a16_gemm(const pta_half* X, const void* tiled, const pta_half* scale, pta_half* Y,
                    int M, int K, int N, const pta_fusion* fuse, pta_stream_t stream);
 
@@ -135,7 +135,7 @@ int pta_w4a16_gemm_swiglu(const pta_half* X, const void* tiled_gate, const pta_h
 /* `w` is fp16 [N, K] (the [out, in] orientation of the state dict, layers/linear.py:30-33). */
 size_t pta_f16_tiled_bytes(int N, int K);
 int pta_f16_tile(const pta_half* w, void* tiled, int N, int K, pta_stream_t stream);
-/* Y[M,N] = fp16(X[M,K] @ w^T), fp32 accumulation. 1 <= M <= 256. */
+/* Y[M,N] = fp16(X[M,K] @ w^T), fp32 accumulation. 1 <= M <= 4096. */
 int pta_f16_gemm(const pta_half* X, const void* tiled, pta_half* Y, int M, int K, int N,
                  const pta_fusion* fuse, pta_stream_t stream);
 
@@ -357,7 +357,7 @@ int pta_fp8_tile(const uint8_t* w, void* tiled, int N, int K, int w_is_kn, pta_s
 
 /* FP8MatMul (ops/customized.py:137-148; custom_ops/matmul_fp8.cpp:177-250, 885-1003).
  * lhs is fp16 [M, K] (lhs_is_fp8 == 0: the weight is cast to fp16, then an fp16 MatMul) or uint8
- * [M, K] (both operands FP8).  Y fp16 [M, N], fp32 accumulation.  1 <= M <= 256.
+ * [M, K] (both operands FP8).  Y fp16 [M, N], fp32 accumulation.  1 <= M <= 4096.
  * workspace: pta_fp8_gemm_workspace_bytes(M, K) bytes, 16-byte aligned.  `fuse` may be NULL. */
 size_t pta_fp8_gemm_workspace_bytes(int M, int K);
 int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_rhs, pta_half* Y, int M, int K, int N,

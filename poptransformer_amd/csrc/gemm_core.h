@@ -119,7 +119,7 @@ struct GemmArgs {
   int ksplit;          // 0 or 1: no split
 };
 constexpr int GEMM_MAX_KSPLIT = 4;
-constexpr int GEMM_MAX_ROWS = 256;
+constexpr int GEMM_MAX_ROWS = 4096;
 
 template <class Fmt, int MT, int NW, bool PAIR>
 __global__ __launch_bounds__(NW * 64) void gemv_mfma_kernel(GemmArgs a) {
@@ -933,6 +933,196 @@ static int launch_gemm_tile(const GemmArgs& a, int total_nb, hipStream_t s, cons
   return PTA_OK;
 }
 
+// ------------------------------------------------------------------------------------------
+// Variant for many rows (prompt passes): the activation fragments live in registers, the weights go through
+// LDS decoded.  A workgroup of 8 waves owns 8 weight streams of 16 channels (8 channel blocks of one matrix,
+// or the gate and up weights of 4 blocks) and 8 * RG * 16 rows.  Per 128-feature tile, wave w
+//   - fetches the tile of stream w, decodes it ONCE into the four fp16 A operands of its MFMA steps and puts
+//     them into LDS (double-buffered, one barrier per tile) - every weight is decoded once per workgroup, not
+//     once per wave and row group: with the decode in the product loop a wave spends 13 VALU instructions per
+//     step for RG MFMAs and the kernel is bound by those (measured: 262 TFLOP/s at 256 rows);
+//   - holds the B operands of ITS RG row groups in registers (fetched with whole-row loads, turned into
+//     fragment order through a strip of LDS of its own) and multiplies them with every stream's operands.
+// ------------------------------------------------------------------------------------------
+constexpr int ROWS_WAVES = 8;
+constexpr int ROWS_CB = 8;                  // streams per workgroup: one per wave
+constexpr int ROWS_XSTRIDE = 128 + 8;
+constexpr int ROWS_AVEC = ROWS_CB * 4 * 64; // A operands (16 bytes each) of one feature tile: [stream][step][lane]
+
+// (two waves per SIMD: the whole register file of 256 per lane is this kernel's to use)
+template <class Fmt, int RG, bool PAIR>
+__global__ __launch_bounds__(ROWS_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_rows_kernel(GemmArgs a, int groups, int row_blocks) {
+  constexpr int KV = Fmt::kVec;
+  constexpr int XROWS = RG * 16;
+  static_assert(ROWS_CB == ROWS_WAVES, "wave w decodes stream w");
+  extern __shared__ __align__(16) unsigned char smem[];
+  f16x8* abuf = reinterpret_cast<f16x8*>(smem);                                          // [2][ROWS_AVEC]
+  f16* xbuf = reinterpret_cast<f16*>(smem + (size_t)2 * ROWS_AVEC * 16);                 // [waves][XROWS][ROWS_XSTRIDE]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int K = a.K, M = a.M;
+  // Workgroups are dealt to the eight XCDs (each with an L2 of its own) in turn: workgroup id of the launch takes
+  // tile (id % 8) * per + id / 8 of the list (row block, channel group), row block slowest - so an XCD works through
+  // a contiguous stretch of the list, i.e. on one row block at a time, whose activations stay in its L2.
+  const int per = (int)gridDim.x / 8;
+  const int tile = ((int)blockIdx.x % 8) * per + (int)blockIdx.x / 8;
+  if (tile >= groups * row_blocks) return;
+  const int group = tile % groups, row_block = tile / groups;
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  const int per_slice = (a.KT + nsl - 1) / nsl;
+  const int kt_first = (int)blockIdx.y * per_slice;
+  const int kt_end = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;
+  const int steps = kt_end - kt_first;
+
+  int mi = 0;
+  const int first_blk = group * (PAIR ? ROWS_CB / 2 : ROWS_CB);
+  if (!PAIR) {
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (i < a.count && first_blk >= a.mat[i].nb_begin) mi = i;
+  }
+  // stream st: its matrix and channel block
+  auto stream_mat = [&](int st) -> const GemmMat& { return a.mat[PAIR ? (st < ROWS_CB / 2 ? 0 : 1) : mi]; };
+  auto stream_blk = [&](int st) { return PAIR ? first_blk + st % (ROWS_CB / 2) : first_blk - a.mat[mi].nb_begin + st; };
+  const GemmMat& own = stream_mat(wave);
+  const typename Fmt::Scale own_sc = Fmt::load_scale(own.scale, a.x_scale, stream_blk(wave) * 16 + (lane & 15), own.N);
+  const u32x4* own_w = reinterpret_cast<const u32x4*>(own.tiled) + (size_t)stream_blk(wave) * a.KT * (KV * 64) + lane;
+  const f16* X = a.mat[mi].X ? a.mat[mi].X : a.X;
+  const int row0 = (row_block * ROWS_WAVES + wave) * XROWS;      // first row of this wave
+  f16* xw = xbuf + (size_t)wave * XROWS * ROWS_XSTRIDE;
+
+  auto fetch_w = [&](int kt, u32x4 (&wv)[KV]) {
+#pragma unroll
+    for (int v = 0; v < KV; ++v) wv[v] = __builtin_nontemporal_load(own_w + ((size_t)kt * KV + v) * 64);
+  };
+  auto decode_w = [&](f16x8* buf, const u32x4 (&wv)[KV]) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m) buf[(wave * 4 + m) * 64 + lane] = Fmt::a_operand(wv, m, own_sc);
+  };
+  // whole-row loads: instruction j covers rows 4 j .. 4 j + 3 of the wave, 256 bytes each
+  auto fetch_x = [&](int kt, u32x4 (&xr)[RG * 4]) {
+#pragma unroll
+    for (int j = 0; j < RG * 4; ++j) {
+      const int row = row0 + j * 4 + (lane >> 4), k = kt * 128 + (lane & 15) * 8;
+      xr[j] = (row < M && k < K) ? *reinterpret_cast<const u32x4*>(X + (size_t)row * K + k) : u32x4{0, 0, 0, 0};
+    }
+  };
+  // through the wave's own strip of LDS into fragment order (a wave's LDS accesses complete in order)
+  auto to_fragments = [&](const u32x4 (&xr)[RG * 4], f16x8 (&xf)[RG][4]) {
+#pragma unroll
+    for (int j = 0; j < RG * 4; ++j)
+      *reinterpret_cast<u32x4*>(xw + (j * 4 + (lane >> 4)) * ROWS_XSTRIDE + (lane & 15) * 8) = xr[j];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        xf[rg][m] = *reinterpret_cast<const f16x8*>(xw + (rg * 16 + (lane & 15)) * ROWS_XSTRIDE + m * 32 + (lane >> 4) * 8);
+  };
+
+  f32x4 acc[RG][ROWS_CB];
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+    for (int st = 0; st < ROWS_CB; ++st) acc[rg][st] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 wv[KV], xr[RG * 4];
+  f16x8 xf[RG][4];
+  if (steps > 0) {
+    fetch_w(kt_first, wv);
+    fetch_x(kt_first, xr);
+    decode_w(abuf, wv);
+    to_fragments(xr, xf);
+  }
+  __syncthreads();
+  for (int i = 0; i < steps; ++i) {
+    const bool more = i + 1 < steps;
+    if (more) { fetch_w(kt_first + i + 1, wv); fetch_x(kt_first + i + 1, xr); }
+    const f16x8* cur = abuf + (size_t)(i & 1) * ROWS_AVEC;
+#pragma unroll
+    for (int st = 0; st < ROWS_CB; ++st) {
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const f16x8 av = cur[(st * 4 + m) * 64 + lane];
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) acc[rg][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xf[rg][m], acc[rg][st], 0, 0, 0);
+      }
+    }
+    if (more) {
+      decode_w(abuf + (size_t)((i + 1) & 1) * ROWS_AVEC, wv);
+      to_fragments(xr, xf);
+    }
+    __syncthreads();
+  }
+
+  // Lane l holds channels (l / 16) * 4 + r, r = 0..3, of row l % 16 of each row group, for every stream.  The sums
+  // go to the wave's strip of LDS first (the operand buffers are free after the last barrier) and one copy of the
+  // epilogue walks over them: unrolled RG * 8 * 4 times the epilogue is too large to unroll, and an accumulator
+  // array that is indexed by a loop counter lives in scratch memory - for the whole kernel.
+  f32x4* sums = reinterpret_cast<f32x4*>(smem) + (size_t)wave * (RG * ROWS_CB * 64);
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+    for (int st = 0; st < ROWS_CB; ++st) sums[(rg * ROWS_CB + st) * 64 + lane] = acc[rg][st];
+  if constexpr (PAIR) {
+    const GemmMat& mat = a.mat[0];
+    const typename Fmt::Scale sg = Fmt::load_scale(a.mat[0].scale, a.x_scale, 0, 1), su = Fmt::load_scale(a.mat[1].scale, a.x_scale, 0, 1);
+#pragma unroll 1
+    for (int i = 0; i < RG * ROWS_CB / 2; ++i) {
+      const int rg = i / (ROWS_CB / 2), st = i % (ROWS_CB / 2);
+      const int m = row0 + rg * 16 + (lane & 15);
+      const f32x4 g4 = sums[(rg * ROWS_CB + st) * 64 + lane], u4 = sums[(rg * ROWS_CB + st + ROWS_CB / 2) * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = (first_blk + st) * 16 + (lane >> 4) * 4 + r;
+        if (m >= M || n >= mat.N) continue;
+        mat.Y[(size_t)m * mat.N + n] = swiglu_out(a.epi, (f16)Fmt::finish(g4[r], sg), (f16)Fmt::finish(u4[r], su));
+      }
+    }
+  } else {
+    const GemmMat& mat = a.mat[mi];
+    const int N = mat.N;
+    const typename Fmt::Scale s1 = Fmt::load_scale(mat.scale, a.x_scale, 0, 1);      // no format's finish uses the per-channel part
+#pragma unroll 1
+    for (int i = 0; i < RG * ROWS_CB; ++i) {
+      const int rg = i / ROWS_CB, st = i % ROWS_CB;
+      const int m = row0 + rg * 16 + (lane & 15);
+      const f32x4 v4 = sums[i * 64 + lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = stream_blk(st) * 16 + (lane >> 4) * 4 + r;
+        if (m >= M || n >= N) continue;
+        if (nsl > 1) { a.part[((size_t)blockIdx.y * M + m) * N + n] = v4[r]; continue; }
+        f16 y0 = (f16)Fmt::finish(v4[r], s1);
+        if (mat.bias) y0 = y0 + mat.bias[n];
+        y0 = apply_act(mat.act, y0);
+        mat.Y[(size_t)m * N + n] = apply_epilogue(a.epi, y0, m, n, N);
+      }
+    }
+  }
+}
+
+template <class Fmt, int RG, bool PAIR>
+static int launch_gemm_rows(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  static bool ready = false;
+  const size_t smem = (size_t)2 * ROWS_AVEC * 16 + (size_t)ROWS_WAVES * RG * 16 * ROWS_XSTRIDE * 2;
+  static_assert((size_t)2 * ROWS_AVEC * 16 + (size_t)ROWS_WAVES * RG * 16 * ROWS_XSTRIDE * 2 <= 160 * 1024, "LDS");
+  if (!ready) {
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_rows_kernel<Fmt, RG, PAIR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem) == hipSuccess,
+                "%s: cannot reserve %zu bytes of LDS", name, smem);
+    ready = true;
+  }
+  const int groups = total_nb / (PAIR ? ROWS_CB / 2 : ROWS_CB);
+  const int row_blocks = (a.M + ROWS_WAVES * RG * 16 - 1) / (ROWS_WAVES * RG * 16);
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  const int per = (groups * row_blocks + 7) / 8;
+  hipLaunchKernelGGL((gemm_rows_kernel<Fmt, RG, PAIR>), dim3(per * 8, nsl), dim3(ROWS_WAVES * 64), smem, s, a, groups, row_blocks);
+  if (nsl > 1) {
+    const size_t total = (size_t)a.M * a.mat[0].N;
+    hipLaunchKernelGGL((splitk_finish_kernel<Fmt>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+  }
+  return PTA_OK;
+}
+
 // whether the launch fits gemm_tile_kernel with `per_wg` channel blocks per workgroup: every matrix
 // a whole number of workgroups, enough feature tiles for the K groups
 static inline bool tile_fits(const GemmArgs& a, int per_wg, int kq, bool pair) {
@@ -992,6 +1182,22 @@ static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, co
   const int cus = device_compute_units();
   const int per_wg = PAIR ? 4 : 8;
   const bool tiles = a.epi.norm == PTA_NORM_NONE && tile_fits(a, per_wg, 2, PAIR);
+  if (tiles) {
+    // fragments in registers, weights through LDS: 256 rows per workgroup where that still fills the machine,
+    // else 128; few workgroups and one matrix: K in slices as well
+    const int groups = total_nb / per_wg;
+    const bool two = a.M > 128 && (long)groups * ((a.M + 255) / 256) * 2 >= (long)cus;
+    const int wgs = groups * (two ? (a.M + 255) / 256 : (a.M + 127) / 128);
+    GemmArgs b = a;
+    int nsl = wgs > 0 ? cus / wgs : 1;
+    nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
+    while (nsl > 1 && a.KT < nsl * 8) --nsl;
+    if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
+    const int rc = two ? launch_gemm_rows<Fmt, 2, PAIR>(b, total_nb, s, name) : launch_gemm_rows<Fmt, 1, PAIR>(b, total_nb, s, name);
+    if (rc) return rc;
+    PTA_CHECK_LAUNCH(name);
+    return PTA_OK;
+  }
   if (tiles && a.M <= 128) {
     GemmArgs b = a;
     const int wgs = total_nb / per_wg;

@@ -401,8 +401,8 @@ class FusedDecoder(LayerOps):
         if n == 0:
             return 0
         R = max(1, 64 // s.batch) if rows_per_pass is None else int(rows_per_pass)
-        if R < 1 or R * s.batch > 256:
-            raise ValueError(f"consume_prompt: rows_per_pass * batch must lie in [1, 256], got {R} * {s.batch}")
+        if R < 1 or R * s.batch > 2048:
+            raise ValueError(f"consume_prompt: rows_per_pass * batch must lie in [1, 2048], got {R} * {s.batch}")
         if not hasattr(self, "_prompt_passes"):
             self._prompt_passes = {}
         with torch.cuda.stream(self._stream):

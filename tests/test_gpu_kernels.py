@@ -263,7 +263,7 @@ def test_w4a16_guards(K):
     with pytest.raises(ValueError):
         K.w4a16_gemm(dev(np.zeros((1, 64), np.float16)), w)
     with pytest.raises(ValueError):
-        K.w4a16_gemm(dev(np.zeros((257, 128), np.float16)), w)
+        K.w4a16_gemm(dev(np.zeros((4097, 128), np.float16)), w)
 
 
 # ---------------------------------------------------------------- FP16 GEMM
@@ -1010,13 +1010,14 @@ def test_fp8_products_pair_multi_and_nan(K):
     assert np.abs(got[ok].astype(np.float64) - ref[ok].astype(np.float64)).max() <= 2.0 ** -10 * np.abs(ref[ok].astype(np.float64)).max()
 
 
-# ---------------------------------------------------------------- 65..256 rows
-@pytest.mark.parametrize("M", [65, 128, 200, 256])
+# ---------------------------------------------------------------- more than 64 rows
+@pytest.mark.parametrize("M", [65, 128, 200, 256, 600, 1024])
 @pytest.mark.parametrize("Kdim,N", [(4096, 4096), (1160, 8192), (11008, 4096), (512, 100)])
 def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
-    """More than 64 rows: the staged kernel with 8 or 16 row groups (with and without the K split that a workspace
-    allows; 1160 features = a ragged last tile), and for channel counts that do not divide into its workgroup tiles
-    (100) the 64-row paths over the rows in turn.  Bias, and a residual that aliases the output."""
+    """More than 64 rows: the kernel that keeps the activation fragments in registers (128 or 256 rows per workgroup,
+    with and without the K split that a workspace allows; 1160 features = a ragged last tile; 200 and 600 rows = a
+    ragged last row block), and for channel counts that do not divide into its workgroup tiles (100) the 64-row
+    paths over the rows in turn.  Bias, and a residual that aliases the output."""
     x, packed, scale = _w4_case(M + Kdim + N, M, Kdim, N)
     rng = np.random.default_rng(M * N)
     bias = rng.standard_normal(N).astype(np.float16)
@@ -1033,7 +1034,7 @@ def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
 
 def test_gemm_up_to_256_rows_exact_integers_pair_and_other_formats(K):
     rng = np.random.default_rng(61)
-    for M in (96, 256):
+    for M in (96, 256, 520):
         Kdim, N = 1024, 8192
         x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
         q = rng.integers(-8, 8, size=(N, Kdim))
@@ -1056,4 +1057,4 @@ def test_gemm_up_to_256_rows_exact_integers_pair_and_other_formats(K):
         fw = K.F8Weight(dev(w8), dev(np.array([-1], np.int32)), "F143", kn=True)
         assert rel_err(host(K.fp8_gemm(dev(xr), fw, K.fp8_gemm_workspace(M, Kdim, "cuda"))), O.fp8_matmul(xr, w8, [-1], [-1])) <= 1e-2
     with pytest.raises(ValueError):
-        K.w4a16_gemm(dev(rng.standard_normal((257, 1024)).astype(np.float16)), w)
+        K.w4a16_gemm(dev(rng.standard_normal((4097, 1024)).astype(np.float16)), w)

@@ -259,7 +259,7 @@ def test_prompt_passes_stop_before_an_end_token_and_check_their_arguments():
     with pytest.raises(ValueError):
         dec.consume_prompt(9)
     with pytest.raises(ValueError):
-        dec.consume_prompt(4, rows_per_pass=130)      # 260 rows
+        dec.consume_prompt(4, rows_per_pass=1030)     # 2060 rows
     assert dec.consume_prompt(8) == 8
     with pytest.raises(RuntimeError):
         dec.consume_prompt(1)                         # only directly after reset
