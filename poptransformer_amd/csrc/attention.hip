@@ -397,6 +397,136 @@ static int attn_splits(int B, int Hq, int max_len) {
   return n > cap ? cap : n;
 }
 
+// ------------------------------------------------------------------------------------------
+// Attention of many rows at once (the prompt passes) on the matrix unit, head size 128, fp16 cache.
+// One workgroup of four waves per (sequence, query head, 64 rows of the pass); wave w owns 16 of the rows.
+// The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes
+//   S^T = K Q^T     (two 16 x 16 tiles, 4 MFMAs each: lane l then holds the scores of query row l % 16 for
+//                    cache rows (l / 16) * 4 + 0..3 of each tile - which IS the layout of an A operand whose
+//                    k index runs over those eight cache rows),
+//   the roundings of the reference on the scores (fp16 MatMul output, fp16 multiply by 1/sqrt(D)), the online
+//   softmax in fp32 per query row (partners: lanes l ^ 16, l ^ 32), probabilities rounded to fp16 (the
+//   reference's softmax output is fp16),
+//   O += P V        (eight 16 x 16 tiles over the head size, B operands from the transposed V rows).
+// Row r of the pass sits at position step + r and attends to cache rows [0, min(step + r + 1, max_len)), as in
+// attn_partial_kernel.  Outputs differ from that kernel in the last bits (another summation order, fp16
+// probabilities); both are held to 1e-2 against the oracle.
+// ------------------------------------------------------------------------------------------
+constexpr int PA_THREADS = 256;
+constexpr int PA_KSTRIDE = 128 + 8;      // halves per staged K row
+constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
+
+__global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnArgs a) {
+  constexpr int D = 128;
+  __shared__ __align__(16) f16 ks[32 * PA_KSTRIDE];
+  __shared__ __align__(16) f16 vt[D * PA_VSTRIDE];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int kvh = h / (a.Hq / a.Hkv);
+  const int step0 = *a.step;
+  const int r0 = (int)blockIdx.x * 64 + wave * 16;          // first row of this wave within the pass
+  const int qrow = r0 + (lane & 15);
+  f16x8 qf[4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    qf[m] = f16x8{};
+    if (qrow < a.rows) qf[m] = *reinterpret_cast<const f16x8*>(a.q + (((size_t)b * a.rows + qrow) * a.Hq + h) * D + m * 32 + (lane >> 4) * 8);
+  }
+  auto valid_of = [&](int row) { const int v = step0 + row + 1; return row < a.rows ? (v < a.max_len ? v : a.max_len) : 0; };
+  const int my_valid = valid_of(qrow);
+  const int last_of_wave = r0 + 15 < a.rows ? r0 + 15 : a.rows - 1;
+  const int wave_valid = r0 < a.rows ? valid_of(last_of_wave) : 0;
+  const int last_of_wg = (int)blockIdx.x * 64 + 63 < a.rows ? (int)blockIdx.x * 64 + 63 : a.rows - 1;
+  const int wg_valid = valid_of(last_of_wg);
+  const f16* kbase = a.kring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
+  const f16* vbase = a.vring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
+
+  float run_m = -INFINITY, run_l = 0.f;
+  f32x4 o[8];
+#pragma unroll
+  for (int jd = 0; jd < 8; ++jd) o[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int p0 = 0; p0 < wg_valid; p0 += 32) {
+    __syncthreads();
+    // stage cache rows p0 .. p0 + 31: 512 vectors of 16 bytes each of K and V, two per thread
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = (int)threadIdx.x + i * PA_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
+      f16x8 kv = f16x8{}, vv = f16x8{};
+      if (p0 + row < wg_valid) {
+        kv = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p0 + row) * D + col);
+        vv = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p0 + row) * D + col);
+      }
+      *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(col + e) * PA_VSTRIDE + row] = vv[e];
+    }
+    __syncthreads();
+    if (p0 >= wave_valid) continue;
+    float x[8];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const f16x8 kf = *reinterpret_cast<const f16x8*>(ks + (hh * 16 + (lane & 15)) * PA_KSTRIDE + m * 32 + (lane >> 4) * 8);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], sc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        f16 s16 = (f16)sc[r];                       // fp16 output of the q.K^T MatMul
+        if (a.use_scale) s16 = s16 * a.scale;       // fp16 multiply by fp16(1/sqrt(D))
+        const int pos = p0 + hh * 16 + (lane >> 4) * 4 + r;
+        x[hh * 4 + r] = pos < my_valid ? (float)s16 : -INFINITY;
+      }
+    }
+    float mx = x[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float new_m = fmaxf(run_m, mx);
+    const float corr = run_m == -INFINITY ? 0.f : __expf(run_m - new_m);
+    float psum = 0.f;
+    f16x8 pa;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = x[e] == -INFINITY ? 0.f : __expf(x[e] - new_m);
+      psum += pe;
+      pa[e] = (f16)pe;
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    run_l = run_l * corr + psum;
+    run_m = new_m;
+    // the accumulators' rows are query rows (lane / 16) * 4 + r: their correction factors sit in lanes of that index
+    float cr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, (lane >> 4) * 4 + r, 64);
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) {
+      const f16* vrow = vt + (jd * 16 + (lane & 15)) * PA_VSTRIDE + (lane >> 4) * 4;
+      const f16x4 v0 = *reinterpret_cast<const f16x4*>(vrow), v1 = *reinterpret_cast<const f16x4*>(vrow + 16);
+      const f16x8 vb = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[jd][r] *= cr[r];
+      o[jd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[jd], 0, 0, 0);
+    }
+  }
+  float lr[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) lr[r] = __shfl(run_l, (lane >> 4) * 4 + r, 64);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = r0 + (lane >> 4) * 4 + r;
+    if (row >= a.rows) continue;
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd)
+      a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] = attn_result(a, (f16)(o[jd][r] / lr[r]));
+  }
+}
+
 extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int max_len) {
   if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
   const int chunk = 64;
@@ -425,7 +555,8 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   PTA_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0, "%s: bad head counts %d/%d", name, Hq, Hkv);
   PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
   PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
-  PTA_REQUIRE(rows > 0 && rows <= max_len && (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
+  PTA_REQUIRE(rows > 0 && rows <= max_len, "%s: rows = %d must lie in [1, max_len = %d]", name, rows, max_len);
+  PTA_REQUIRE((rows >= 16 && D == 128 && !kv8) || (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
   PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "%s: q and kv_ring must be 16-byte aligned", name);
   PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
   const size_t ring_elems = (size_t)B * Hkv * max_len * D;
@@ -436,6 +567,11 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B * rows, Hq, max_len); a.rows = rows;
   a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
+  if (rows >= 16 && D == 128 && !kv8) {        // many rows: on the matrix unit, no splits, no workspace
+    hipLaunchKernelGGL(prompt_attention_mfma_kernel, dim3((rows + 63) / 64, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    PTA_CHECK_LAUNCH(name);
+    return PTA_OK;
+  }
   launch_attention<false>(a, D, kv8 != 0, B * rows * Hq, (hipStream_t)stream);
   PTA_CHECK_LAUNCH(name);
   return PTA_OK;

@@ -1037,14 +1037,25 @@ __global__ __launch_bounds__(ROWS_WAVES * 64) __attribute__((amdgpu_waves_per_eu
     const bool more = i + 1 < steps;
     if (more) { fetch_w(kt_first + i + 1, wv); fetch_x(kt_first + i + 1, xr); }
     const f16x8* cur = abuf + (size_t)(i & 1) * ROWS_AVEC;
+    // the operands of stream st + 1 are read while stream st is multiplied (left to itself the compiler reads two
+    // operands, waits, multiplies, and the LDS latency shows after every fourth MFMA)
+    f16x8 av[4], avn[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) av[m] = cur[m * 64 + lane];
 #pragma unroll
     for (int st = 0; st < ROWS_CB; ++st) {
+      if (st + 1 < ROWS_CB) {
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const f16x8 av = cur[(st * 4 + m) * 64 + lane];
-#pragma unroll
-        for (int rg = 0; rg < RG; ++rg) acc[rg][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xf[rg][m], acc[rg][st], 0, 0, 0);
+        for (int m = 0; m < 4; ++m) avn[m] = cur[((st + 1) * 4 + m) * 64 + lane];
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) acc[rg][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[m], xf[rg][m], acc[rg][st], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) av[m] = avn[m];
     }
     if (more) {
       decode_w(abuf + (size_t)((i + 1) & 1) * ROWS_AVEC, wv);

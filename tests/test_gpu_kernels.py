@@ -624,7 +624,9 @@ def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, H
 
 
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,first,rows", [("llama", 2, 4, 4, 128, 160, 0, 32), ("llama", 1, 4, 4, 128, 160, 70, 64),
-                                                                  ("gpt2", 3, 4, 4, 64, 64, 5, 21), ("glm2", 2, 8, 2, 128, 200, 64, 17)])
+                                                                  ("gpt2", 3, 4, 4, 64, 64, 5, 21), ("glm2", 2, 8, 2, 128, 200, 64, 17),
+                                                                  ("llama", 1, 4, 4, 128, 300, 3, 200), ("glm2", 2, 8, 2, 128, 256, 30, 130),
+                                                                  ("llama", 2, 2, 2, 128, 64, 0, 15), ("llama", 1, 2, 2, 128, 64, 0, 16)])
 def test_prompt_rows_equal_the_loop(K, family, B, Hq, Hkv, D, max_len, first, rows):
     """pta_prompt_rope_append + pta_prompt_attention over `rows` positions at once against the oracle's
     position-by-position attention (1e-2) and against the per-position calls: the ring is bit-identical, the
