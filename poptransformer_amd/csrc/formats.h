@@ -48,7 +48,8 @@ struct FmtW4 {
   static constexpr int kVec = 1;
   typedef f16x2 Scale;
   static __device__ __forceinline__ Scale load_scale(const void* scale, const int32_t*, int row, int N) {
-    const f16 s = row < N ? reinterpret_cast<const f16*>(scale)[row] : (f16)0.0f;
+    const f16 v = reinterpret_cast<const f16*>(scale)[row < N ? row : N - 1];      // (a load without a branch round it)
+    const f16 s = row < N ? v : (f16)0.0f;
     return f16x2{s, s};
   }
   static __device__ __forceinline__ f16x8 a_operand(const u32x4 (&raw)[1], int j, Scale s) {

@@ -1134,6 +1134,311 @@ static int launch_gemm_rows(const GemmArgs& a, int total_nb, hipStream_t s, cons
   return PTA_OK;
 }
 
+// ------------------------------------------------------------------------------------------
+// Variant for hundreds of rows: the roles turned round.  The tiled weight format IS the A operand order, so a
+// wave fetches the tiles of its own NST channel blocks straight into registers (1 KiB per instruction, no LDS)
+// and decodes them there; the 128 activation rows of the workgroup go through LDS once per 128-feature tile
+// (whole-row loads, double-buffered, one barrier per tile) and every wave reads all of them as B operands.
+// A wave's tile is 128 rows x NST * 16 channels: one B operand read from LDS feeds NST MFMAs and one decoded
+// A operand feeds 8, which is what keeps both LDS (128 bytes per clock and compute unit) and the vector ALU
+// behind the matrix unit.  (With the weights through LDS and the rows in registers - gemm_rows_kernel - every
+// wave reads every decoded weight: 1 KiB of LDS per 2 MFMAs, more than the LDS delivers.)
+// PAIR: a wave owns NST / 2 gate blocks and the same blocks of the up weight.
+// ------------------------------------------------------------------------------------------
+constexpr int PANEL_WAVES = 8;
+constexpr int PANEL_RG = 8;                       // row groups of 16: every wave multiplies all of them
+constexpr int PANEL_ROWS = PANEL_RG * 16;
+constexpr int PANEL_XBUF = PANEL_ROWS * 128;        // halves of one buffer of staged rows
+static_assert(PANEL_RG == 8, "the epilogue's switch names the row groups");
+
+template <class Fmt, int NST, bool PAIR>
+__global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_panel_kernel(GemmArgs a, int groups, int row_blocks, int units) {
+  constexpr int KV = Fmt::kVec;
+  constexpr int SW = NST * 16 + 4;                // floats per row of a wave's epilogue strip
+  static_assert(!PAIR || NST % 2 == 0, "gate and up blocks in equal numbers");
+  static_assert(PANEL_WAVES * 16 * SW * 4 <= 2 * PANEL_XBUF * 2, "the epilogue strips reuse the row buffers");
+  extern __shared__ __align__(16) unsigned char smem[];
+  f16* xbuf = reinterpret_cast<f16*>(smem);                                              // [2][PANEL_ROWS][128], pieces exchanged (see fetch_x)
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int K = a.K, M = a.M;
+  // workgroup id -> tile as in gemm_rows_kernel (contiguous stretches of the tile list per XCD); the row block runs
+  // fastest, so the workgroups that are resident together multiply the same weights and those come from L2
+  const int per = (int)gridDim.x / 8;
+  const int tile = ((int)blockIdx.x % 8) * per + (int)blockIdx.x / 8;
+  if (tile >= groups * row_blocks) return;
+  const int row_block = tile % row_blocks, group = tile / row_blocks;
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  const int per_slice = (a.KT + nsl - 1) / nsl;
+  const int kt_first = (int)blockIdx.y * per_slice;
+  const int kt_end = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;
+  const int steps = kt_end - kt_first;
+
+  // this wave's channel blocks: unit `wu` of the launch; waves past the last unit only help with the rows
+  const int wu = group * PANEL_WAVES + wave;
+  const bool active = wu < units;
+  const int gb = (active ? wu : 0) * (PAIR ? NST / 2 : NST);      // first block (of the launch; of the pair's matrices)
+  int mi = 0;
+  if (!PAIR) {
+#pragma unroll
+    for (int i = 1; i < 4; ++i)
+      if (i < a.count && gb >= a.mat[i].nb_begin) mi = i;
+  }
+  const int blk0 = PAIR ? gb : gb - a.mat[mi].nb_begin;           // first block within its matrix
+  // Loads through buffer descriptors: the descriptor and the tile's offset travel in scalar registers and one
+  // 32-bit offset per lane serves all streams, another all rows (with 64-bit addresses per lane the loop keeps a
+  // pointer per stream and row in vector registers, which this kernel does not have).  Rows past M lie past
+  // the end of the rows' descriptor and read as zero.
+  constexpr int NBW = PAIR ? NST / 2 : NST;                        // consecutive blocks behind one descriptor
+  const uint32_t blk_bytes = (uint32_t)a.KT * (KV * 1024);
+  const unsigned char* w0 = reinterpret_cast<const unsigned char*>(a.mat[PAIR ? 0 : mi].tiled) + (size_t)blk0 * blk_bytes;
+  const unsigned char* w1 = reinterpret_cast<const unsigned char*>(a.mat[PAIR ? 1 : mi].tiled) + (size_t)blk0 * blk_bytes;
+  const __amdgpu_buffer_rsrc_t wr0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(w0), 0, (int)(NBW * blk_bytes), 0x00020000);
+  const __amdgpu_buffer_rsrc_t wr1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(w1), 0, (int)(NBW * blk_bytes), 0x00020000);
+  const int wlane = lane * 16;
+  const int row0 = row_block * PANEL_ROWS;
+  const int rows_here = M - row0 < PANEL_ROWS ? M - row0 : PANEL_ROWS;
+  const __amdgpu_buffer_rsrc_t xr0 = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<f16*>(a.X + (size_t)row0 * K), 0, (int)((size_t)rows_here * K * 2), 0x00020000);
+
+  auto fetch_w = [&](int kt, u32x4 (&wv)[NST][KV]) {
+#pragma unroll
+    for (int st = 0; st < NST; ++st)
+#pragma unroll
+      for (int v = 0; v < KV; ++v)
+        wv[st][v] = __builtin_amdgcn_raw_buffer_load_b128(PAIR && st >= NST / 2 ? wr1 : wr0, wlane,
+                                                          (int)((PAIR ? st % (NST / 2) : st) * blk_bytes + (uint32_t)(kt * KV + v) * 1024), 0);
+  };
+  // The rows go from memory into LDS without passing through registers: instruction j of wave w brings rows
+  // 32 j + 4 w .. + 3 of the workgroup, 256 bytes each, lane l the 16 bytes that belong at position l % 16 of row
+  // l / 16 - LDS receives the lanes' data one after the other, so a row takes 256 bytes and its 16-byte pieces are
+  // stored exchanged among themselves: piece c of row r at position c ^ (r % 16).  The sixteen rows of a B operand
+  // read then fall into sixteen different groups of four banks, without padding.
+  auto fetch_x = [&](int kt, f16* xb) {
+    const int row = wave * 4 + (lane >> 4);
+    const int piece = (lane & 15) ^ (row & 15);                   // (32 j does not change row % 16)
+    const bool in_k = kt * 128 + piece * 8 < K;
+    const int off = in_k ? row * K * 2 + piece * 16 : -1;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xr0, (__attribute__((address_space(3))) void*)(xb + (j * 32 + wave * 4) * 128), 16,
+                                           in_k ? off + j * 32 * K * 2 : -1, kt * 256, 0, 0);
+  };
+
+  f32x4 acc[PANEL_RG][NST];
+#pragma unroll
+  for (int rg = 0; rg < PANEL_RG; ++rg)
+#pragma unroll
+    for (int st = 0; st < NST; ++st) acc[rg][st] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // The product runs as one pipeline over all feature tiles: 4 * NST blocks of eight MFMAs per tile (one decoded A
+  // operand each); the A operand of the next block is decoded among the MFMAs of this one, and during the last
+  // block of a step every B operand is replaced by the next step's as soon as its MFMA has been issued - across the
+  // tile boundary too.  So the tile's one barrier stands before its last step: by then every wave has read the
+  // last B operands from this tile's buffer (which the loads of the tile after next may then overwrite) and the next
+  // tile's rows, requested when this tile began, must have landed.
+  u32x4 wa[NST][KV], wb[NST][KV];
+  f16x8 xf[PANEL_RG];
+  f16x8 avc;
+  const int xat = (lane & 15) * 128;                               // this lane's row within a row group, in halves
+  auto b_piece = [&](int m) { return ((m * 4 + (lane >> 4)) ^ (lane & 15)) * 8; };
+  if (steps > 0) {
+    if (active) fetch_w(kt_first, wa);
+    fetch_x(kt_first, xbuf);
+  }
+  typename Fmt::Scale sc[NST];             // (requested behind the first tile: one round trip to memory, not two)
+#pragma unroll
+  for (int st = 0; st < NST; ++st) {
+    const GemmMat& mt = a.mat[PAIR ? (st < NST / 2 ? 0 : 1) : mi];
+    sc[st] = Fmt::load_scale(mt.scale, a.x_scale, (blk0 + (PAIR ? st % (NST / 2) : st)) * 16 + (lane & 15), mt.N);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): the rows have landed in LDS
+  __syncthreads();
+  if (active && steps > 0) {
+#pragma unroll
+    for (int rg = 0; rg < PANEL_RG; ++rg) xf[rg] = *reinterpret_cast<const f16x8*>(xbuf + xat + rg * 16 * 128 + b_piece(0));
+    avc = Fmt::a_operand(wa[0], 0, sc[0]);
+  }
+  auto feature_tile = [&](int i, const u32x4 (&wc)[NST][KV], u32x4 (&wn)[NST][KV]) {
+    const bool more = i + 1 < steps;
+    const f16* xc = xbuf + (size_t)(i & 1) * PANEL_XBUF + xat;
+    const f16* xn = xbuf + (size_t)((i + 1) & 1) * PANEL_XBUF + xat;
+    if (more) {
+      if (active) fetch_w(kt_first + i + 1, wn);
+      fetch_x(kt_first + i + 1, xbuf + (size_t)((i + 1) & 1) * PANEL_XBUF);
+    }
+    auto blocks = [&](int first, int last) {
+#pragma unroll
+      for (int blk = first; blk < last; ++blk) {
+        const int m = blk / NST, st = blk % NST;
+        f16x8 avn = avc;
+        if (blk + 1 < 4 * NST) avn = Fmt::a_operand(wc[(blk + 1) % NST], (blk + 1) / NST, sc[(blk + 1) % NST]);
+        else if (more) avn = Fmt::a_operand(wn[0], 0, sc[0]);
+#pragma unroll
+        for (int rg = 0; rg < PANEL_RG; ++rg) {
+          acc[rg][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(avc, xf[rg], acc[rg][st], 0, 0, 0);
+          if (st == NST - 1) {
+            if (m < 3) xf[rg] = *reinterpret_cast<const f16x8*>(xc + rg * 16 * 128 + b_piece(m + 1));
+            else if (more) xf[rg] = *reinterpret_cast<const f16x8*>(xn + rg * 16 * 128 + b_piece(0));
+          }
+        }
+        avc = avn;
+      }
+    };
+    if (active) blocks(0, 3 * NST);
+    __builtin_amdgcn_s_waitcnt(0x0f70);    // vmcnt(0): the next tile's rows have landed (and its weights)
+    __syncthreads();
+    if (active) blocks(3 * NST, 4 * NST);
+  };
+  for (int i = 0; i < steps; i += 2) {
+    feature_tile(i, wa, wb);
+    if (i + 1 < steps) feature_tile(i + 1, wb, wa);
+  }
+  __syncthreads();                         // (the epilogue's strips lie in the row buffers)
+  if (!active) return;
+
+  // Lane l holds channels st * 16 + (l / 16) * 4 + r of row l % 16 of each row group.  Row group by row group the
+  // sums pass through a strip of LDS of the wave's own (the row buffers are free after the last barrier) and come
+  // back with eight consecutive channels of one row per lane: one 16-byte store per lane, whole 128-byte stretches
+  // of a row per wave.  (A wave's LDS accesses complete in order.)
+  float* strip = reinterpret_cast<float*>(smem) + (size_t)wave * (16 * SW);
+  const GemmMat& mat = a.mat[PAIR ? 0 : mi];
+  const int N = mat.N;
+  const bool direct = !mat.bias && mat.act == PTA_ACT_NONE && !a.epi.bias && a.epi.act == PTA_ACT_NONE && !a.epi.mul &&
+                      a.epi.post_scale == 0.0f && !a.epi.out_fp8_scale;
+  const typename Fmt::Scale s0 = Fmt::load_scale(a.mat[PAIR ? 0 : mi].scale, a.x_scale, 0, 1);   // no format's finish uses the per-channel part
+  const typename Fmt::Scale s1 = Fmt::load_scale(a.mat[PAIR ? 1 : mi].scale, a.x_scale, 0, 1);
+  auto put = [&](const f32x4 (&sums)[NST]) {
+#pragma unroll
+    for (int st = 0; st < NST; ++st)
+      *reinterpret_cast<f32x4*>(strip + (lane & 15) * SW + st * 16 + (lane >> 4) * 4) = sums[st];
+  };
+  // (one copy of the epilogue code: unrolled over the row groups it is too large to unroll, and an accumulator
+  // array indexed by a loop counter lives in scratch memory for the whole kernel - hence the switch)
+#pragma unroll 1
+  for (int rg = 0; rg < PANEL_RG; ++rg) {
+    switch (rg) {
+      case 0: put(acc[0]); break;
+      case 1: put(acc[1]); break;
+      case 2: put(acc[2]); break;
+      case 3: put(acc[3]); break;
+      case 4: put(acc[4]); break;
+      case 5: put(acc[5]); break;
+      case 6: put(acc[6]); break;
+      default: put(acc[7]); break;
+    }
+    if constexpr (PAIR) {
+      constexpr int LPR = NST / 2 * 16 / 8;                      // lanes per row: eight output channels each
+      constexpr int RPP = 64 / LPR;                              // rows per pass
+#pragma unroll 1
+      for (int it = 0; it < 16 / RPP; ++it) {
+        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
+        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
+        if (rr >= 16) continue;
+        const f32x4 g0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), g1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
+        const f32x4 u0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0), u1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0 + 4);
+        if (m >= M) continue;
+        f16x8 y;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          y[j] = swiglu_out(a.epi, (f16)Fmt::finish(j < 4 ? g0[j & 3] : g1[j & 3], s0), (f16)Fmt::finish(j < 4 ? u0[j & 3] : u1[j & 3], s1));
+        if (n + 8 <= N && (N & 7) == 0) {
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
+        }
+      }
+    } else {
+      constexpr int LPR = NST * 16 / 8;
+      constexpr int RPP = 64 / LPR;
+#pragma unroll 1
+      for (int it = 0; it < (16 + RPP - 1) / RPP; ++it) {
+        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
+        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
+        if (rr >= 16) continue;
+        const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), v1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
+        if (m >= M) continue;
+        if (nsl > 1) {
+          float* p = a.part + ((size_t)blockIdx.y * M + m) * N + n;
+          if (n + 8 <= N && (N & 3) == 0) {
+            *reinterpret_cast<f32x4*>(p) = v0;
+            *reinterpret_cast<f32x4*>(p + 4) = v1;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (n + j < N) p[j] = j < 4 ? v0[j & 3] : v1[j & 3];
+          }
+          continue;
+        }
+        f16x8 y;
+        if (direct && n + 8 <= N && (N & 7) == 0) {                // nothing but the residual stream to add: whole vectors
+          f16x8 res;
+          if (a.epi.residual) res = *reinterpret_cast<const f16x8*>(a.epi.residual + (size_t)m * N + n);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            y[j] = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
+            if (a.epi.residual) y[j] = y[j] + res[j];
+          }
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+          continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          f16 y0 = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
+          if (n + j < N) {
+            if (mat.bias) y0 = y0 + mat.bias[n + j];
+            y0 = apply_act(mat.act, y0);
+            y0 = apply_epilogue(a.epi, y0, m, n + j, N);
+          }
+          y[j] = y0;
+        }
+        if (n + 8 <= N && (N & 7) == 0) {
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
+        }
+      }
+    }
+  }
+}
+
+// whether every matrix of the launch is a whole number of wave tiles of `nst` channel blocks and all share one input
+static inline bool panel_fits(const GemmArgs& a, int nst, bool pair) {
+  if (a.epi.norm != PTA_NORM_NONE || a.KT < 2) return false;
+  if (pair) return ((a.mat[0].N + 15) / 16) % (nst / 2) == 0;
+  for (int i = 0; i < a.count; ++i) {
+    if (((a.mat[i].N + 15) / 16) % nst != 0) return false;
+    if (a.mat[i].X && a.mat[i].X != a.X) return false;
+  }
+  return true;
+}
+
+template <class Fmt, int NST, bool PAIR>
+static int launch_gemm_panel(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+  static bool ready = false;
+  const size_t smem = (size_t)2 * PANEL_XBUF * 2;
+  if (!ready) {
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_panel_kernel<Fmt, NST, PAIR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem) == hipSuccess,
+                "%s: cannot reserve %zu bytes of LDS", name, smem);
+    ready = true;
+  }
+  const int units = PAIR ? total_nb / (NST / 2) : total_nb / NST;
+  const int groups = (units + PANEL_WAVES - 1) / PANEL_WAVES;
+  const int row_blocks = (a.M + PANEL_ROWS - 1) / PANEL_ROWS;
+  const int nsl = a.ksplit > 1 ? a.ksplit : 1;
+  const int per = (groups * row_blocks + 7) / 8;
+  hipLaunchKernelGGL((gemm_panel_kernel<Fmt, NST, PAIR>), dim3(per * 8, nsl), dim3(PANEL_WAVES * 64), smem, s, a, groups, row_blocks, units);
+  if (nsl > 1) {
+    const size_t total = (size_t)a.M * a.mat[0].N;
+    hipLaunchKernelGGL((splitk_finish_kernel<Fmt>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+  }
+  return PTA_OK;
+}
+
 // whether the launch fits gemm_tile_kernel with `per_wg` channel blocks per workgroup: every matrix
 // a whole number of workgroups, enough feature tiles for the K groups
 static inline bool tile_fits(const GemmArgs& a, int per_wg, int kq, bool pair) {
@@ -1183,16 +1488,32 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name);
 
-// 65..256 rows.  Up to 128 rows, where the channel blocks divide into workgroup tiles: the staged kernel with 8 row
-// groups (2 K groups of 4 waves; 8 channel blocks or 4 SwiGLU pairs per workgroup), every weight tile decoded once for
-// all rows; a single matrix with few channels also splits K when a workspace is at hand.  Otherwise, and beyond 128
-// rows, the rows go through the smaller paths in turn, 128 or 64 at a time.  (A variant with 16 row groups per wave
-// was measured: it needs more registers than a wave has - 41..53 spilled - and ran 10 times slower.)
+// More than 64 rows.  Beyond 256 rows gemm_panel_kernel, up to 256 gemm_rows_kernel, where the channel blocks divide
+// into their workgroup tiles; a single matrix with few channels also splits K when a workspace is at hand.  Otherwise
+// the rows go through the smaller paths in turn, 64 at a time.
 template <class Fmt, bool PAIR>
 static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   const int cus = device_compute_units();
   const int per_wg = PAIR ? 4 : 8;
   const bool tiles = a.epi.norm == PTA_NORM_NONE && tile_fits(a, per_wg, 2, PAIR);
+  // More than 256 rows (measured on whole prompt passes of the 7B shape: 8.7 against 10.4 ms at 256 rows, 14.3
+  // against 11.3 at 384): 128-row panels through LDS, the weights straight into registers.  Formats of up to two
+  // vectors per tile only - with four (fp16) two tiles of four streams do not fit the registers.
+  if constexpr (Fmt::kVec <= 2) {
+    if (a.M > 256 && panel_fits(a, 4, PAIR)) {
+      const int units = PAIR ? total_nb / 2 : total_nb / 4;
+      const int wgs = ((units + PANEL_WAVES - 1) / PANEL_WAVES) * ((a.M + PANEL_ROWS - 1) / PANEL_ROWS);
+      GemmArgs b = a;
+      int nsl = wgs > 0 ? cus / wgs : 1;
+      nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
+      while (nsl > 1 && a.KT < nsl * 8) --nsl;
+      if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
+      const int rc = launch_gemm_panel<Fmt, 4, PAIR>(b, total_nb, s, name);
+      if (rc) return rc;
+      PTA_CHECK_LAUNCH(name);
+      return PTA_OK;
+    }
+  }
   if (tiles) {
     // fragments in registers, weights through LDS: 256 rows per workgroup where that still fills the machine,
     // else 128; few workgroups and one matrix: K in slices as well
@@ -1209,19 +1530,7 @@ static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, co
     PTA_CHECK_LAUNCH(name);
     return PTA_OK;
   }
-  if (tiles && a.M <= 128) {
-    GemmArgs b = a;
-    const int wgs = total_nb / per_wg;
-    int nsl = wgs > 0 ? cus / wgs : 1;
-    nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
-    while (nsl > 1 && a.KT < nsl * 8) --nsl;
-    if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
-    const int rc = launch_gemm_tile<Fmt, 8, 2, PAIR>(b, total_nb, s, name);
-    if (rc) return rc;
-    PTA_CHECK_LAUNCH(name);
-    return PTA_OK;
-  }
-  const int chunk = tiles ? 128 : 64;
+  const int chunk = 64;
   for (int m0 = 0; m0 < a.M; m0 += chunk) {
     GemmArgs b = a;
     b.M = a.M - m0 < chunk ? a.M - m0 : chunk;

@@ -1016,10 +1016,12 @@ def test_fp8_products_pair_multi_and_nan(K):
 @pytest.mark.parametrize("M", [65, 128, 200, 256, 600, 1024])
 @pytest.mark.parametrize("Kdim,N", [(4096, 4096), (1160, 8192), (11008, 4096), (512, 100)])
 def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
-    """More than 64 rows: the kernel that keeps the activation fragments in registers (128 or 256 rows per workgroup,
+    """More than 64 rows: up to 256 the kernel that keeps the activation fragments in registers (128 or 256 rows per
+    workgroup), beyond them the kernel that takes 128-row panels through LDS and the weights straight into registers;
     with and without the K split that a workspace allows; 1160 features = a ragged last tile; 200 and 600 rows = a
-    ragged last row block), and for channel counts that do not divide into its workgroup tiles (100) the 64-row
-    paths over the rows in turn.  Bias, and a residual that aliases the output."""
+    ragged last row block, and for channel counts that do not divide into the workgroup tiles (100) the 64-row
+    paths over the rows in turn.  Bias and a residual that aliases the output; the residual alone (the epilogue
+    that moves whole vectors)."""
     x, packed, scale = _w4_case(M + Kdim + N, M, Kdim, N)
     rng = np.random.default_rng(M * N)
     bias = rng.standard_normal(N).astype(np.float16)
@@ -1032,6 +1034,22 @@ def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
     y = dev(res.copy())
     K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=y, out=y, workspace=ws)
     assert rel_err(host(y), ref) <= 1e-2
+    ref = (O.w4a16_matmul(x, packed, scale) + res).astype(np.float16)
+    y = dev(res.copy())
+    K.w4a16_gemm(dev(x), w, residual=y, out=y)
+    assert rel_err(host(y), ref) <= 1e-2
+
+
+def test_w4a16_gemm_most_rows_few_channels_exact_integers(K):
+    """4096 rows (the most a launch takes) and 256 channels: a workgroup of the panel kernel in which half the waves
+    have no channel blocks and only help to bring the rows in; 3000 rows = a ragged last panel."""
+    rng = np.random.default_rng(77)
+    for M in (4096, 3000):
+        Kdim, N = 512, 256
+        x = rng.integers(-2, 3, size=(M, Kdim)).astype(np.float16)
+        q = rng.integers(-8, 8, size=(N, Kdim))
+        w = K.W4Weight(dev(O.pack_int4(q)), dev(np.ones(N, np.float16)))
+        assert np.array_equal(host(K.w4a16_gemm(dev(x), w)).astype(np.int64), x.astype(np.int64) @ q.T.astype(np.int64))
 
 
 def test_gemm_up_to_256_rows_exact_integers_pair_and_other_formats(K):
