@@ -31,13 +31,15 @@ struct QkvArgs {
 // Llama: angle = fp16(fp16(step) * inv_freq16) (an fp16 MatMul of a 1x1 by a 1xD/2 matrix,
 // llama2/attention.py:28-38), sin/cos rounded to fp16, rotate-half over the whole head
 // (llama2/attention.py:40-56): y = fp16(fp16(x*cos) + fp16(rot(x)*sin)).
+__device__ __forceinline__ f16 rope_mix(f16 x, f16 rot, f16 c, f16 s) { return x * c + rot * s; }
+__device__ __forceinline__ f16 rope_llama_angle(int step, f16 inv_freq) { return (f16)((float)(f16)(float)step * (float)inv_freq); }
 __device__ __forceinline__ f16 rope_llama_value(const f16* x, int d, int D, int step, const f16* inv_freq) {
   const int half = D >> 1;
   const int i = d < half ? d : d - half;
-  const f16 ang = (f16)((float)(f16)(float)step * (float)inv_freq[i]);
+  const f16 ang = rope_llama_angle(step, inv_freq[i]);
   const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
   const f16 rot = d < half ? -x[d + half] : x[d - half];
-  return x[d] * c + rot * s;
+  return rope_mix(x[d], rot, c, s);
 }
 __device__ __forceinline__ void rope_llama(const f16* x, f16* y, int d, int D, int step, const f16* inv_freq) {
   y[d] = rope_llama_value(x, d, D, step, inv_freq);
@@ -52,7 +54,7 @@ __device__ __forceinline__ f16 rope_glm2_value(const f16* x, int d, int D, int s
   const f16 ang = (f16)((float)step * inv_freq[j]);
   const f16 c = (f16)cosf((float)ang), s = (f16)sinf((float)ang);
   const f16 rot = (d & 1) ? x[d - 1] : -x[d + 1];
-  return x[d] * c + rot * s;
+  return rope_mix(x[d], rot, c, s);
 }
 __device__ __forceinline__ void rope_glm2(const f16* x, f16* y, int d, int D, int step, const float* inv_freq) {
   y[d] = rope_glm2_value(x, d, D, step, inv_freq);
@@ -109,6 +111,65 @@ __global__ __launch_bounds__(256) void qkv_rope_append_kernel(QkvArgs a) {
   else a.vring[at] = y;
 }
 
+// The same for many rows (prompt passes): one workgroup per row.  The angles of a position are the same for every
+// head, so their cosines and sines are worked out once per row into LDS (the kernel above evaluates both for every
+// element), and every thread moves vectors of eight features.  The arithmetic per element is that of the kernel
+// above, so both leave the same bits.
+__global__ __launch_bounds__(256) void qkv_rope_append_rows_kernel(QkvArgs a) {
+  __shared__ f16 cs[2][256];
+  const int D = a.D, tid = threadIdx.x;
+  const int row = blockIdx.x;
+  const int b = row / a.rows;
+  const int step = *a.step + row % a.rows;
+  const int pos = step % a.max_len;
+  if (a.rope == PTA_ROPE_LLAMA && tid < (D >> 1)) {
+    const f16 ang = rope_llama_angle(step, ((const f16*)a.inv_freq)[tid]);
+    cs[0][tid] = (f16)cosf((float)ang); cs[1][tid] = (f16)sinf((float)ang);
+  } else if (a.rope == PTA_ROPE_GLM2 && tid < (D >> 2)) {
+    const f16 ang = (f16)((float)step * ((const float*)a.inv_freq)[tid]);
+    cs[0][tid] = (f16)cosf((float)ang); cs[1][tid] = (f16)sinf((float)ang);
+  }
+  __syncthreads();
+  const int nq = a.Hq * D, nk = a.Hkv * D;
+  for (int r = tid * 8; r < nq + 2 * nk; r += 256 * 8) {
+    const int sect = r < nq ? 0 : (r < nq + nk ? 1 : 2);
+    const int e = r - (sect == 0 ? 0 : (sect == 1 ? nq : nq + nk));
+    const int h = e / D, d0 = e % D;
+    const f16* x = sect == 0 ? a.q + (size_t)row * a.q_stride + h * D
+                 : sect == 1 ? a.k + (size_t)row * a.k_stride + h * D : a.v + (size_t)row * a.v_stride + h * D;
+    f16x8 y = *reinterpret_cast<const f16x8*>(x + d0);
+    if (sect < 2 && a.rope == PTA_ROPE_LLAMA) {
+      const int half = D >> 1;
+      const bool low = d0 < half;
+      const f16x8 o = *reinterpret_cast<const f16x8*>(x + (low ? d0 + half : d0 - half));
+      const int i0 = low ? d0 : d0 - half;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = rope_mix(y[j], low ? -o[j] : o[j], cs[0][i0 + j], cs[1][i0 + j]);
+    } else if (sect < 2 && a.rope == PTA_ROPE_GLM2 && d0 < (D >> 1)) {
+      const f16x8 xin = y;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = rope_mix(xin[j], (j & 1) ? xin[j - 1] : -xin[j + 1], cs[0][(d0 + j) >> 1], cs[1][(d0 + j) >> 1]);
+    }
+    if (sect == 0) {
+      *reinterpret_cast<f16x8*>(a.q_out + ((size_t)row * a.Hq + h) * D + d0) = y;
+      continue;
+    }
+    const size_t at = (((size_t)b * a.Hkv + h) * a.max_len + pos) * D + d0;
+    f16* ring = sect == 1 ? a.kring : a.vring;
+    if (a.kv8) {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        lo |= (uint32_t)kv8_encode(y[j], a.kv_scale) << (8 * j);
+        hi |= (uint32_t)kv8_encode(y[4 + j], a.kv_scale) << (8 * j);
+      }
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint8_t*>(ring) + at) = make_uint2(lo, hi);
+    } else {
+      *reinterpret_cast<f16x8*>(ring + at) = y;
+    }
+  }
+}
+
 static int rope_append_rows(const char* name, const pta_half* q, const pta_half* k, const pta_half* v, int q_stride,
                             int k_stride, int v_stride, pta_half* q_out, pta_half* kv_ring, const int32_t* step,
                             const void* inv_freq, int B, int rows, int Hq, int Hkv, int D, int max_len, int rope,
@@ -125,7 +186,13 @@ static int rope_append_rows(const char* name, const pta_half* q, const pta_half*
   QkvArgs a{(const f16*)q, (const f16*)k, (const f16*)v, q_stride, k_stride, v_stride, (f16*)q_out,
             (f16*)kv_ring, vring, step, inv_freq, B, Hq, Hkv, D, max_len, rope, rows, kv8 ? 1 : 0, kv_scale};
   const long total = (long)B * rows * (Hq + 2 * Hkv) * D;
-  hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
+  const bool vectors = D % 16 == 0 && D <= 512 && q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 &&
+                       (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)q_out | (uintptr_t)kv_ring) & 15) == 0 &&
+                       (!kv8 || ring_elems % 8 == 0);
+  if (vectors && (long)B * rows >= 64)
+    hipLaunchKernelGGL(qkv_rope_append_rows_kernel, dim3((unsigned)(B * rows)), dim3(256), 0, (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL(qkv_rope_append_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
   PTA_CHECK_LAUNCH(name);
   return PTA_OK;
 }
