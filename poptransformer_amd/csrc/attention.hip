@@ -466,22 +466,31 @@ static int attn_splits(int B, int Hq, int max_len) {
 
 // ------------------------------------------------------------------------------------------
 // Attention of many rows at once (the prompt passes) on the matrix unit, head size 128, fp16 cache.
-// One workgroup of four waves per (sequence, query head, 64 rows of the pass); wave w owns 16 of the rows.
-// The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes
+// One workgroup of four waves per (sequence, query head, 128 rows of the pass); wave w owns 32 of the rows, two
+// groups of 16.  The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes,
+// for each of its row groups,
 //   S^T = K Q^T     (two 16 x 16 tiles, 4 MFMAs each: lane l then holds the scores of query row l % 16 for
 //                    cache rows (l / 16) * 4 + 0..3 of each tile - which IS the layout of an A operand whose
 //                    k index runs over those eight cache rows),
 //   the roundings of the reference on the scores (fp16 MatMul output, fp16 multiply by 1/sqrt(D)), the online
 //   softmax in fp32 per query row (partners: lanes l ^ 16, l ^ 32), probabilities rounded to fp16 (the
 //   reference's softmax output is fp16),
-//   O += P V        (eight 16 x 16 tiles over the head size, B operands from the transposed V rows).
+//   O += P V        (eight 16 x 16 tiles over the head size, B operands from the transposed V rows);
+// every K and V operand read from LDS serves both row groups.
 // Row r of the pass sits at position step + r and attends to cache rows [0, min(step + r + 1, max_len)), as in
 // attn_partial_kernel.  Outputs differ from that kernel in the last bits (another summation order, fp16
 // probabilities); both are held to 1e-2 against the oracle.
 // ------------------------------------------------------------------------------------------
 constexpr int PA_THREADS = 256;
+constexpr int PA_RG = 2;                 // row groups of 16 per wave
+constexpr int PA_ROWS = 4 * PA_RG * 16;  // rows of the pass per workgroup
 constexpr int PA_KSTRIDE = 128 + 8;      // halves per staged K row
 constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
+
+// V^T in LDS: feature d, cache row p (of the 32 staged) at d * PA_VSTRIDE + (((p / 2) ^ (2 * (d / 16))) * 2 + p % 2.
+// Exchanging the dwords of a row by its feature group spreads the 2-byte stores of the transposition (which go
+// down the features, 8 * PA_VSTRIDE halves apart) over the banks; pairs of dwords stay together for the 8-byte reads.
+__device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + ((((p >> 1) ^ ((d >> 4) << 1))) << 1) + (p & 1); }
 
 __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnArgs a) {
   constexpr int D = 128;
@@ -491,27 +500,35 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   const int h = blockIdx.y, b = blockIdx.z;
   const int kvh = h / (a.Hq / a.Hkv);
   const int step0 = *a.step;
-  const int r0 = (int)blockIdx.x * 64 + wave * 16;          // first row of this wave within the pass
-  const int qrow = r0 + (lane & 15);
-  f16x8 qf[4];
-#pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    qf[m] = f16x8{};
-    if (qrow < a.rows) qf[m] = *reinterpret_cast<const f16x8*>(a.q + (((size_t)b * a.rows + qrow) * a.Hq + h) * D + m * 32 + (lane >> 4) * 8);
-  }
+  const int r0 = (int)blockIdx.x * PA_ROWS + wave * (PA_RG * 16);          // first row of this wave within the pass
   auto valid_of = [&](int row) { const int v = step0 + row + 1; return row < a.rows ? (v < a.max_len ? v : a.max_len) : 0; };
-  const int my_valid = valid_of(qrow);
-  const int last_of_wave = r0 + 15 < a.rows ? r0 + 15 : a.rows - 1;
+  f16x8 qf[PA_RG][4];
+  int my_valid[PA_RG];
+#pragma unroll
+  for (int g = 0; g < PA_RG; ++g) {
+    const int qrow = r0 + g * 16 + (lane & 15);
+    my_valid[g] = valid_of(qrow);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      qf[g][m] = f16x8{};
+      if (qrow < a.rows) qf[g][m] = *reinterpret_cast<const f16x8*>(a.q + (((size_t)b * a.rows + qrow) * a.Hq + h) * D + m * 32 + (lane >> 4) * 8);
+    }
+  }
+  const int last_of_wave = r0 + PA_RG * 16 - 1 < a.rows ? r0 + PA_RG * 16 - 1 : a.rows - 1;
   const int wave_valid = r0 < a.rows ? valid_of(last_of_wave) : 0;
-  const int last_of_wg = (int)blockIdx.x * 64 + 63 < a.rows ? (int)blockIdx.x * 64 + 63 : a.rows - 1;
+  const int last_of_wg = (int)blockIdx.x * PA_ROWS + PA_ROWS - 1 < a.rows ? (int)blockIdx.x * PA_ROWS + PA_ROWS - 1 : a.rows - 1;
   const int wg_valid = valid_of(last_of_wg);
   const f16* kbase = a.kring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
   const f16* vbase = a.vring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
 
-  float run_m = -INFINITY, run_l = 0.f;
-  f32x4 o[8];
+  float run_m[PA_RG], run_l[PA_RG];
+  f32x4 o[PA_RG][8];
 #pragma unroll
-  for (int jd = 0; jd < 8; ++jd) o[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int g = 0; g < PA_RG; ++g) {
+    run_m[g] = -INFINITY; run_l[g] = 0.f;
+#pragma unroll
+    for (int jd = 0; jd < 8; ++jd) o[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   for (int p0 = 0; p0 < wg_valid; p0 += 32) {
     __syncthreads();
@@ -527,70 +544,86 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
       }
       *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(col + e) * PA_VSTRIDE + row] = vv[e];
+      for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[e];
     }
     __syncthreads();
     if (p0 >= wave_valid) continue;
-    float x[8];
+    f32x4 sc[PA_RG][2];
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
-      f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < PA_RG; ++g) sc[g][hh] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const f16x8 kf = *reinterpret_cast<const f16x8*>(ks + (hh * 16 + (lane & 15)) * PA_KSTRIDE + m * 32 + (lane >> 4) * 8);
-        sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], sc, 0, 0, 0);
-      }
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        f16 s16 = (f16)sc[r];                       // fp16 output of the q.K^T MatMul
-        if (a.use_scale) s16 = s16 * a.scale;       // fp16 multiply by fp16(1/sqrt(D))
-        const int pos = p0 + hh * 16 + (lane >> 4) * 4 + r;
-        x[hh * 4 + r] = pos < my_valid ? (float)s16 : -INFINITY;
+        for (int g = 0; g < PA_RG; ++g) sc[g][hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[g][m], sc[g][hh], 0, 0, 0);
       }
     }
-    float mx = x[0];
+    f16x8 pa[PA_RG];
+    float cr[PA_RG][4];
 #pragma unroll
-    for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float new_m = fmaxf(run_m, mx);
-    const float corr = run_m == -INFINITY ? 0.f : __expf(run_m - new_m);
-    float psum = 0.f;
-    f16x8 pa;
+    for (int g = 0; g < PA_RG; ++g) {
+      float x[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float pe = x[e] == -INFINITY ? 0.f : __expf(x[e] - new_m);
-      psum += pe;
-      pa[e] = (f16)pe;
+      for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          f16 s16 = (f16)sc[g][hh][r];                // fp16 output of the q.K^T MatMul
+          if (a.use_scale) s16 = s16 * a.scale;       // fp16 multiply by fp16(1/sqrt(D))
+          const int pos = p0 + hh * 16 + (lane >> 4) * 4 + r;
+          x[hh * 4 + r] = pos < my_valid[g] ? (float)s16 : -INFINITY;
+        }
+      float mx = x[0];
+#pragma unroll
+      for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float new_m = fmaxf(run_m[g], mx);
+      const float corr = run_m[g] == -INFINITY ? 0.f : __expf(run_m[g] - new_m);
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pe = x[e] == -INFINITY ? 0.f : __expf(x[e] - new_m);
+        psum += pe;
+        pa[g][e] = (f16)pe;
+      }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      run_l[g] = run_l[g] * corr + psum;
+      run_m[g] = new_m;
+      // the accumulators' rows are query rows (lane / 16) * 4 + r: their correction factors sit in lanes of that index
+#pragma unroll
+      for (int r = 0; r < 4; ++r) cr[g][r] = __shfl(corr, (lane >> 4) * 4 + r, 64);
     }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
-    run_l = run_l * corr + psum;
-    run_m = new_m;
-    // the accumulators' rows are query rows (lane / 16) * 4 + r: their correction factors sit in lanes of that index
-    float cr[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, (lane >> 4) * 4 + r, 64);
 #pragma unroll
     for (int jd = 0; jd < 8; ++jd) {
-      const f16* vrow = vt + (jd * 16 + (lane & 15)) * PA_VSTRIDE + (lane >> 4) * 4;
-      const f16x4 v0 = *reinterpret_cast<const f16x4*>(vrow), v1 = *reinterpret_cast<const f16x4*>(vrow + 16);
+      // cache rows (lane / 16) * 4 + 0..3 and 16 + the same of feature jd * 16 + lane % 16
+      const int d = jd * 16 + (lane & 15);
+      const f16x4 v0 = *reinterpret_cast<const f16x4*>(vt + pa_vt_at(d, (lane >> 4) * 4));
+      const f16x4 v1 = *reinterpret_cast<const f16x4*>(vt + pa_vt_at(d, 16 + (lane >> 4) * 4));
       const f16x8 vb = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
 #pragma unroll
-      for (int r = 0; r < 4; ++r) o[jd][r] *= cr[r];
-      o[jd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[jd], 0, 0, 0);
+      for (int g = 0; g < PA_RG; ++g) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[g][jd][r] *= cr[g][r];
+        o[g][jd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa[g], vb, o[g][jd], 0, 0, 0);
+      }
     }
   }
-  float lr[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) lr[r] = __shfl(run_l, (lane >> 4) * 4 + r, 64);
+  for (int g = 0; g < PA_RG; ++g) {
+    float lr[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int row = r0 + (lane >> 4) * 4 + r;
-    if (row >= a.rows) continue;
+    for (int r = 0; r < 4; ++r) lr[r] = __shfl(run_l[g], (lane >> 4) * 4 + r, 64);
 #pragma unroll
-    for (int jd = 0; jd < 8; ++jd)
-      a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] = attn_result(a, (f16)(o[jd][r] / lr[r]));
+    for (int r = 0; r < 4; ++r) {
+      const int row = r0 + g * 16 + (lane >> 4) * 4 + r;
+      if (row >= a.rows) continue;
+#pragma unroll
+      for (int jd = 0; jd < 8; ++jd)
+        a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] = attn_result(a, (f16)(o[g][jd][r] / lr[r]));
+    }
   }
 }
 
@@ -635,7 +668,7 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   if (rows >= 16 && D == 128 && !kv8) {        // many rows: on the matrix unit, no splits, no workspace
-    hipLaunchKernelGGL(prompt_attention_mfma_kernel, dim3((rows + 63) / 64, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(prompt_attention_mfma_kernel, dim3((rows + PA_ROWS - 1) / PA_ROWS, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
     PTA_CHECK_LAUNCH(name);
     return PTA_OK;
   }
