@@ -400,7 +400,9 @@ class FusedDecoder(LayerOps):
             raise RuntimeError("consume_prompt must follow reset()")
         if n == 0:
             return 0
-        R = max(1, 64 // s.batch) if rows_per_pass is None else int(rows_per_pass)
+        # by default passes of up to 1024 rows: from a few hundred rows on the projections run on the kernel whose
+        # workgroups take 128-row panels, at 2-3 times the rate per row of the 64-row kernels
+        R = max(1, min(n, 1024 // s.batch)) if rows_per_pass is None else int(rows_per_pass)
         if R < 1 or R * s.batch > 2048:
             raise ValueError(f"consume_prompt: rows_per_pass * batch must lie in [1, 2048], got {R} * {s.batch}")
         if not hasattr(self, "_prompt_passes"):

@@ -7,7 +7,7 @@ two-stage ChatGLM model runs the same layer stack once over the whole prompt wit
 (models/chatglm/model.py:301-330, models/chatglm/attention.py:89-140) before the loop starts.
 
 `PromptPass` is that first stage for the decoders here: R consecutive positions of every sequence
-(B*R <= 64 rows) go through each layer together - the projections as GEMMs over B*R rows, which read
+(B*R <= 2048 rows) go through each layer together - the projections as GEMMs over B*R rows, which read
 each weight once per pass, the rotary embedding and cache append per row at its own position, and
 causal attention of row r over positions 0..p0+r.  The final norm, the head and the token selection
 are skipped: the loop would discard their result.  What it leaves in the KV rings is what R iterations
