@@ -1146,20 +1146,29 @@ static int launch_gemm_rows(const GemmArgs& a, int total_nb, hipStream_t s, cons
 // PAIR: a wave owns NST / 2 gate blocks and the same blocks of the up weight.
 // ------------------------------------------------------------------------------------------
 constexpr int PANEL_WAVES = 8;
-constexpr int PANEL_RG = 8;                       // row groups of 16: every wave multiplies all of them
-constexpr int PANEL_ROWS = PANEL_RG * 16;
-constexpr int PANEL_XBUF = PANEL_ROWS * 128;        // halves of one buffer of staged rows
-static_assert(PANEL_RG == 8, "the epilogue's switch names the row groups");
 
-template <class Fmt, int NST, bool PAIR>
+// RG: row groups of 16 per workgroup (every wave multiplies all of them); KH: parts of K inside the workgroup - the
+// waves are 8 / KH channel units x KH parts, part kh takes the feature tiles kh, kh + KH, ... of the workgroup's
+// range and the parts' sums meet in LDS at the end.  KH > 1 is for launches with few channels: it halves or
+// quarters the channels of a workgroup tile, so more workgroups, without the fp32 round trip through memory that
+// slices of workgroups (ksplit) cost.
+template <class Fmt, int NST, int RG, int KH, bool PAIR>
 __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_panel_kernel(GemmArgs a, int groups, int row_blocks, int units) {
   constexpr int KV = Fmt::kVec;
+  constexpr int CW = PANEL_WAVES / KH;            // channel units (waves side by side) per workgroup
+  constexpr int ROWS = RG * 16;
+  constexpr int XPART = ROWS * 128;               // halves of one feature tile of the workgroup's rows
+  constexpr int XSTAGE = KH * XPART;              // one stage: a tile per part
+  constexpr int QN = KH * RG / 2;                 // row loads (4 rows each) per wave and stage
   constexpr int SW = NST * 16 + 4;                // floats per row of a wave's epilogue strip
   static_assert(!PAIR || NST % 2 == 0, "gate and up blocks in equal numbers");
-  static_assert(PANEL_WAVES * 16 * SW * 4 <= 2 * PANEL_XBUF * 2, "the epilogue strips reuse the row buffers");
+  static_assert(KH == 1 || KH == 2 || KH == 4, "parts of K");
+  static_assert((KH * RG) % 2 == 0 && RG <= 8, "row loads per wave");
+  static_assert(KH == 1 || (KH - 1) * CW * RG * NST * 1024 <= 2 * XSTAGE * 2, "the parts' sums meet in the row buffers");
   extern __shared__ __align__(16) unsigned char smem[];
-  f16* xbuf = reinterpret_cast<f16*>(smem);                                              // [2][PANEL_ROWS][128], pieces exchanged (see fetch_x)
+  f16* xbuf = reinterpret_cast<f16*>(smem);                                              // [2][KH][ROWS][128], pieces exchanged (see fetch_x)
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int cw = wave % CW, kh = wave / CW;
   const int K = a.K, M = a.M;
   // workgroup id -> tile as in gemm_rows_kernel (contiguous stretches of the tile list per XCD); the row block runs
   // fastest, so the workgroups that are resident together multiply the same weights and those come from L2
@@ -1171,10 +1180,10 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
   const int per_slice = (a.KT + nsl - 1) / nsl;
   const int kt_first = (int)blockIdx.y * per_slice;
   const int kt_end = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;
-  const int steps = kt_end - kt_first;
+  const int steps = kt_end > kt_first ? (kt_end - kt_first + KH - 1) / KH : 0;      // a tile per part and step
 
   // this wave's channel blocks: unit `wu` of the launch; waves past the last unit only help with the rows
-  const int wu = group * PANEL_WAVES + wave;
+  const int wu = group * CW + cw;
   const bool active = wu < units;
   const int gb = (active ? wu : 0) * (PAIR ? NST / 2 : NST);      // first block (of the launch; of the pair's matrices)
   int mi = 0;
@@ -1195,55 +1204,61 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
   const __amdgpu_buffer_rsrc_t wr0 = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(w0), 0, (int)(NBW * blk_bytes), 0x00020000);
   const __amdgpu_buffer_rsrc_t wr1 = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(w1), 0, (int)(NBW * blk_bytes), 0x00020000);
   const int wlane = lane * 16;
-  const int row0 = row_block * PANEL_ROWS;
-  const int rows_here = M - row0 < PANEL_ROWS ? M - row0 : PANEL_ROWS;
+  const int row0 = row_block * ROWS;
+  const int rows_here = M - row0 < ROWS ? M - row0 : ROWS;
   const __amdgpu_buffer_rsrc_t xr0 = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<f16*>(a.X + (size_t)row0 * K), 0, (int)((size_t)rows_here * K * 2), 0x00020000);
 
-  auto fetch_w = [&](int kt, u32x4 (&wv)[NST][KV]) {
+  // this wave's weight tiles of step i (past the end of the range: zeros - the rows of that tile are zeros too)
+  auto fetch_w = [&](int i, u32x4 (&wv)[NST][KV]) {
+    const int kt = kt_first + i * KH + kh;
 #pragma unroll
     for (int st = 0; st < NST; ++st)
 #pragma unroll
       for (int v = 0; v < KV; ++v)
-        wv[st][v] = __builtin_amdgcn_raw_buffer_load_b128(PAIR && st >= NST / 2 ? wr1 : wr0, wlane,
-                                                          (int)((PAIR ? st % (NST / 2) : st) * blk_bytes + (uint32_t)(kt * KV + v) * 1024), 0);
+        wv[st][v] = kt < kt_end ? __builtin_amdgcn_raw_buffer_load_b128(PAIR && st >= NST / 2 ? wr1 : wr0, wlane,
+                                      (int)((PAIR ? st % (NST / 2) : st) * blk_bytes + (uint32_t)(kt * KV + v) * 1024), 0)
+                                : u32x4{0, 0, 0, 0};
   };
-  // The rows go from memory into LDS without passing through registers: instruction j of wave w brings rows
-  // 32 j + 4 w .. + 3 of the workgroup, 256 bytes each, lane l the 16 bytes that belong at position l % 16 of row
-  // l / 16 - LDS receives the lanes' data one after the other, so a row takes 256 bytes and its 16-byte pieces are
-  // stored exchanged among themselves: piece c of row r at position c ^ (r % 16).  The sixteen rows of a B operand
-  // read then fall into sixteen different groups of four banks, without padding.
-  auto fetch_x = [&](int kt, f16* xb) {
-    const int row = wave * 4 + (lane >> 4);
-    const int piece = (lane & 15) ^ (row & 15);                   // (32 j does not change row % 16)
-    const bool in_k = kt * 128 + piece * 8 < K;
-    const int off = in_k ? row * K * 2 + piece * 16 : -1;
+  // The rows go from memory into LDS without passing through registers: load q = 8 j + w (w: the wave) of a stage
+  // brings rows 4 (q % (4 RG)) .. + 3 of the tile of part q / (4 RG), 256 bytes each, lane l the 16 bytes that
+  // belong at position l % 16 of row l / 16 - LDS receives the lanes' data one after the other, so a row takes 256
+  // bytes and its 16-byte pieces are stored exchanged among themselves: piece c of row r at position c ^ (r % 16).
+  // The sixteen rows of a B operand read then fall into sixteen different groups of four banks, without padding.
+  auto fetch_x = [&](int i, f16* stage) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(xr0, (__attribute__((address_space(3))) void*)(xb + (j * 32 + wave * 4) * 128), 16,
-                                           in_k ? off + j * 32 * K * 2 : -1, kt * 256, 0, 0);
+    for (int j = 0; j < QN; ++j) {
+      const int q = j * PANEL_WAVES + wave;
+      const int part = q / (4 * RG), rb = q % (4 * RG);
+      const int row = rb * 4 + (lane >> 4);
+      const int piece = (lane & 15) ^ (row & 15);
+      const int kt = kt_first + i * KH + part;
+      const bool in_k = kt < kt_end && kt * 128 + piece * 8 < K;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(xr0, (__attribute__((address_space(3))) void*)(stage + part * XPART + rb * 4 * 128), 16,
+                                               in_k ? row * K * 2 + piece * 16 : -1, kt * 256, 0, 0);
+    }
   };
 
-  f32x4 acc[PANEL_RG][NST];
+  f32x4 acc[RG][NST];
 #pragma unroll
-  for (int rg = 0; rg < PANEL_RG; ++rg)
+  for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
     for (int st = 0; st < NST; ++st) acc[rg][st] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The product runs as one pipeline over all feature tiles: 4 * NST blocks of eight MFMAs per tile (one decoded A
-  // operand each); the A operand of the next block is decoded among the MFMAs of this one, and during the last
-  // block of a step every B operand is replaced by the next step's as soon as its MFMA has been issued - across the
-  // tile boundary too.  So the tile's one barrier stands before its last step: by then every wave has read the
-  // last B operands from this tile's buffer (which the loads of the tile after next may then overwrite) and the next
-  // tile's rows, requested when this tile began, must have landed.
+  // The product runs as one pipeline over all steps: 4 * NST blocks of RG MFMAs per tile (one decoded A operand
+  // each); the A operand of the next block is decoded among the MFMAs of this one, and during the last block of a
+  // 32-feature step every B operand is replaced by the next one's as soon as its MFMA has been issued - across the
+  // tile boundary too.  So the tile's one barrier stands before its last 32 features: by then every wave has read
+  // the last B operands from this stage (which the loads of the stage after next may then overwrite) and the next
+  // stage's rows, requested when this one began, must have landed.
   u32x4 wa[NST][KV], wb[NST][KV];
-  f16x8 xf[PANEL_RG];
+  f16x8 xf[RG];
   f16x8 avc;
-  const int xat = (lane & 15) * 128;                               // this lane's row within a row group, in halves
+  const int xat = kh * XPART + (lane & 15) * 128;                  // this lane's row within a row group of its part, in halves
   auto b_piece = [&](int m) { return ((m * 4 + (lane >> 4)) ^ (lane & 15)) * 8; };
   if (steps > 0) {
-    if (active) fetch_w(kt_first, wa);
-    fetch_x(kt_first, xbuf);
+    if (active) fetch_w(0, wa);
+    fetch_x(0, xbuf);
   }
   typename Fmt::Scale sc[NST];             // (requested behind the first tile: one round trip to memory, not two)
 #pragma unroll
@@ -1255,16 +1270,16 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
   __syncthreads();
   if (active && steps > 0) {
 #pragma unroll
-    for (int rg = 0; rg < PANEL_RG; ++rg) xf[rg] = *reinterpret_cast<const f16x8*>(xbuf + xat + rg * 16 * 128 + b_piece(0));
+    for (int rg = 0; rg < RG; ++rg) xf[rg] = *reinterpret_cast<const f16x8*>(xbuf + xat + rg * 16 * 128 + b_piece(0));
     avc = Fmt::a_operand(wa[0], 0, sc[0]);
   }
   auto feature_tile = [&](int i, const u32x4 (&wc)[NST][KV], u32x4 (&wn)[NST][KV]) {
     const bool more = i + 1 < steps;
-    const f16* xc = xbuf + (size_t)(i & 1) * PANEL_XBUF + xat;
-    const f16* xn = xbuf + (size_t)((i + 1) & 1) * PANEL_XBUF + xat;
+    const f16* xc = xbuf + (size_t)(i & 1) * XSTAGE + xat;
+    const f16* xn = xbuf + (size_t)((i + 1) & 1) * XSTAGE + xat;
     if (more) {
-      if (active) fetch_w(kt_first + i + 1, wn);
-      fetch_x(kt_first + i + 1, xbuf + (size_t)((i + 1) & 1) * PANEL_XBUF);
+      if (active) fetch_w(i + 1, wn);
+      fetch_x(i + 1, xbuf + (size_t)((i + 1) & 1) * XSTAGE);
     }
     auto blocks = [&](int first, int last) {
 #pragma unroll
@@ -1274,7 +1289,7 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
         if (blk + 1 < 4 * NST) avn = Fmt::a_operand(wc[(blk + 1) % NST], (blk + 1) / NST, sc[(blk + 1) % NST]);
         else if (more) avn = Fmt::a_operand(wn[0], 0, sc[0]);
 #pragma unroll
-        for (int rg = 0; rg < PANEL_RG; ++rg) {
+        for (int rg = 0; rg < RG; ++rg) {
           acc[rg][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(avc, xf[rg], acc[rg][st], 0, 0, 0);
           if (st == NST - 1) {
             if (m < 3) xf[rg] = *reinterpret_cast<const f16x8*>(xc + rg * 16 * 128 + b_piece(m + 1));
@@ -1285,7 +1300,7 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
       }
     };
     if (active) blocks(0, 3 * NST);
-    __builtin_amdgcn_s_waitcnt(0x0f70);    // vmcnt(0): the next tile's rows have landed (and its weights)
+    __builtin_amdgcn_s_waitcnt(0x0f70);    // vmcnt(0): the next stage's rows have landed (and its weights)
     __syncthreads();
     if (active) blocks(3 * NST, 4 * NST);
   };
@@ -1293,14 +1308,39 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
     feature_tile(i, wa, wb);
     if (i + 1 < steps) feature_tile(i + 1, wb, wa);
   }
-  __syncthreads();                         // (the epilogue's strips lie in the row buffers)
+  __syncthreads();                         // (what follows reuses the row buffers)
+  if constexpr (KH > 1) {
+    // the sums of parts 1 .. KH - 1 go to part 0's wave of the same channel unit
+    f32x4* ex = reinterpret_cast<f32x4*>(smem);                   // [(KH - 1) * CW][RG * NST][64]
+    if (kh > 0 && active) {
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+        for (int st = 0; st < NST; ++st) ex[(((kh - 1) * CW + cw) * (RG * NST) + rg * NST + st) * 64 + lane] = acc[rg][st];
+    }
+    __syncthreads();
+    if (kh == 0 && active) {
+#pragma unroll
+      for (int k = 1; k < KH; ++k)
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+          for (int st = 0; st < NST; ++st) {
+            const f32x4 other = ex[(((k - 1) * CW + cw) * (RG * NST) + rg * NST + st) * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[rg][st][r] += other[r];
+          }
+    }
+    __syncthreads();
+    if (kh > 0) return;
+  }
   if (!active) return;
 
   // Lane l holds channels st * 16 + (l / 16) * 4 + r of row l % 16 of each row group.  Row group by row group the
   // sums pass through a strip of LDS of the wave's own (the row buffers are free after the last barrier) and come
   // back with eight consecutive channels of one row per lane: one 16-byte store per lane, whole 128-byte stretches
   // of a row per wave.  (A wave's LDS accesses complete in order.)
-  float* strip = reinterpret_cast<float*>(smem) + (size_t)wave * (16 * SW);
+  float* strip = reinterpret_cast<float*>(smem) + (size_t)cw * (16 * SW);
   const GemmMat& mat = a.mat[PAIR ? 0 : mi];
   const int N = mat.N;
   const bool direct = !mat.bias && mat.act == PTA_ACT_NONE && !a.epi.bias && a.epi.act == PTA_ACT_NONE && !a.epi.mul &&
@@ -1313,19 +1353,12 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
       *reinterpret_cast<f32x4*>(strip + (lane & 15) * SW + st * 16 + (lane >> 4) * 4) = sums[st];
   };
   // (one copy of the epilogue code: unrolled over the row groups it is too large to unroll, and an accumulator
-  // array indexed by a loop counter lives in scratch memory for the whole kernel - hence the switch)
+  // array indexed by a loop counter lives in scratch memory for the whole kernel - hence the chain of comparisons)
 #pragma unroll 1
-  for (int rg = 0; rg < PANEL_RG; ++rg) {
-    switch (rg) {
-      case 0: put(acc[0]); break;
-      case 1: put(acc[1]); break;
-      case 2: put(acc[2]); break;
-      case 3: put(acc[3]); break;
-      case 4: put(acc[4]); break;
-      case 5: put(acc[5]); break;
-      case 6: put(acc[6]); break;
-      default: put(acc[7]); break;
-    }
+  for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+      if (r == rg) put(acc[r]);
     if constexpr (PAIR) {
       constexpr int LPR = NST / 2 * 16 / 8;                      // lanes per row: eight output channels each
       constexpr int RPP = 64 / LPR;                              // rows per pass
@@ -1416,22 +1449,25 @@ static inline bool panel_fits(const GemmArgs& a, int nst, bool pair) {
   return true;
 }
 
-template <class Fmt, int NST, bool PAIR>
+template <class Fmt, int NST, int RG, int KH, bool PAIR>
 static int launch_gemm_panel(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   static bool ready = false;
-  const size_t smem = (size_t)2 * PANEL_XBUF * 2;
+  constexpr int CW = PANEL_WAVES / KH;
+  constexpr size_t rows_bytes = (size_t)2 * KH * RG * 16 * 128 * 2, strips = (size_t)CW * 16 * (NST * 16 + 4) * 4;
+  constexpr size_t smem = rows_bytes > strips ? rows_bytes : strips;
+  static_assert(smem <= 160 * 1024, "LDS");
   if (!ready) {
-    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_panel_kernel<Fmt, NST, PAIR>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_panel_kernel<Fmt, NST, RG, KH, PAIR>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)smem) == hipSuccess,
                 "%s: cannot reserve %zu bytes of LDS", name, smem);
     ready = true;
   }
   const int units = PAIR ? total_nb / (NST / 2) : total_nb / NST;
-  const int groups = (units + PANEL_WAVES - 1) / PANEL_WAVES;
-  const int row_blocks = (a.M + PANEL_ROWS - 1) / PANEL_ROWS;
+  const int groups = (units + CW - 1) / CW;
+  const int row_blocks = (a.M + RG * 16 - 1) / (RG * 16);
   const int nsl = a.ksplit > 1 ? a.ksplit : 1;
   const int per = (groups * row_blocks + 7) / 8;
-  hipLaunchKernelGGL((gemm_panel_kernel<Fmt, NST, PAIR>), dim3(per * 8, nsl), dim3(PANEL_WAVES * 64), smem, s, a, groups, row_blocks, units);
+  hipLaunchKernelGGL((gemm_panel_kernel<Fmt, NST, RG, KH, PAIR>), dim3(per * 8, nsl), dim3(PANEL_WAVES * 64), smem, s, a, groups, row_blocks, units);
   if (nsl > 1) {
     const size_t total = (size_t)a.M * a.mat[0].N;
     hipLaunchKernelGGL((splitk_finish_kernel<Fmt>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
@@ -1502,13 +1538,16 @@ static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, co
   if constexpr (Fmt::kVec <= 2) {
     if (a.M > 256 && panel_fits(a, 4, PAIR)) {
       const int units = PAIR ? total_nb / 2 : total_nb / 4;
-      const int wgs = ((units + PANEL_WAVES - 1) / PANEL_WAVES) * ((a.M + PANEL_ROWS - 1) / PANEL_ROWS);
+      const int row_blocks = (a.M + 127) / 128;
+      // few workgroup tiles (4096 channels: 8 per row block): K in halves inside the workgroup, tiles of half the channels
+      const bool halves = ((units + 7) / 8) * row_blocks * 2 <= cus && a.KT >= 16;
+      const int wgs = ((units + (halves ? 3 : 7)) / (halves ? 4 : 8)) * row_blocks;
       GemmArgs b = a;
       int nsl = wgs > 0 ? cus / wgs : 1;
       nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
-      while (nsl > 1 && a.KT < nsl * 8) --nsl;
+      while (nsl > 1 && a.KT < nsl * 16) --nsl;
       if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
-      const int rc = launch_gemm_panel<Fmt, 4, PAIR>(b, total_nb, s, name);
+      const int rc = halves ? launch_gemm_panel<Fmt, 4, 8, 2, PAIR>(b, total_nb, s, name) : launch_gemm_panel<Fmt, 4, 8, 1, PAIR>(b, total_nb, s, name);
       if (rc) return rc;
       PTA_CHECK_LAUNCH(name);
       return PTA_OK;
