@@ -335,7 +335,7 @@ def main():
                     help="operators executor: run the norms inside the projections that consume them (default: the decoder's choice)")
     ap.add_argument("--prompt-loop", action="store_true",
                     help="decode workload: consume the (untimed) prompt one loop iteration per position, as the reference's "
-                         "loop does, instead of in passes of up to 64 rows (FusedDecoder.consume_prompt)")
+                         "loop does, instead of in passes of up to 1024 rows (FusedDecoder.consume_prompt)")
     ap.add_argument("--no-batch16", action="store_true",
                     help="default run only: skip the second, batch-16 measurement that is reported beside the headline")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -467,7 +467,7 @@ def main():
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"Llama2-7B INT4 greedy decode, batch {B}, timed context {t_first}..{t_first + args.steps - 1} "
                                f"after the {prompt}-token prompt (untimed, "
-                               f"{'passes of <= 64 rows' if in_passes else 'token by token'}), "
+                               f"{'one pass per sequence batch' if in_passes else 'token by token'}), "
                                f"{'F143' if args.fp8_cache else 'fp16'} KV cache of {MAX_LEN}",
                    "batch": B, "kv_cache_len": MAX_LEN, "executor": executor},
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
