@@ -467,7 +467,7 @@ def main():
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"Llama2-7B INT4 greedy decode, batch {B}, timed context {t_first}..{t_first + args.steps - 1} "
                                f"after the {prompt}-token prompt (untimed, "
-                               f"{'one pass per sequence batch' if in_passes else 'token by token'}), "
+                               f"{'in one pass' if in_passes else 'token by token'}), "
                                f"{'F143' if args.fp8_cache else 'fp16'} KV cache of {MAX_LEN}",
                    "batch": B, "kv_cache_len": MAX_LEN, "executor": executor},
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
