@@ -1153,7 +1153,7 @@ constexpr int PANEL_WAVES = 8;
 // quarters the channels of a workgroup tile, so more workgroups, without the fp32 round trip through memory that
 // slices of workgroups (ksplit) cost.
 template <class Fmt, int NST, int RG, int KH, bool PAIR>
-__global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_panel_kernel(GemmArgs a, int groups, int row_blocks, int units) {
+__global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_panel_kernel(GemmArgs a, int groups, int row_blocks, int unit0, int units) {
   constexpr int KV = Fmt::kVec;
   constexpr int CW = PANEL_WAVES / KH;            // channel units (waves side by side) per workgroup
   constexpr int ROWS = RG * 16;
@@ -1182,8 +1182,9 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
   const int kt_end = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;
   const int steps = kt_end > kt_first ? (kt_end - kt_first + KH - 1) / KH : 0;      // a tile per part and step
 
-  // this wave's channel blocks: unit `wu` of the launch; waves past the last unit only help with the rows
-  const int wu = group * CW + cw;
+  // this wave's channel blocks: unit `wu` of the matrices (the launch covers units unit0 .. units - 1); waves past the
+  // last unit only help with the rows
+  const int wu = unit0 + group * CW + cw;
   const bool active = wu < units;
   const int gb = (active ? wu : 0) * (PAIR ? NST / 2 : NST);      // first block (of the launch; of the pair's matrices)
   int mi = 0;
@@ -1449,8 +1450,9 @@ static inline bool panel_fits(const GemmArgs& a, int nst, bool pair) {
   return true;
 }
 
+// units [unit0, unit1) of the launch's matrices (a unit: NST channel blocks, or NST / 2 gate and up blocks)
 template <class Fmt, int NST, int RG, int KH, bool PAIR>
-static int launch_gemm_panel(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
+static int launch_gemm_panel(const GemmArgs& a, int unit0, int unit1, hipStream_t s, const char* name) {
   static bool ready = false;
   constexpr int CW = PANEL_WAVES / KH;
   constexpr size_t rows_bytes = (size_t)2 * KH * RG * 16 * 128 * 2, strips = (size_t)CW * 16 * (NST * 16 + 4) * 4;
@@ -1462,12 +1464,11 @@ static int launch_gemm_panel(const GemmArgs& a, int total_nb, hipStream_t s, con
                 "%s: cannot reserve %zu bytes of LDS", name, smem);
     ready = true;
   }
-  const int units = PAIR ? total_nb / (NST / 2) : total_nb / NST;
-  const int groups = (units + CW - 1) / CW;
+  const int groups = (unit1 - unit0 + CW - 1) / CW;
   const int row_blocks = (a.M + RG * 16 - 1) / (RG * 16);
   const int nsl = a.ksplit > 1 ? a.ksplit : 1;
   const int per = (groups * row_blocks + 7) / 8;
-  hipLaunchKernelGGL((gemm_panel_kernel<Fmt, NST, RG, KH, PAIR>), dim3(per * 8, nsl), dim3(PANEL_WAVES * 64), smem, s, a, groups, row_blocks, units);
+  hipLaunchKernelGGL((gemm_panel_kernel<Fmt, NST, RG, KH, PAIR>), dim3(per * 8, nsl), dim3(PANEL_WAVES * 64), smem, s, a, groups, row_blocks, unit0, unit1);
   if (nsl > 1) {
     const size_t total = (size_t)a.M * a.mat[0].N;
     hipLaunchKernelGGL((splitk_finish_kernel<Fmt>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
@@ -1540,14 +1541,26 @@ static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, co
       const int units = PAIR ? total_nb / 2 : total_nb / 4;
       const int row_blocks = (a.M + 127) / 128;
       // few workgroup tiles (4096 channels: 8 per row block): K in halves inside the workgroup, tiles of half the channels
-      const bool halves = ((units + 7) / 8) * row_blocks * 2 <= cus && a.KT >= 16;
+      const int groups = (units + 7) / 8, tiles_all = groups * row_blocks;
+      const bool halves = tiles_all * 2 <= cus && a.KT >= 16;
       const int wgs = ((units + (halves ? 3 : 7)) / (halves ? 4 : 8)) * row_blocks;
       GemmArgs b = a;
       int nsl = wgs > 0 ? cus / wgs : 1;
       nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
       while (nsl > 1 && a.KT < nsl * 16) --nsl;
       if (!PAIR && a.count == 1 && a.part && nsl > 1 && a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) b.ksplit = nsl;
-      const int rc = halves ? launch_gemm_panel<Fmt, 4, 8, 2, PAIR>(b, total_nb, s, name) : launch_gemm_panel<Fmt, 4, 8, 1, PAIR>(b, total_nb, s, name);
+      // More tiles than compute units and a last round that fills at most half of them (344 tiles are 1.34 rounds
+      // of 256 and would take 2): the channel groups of the whole rounds in one launch, the rest with K in halves -
+      // twice the workgroups, each half as long.
+      const int whole = (tiles_all / cus) * cus / row_blocks;             // channel groups within the whole rounds
+      const int rest = (groups - whole) * row_blocks;
+      int rc;
+      if (!halves && whole > 0 && rest > 0 && rest * 2 <= cus && a.KT >= 16 && b.ksplit <= 1) {
+        rc = launch_gemm_panel<Fmt, 4, 8, 1, PAIR>(b, 0, whole * 8, s, name);
+        if (!rc) rc = launch_gemm_panel<Fmt, 4, 8, 2, PAIR>(b, whole * 8, units, s, name);
+      } else {
+        rc = halves ? launch_gemm_panel<Fmt, 4, 8, 2, PAIR>(b, 0, units, s, name) : launch_gemm_panel<Fmt, 4, 8, 1, PAIR>(b, 0, units, s, name);
+      }
       if (rc) return rc;
       PTA_CHECK_LAUNCH(name);
       return PTA_OK;
