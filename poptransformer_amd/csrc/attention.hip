@@ -530,22 +530,33 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
     for (int jd = 0; jd < 8; ++jd) o[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int p0 = 0; p0 < wg_valid; p0 += 32) {
-    __syncthreads();
-    // stage cache rows p0 .. p0 + 31: 512 vectors of 16 bytes each of K and V, two per thread
+  // cache rows p .. p + 31: 512 vectors of 16 bytes each of K and V, two per thread; they are requested one step
+  // ahead, so that their way from memory runs beside the step's arithmetic
+  f16x8 kv[2], vv[2];
+  auto request = [&](int p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int c = (int)threadIdx.x + i * PA_THREADS;
       const int row = c >> 4, col = (c & 15) * 8;
-      f16x8 kv = f16x8{}, vv = f16x8{};
-      if (p0 + row < wg_valid) {
-        kv = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p0 + row) * D + col);
-        vv = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p0 + row) * D + col);
+      kv[i] = f16x8{}; vv[i] = f16x8{};
+      if (p + row < wg_valid) {
+        kv[i] = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p + row) * D + col);
+        vv[i] = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p + row) * D + col);
       }
-      *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[e];
     }
+  };
+  request(0);
+  for (int p0 = 0; p0 < wg_valid; p0 += 32) {
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int c = (int)threadIdx.x + i * PA_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
+      *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv[i];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[i][e];
+    }
+    if (p0 + 32 < wg_valid) request(p0 + 32);
     __syncthreads();
     if (p0 >= wave_valid) continue;
     f32x4 sc[PA_RG][2];
