@@ -466,8 +466,8 @@ static int attn_splits(int B, int Hq, int max_len) {
 
 // ------------------------------------------------------------------------------------------
 // Attention of many rows at once (the prompt passes) on the matrix unit, head size 128, fp16 cache.
-// One workgroup of four waves per (sequence, query head, 128 rows of the pass); wave w owns 32 of the rows, two
-// groups of 16.  The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes,
+// One workgroup of four waves per (sequence, query head, 64 or 128 rows of the pass); wave w owns one or two
+// groups of 16 rows.  The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes,
 // for each of its row groups,
 //   S^T = K Q^T     (two 16 x 16 tiles, 4 MFMAs each: lane l then holds the scores of query row l % 16 for
 //                    cache rows (l / 16) * 4 + 0..3 of each tile - which IS the layout of an A operand whose
@@ -476,14 +476,12 @@ static int attn_splits(int B, int Hq, int max_len) {
 //   softmax in fp32 per query row (partners: lanes l ^ 16, l ^ 32), probabilities rounded to fp16 (the
 //   reference's softmax output is fp16),
 //   O += P V        (eight 16 x 16 tiles over the head size, B operands from the transposed V rows);
-// every K and V operand read from LDS serves both row groups.
+// every K and V operand read from LDS serves all row groups of the wave.
 // Row r of the pass sits at position step + r and attends to cache rows [0, min(step + r + 1, max_len)), as in
 // attn_partial_kernel.  Outputs differ from that kernel in the last bits (another summation order, fp16
 // probabilities); both are held to 1e-2 against the oracle.
 // ------------------------------------------------------------------------------------------
 constexpr int PA_THREADS = 256;
-constexpr int PA_RG = 2;                 // row groups of 16 per wave
-constexpr int PA_ROWS = 4 * PA_RG * 16;  // rows of the pass per workgroup
 constexpr int PA_KSTRIDE = 128 + 8;      // halves per staged K row
 constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
 
@@ -492,8 +490,13 @@ constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
 // down the features, 8 * PA_VSTRIDE halves apart) over the banks; pairs of dwords stay together for the 8-byte reads.
 __device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + ((((p >> 1) ^ ((d >> 4) << 1))) << 1) + (p & 1); }
 
+// PA_RG: row groups of 16 per wave (a workgroup takes 4 * PA_RG * 16 rows of the pass).  Two where that still gives every
+// compute unit two workgroups or more (a wave's dependent chains - MFMA, maximum, exponentials, MFMA - need company
+// on their SIMD), else one.
+template <int PA_RG>
 __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnArgs a) {
   constexpr int D = 128;
+  constexpr int PA_ROWS = 4 * PA_RG * 16;
   __shared__ __align__(16) f16 ks[32 * PA_KSTRIDE];
   __shared__ __align__(16) f16 vt[D * PA_VSTRIDE];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -679,7 +682,12 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
   if (rows >= 16 && D == 128 && !kv8) {        // many rows: on the matrix unit, no splits, no workspace
-    hipLaunchKernelGGL(prompt_attention_mfma_kernel, dim3((rows + PA_ROWS - 1) / PA_ROWS, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    if ((long)((rows + 127) / 128) * Hq * B >= 2L * cus)
+      hipLaunchKernelGGL(prompt_attention_mfma_kernel<2>, dim3((rows + 127) / 128, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    else
+      hipLaunchKernelGGL(prompt_attention_mfma_kernel<1>, dim3((rows + 63) / 64, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
     PTA_CHECK_LAUNCH(name);
     return PTA_OK;
   }
