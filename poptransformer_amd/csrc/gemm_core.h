@@ -1525,19 +1525,20 @@ static void launch_gemv(const GemmArgs& a, int total_nb, hipStream_t s) {
 template <class Fmt, bool PAIR>
 static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const char* name);
 
-// More than 64 rows.  Beyond 256 rows gemm_panel_kernel, up to 256 gemm_rows_kernel, where the channel blocks divide
-// into their workgroup tiles; a single matrix with few channels also splits K when a workspace is at hand.  Otherwise
+// More than 64 rows.  Beyond 128 rows gemm_panel_kernel, up to 128 (fp16 weights: any number) gemm_rows_kernel, where
+// the channel blocks divide into their workgroup tiles; a single matrix with few channels also splits K when a workspace is at hand.  Otherwise
 // the rows go through the smaller paths in turn, 64 at a time.
 template <class Fmt, bool PAIR>
 static int dispatch_many_rows(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   const int cus = device_compute_units();
   const int per_wg = PAIR ? 4 : 8;
   const bool tiles = a.epi.norm == PTA_NORM_NONE && tile_fits(a, per_wg, 2, PAIR);
-  // More than 256 rows (measured on whole prompt passes of the 7B shape: 8.7 against 10.4 ms at 256 rows, 14.3
-  // against 11.3 at 384): 128-row panels through LDS, the weights straight into registers.  Formats of up to two
-  // vectors per tile only - with four (fp16) two tiles of four streams do not fit the registers.
+  // More than 128 rows (measured on whole prompt passes of the 7B shape, gemm_rows_kernel against this: 6.5 against
+  // 7.2 ms at 128 rows, 7.7 against 7.3 at 192, 8.1 against 7.5 at 256): 128-row panels through LDS, the weights
+  // straight into registers.  Formats of up to two vectors per tile only - with four (fp16) two tiles of four
+  // streams do not fit the registers.
   if constexpr (Fmt::kVec <= 2) {
-    if (a.M > 256 && panel_fits(a, 4, PAIR)) {
+    if (a.M > 128 && panel_fits(a, 4, PAIR)) {
       const int units = PAIR ? total_nb / 2 : total_nb / 4;
       const int row_blocks = (a.M + 127) / 128;
       // few workgroup tiles (4096 channels: 8 per row block): K in halves inside the workgroup, tiles of half the channels

@@ -1016,8 +1016,8 @@ def test_fp8_products_pair_multi_and_nan(K):
 @pytest.mark.parametrize("M", [65, 128, 200, 256, 600, 1024])
 @pytest.mark.parametrize("Kdim,N", [(4096, 4096), (1160, 8192), (11008, 4096), (512, 100)])
 def test_w4a16_gemm_up_to_256_rows(K, M, Kdim, N):
-    """More than 64 rows: up to 256 the kernel that keeps the activation fragments in registers (128 or 256 rows per
-    workgroup), beyond them the kernel that takes 128-row panels through LDS and the weights straight into registers;
+    """More than 64 rows: up to 128 the kernel that keeps the activation fragments in registers, beyond them the
+    kernel that takes 128-row panels through LDS and the weights straight into registers;
     with and without the K split that a workspace allows; 1160 features = a ragged last tile; 200 and 600 rows = a
     ragged last row block, and for channel counts that do not divide into the workgroup tiles (100) the 64-row
     paths over the rows in turn.  Bias and a residual that aliases the output; the residual alone (the epilogue
