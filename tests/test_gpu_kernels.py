@@ -1052,6 +1052,26 @@ def test_w4a16_gemm_most_rows_few_channels_exact_integers(K):
         assert np.array_equal(host(K.w4a16_gemm(dev(x), w)).astype(np.int64), x.astype(np.int64) @ q.T.astype(np.int64))
 
 
+def test_w4a16_gemm_last_round_of_tiles_in_a_launch_of_its_own(K):
+    """More workgroup tiles than compute units with a last round that fills at most half of them: the channel groups
+    of the whole rounds run in one launch, the rest in a second one with K in halves inside the workgroup (its
+    units start in the middle of the matrices).  11008 channels at 2048 rows (352 tiles of 128 rows x 512 channels),
+    the SwiGLU pair at 1024 rows (344 tiles), and three matrices in one launch at 2048 rows."""
+    rng = np.random.default_rng(91)
+    Kdim = 1024
+    mats = [(rng.integers(-128, 128, size=(n, Kdim // 2), dtype=np.int8), rng.uniform(0.005, 0.02, size=(n,)).astype(np.float16))
+            for n in (11008, 11008, 4096, 4096)]
+    ws = [K.W4Weight(dev(p), dev(s_)) for p, s_ in mats]
+    x = rng.standard_normal((2048, Kdim)).astype(np.float16)
+    assert rel_err(host(K.w4a16_gemm(dev(x), ws[0])), O.w4a16_matmul(x, *mats[0])) <= 1e-2
+    for (p, s_), o in zip(mats[1:], K.w4a16_gemm_multi(dev(x), ws[1:])):
+        assert rel_err(host(o), O.w4a16_matmul(x, p, s_)) <= 1e-2
+    x = x[:1024].copy()
+    got = host(K.w4a16_gemm_swiglu(dev(x), ws[0], ws[1]))
+    ref = (O.w4a16_matmul(x, *mats[1]) * O.swish(O.w4a16_matmul(x, *mats[0]))).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+
+
 def test_gemm_up_to_256_rows_exact_integers_pair_and_other_formats(K):
     rng = np.random.default_rng(61)
     for M in (96, 256, 520):
