@@ -375,7 +375,7 @@ def main():
     B, cfg = args.batch, LLAMA2_7B
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
-    executor = args.executor or ("persistent" if B <= 16 and not args.fp8_cache else "operators")
+    executor = args.executor or ("persistent" if B <= 16 else "operators")
     if args.fuse_norm is not None:
         dec.fuse_norm = args.fuse_norm == "on"
     if executor == "persistent":

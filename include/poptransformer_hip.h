@@ -474,6 +474,13 @@ size_t pta_decode_step_workspace_bytes(const pta_decode_model* model);
 int pta_llama_decode_step(const pta_decode_model* model, const pta_decode_state* state, void* workspace,
                           pta_stream_t stream);
 
+/* The same iteration with FP8 KV rings (KVCacheOp with fp8 = true, custom_ops/kv_cache.cpp:43-74,103-105;
+ * the cache layout and numerics of pta_decode_attention_qkv_f8): every layer's kv_ring holds F143 bytes
+ * [2 * batch * n_head, max_len, head_dim] of value * 2^-kv_scale, kv_scale in [-16, 16] (the reference's
+ * metadata scale is the constant 1).  Same workspace, same conditions. */
+int pta_llama_decode_step_f8(const pta_decode_model* model, const pta_decode_state* state, int kv_scale, void* workspace,
+                             pta_stream_t stream);
+
 /* Copies the failure word of the workspace to *failed (synchronises with `stream`). */
 int pta_decode_step_failed(const void* workspace, int* failed, pta_stream_t stream);
 

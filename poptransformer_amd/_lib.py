@@ -125,6 +125,7 @@ SIGNATURES = {
                                 c_int, c_int, c_int, c_void_p]),
     "pta_decode_step_workspace_bytes": (c_size_t, [POINTER(DecodeModel)]),
     "pta_llama_decode_step": (c_int, [POINTER(DecodeModel), POINTER(DecodeState), c_void_p, c_void_p]),
+    "pta_llama_decode_step_f8": (c_int, [POINTER(DecodeModel), POINTER(DecodeState), c_int, c_void_p, c_void_p]),
     "pta_decode_step_failed": (c_int, [c_void_p, POINTER(c_int), c_void_p]),
     "pta_llama_decode_step_static": (c_int, [POINTER(DecodeModel), POINTER(DecodeState), c_int, c_void_p]),
 }

@@ -87,6 +87,7 @@ struct DsArgs {
   uint32_t* best;        // [workgroups][16 rows][2]: value bits and index of each workgroup's largest logit per row (wide kernel)
   unsigned* sync;
   int nsplit;
+  int kv_scale;          // KV8 kernels: the rings hold F143 bytes of value * 2^-kv_scale (custom_ops/kv_cache.cpp:43-74)
   int region0;           // bytes of the activation / attention area at the start of LDS
   unsigned long long* trace;
 };
@@ -680,7 +681,63 @@ __device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8],
 // angles), append of the new K/V row to the ring by the split whose range holds it, online-softmax
 // attention over this split's rows.  Split 0 of a head collects the partials of the other splits
 // that have rows and writes the head's output.
-template <bool GROUPED = false>
+// FP8 KV rings (KVCacheOp with fp8 = true, custom_ops/kv_cache.cpp:43-74,103-105), as in attention.hip: a row is
+// stored as the F143 bytes of value * 2^-kv_scale; the kernels take decode(byte) as the row, multiply the fp32 score
+// by 2^kv_scale before it is rounded to fp16 and the weighted sum of the values by 2^kv_scale at the end (powers of
+// two: exact).  This step's own row enters LDS as decode(byte) too, so the pass sees what the cache will hold.
+__device__ __forceinline__ uint8_t ring_code(f16 v, int kv_scale) { return F8<0>::encode(ldexpf((float)v, -kv_scale)); }
+template <bool KV8> struct RingRow;
+template <> struct RingRow<false> {
+  typedef f16x8 type;
+  static __device__ __forceinline__ f16x8 values(f16x8 r) { return r; }
+};
+template <> struct RingRow<true> {
+  typedef u32x2 type;
+  static __device__ __forceinline__ f16x8 values(u32x2 r) { return f143_decode8(r[0], r[1]); }
+};
+template <bool KV8>
+__device__ __forceinline__ void ring_rows(const f16* kring, const f16* vring, size_t at, f16x8& k8, f16x8& v8) {
+  if constexpr (KV8) {
+    const u32x2 kr = *reinterpret_cast<const DS_GLOBAL u32x2*>(as_global(reinterpret_cast<const uint8_t*>(kring)) + at);
+    const u32x2 vr = *reinterpret_cast<const DS_GLOBAL u32x2*>(as_global(reinterpret_cast<const uint8_t*>(vring)) + at);
+    k8 = f143_decode8(kr[0], kr[1]);
+    v8 = f143_decode8(vr[0], vr[1]);
+  } else {
+    k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + at);
+    v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + at);
+  }
+}
+// the rings of (sequence b, head h): element pointers (fp16) or byte pointers carried as f16* (KV8)
+template <bool KV8>
+__device__ __forceinline__ void ring_of(const DsArgs& a, f16* kring_base, int b, int h, f16*& kring, f16*& vring) {
+  const size_t head = ((size_t)b * a.H + h) * a.max_len * DS_D, all = (size_t)a.B * a.H * a.max_len * DS_D;
+  if constexpr (KV8) {
+    kring = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(kring_base) + head);
+    vring = reinterpret_cast<f16*>(reinterpret_cast<uint8_t*>(kring) + all);
+  } else {
+    kring = kring_base + head;
+    vring = kring + all;
+  }
+}
+// element d of row pos of a ring: y goes in, what the cache holds of it comes back
+template <bool KV8>
+__device__ __forceinline__ f16 ring_put(f16* ring, size_t at, f16 y, int kv_scale) {
+  if constexpr (KV8) {
+    const uint8_t code = ring_code(y, kv_scale);
+    as_global(reinterpret_cast<uint8_t*>(ring))[at] = code;
+    return (f16)F8<0>::decode(code);
+  } else {
+    as_global(ring)[at] = y;
+    return y;
+  }
+}
+template <bool KV8>
+__device__ __forceinline__ f16 ring_value(f16 y, int kv_scale) {
+  if constexpr (KV8) return (f16)F8<0>::decode(ring_code(y, kv_scale));
+  else return y;
+}
+
+template <bool GROUPED = false, bool KV8 = false>
 __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kring_base, int unit, int step, float* lds,
                                                const f16* cs, Waiter& w) {
   constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2;
@@ -701,8 +758,9 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
   float* sm_l = sm_m + DS_WAVES;
   float* sm_acc = sm_l + DS_WAVES;                    // [DS_WAVES][D]
   const f16* qrow = a.qkv + ((size_t)li * a.B + b) * 3 * a.d + h * D;
-  f16* kring = kring_base + ((size_t)b * a.H + h) * a.max_len * D;
-  f16* vring = kring + (size_t)a.B * a.H * a.max_len * D;
+  f16 *kring, *vring;
+  ring_of<KV8>(a, kring_base, b, h, kring, vring);
+  const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
   const bool owner = pos >= c0 && pos < c0 + chunk;
   {
     // waves 0-1: q, waves 2-3: k, waves 4-5: v; a rotated element needs x[d] and x[d +- D/2]
@@ -719,9 +777,9 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
         const f16 rot = d_ < HALF ? -x1 : x1;
         y = x0 * cs[i] + rot * cs[HALF + i];
       }
+      if (which == 1) y = owner ? ring_put<KV8>(kring, (size_t)pos * D + d_, y, a.kv_scale) : ring_value<KV8>(y, a.kv_scale);
+      if (which == 2) y = owner ? ring_put<KV8>(vring, (size_t)pos * D + d_, y, a.kv_scale) : ring_value<KV8>(y, a.kv_scale);
       q_s[which * D + d_] = y;
-      if (which == 1 && owner) as_global(kring)[(size_t)pos * D + d_] = y;
-      if (which == 2 && owner) as_global(vring)[(size_t)pos * D + d_] = y;
     }
   }
   wg_sync();
@@ -743,14 +801,14 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
         k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
         v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
       } else {
-        k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)pc * D + d0);
-        v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)pc * D + d0);
+        ring_rows<KV8>(kring, vring, (size_t)pc * D + d0, k8, v8);
       }
       float s = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
 #pragma unroll
       for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      if (KV8) s *= kv_mul;
       f16 s16 = (f16)s;          // fp16 output of the q.K^T MatMul
       s16 = s16 * scale;         // fp16 multiply by fp16(1/sqrt(D))
       const float x = on ? (float)s16 : -INFINITY;
@@ -815,6 +873,7 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
         As = As * ca + as * cb;
         Mx = mn;
       }
+      if (KV8) As *= kv_mul;
       if constexpr (GROUPED) put(a.ctx + (size_t)li * 16 * a.d + grouped_at(b, h * D + d_), (f16)(As / Ls));
       else put(a.ctx + ((size_t)li * a.B + b) * a.d + h * D + d_, (f16)(As / Ls));
     }
@@ -826,6 +885,7 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
 // units as workgroups): the same arithmetic as attention_unit per unit - the online-softmax state of a row group
 // depends on the rows it visits, so the outputs differ from a sixteen-wave pass in the last bits, as they do between
 // split counts.  bh1 < 0: the second half of the workgroup has no unit.
+template <bool KV8 = false>
 __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* kring_base, int bh0, int bh1, int step, float* lds,
                                               const f16* cs, Waiter& w) {
   constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2, WPU = DS_WAVES / 2;
@@ -843,23 +903,25 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
   float* sm_l = sm_m + DS_WAVES;
   float* sm_acc = sm_l + DS_WAVES;                             // [DS_WAVES][D]
   const f16* qrow = a.qkv + ((size_t)li * a.B + b) * 3 * a.d + h * D;
-  f16* kring = kring_base + ((size_t)b * a.H + h) * a.max_len * D;
-  f16* vring = kring + (size_t)a.B * a.H * a.max_len * D;
+  f16 *kring, *vring;
+  ring_of<KV8>(a, kring_base, b, h, kring, vring);
+  const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
   // The cache rows of the first NPRE rounds (a round: four rows per wave) are requested before q, k and v are waited
   // for: the rows are known, and they travel while the producers' values do.  (More rounds, or a window that is
   // requested again as it is visited, do not fit the registers next to the weight tiles in flight.)
   constexpr int NPRE = 4;
-  f16x8 kp[NPRE], vp[NPRE];
+  typedef typename RingRow<KV8>::type Row;       // eight elements of a cache row as they are stored (decoded at the visit)
+  Row kp[NPRE], vp[NPRE];
   {
     const int grp = lane / LPP, d0 = (lane % LPP) * 8;
 #pragma unroll
     for (int it = 0; it < NPRE; ++it) {
       const int p = wv * PPW + grp + it * WPU * PPW;
-      kp[it] = f16x8{};
-      vp[it] = f16x8{};
+      kp[it] = Row{};
+      vp[it] = Row{};
       if (active && p < valid && p != pos) {
-        kp[it] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)p * D + d0);
-        vp[it] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)p * D + d0);
+        kp[it] = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(kring)) + ((size_t)p * D + d0) * (KV8 ? 1 : 2));
+        vp[it] = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(vring)) + ((size_t)p * D + d0) * (KV8 ? 1 : 2));
       }
     }
   }
@@ -877,9 +939,9 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
         const f16 rot = d_ < HALF ? -x1 : x1;
         y = x0 * cs[i] + rot * cs[HALF + i];
       }
+      if (which == 1) y = ring_put<KV8>(kring, (size_t)pos * D + d_, y, a.kv_scale);
+      if (which == 2) y = ring_put<KV8>(vring, (size_t)pos * D + d_, y, a.kv_scale);
       q_s[which * D + d_] = y;
-      if (which == 1) as_global(kring)[(size_t)pos * D + d_] = y;
-      if (which == 2) as_global(vring)[(size_t)pos * D + d_] = y;
     }
   }
   wg_sync();
@@ -898,6 +960,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
       for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[e], s);
 #pragma unroll
       for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      if (KV8) s *= kv_mul;
       f16 s16 = (f16)s;          // fp16 output of the q.K^T MatMul
       s16 = s16 * scale;         // fp16 multiply by fp16(1/sqrt(D))
       const float x = on ? (float)s16 : -INFINITY;
@@ -915,7 +978,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
       if (p0 < valid) {
         const int p = p0 + grp;
         const bool on = p < valid;
-        f16x8 k8 = kp[it], v8 = vp[it];
+        f16x8 k8 = RingRow<KV8>::values(kp[it]), v8 = RingRow<KV8>::values(vp[it]);
         if ((on ? p : valid - 1) == pos) {      // this step's row: taken from LDS, its global copy is being written
           k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
           v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
@@ -932,8 +995,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
         k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
         v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
       } else {
-        k8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(kring) + (size_t)pc * D + d0);
-        v8 = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(vring) + (size_t)pc * D + d0);
+        ring_rows<KV8>(kring, vring, (size_t)pc * D + d0, k8, v8);
       }
       visit(k8, v8, on);
     }
@@ -958,6 +1020,7 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
         Ls = __builtin_fmaf(sm_l[half * WPU + i], wgt, Ls);
         As = __builtin_fmaf(sm_acc[(half * WPU + i) * D + d_], wgt, As);
       }
+      if (KV8) As *= kv_mul;
       put(a.ctx + (size_t)li * 16 * a.d + grouped_at(b, h * D + d_), (f16)(As / Ls));      // the layout of decode_step_wide_kernel
     }
   }
@@ -1068,7 +1131,7 @@ __device__ __forceinline__ bool select_and_advance(const DsArgs& a, float* lds, 
 // TPW_D / TPW_F: K tiles per wave for K = hidden / ffn; U_F: gate/up row-blocks per workgroup;
 // MAXB: largest batch the instance serves.  Hidden row-blocks (q/k/v, o_proj, down) are at most
 // one per workgroup.
-template <int TPW_D, int TPW_F, int U_F, int MAXB>
+template <int TPW_D, int TPW_F, int U_F, int MAXB, bool KV8 = false>
 __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   constexpr int NS_D = (MAXB * TPW_D * DS_WAVES * 16 + DS_THREADS - 1) / DS_THREADS;
   constexpr int NS_F = (MAXB * TPW_F * DS_WAVES * 16 + DS_THREADS - 1) / DS_THREADS;
@@ -1196,7 +1259,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
-      for (int u = wg; u < units; u += G) attention_unit(a, li, kring, u, step, att_lds, cs, w);
+      for (int u = wg; u < units; u += G) attention_unit<false, KV8>(a, li, kring, u, step, att_lds, cs, w);
       if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
@@ -1547,7 +1610,7 @@ __device__ __forceinline__ f16 wide_unit(const u32x4 (&S)[NSLOT], const float* s
   return wide_finish<NRB, EPI>(out, ostride, res, u, N, M, rb, xsum, scl);
 }
 
-template <int TPW_D, int TPW_F, int U_F>
+template <int TPW_D, int TPW_F, int U_F, bool KV8 = false>
 __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   if (*a.keep_going == 0) return;
@@ -1691,9 +1754,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
       if (a.nsplit == 1) {
-        for (int u = wg; u < units; u += 2 * G) attention_two(a, li, kring, u, u + G < units ? u + G : -1, step, att_lds, cs, w);
+        for (int u = wg; u < units; u += 2 * G) attention_two<KV8>(a, li, kring, u, u + G < units ? u + G : -1, step, att_lds, cs, w);
       } else {
-        for (int u = wg; u < units; u += G) attention_unit<true>(a, li, kring, u, step, att_lds, cs, w);
+        for (int u = wg; u < units; u += G) attention_unit<true, KV8>(a, li, kring, u, step, att_lds, cs, w);
       }
       // the head outputs are stored by waves 0, 1 and (second unit of attention_two) 8, 9
       announce(phase_rows(4 * li + 1), a.flag_words, wg, wave < 2 || wave == 8 || wave == 9);
@@ -1916,15 +1979,21 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 
 struct Variant {
   int tpw_d, tpw_f, u_f, minb, maxb;
+  bool kv8;              // FP8 (F143) KV rings
   void (*kern)(DsArgs);
   bool ready;
 };
 Variant g_variants[] = {
-    {1, 1, 1, 1, 4, decode_step_kernel<1, 1, 1, 4>, false},        // small test shapes
-    {2, 6, 3, 1, 1, decode_step_kernel<2, 6, 3, 1>, false},        // 7B: hidden 4096, ffn 11008, batch 1
-    {2, 6, 3, 2, 4, decode_step_kernel<2, 6, 3, 4>, false},        // 7B, batch 2..4
-    {1, 1, 1, 5, 16, decode_step_wide_kernel<1, 1, 1>, false},     // small test shapes, batch 5..16
-    {2, 6, 3, 5, 16, decode_step_wide_kernel<2, 6, 3>, false},     // 7B, batch 5..16
+    {1, 1, 1, 1, 4, false, decode_step_kernel<1, 1, 1, 4>, false},        // small test shapes
+    {2, 6, 3, 1, 1, false, decode_step_kernel<2, 6, 3, 1>, false},        // 7B: hidden 4096, ffn 11008, batch 1
+    {2, 6, 3, 2, 4, false, decode_step_kernel<2, 6, 3, 4>, false},        // 7B, batch 2..4
+    {1, 1, 1, 5, 16, false, decode_step_wide_kernel<1, 1, 1>, false},     // small test shapes, batch 5..16
+    {2, 6, 3, 5, 16, false, decode_step_wide_kernel<2, 6, 3>, false},     // 7B, batch 5..16
+    {1, 1, 1, 1, 4, true, decode_step_kernel<1, 1, 1, 4, true>, false},   // the same with FP8 KV rings
+    {2, 6, 3, 1, 1, true, decode_step_kernel<2, 6, 3, 1, true>, false},
+    {2, 6, 3, 2, 4, true, decode_step_kernel<2, 6, 3, 4, true>, false},
+    {1, 1, 1, 5, 16, true, decode_step_wide_kernel<1, 1, 1, true>, false},
+    {2, 6, 3, 5, 16, true, decode_step_wide_kernel<2, 6, 3, true>, false},
 };
 
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -1979,7 +2048,8 @@ extern "C" size_t pta_decode_step_workspace_bytes(const pta_decode_model* model)
   return layout_for(model, cus).total;
 }
 
-static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace, pta_stream_t stream) {
+static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace, pta_stream_t stream,
+                              bool kv8 = false, int kv_scale = 0) {
   PTA_REQUIRE(mdl && st && workspace, "pta_llama_decode_step: null pointer");
   PTA_REQUIRE(mdl->layers && mdl->n_layer > 0 && mdl->embed && mdl->final_norm && mdl->head && mdl->inv_freq,
               "pta_llama_decode_step: incomplete model");
@@ -1998,7 +2068,7 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   const int u_f = (nb_f + cus - 1) / cus;
   Variant* var = nullptr;
   for (Variant& v : g_variants)
-    if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B >= v.minb && B <= v.maxb && !var) var = &v;
+    if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B >= v.minb && B <= v.maxb && v.kv8 == kv8 && !var) var = &v;
   if (!shape_ok(mdl) || nb_d > cus || !var) {
     pta_set_error("pta_llama_decode_step: supports batch <= %d, head size %d, hidden = heads * head size <= %d, ffn "
                   "and vocabulary sizes that are multiples of 8, and the (hidden, ffn) of the 7B model or small test "
@@ -2031,6 +2101,7 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.flag_words = (int)flag_words_for(cus);
   a.best = (uint32_t*)(ws + lay.best);
   a.nsplit = splits_for(cus, B, H);
+  a.kv_scale = kv_scale;
   const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
   size_t region0 = wide ? 0 : (size_t)B * xstride * 2;
@@ -2062,6 +2133,12 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
 extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
                                      pta_stream_t stream) {
   return decode_step_launch(mdl, st, workspace, stream);
+}
+
+extern "C" int pta_llama_decode_step_f8(const pta_decode_model* mdl, const pta_decode_state* st, int kv_scale, void* workspace,
+                                        pta_stream_t stream) {
+  PTA_REQUIRE(kv_scale >= -16 && kv_scale <= 16, "pta_llama_decode_step_f8: kv_scale %d outside [-16, 16]", kv_scale);
+  return decode_step_launch(mdl, st, workspace, stream, true, kv_scale);
 }
 
 // ------------------------------------------------------------------------------------------ the same step without a workspace argument

@@ -453,9 +453,27 @@ def compile_graph(graph, anchors, batches_per_step=1, allow_fused=True, strict=F
             # the executor is checked against the graph with fp16 caches first, then switched
             plain = fused.FusedDecoder(dataclasses.replace(spec, fp8_cache=False), weights)
             _validate_greedy_up_to_a_tie(plain, prog, facts, steps, passes, "the fused executor")
-            del plain
             decoder.capture()
             kind = f"fused:{family}"
+            if persistent and hasattr(decoder, "enable_persistent"):
+                # the persistent step likewise: checked with fp16 caches, used with FP8 ones
+                try:
+                    plain.enable_persistent()
+                    plain.capture()
+                    _validate_greedy_up_to_a_tie(plain, prog, facts, steps, passes, "the persistent decode step")
+                    decoder.enable_persistent()
+                    decoder.capture()
+                    kind += ":persistent"
+                except NotImplementedError as e:
+                    prog.persistent_reason = str(e)
+                except (ValueError, RuntimeError) as e:
+                    if strict:
+                        raise
+                    log.warning("the persistent decode step is not used: %s", e)
+                    prog.persistent_reason = str(e)
+                    decoder.persistent = None
+                    decoder.capture()
+            del plain
         else:
             # validation: identical ids over a few iterations (up to a near tie), eager and replayed
             _validate_greedy_up_to_a_tie(decoder, prog, facts, steps, passes, "the fused executor")

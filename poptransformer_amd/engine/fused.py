@@ -297,8 +297,6 @@ class FusedDecoder(LayerOps):
         s, w = self.spec, self.w
         if s.topk != 1:
             raise NotImplementedError("the persistent decode step selects greedily (topk = 1)")
-        if s.fp8_cache:
-            raise NotImplementedError("the persistent decode step keeps its KV cache in fp16")
         if s.family != "llama2" or s.n_kv_head != s.n_head:
             raise NotImplementedError("the persistent decode step covers Llama-2 blocks with as many KV heads as heads")
         lins = [lw for b in w.blocks for lw in b.qkv + [b.out] + b.mlp_in + [b.mlp_out]]
@@ -318,7 +316,7 @@ class FusedDecoder(LayerOps):
                      keep_going=self.keep_going, next_ids=self.next_ids, logits=self.logits)
         self.persistent = K.DecodeStep(layers, w.embed, w.final_norm[0], w.head.w.tiled, w.inv_freq, s.batch, s.d_model,
                                        s.n_head, s.head_dim, w.blocks[0].mlp_out.K, s.vocab, s.max_len, s.eps, s.pad_id,
-                                       s.eos_id, s.early_stop, state)
+                                       s.eos_id, s.early_stop, state, kv_scale=self.kv_scale)
         return self
 
     def step_fn(self):

@@ -599,8 +599,9 @@ class DecodeStep:
     raises NotImplementedError for shapes the kernel does not cover."""
 
     def __init__(self, layers, embed, final_norm, head, inv_freq, batch, hidden, n_head, head_dim, ffn, vocab, max_len,
-                 eps, pad_id, eos_id, early_stop, state):
+                 eps, pad_id, eos_id, early_stop, state, kv_scale=None):
         lib = _lib.load()
+        self.kv_scale = kv_scale            # not None: the layers' KV rings hold F143 bytes (pta_llama_decode_step_f8)
         dev = embed.device
         arr = (_lib.DecodeLayer * len(layers))()
         for dst, src in zip(arr, layers):
@@ -619,12 +620,18 @@ class DecodeStep:
         self.state = _lib.DecodeState(**{k: v.data_ptr() for k, v in state.items()})
 
     def launch(self):
+        if self.kv_scale is not None:
+            check(_lib.load().pta_llama_decode_step_f8(ctypes.byref(self.model), ctypes.byref(self.state), int(self.kv_scale),
+                                                       _p(self.workspace), _stream()))
+            return
         check(_lib.load().pta_llama_decode_step(ctypes.byref(self.model), ctypes.byref(self.state), _p(self.workspace),
                                                 _stream()))
 
     def launch_static(self, clear_failure=False):
         """The same iteration through the entry point that allocates nothing: its workspace is the array built
         into the library, not `self.workspace` (pta_llama_decode_step_static)."""
+        if self.kv_scale is not None:
+            raise NotImplementedError("the entry point without a workspace keeps fp16 KV rings")
         check(_lib.load().pta_llama_decode_step_static(ctypes.byref(self.model), ctypes.byref(self.state),
                                                        1 if clear_failure else 0, _stream()))
 

@@ -22,7 +22,7 @@ class Session:
         #   persistent    one launch per loop iteration where the model allows it (INT4 Llama 2, batch <= 16); that
         #                 kernel occupies every compute unit while it runs: nothing else may run on the device beside it
         #   prompt_passes take the prompt's positions in passes of up to 1024 rows instead of one per iteration
-        #   fp8_cache     KV caches hold F143 bytes, as the KVCache op does with fp8 = true
+        #   fp8_cache     KV caches hold F143 bytes, as the KVCache op does with fp8 = true (per operator and persistent)
         self.allow_fused = kwargs.get("allow_fused", True)
         self.executor_options = {k: kwargs[k] for k in ("strict", "persistent", "prompt_passes", "fp8_cache") if k in kwargs}
         self.enable_pipeline = REGISTRY.get("enable_pipeline")

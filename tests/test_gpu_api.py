@@ -102,8 +102,7 @@ def test_llama2_int4_batch_6_through_the_operator_api():
 
 def test_llama2_session_options_choose_the_executor():
     """persistent = False keeps one launch per operator; fp8_cache = True makes the KV caches F143 bytes (the
-    KVCache op with fp8 = true), which the persistent step does not cover: per-operator executor, tokens equal to
-    the oracle's with an FP8 cache."""
+    KVCache op with fp8 = true), on the persistent step too: tokens equal to the oracle's with an FP8 cache."""
     from poptransformer_amd.models.llama2 import LLAMA2DecModel
     B, L, steps, pad, eos = 2, 32, 20, 0, 2
     sd = OM.make_llama2_state_dict(LLAMA, seed=21, int4=True)
@@ -112,7 +111,8 @@ def test_llama2_session_options_choose_the_executor():
     session, model = _session(LLAMA2DecModel, "int4", B, kw, True, persistent=False, strict=True)
     assert session.executor_kind == "fused:llama2" and session.session.executor.decoder.persistent is None
     session, model = _session(LLAMA2DecModel, "int4", B, kw, True, fp8_cache=True, strict=True)
-    assert session.executor_kind == "fused:llama2" and session.session.executor.decoder.spec.fp8_cache
+    assert session.executor_kind == "fused:llama2:persistent" and session.session.executor.decoder.spec.fp8_cache
+    assert session.session.executor.decoder.persistent.kv_scale == 1
     probe, ref_c, ref_s, cols = _robust_reference(lambda: OM.Llama2Oracle(sd, LLAMA, L, B, fp8_cache=True), ids, L, steps, pad, eos)
     session.run(model.build_input_dict(input_ids=[list(r[r != pad]) for r in probe]))
     got = session.anchor_arrays["Loop:0"]

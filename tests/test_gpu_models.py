@@ -286,5 +286,4 @@ def test_llama2_fp8_kv_cache_matches_oracle(B):
     reference = dec.container.cpu().numpy().copy()
     _prompt_then_loop(dec, ids, steps)
     assert np.array_equal(dec.container.cpu().numpy(), reference)
-    with pytest.raises(NotImplementedError):
-        dec.enable_persistent()
+

@@ -10,10 +10,10 @@ from tests.test_gpu_models import LLAMA_TINY, _prompt, _compare
 pytestmark = pytest.mark.gpu
 
 
-def _decoders(B, L, pad, eos, seed, early_stop=False):
+def _decoders(B, L, pad, eos, seed, early_stop=False, fp8_cache=False):
     from poptransformer_amd.engine import fused, loader
     sd = OM.make_llama2_state_dict(LLAMA_TINY, seed=seed, int4=True)
-    spec = loader.llama2_spec(LLAMA_TINY, L, B, pad, eos)
+    spec = loader.llama2_spec(LLAMA_TINY, L, B, pad, eos, fp8_cache=fp8_cache)
     spec.early_stop = early_stop
     w = loader.llama2_weights(sd, LLAMA_TINY)
     return sd, fused.FusedDecoder(spec, w), fused.FusedDecoder(spec, w).enable_persistent()
@@ -29,6 +29,45 @@ def test_persistent_step_matches_oracle(B):
     ids = _prompt(np.random.default_rng(7), B, L, 8, LLAMA_TINY["vocab_size"], pad)
     _compare(dec, oracle, ids, L, steps, pad, eos)
     assert not dec.persistent.failed()
+
+
+@pytest.mark.parametrize("B", [1, 3, 6, 16])
+def test_persistent_step_with_fp8_kv_cache(B):
+    """KV rings of F143 bytes (pta_llama_decode_step_f8).  Up to 4 sequences against the oracle (KVCache with
+    fp8 = true): greedy ids identical over the first 32 steps, logits within 3e-2 (measured up to 1.8e-2: this kernel's
+    INT4 projections agree with the oracle's to the last fp16 bit or differ in it, and where such a k or v element
+    lies at an FP8 rounding boundary its byte - three mantissa bits - comes out one step away; the per-operator path,
+    whose projections round as the oracle's do, is held to 1e-2 in test_llama2_fp8_kv_cache_matches_oracle).  Every
+    batch size step by step against the per-operator path of the same cache format, fed the same tokens: logits
+    within 3e-2 of their largest magnitude, ids equal wherever the reference's best two candidates are further
+    apart than that; after 40 steps at least 99 % of the first layer's ring bytes are equal (measured 99.5 %) and at
+    least 85 % of every later layer's (their inputs already differ by what those bytes changed: measured 92-94 %),
+    and nothing is written past the steps taken."""
+    L, steps, pad, eos = 48, 32, 0, 2
+    print("case: persistent step with FP8 KV cache, batch", B, flush=True)
+    sd, ref, dec = _decoders(B, L, pad, eos, seed=1, fp8_cache=True)
+    ids = _prompt(np.random.default_rng(7), B, L, 12, LLAMA_TINY["vocab_size"], pad)
+    if B <= 4:
+        _compare(dec, OM.Llama2Oracle(sd, LLAMA_TINY, L, B, fp8_cache=True), ids, L, steps, pad, eos, tol=3e-2)
+    ref.reset(ids)
+    dec.reset(ids)
+    for it in range(40):
+        ref.step_fn()
+        dec.step_fn()
+        torch.cuda.synchronize()
+        a = ref.logits.float().cpu().numpy()
+        b = dec.logits.float().cpu().numpy()
+        scale, tol = np.abs(a).max(), 3e-2
+        assert np.abs(a - b).max() <= tol * scale, f"logits differ at step {it}"
+        top2 = np.sort(a, axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 2 * tol * scale
+        assert np.array_equal(ref.next_ids.cpu().numpy()[clear], dec.next_ids.cpu().numpy()[clear]), f"ids differ at step {it}"
+        dec.container.copy_(ref.container)          # after a near tie: follow the reference's choice
+    assert not dec.persistent.failed()
+    for li, (ra, rb) in enumerate(zip(ref.rings, dec.rings)):
+        a, b = ra[:, :40].cpu().numpy(), rb[:, :40].cpu().numpy()
+        assert a.dtype == np.uint8 and (a == b).mean() >= (0.99 if li == 0 else 0.85), f"layer {li}"
+        assert torch.equal(ra[:, 41:], rb[:, 41:])          # nothing written past the steps taken
 
 
 @pytest.mark.parametrize("B", [1, 4, 7, 16])
