@@ -483,13 +483,12 @@ static int attn_splits(int B, int Hq, int max_len) {
 // ------------------------------------------------------------------------------------------
 constexpr int PA_THREADS = 256;
 constexpr int PA_KSTRIDE = 128 + 8;      // halves per staged K row
-constexpr int PA_VSTRIDE = 32 + 4;       // halves per staged row of V^T (18 dwords: eight rows lie 16 banks apart)
+constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
 
-// V^T in LDS: feature d, cache row p (of the 32 staged) in dword ((p / 2) + 4 * (d / 32)) % 16 of row d, half p % 2.
-// A thread stages two consecutive cache rows of eight features and stores dwords (both rows of one feature): with
-// the row stride of 18 dwords and the rotation by feature group, the 64 stores of a wave fall into 64 banks; pairs
-// of dwords stay together for the 8-byte reads.
-__device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + ((((p >> 1) + 4 * (d >> 5)) & 15) << 1) + (p & 1); }
+// V^T in LDS: feature d, cache row p (of the 32 staged) at d * PA_VSTRIDE + (((p / 2) ^ (2 * (d / 16))) * 2 + p % 2.
+// Exchanging the dwords of a row by its feature group spreads the 2-byte stores of the transposition (which go
+// down the features, 8 * PA_VSTRIDE halves apart) over the banks; pairs of dwords stay together for the 8-byte reads.
+__device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + ((((p >> 1) ^ ((d >> 4) << 1))) << 1) + (p & 1); }
 
 // PA_RG: row groups of 16 per wave (a workgroup takes 4 * PA_RG * 16 rows of the pass).  Two where that still gives every
 // compute unit two workgroups or more (a wave's dependent chains - MFMA, maximum, exponentials, MFMA - need company
@@ -534,32 +533,31 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
     for (int jd = 0; jd < 8; ++jd) o[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // cache rows p .. p + 31: 512 vectors of 16 bytes each of K and V, two per thread (K: rows t / 16 and 16 + t / 16,
-  // V: rows 2 (t / 16) and the next); they are requested one step ahead, so that their way from memory runs beside
-  // the step's arithmetic
+  // cache rows p .. p + 31: 512 vectors of 16 bytes each of K and V, two per thread; they are requested one step
+  // ahead, so that their way from memory runs beside the step's arithmetic
   f16x8 kv[2], vv[2];
   auto request = [&](int p) {
-    const int col = ((int)threadIdx.x & 15) * 8;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int krow = ((int)threadIdx.x >> 4) + i * 16, vrow = ((int)threadIdx.x >> 4) * 2 + i;
+      const int c = (int)threadIdx.x + i * PA_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
       kv[i] = f16x8{}; vv[i] = f16x8{};
-      if (p + krow < wg_valid) kv[i] = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p + krow) * D + col);
-      if (p + vrow < wg_valid) vv[i] = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p + vrow) * D + col);
+      if (p + row < wg_valid) {
+        kv[i] = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p + row) * D + col);
+        vv[i] = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p + row) * D + col);
+      }
     }
   };
   request(0);
   for (int p0 = 0; p0 < wg_valid; p0 += 32) {
     __syncthreads();
-    {
-      const int col = ((int)threadIdx.x & 15) * 8, rp = (int)threadIdx.x >> 4;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) *reinterpret_cast<f16x8*>(ks + (rp + i * 16) * PA_KSTRIDE + col) = kv[i];
+    for (int i = 0; i < 2; ++i) {
+      const int c = (int)threadIdx.x + i * PA_THREADS;
+      const int row = c >> 4, col = (c & 15) * 8;
+      *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv[i];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const f16x2 two = {vv[0][e], vv[1][e]};
-        *reinterpret_cast<f16x2*>(vt + pa_vt_at(col + e, 2 * rp)) = two;
-      }
+      for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[i][e];
     }
     if (p0 + 32 < wg_valid) request(p0 + 32);
     __syncthreads();
