@@ -117,7 +117,9 @@ struct GemmArgs {
   float* part;
   size_t part_bytes;
   int ksplit;          // 0 or 1: no split
+  int prefer_stream;   // host side: up to 16 rows go to gemv_stream_kernel wherever it fits
 };
+static inline int device_compute_units();
 constexpr int GEMM_MAX_KSPLIT = 4;
 constexpr int GEMM_MAX_ROWS = 4096;
 
@@ -665,6 +667,10 @@ static int launch_gemv_wide(const GemmArgs& a, int total_nb, hipStream_t s, cons
 
 // blocks per workgroup: the launch's share per compute unit, capped by what the registers of a wave
 // (weight tiles in flight) and the LDS reduction buffer (8 KiB-groups of partial sums) hold
+// the longest chain of channel blocks a compute unit multiplies under launch_gemv_wide_for (M <= 16)
+template <class Fmt, bool PAIR>
+static int wide_block_times(int total_nb, int per_cu);
+
 template <class Fmt, int MT, bool PAIR, bool NORM = false>
 static int launch_gemv_wide_for(const GemmArgs& a, int total_nb, int per_cu, hipStream_t s, const char* name) {
   constexpr int NACC = PAIR ? 2 : 1;
@@ -674,6 +680,228 @@ static int launch_gemv_wide_for(const GemmArgs& a, int total_nb, int per_cu, hip
   if (per_cu <= 1 || cap == 1) return launch_gemv_wide<Fmt, MT, 1, PAIR, NORM>(a, total_nb, s, name);
   if (per_cu == 2 || cap == 2) return launch_gemv_wide<Fmt, MT, cap >= 2 ? 2 : 1, PAIR, NORM>(a, total_nb, s, name);
   return launch_gemv_wide<Fmt, MT, cap >= 3 ? 3 : 1, PAIR, NORM>(a, total_nb, s, name);
+}
+
+template <class Fmt, bool PAIR>
+static int wide_block_times(int total_nb, int per_cu) {
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int cap_regs = Fmt::kVec * NACC <= 4 ? 3 : 2;
+  constexpr int cap_lds = 8 / NACC;
+  constexpr int cap = cap_regs < cap_lds ? cap_regs : cap_lds;
+  const int nb = per_cu < cap ? per_cu : cap;
+  const int cus = device_compute_units();
+  const int wgs = (total_nb + nb - 1) / nb;
+  return (wgs + cus - 1) / cus * nb;
+}
+
+// ------------------------------------------------------------------------------------------
+// Variant for up to 16 rows, one shared X, K <= 4096 and several channel blocks per compute unit: one workgroup
+// of 8 waves per compute unit walks a contiguous range of the launch's 16-channel blocks.  Wave w takes the
+// feature tiles w, w + 8, ... of every block, U at a time (a step; a block is up to 4 / U steps long).  The
+// weights of the next D - 1 steps are on their way while those of the current one are multiplied, across block
+// boundaries as well, so the stream does not pause for a reduction or for a change of workgroups; the partial
+// sums of a block meet in LDS (two buffers in turn, one barrier per block) and 256 threads finish its 16 x 16
+// outputs while the others go on.  The activation fragments of a wave's tiles are the same for every block
+// and stay in registers (x[p]: those of a block's step p).
+// ------------------------------------------------------------------------------------------
+constexpr int STREAM_WAVES = 8;
+constexpr int STREAM_TILES = 4;          // feature tiles of a block per wave, at most: K <= 8 * 4 * 128
+
+template <class Fmt, int U, int D, bool PAIR>
+__global__ __launch_bounds__(STREAM_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void gemv_stream_kernel(GemmArgs a, int total_nb) {
+  constexpr int XP = STREAM_TILES / U;     // steps of a block, at most
+  static_assert(D % XP == 0, "a step's place in the ring of weight sets tells its place in the block");
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int KV = Fmt::kVec;
+  __shared__ float red[2][STREAM_WAVES][NACC][256];
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int K = a.K, KT = a.KT;
+  const int G = gridDim.x;
+  const int b0 = (int)((long)total_nb * blockIdx.x / G), b1 = (int)((long)total_nb * (blockIdx.x + 1) / G);
+  // steps per block: 1, 2 or 4 (a divisor of the ring's length; a step past the end of K multiplies zeros)
+  const int spb = KT <= STREAM_WAVES * U ? 1 : KT <= 2 * STREAM_WAVES * U ? 2 : XP;
+  const int steps = (b1 - b0) * spb;
+  if (steps == 0) return;
+
+  struct Set {
+    u32x4 w[U][NACC][KV];
+    typename Fmt::Scale sc[NACC];
+    uint16_t e[4];      // epilogue operands of the output this thread finishes: the matrix's bias, then bias, mul, residual
+  };
+  Set ring[D];
+  typename Fmt::Scale sc[NACC];
+  f32x4 acc[NACC];
+#pragma unroll
+  for (int g = 0; g < NACC; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto matrix_of = [&](int blk) {
+    int m_ = 0;
+    if (!PAIR) {
+#pragma unroll
+      for (int i = 1; i < 4; ++i)
+        if (i < a.count && blk >= a.mat[i].nb_begin) m_ = i;
+    }
+    return m_;
+  };
+
+  // The requesting side runs D - 1 steps ahead of the multiplying side.  Every step issues the same loads whatever
+  // the data (a wait for one set of weights then counts the loads issued after it): they go through a buffer
+  // descriptor of the block's matrix, and a tile past the end of K, or a step past the end of the workgroup's
+  // range, is given an offset beyond the descriptor's range - it reads as zero and touches no memory.
+  const uint32_t blk_bytes = (uint32_t)KT * (KV * 1024);
+  int fb = b0, fs = 0;
+  auto fetch = [&](Set& st, bool live) {
+    const int m_ = matrix_of(fb);
+    const int nb = fb - a.mat[m_].nb_begin;
+#pragma unroll
+    for (int g = 0; g < NACC; ++g) {
+      const GemmMat& m = a.mat[PAIR ? g : m_];
+      const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<void*>(m.tiled), 0, (int)((uint32_t)((m.N + 15) / 16) * blk_bytes), 0x00020000);
+      st.sc[g] = Fmt::load_scale(m.scale, a.x_scale, nb * 16 + (lane & 15), m.N);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kt = (fs * U + u) * STREAM_WAVES + wave;
+        const int voff = live && kt < KT ? lane * 16 : -1;
+#pragma unroll
+        for (int v = 0; v < KV; ++v)
+          st.w[u][g][v] = __builtin_amdgcn_raw_buffer_load_b128(wr, voff, (int)((uint32_t)nb * blk_bytes + (uint32_t)(kt * KV + v) * 1024), 2);
+      }
+    }
+    if constexpr (!PAIR) {
+      // The operands of the epilogue travel with the weights of the block's last step: a load issued when the block
+      // is finished would wait for every set of weights requested before it.  Absent operands have an empty range.
+      const GemmMat& mat = a.mat[m_];
+      const int nn = threadIdx.x & 15, m = threadIdx.x >> 4, n = nb * 16 + nn;
+      const bool mine = live && fs == spb - 1 && threadIdx.x < 256 && m < a.M && n < mat.N;
+      const f16* ptr[4] = {mat.bias, a.epi.bias, a.epi.mul, a.epi.residual};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<f16*>(ptr[i]), 0, ptr[i] ? (i < 2 ? mat.N : a.M * mat.N) * 2 : 0, 0x00020000);
+        st.e[i] = __builtin_amdgcn_raw_buffer_load_b16(r, mine ? (i < 2 ? n : m * mat.N + n) * 2 : -1, 0, 0);
+      }
+    }
+    if (++fs == spb) { fs = 0; ++fb; }
+  };
+
+  // B operands: row lane % 16 of X (clamped: padding rows compute values that are never stored), features
+  // (lane / 16) * 8 + 0..7 of every 32; x[p] holds them for the tiles of a block's step p (of its only step, when
+  // a block is one step long).  Requested before the first weights: loads return in the order of their issue, and
+  // the first products need these and one set of weights only.
+  f16x8 x[XP][U][4];
+  {
+    int mrow = lane & 15;
+    mrow = mrow < a.M ? mrow : a.M - 1;
+    const f16* xrow = a.X + (size_t)mrow * K + (lane >> 4) * 8;
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kt = ((p % spb) * U + u) * STREAM_WAVES + wave;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int k = kt * 128 + j * 32;
+          const f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+          x[p][u][j] = kt < KT && k + (lane >> 4) * 8 < K ? *reinterpret_cast<const f16x8*>(xrow + k) : z;
+        }
+      }
+  }
+
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i) fetch(ring[i], i < steps);
+
+  int cb = b0, cs = 0, par = 0;
+  auto multiply = [&](Set& st, const f16x8 (&xs)[U][4]) {
+    if (cs == 0) {
+#pragma unroll
+      for (int g = 0; g < NACC; ++g) sc[g] = st.sc[g];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < NACC; ++g)
+          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Fmt::a_operand(st.w[u][g], j, sc[g]), xs[u][j], acc[g], 0, 0, 0);
+    if (++cs < spb) return;
+    // the block is complete: lane l holds channels (l/16)*4 + r, r = 0..3, for activation row l%16
+#pragma unroll
+    for (int g = 0; g < NACC; ++g)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        red[par][wave][g][r * 64 + lane] = acc[g][r];
+        acc[g][r] = 0.f;
+      }
+    __syncthreads();
+    if (threadIdx.x < 256) {
+      const int m_ = matrix_of(cb);
+      const GemmMat& mat = a.mat[PAIR ? 0 : m_];
+      const int nn = threadIdx.x & 15, m = threadIdx.x >> 4;
+      const int N = mat.N, n = (cb - a.mat[m_].nb_begin) * 16 + nn;
+      if (m < a.M && n < N) {
+        const int r = nn & 3, ln = (nn >> 2) * 16 + m;
+        float sum[NACC];
+#pragma unroll
+        for (int g = 0; g < NACC; ++g) {
+          float t = 0.f;
+#pragma unroll
+          for (int w = 0; w < STREAM_WAVES; ++w) t += red[par][w][g][r * 64 + ln];
+          sum[g] = Fmt::finish(t, sc[g]);        // no format's finish uses the per-channel part of the scale
+        }
+        if (PAIR) {
+          mat.Y[(size_t)m * N + n] = swiglu_out(a.epi, (f16)sum[0], (f16)sum[1]);
+        } else {
+          // as apply_epilogue, with the operands that came with the weights
+          f16 y0 = (f16)sum[0];
+          if (mat.bias) y0 = y0 + bitcast<f16>(st.e[0]);
+          y0 = apply_act(mat.act, y0);
+          if (a.epi.bias) y0 = y0 + bitcast<f16>(st.e[1]);
+          y0 = apply_act(a.epi.act, y0);
+          if (a.epi.mul) y0 = y0 * bitcast<f16>(st.e[2]);
+          if (a.epi.residual) y0 = y0 + bitcast<f16>(st.e[3]);
+          if (a.epi.post_scale != 0.0f) y0 = y0 * (f16)a.epi.post_scale;
+          if (a.epi.out_fp8_scale) y0 = f8_grid_value(y0, a.epi.out_fp8_scale[0], a.epi.out_fp8_format);
+          mat.Y[(size_t)m * N + n] = y0;
+        }
+      }
+    }
+    par ^= 1;
+    cs = 0;
+    ++cb;
+  };
+
+  int t = 0;
+  for (; t + D <= steps; t += D) {
+#pragma unroll
+    for (int i = 0; i < D; ++i) {
+      fetch(ring[(i + D - 1) % D], t + i + D - 1 < steps);
+      multiply(ring[i], x[i % XP]);
+    }
+  }
+  // fewer than D steps are left and their weights are on their way
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i)
+    if (t + i < steps) multiply(ring[i], x[i % XP]);
+}
+
+// the shapes the streaming kernel takes
+static inline bool stream_fits(const GemmArgs& a) {
+  if (a.M > 16 || a.KT < 8 || a.KT > STREAM_WAVES * STREAM_TILES || a.epi.norm != PTA_NORM_NONE) return false;
+  for (int i = 0; i < a.count; ++i)
+    if (a.mat[i].X) return false;
+  return true;
+}
+
+template <class Fmt, bool PAIR>
+static int launch_gemv_stream(const GemmArgs& a, int total_nb, int cus, hipStream_t s, const char* name) {
+  // tiles per step, and four steps in the ring: 96 KiB on their way per compute unit, a ring of 64 registers
+  constexpr int V = Fmt::kVec * (PAIR ? 2 : 1);
+  constexpr int U = V >= 4 ? 1 : V >= 2 ? 2 : 4, D = 4;
+  hipLaunchKernelGGL((gemv_stream_kernel<Fmt, U, D, PAIR>), dim3(total_nb < cus ? total_nb : cus), dim3(STREAM_WAVES * 64), 0, s, a,
+                     total_nb);
+  return PTA_OK;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1646,7 +1874,17 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
     }
     if (shared_x && a.KT >= 8) {
       int rc;
-      if (a.M <= 16 && a.epi.norm != PTA_NORM_NONE) rc = launch_gemv_wide_for<Fmt, 1, PAIR, true>(a, total_nb, per_cu, s, name);
+      bool streamed = false;
+      if constexpr (Fmt::kVec * (PAIR ? 2 : 1) <= 4) {
+        // gemv_stream_kernel where gemv_wide_kernel's rounds of workgroups come out longer than an even share of the
+        // blocks (856 blocks: 286 workgroups of 3 = two rounds = 6 block times, against 4), or on request
+        if (stream_fits(a) && total_nb >= device_compute_units() && (a.prefer_stream || wide_block_times<Fmt, PAIR>(total_nb, per_cu) > per_cu)) {
+          rc = launch_gemv_stream<Fmt, PAIR>(a, total_nb, device_compute_units(), s, name);
+          streamed = true;
+        }
+      }
+      if (streamed) {}
+      else if (a.M <= 16 && a.epi.norm != PTA_NORM_NONE) rc = launch_gemv_wide_for<Fmt, 1, PAIR, true>(a, total_nb, per_cu, s, name);
       else if (a.M <= 16) rc = launch_gemv_wide_for<Fmt, 1, PAIR>(a, total_nb, per_cu, s, name);
       else if (a.M <= 32) rc = launch_gemv_wide_for<Fmt, 2, PAIR>(a, total_nb, per_cu, s, name);
       else rc = launch_gemv_wide_for<Fmt, 4, PAIR>(a, total_nb, per_cu, s, name);

@@ -74,14 +74,17 @@ static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int c
   // Both operands F143: the FP8 matrix instruction.  fp16 grid values are turned into bytes by every workgroup that
   // reads them (about 60 vector instructions per 32-feature step), which pays only when the bytes feed several
   // products.  Measured at the ChatGLM2-6B shape, 8 rows, saturating activations (every step multiplied twice, 224
-  // and 16): the SwiGLU pair 31.2 against 32.5 us on the fp16 instruction with decoded weights; one channel block per
-  // workgroup (4096 x 4096) 16.2 against 11.5 us, q | kv and the lm_head slower as well.  So fp16 grid values take
-  // this path for the SwiGLU pair only; an uint8 left-hand side always comes here.
+  // and 16): the SwiGLU pair 31.2 against 32.5 us for gemv_wide_kernel on the fp16 instruction with decoded weights
+  // - and 25.0 us for gemv_stream_kernel, also with decoded weights, which therefore takes the pair wherever it
+  // fits; one channel block per workgroup (4096 x 4096) 16.2 against 11.5 us, q | kv and the lm_head slower as well.
+  // So fp16 grid values come here for a SwiGLU pair outside that kernel's shapes only; an uint8 left-hand side always.
   const bool several = swiglu != 0;
-  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || (fp8_native_enabled() && several))) {
+  const bool stream_pair = several && !x_bytes && stream_fits(a) && nb >= device_compute_units();
+  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || (fp8_native_enabled() && several && !stream_pair))) {
     if (x_bytes) return swiglu ? dispatch_gemv_f8n<true, true>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, true>(a, nb, s, "pta_linear");
     return swiglu ? dispatch_gemv_f8n<true, false>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, false>(a, nb, s, "pta_linear");
   }
+  a.prefer_stream = stream_pair && (kind == PTA_W_F143 || kind == PTA_W_F152);
   PTA_REQUIRE(!x_bytes, "pta_linear: an uint8 left-hand side needs F143 weights, M <= 16 and K >= 1024");
   switch (kind) {
     case PTA_W_INT4: return run_linear<FmtW4>(a, nb, swiglu, s, "pta_linear");
