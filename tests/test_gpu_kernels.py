@@ -173,6 +173,54 @@ def test_w4a16_gemm_many_rows_multi_swiglu_epilogue(K):
     assert rel_err(got, ref) <= 1e-2
 
 
+@pytest.mark.parametrize("M", [5, 8, 16])
+@pytest.mark.parametrize("Kdim,N", [(4096, 13696), (1160, 13690), (1024, 13696), (2176, 13696)])
+def test_w4a16_gemv_uneven_rounds_of_workgroups(K, M, Kdim, N):
+    """Up to 16 rows and a number of channel blocks (856) that the workgroups of the 16-wave kernel cover in uneven
+    rounds: the kernel in which one workgroup per compute unit walks its share of the blocks.  1160 and 2176 features =
+    a ragged last tile / a block of one, two and four steps; 13690 channels = a ragged last block; bias and a residual
+    that aliases the output."""
+    x, packed, scale = _w4_case(M + Kdim + N, M, Kdim, N)
+    rng = np.random.default_rng(M * N)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    w = K.W4Weight(dev(packed), dev(scale))
+    plain = O.w4a16_matmul(x, packed, scale)
+    assert rel_err(host(K.w4a16_gemm(dev(x), w)), plain) <= 1e-2
+    y = dev(res.copy())
+    K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=y, out=y)
+    assert rel_err(host(y), ((plain + bias).astype(np.float16) + res).astype(np.float16)) <= 1e-2
+
+
+def test_gemv_uneven_rounds_exact_integers_multi_swiglu_f16(K):
+    """The same kernel: integers small enough for exact sums (any wrong tile, step or lane shows), three matrices of
+    different widths with their biases in one launch, the SwiGLU pair, and fp16 weights."""
+    rng = np.random.default_rng(21)
+    M, Kdim, N = 16, 1024, 13696
+    x = rng.integers(-1, 2, size=(M, Kdim)).astype(np.float16)
+    q = rng.integers(-8, 8, size=(N, Kdim))
+    w = K.W4Weight(dev(O.pack_int4(q)), dev(np.ones(N, np.float16)))
+    assert np.array_equal(host(K.w4a16_gemm(dev(x), w)).astype(np.int64), x.astype(np.int64) @ q.T.astype(np.int64))
+    M, Kdim = 7, 4096
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    mats = [(rng.integers(-128, 128, size=(n, Kdim // 2), dtype=np.int8), rng.uniform(0.005, 0.02, size=(n,)).astype(np.float16))
+            for n in (4096, 9000, 520)]
+    ws = [K.W4Weight(dev(p), dev(s)) for p, s in mats]
+    biases = [rng.standard_normal(p.shape[0]).astype(np.float16) for p, _ in mats]
+    outs = [torch.empty((M, p.shape[0]), dtype=torch.float16, device="cuda") for p, _ in mats]
+    K.linear(dev(x), ws, outs, biases=[dev(b) for b in biases])
+    for (p, s), b, o in zip(mats, biases, outs):
+        assert rel_err(host(o), (O.w4a16_matmul(x, p, s) + b).astype(np.float16)) <= 1e-2
+    (pg, sg), (pu, su) = [(rng.integers(-128, 128, size=(N, Kdim // 2), dtype=np.int8),
+                           rng.uniform(0.005, 0.02, size=(N,)).astype(np.float16)) for _ in range(2)]
+    got = host(K.w4a16_gemm_swiglu(dev(x), K.W4Weight(dev(pg), dev(sg)), K.W4Weight(dev(pu), dev(su))))
+    assert rel_err(got, (O.w4a16_matmul(x, pu, su) * O.swish(O.w4a16_matmul(x, pg, sg))).astype(np.float16)) <= 1e-2
+    wf = (rng.standard_normal((Kdim, N)) * 0.05).astype(np.float16)
+    got = host(K.f16_gemm(dev(x), K.F16Weight(dev(np.ascontiguousarray(wf.T)))))
+    ref64 = x.astype(np.float64) @ wf.astype(np.float64)
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
+
+
 def test_w4a16_gemm_epilogue(K):
     x, packed, scale = _w4_case(11, 3, 512, 96)
     rng = np.random.default_rng(12)
