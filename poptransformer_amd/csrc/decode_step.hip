@@ -1400,14 +1400,20 @@ __device__ __forceinline__ bool await_row(const unsigned* rows, int row_words, i
 // fabric.  Nothing of a slot is in a cache before its arrival: the launch starts with an agent-scope acquire (no
 // line of the previous launch survives), no slot of this protocol is written with the filler, and every address is
 // written once per launch.  The slot is laid out for this read (grouped_at): a wave's 64 loads of a step are one
-// contiguous KiB.  Features beyond K and rows beyond M read as zero.
+// contiguous KiB.  Features beyond K (also: a tile beyond the last) and rows beyond M read as zero.
+// The four loads are issued whatever the lane, the row count or the tile: through a buffer descriptor, with an
+// offset beyond its range where the fragment does not exist (that reads zero and touches no memory).  With the
+// loads under a condition the compiler cannot count them, and a wait for an OLDER load - the fragments of the
+// current tile while those of the next are on their way - becomes a wait for all of them.
 __device__ __forceinline__ void load_xtile(const f16* X, int M, int K, int kt, XTile& t) {
   const int lane = lane_id();
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16*>(X), 0, ((K + 127) / 128) * (16 * 128 * 2), 0x00020000);
+  int no_row = (lane & 15) < M ? 0 : -1;      // rows beyond M are never written
+  asm volatile("" : "+v"(no_row));            // (kept a value: as a condition the compiler turns it into two copies of the loads under branches)
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    t.v[j] = f16x8{};
-    if ((lane & 15) < M && kt * 128 + j * 32 + (lane >> 4) * 8 < K)      // rows beyond M are never written
-      t.v[j] = *reinterpret_cast<const DS_GLOBAL f16x8*>(as_global(X) + ((size_t)(kt * 4 + j) * 64 + lane) * 8);
+    const int no_k = kt * 128 + j * 32 + (lane >> 4) * 8 < K ? 0 : -1;
+    t.v[j] = bitcast<f16x8>(__builtin_amdgcn_raw_buffer_load_b128(xr, ((kt * 4 + j) * 64 + lane) * 16 | no_row | no_k, 0, 0));
   }
 }
 
@@ -1730,7 +1736,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 #pragma unroll
       for (int i = 0; i < T; ++i) {
         xt[i] = XTile{};
-        if (wave + i * DS_WAVES < KT_D) load_xtile(x_in, M, a.d, wave + i * DS_WAVES, xt[i]);
+        load_xtile(x_in, M, a.d, wave + i * DS_WAVES, xt[i]);
       }
       if (wave == 0) keep_scales<3>(sv, scl);
     }
@@ -1771,7 +1777,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 #pragma unroll
       for (int i = 0; i < T; ++i) {
         xt[i] = XTile{};
-        if (wave + i * DS_WAVES < KT_D) load_xtile(a.ctx + (size_t)li * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
+        load_xtile(a.ctx + (size_t)li * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
       }
       if (wave == 0) keep_scales<1>(sv, scl + DW_SCL);
     }
@@ -1800,7 +1806,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 #pragma unroll
       for (int i = 0; i < T; ++i) {
         xt[i] = XTile{};
-        if (wave + i * DS_WAVES < KT_D) load_xtile(x_mid, M, a.d, wave + i * DS_WAVES, xt[i]);
+        load_xtile(x_mid, M, a.d, wave + i * DS_WAVES, xt[i]);
       }
       if (wave == 0) {
 #pragma unroll
@@ -1841,9 +1847,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 0, T>(S, mm, wg, nb_d, KT_D); }
 #pragma unroll
       for (int i = 0; i < TPW_F; ++i) {
+        const XTile x1 = ahead;
+        if (i + 1 < TPW_F) load_xtile(actx, M, a.ffn, wave + (i + 1) * DS_WAVES, ahead);      // (a tile beyond the last: zeros)
         if (wave + i * DS_WAVES < KT_F) {
-          const XTile x1 = ahead;
-          if (i + 1 < TPW_F && wave + (i + 1) * DS_WAVES < KT_F) load_xtile(actx, M, a.ffn, wave + (i + 1) * DS_WAVES, ahead);
           const XTile one[1] = {x1};
           s1 += xtiles_rowsum<1>(one);
           wide_tile_product<1, TPW_F>(S, acc, S_D, i, x1);
@@ -1880,7 +1886,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
 #pragma unroll
     for (int i = 0; i < T; ++i) {
       xt[i] = XTile{};
-      if (wave + i * DS_WAVES < KT_D) load_xtile(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
+      load_xtile(a.xres + (size_t)(2 * a.n_layer) * xslot, M, a.d, wave + i * DS_WAVES, xt[i]);
     }
     wg_sync();
     alive = *lds_dead == 0;
