@@ -906,25 +906,24 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
   f16 *kring, *vring;
   ring_of<KV8>(a, kring_base, b, h, kring, vring);
   const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
-  // The cache rows of the first NPRE rounds (a round: four rows per wave) are requested before q, k and v are waited
-  // for: the rows are known, and they travel while the producers' values do.  (More rounds, or a window that is
-  // requested again as it is visited, do not fit the registers next to the weight tiles in flight.)
+  // A window of NPRE rounds of cache rows (a round: four rows per wave) travels ahead of the visits: the first NPRE
+  // rounds are requested before q, k and v are waited for - the rows are known, and they travel while the producers'
+  // values do - and every visit of a round requests the round NPRE later into the registers it frees.  Every
+  // request issues the same loads (a row past the end repeats the last one; this step's own row, whose ring copy is
+  // being written, is loaded like any other and replaced by its LDS copy at the visit), so the wait before a visit
+  // counts the requests issued after that round's and leaves them on their way.
   constexpr int NPRE = 4;
   typedef typename RingRow<KV8>::type Row;       // eight elements of a cache row as they are stored (decoded at the visit)
   Row kp[NPRE], vp[NPRE];
-  {
-    const int grp = lane / LPP, d0 = (lane % LPP) * 8;
+  const int att_grp = lane / LPP, att_d0 = (lane % LPP) * 8;
+  auto request = [&](Row& kr, Row& vr, int round) {
+    const int p = wv * PPW + att_grp + round * WPU * PPW;
+    const size_t at = ((size_t)(p < valid ? p : valid - 1) * D + att_d0) * (KV8 ? 1 : 2);
+    kr = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(kring)) + at);
+    vr = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(vring)) + at);
+  };
 #pragma unroll
-    for (int it = 0; it < NPRE; ++it) {
-      const int p = wv * PPW + grp + it * WPU * PPW;
-      kp[it] = Row{};
-      vp[it] = Row{};
-      if (active && p < valid && p != pos) {
-        kp[it] = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(kring)) + ((size_t)p * D + d0) * (KV8 ? 1 : 2));
-        vp[it] = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(vring)) + ((size_t)p * D + d0) * (KV8 ? 1 : 2));
-      }
-    }
-  }
+  for (int it = 0; it < NPRE; ++it) request(kp[it], vp[it], it);
   {
     const int t = thread_id() - half * WPU * 64;
     const int which = t / D, d_ = t % D;
@@ -972,32 +971,23 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
       for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
       m = mn;
     };
+    const int rounds = (valid + WPU * PPW - 1) / (WPU * PPW);
+    for (int r0 = 0; r0 < rounds; r0 += NPRE) {
 #pragma unroll
-    for (int it = 0; it < NPRE; ++it) {
-      const int p0 = wv * PPW + it * WPU * PPW;
-      if (p0 < valid) {
-        const int p = p0 + grp;
-        const bool on = p < valid;
-        f16x8 k8 = RingRow<KV8>::values(kp[it]), v8 = RingRow<KV8>::values(vp[it]);
-        if ((on ? p : valid - 1) == pos) {      // this step's row: taken from LDS, its global copy is being written
-          k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
-          v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
+      for (int it = 0; it < NPRE; ++it) {
+        const int p0 = wv * PPW + (r0 + it) * WPU * PPW;
+        if (p0 < valid) {
+          const int p = p0 + grp;
+          const bool on = p < valid;
+          f16x8 k8 = RingRow<KV8>::values(kp[it]), v8 = RingRow<KV8>::values(vp[it]);
+          if ((on ? p : valid - 1) == pos) {      // this step's row: taken from LDS, its global copy is being written
+            k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
+            v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
+          }
+          visit(k8, v8, on);
         }
-        visit(k8, v8, on);
+        request(kp[it], vp[it], r0 + it + NPRE);
       }
-    }
-    for (int p0 = wv * PPW + NPRE * WPU * PPW; p0 < valid; p0 += WPU * PPW) {
-      const int p = p0 + grp;
-      const bool on = p < valid;
-      const int pc = on ? p : valid - 1;
-      f16x8 k8, v8;
-      if (pc == pos) {
-        k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
-        v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
-      } else {
-        ring_rows<KV8>(kring, vring, (size_t)pc * D + d0, k8, v8);
-      }
-      visit(k8, v8, on);
     }
     merge_lanes(m, l, acc, 16);
     merge_lanes(m, l, acc, 32);
