@@ -70,6 +70,35 @@ def test_persistent_step_with_fp8_kv_cache(B):
         assert torch.equal(ra[:, 41:], rb[:, 41:])          # nothing written past the steps taken
 
 
+@pytest.mark.parametrize("B", [6, 16])
+def test_persistent_step_with_fp8_kv_cache_over_a_long_context(B):
+    """The FP8 rings up to a context of 200 rows, step by step against the per-operator path of the same cache
+    format, fed the same tokens (tolerances as in test_persistent_step_with_fp8_kv_cache): at 16 sequences the
+    attention visits its cache rows in rounds of 32 with a window of four rounds requested ahead, so from 128 rows
+    on every visit uses registers that an earlier round has been through."""
+    L, pad, eos = 200, 0, 2
+    print("case: persistent step with FP8 KV cache over a long context, batch", B, flush=True)
+    _, ref, dec = _decoders(B, L, pad, eos, seed=3, fp8_cache=True)
+    ids = _prompt(np.random.default_rng(13), B, L, 6, LLAMA_TINY["vocab_size"], pad)
+    ref.reset(ids)
+    dec.reset(ids)
+    for it in range(L - 2):
+        ref.step_fn()
+        dec.step_fn()
+        torch.cuda.synchronize()
+        a = ref.logits.float().cpu().numpy()
+        b = dec.logits.float().cpu().numpy()
+        scale, tol = np.abs(a).max(), 3e-2
+        assert np.abs(a - b).max() <= tol * scale, f"logits differ at step {it}"
+        top2 = np.sort(a, axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 2 * tol * scale
+        assert np.array_equal(ref.next_ids.cpu().numpy()[clear], dec.next_ids.cpu().numpy()[clear]), f"ids differ at step {it}"
+        dec.container.copy_(ref.container)          # after a near tie: follow the reference's choice
+    assert not dec.persistent.failed()
+    a, b = ref.rings[0].cpu().numpy(), dec.rings[0].cpu().numpy()
+    assert (a == b).mean() >= 0.99
+
+
 @pytest.mark.parametrize("B", [1, 4, 7, 16])
 def test_persistent_step_follows_the_per_operator_path(B):
     """Step by step over a long generation: logits agree to 2e-3 of their largest magnitude (the two
