@@ -792,16 +792,24 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    for (int p0 = c0 + wave * PPW; p0 < c1; p0 += DS_WAVES * PPW) {
+    // The rows of the next visit are requested before those of the current one are used (two sets of registers in
+    // turn).  Every request issues the same loads: a row past the end of the range repeats its last row, and this
+    // step's own row, whose ring copy is being written, is loaded like any other and replaced by its LDS copy at
+    // the visit - so the wait before a visit leaves the next request on its way.
+    typedef typename RingRow<KV8>::type Row;
+    auto request = [&](Row& kr, Row& vr, int p0) {
+      const int p = p0 + grp;
+      const size_t at = ((size_t)(p < c1 ? p : c1 - 1) * D + d0) * (KV8 ? 1 : 2);
+      kr = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(kring)) + at);
+      vr = *reinterpret_cast<const DS_GLOBAL Row*>(as_global(reinterpret_cast<const uint8_t*>(vring)) + at);
+    };
+    auto visit = [&](const Row& kr, const Row& vr, int p0) {
       const int p = p0 + grp;
       const bool on = p < c1;
-      const int pc = on ? p : c1 - 1;
-      f16x8 k8, v8;
-      if (pc == pos) {      // this step's row: taken from LDS, its global copy is being written
+      f16x8 k8 = RingRow<KV8>::values(kr), v8 = RingRow<KV8>::values(vr);
+      if ((on ? p : c1 - 1) == pos) {      // this step's row: taken from LDS, its global copy is being written
         k8 = *reinterpret_cast<const f16x8*>(k_s + d0);
         v8 = *reinterpret_cast<const f16x8*>(v_s + d0);
-      } else {
-        ring_rows<KV8>(kring, vring, (size_t)pc * D + d0, k8, v8);
       }
       float s = 0.f;
 #pragma unroll
@@ -819,6 +827,23 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(pe, (float)v8[e], acc[e] * corr);
       m = mn;
+    };
+    {
+      constexpr int VISIT = DS_WAVES * PPW;
+      Row ka, va, kb, vb;
+      int p0 = c0 + wave * PPW;
+      request(ka, va, p0);
+      if (c1 - c0 <= VISIT) {              // one visit (batch 1 up to 512 rows of context): nothing to request ahead
+        if (p0 < c1) visit(ka, va, p0);
+      } else {
+        for (; p0 < c1; p0 += 2 * VISIT) {
+          request(kb, vb, p0 + VISIT);
+          visit(ka, va, p0);
+          if (p0 + VISIT >= c1) break;
+          request(ka, va, p0 + 2 * VISIT);
+          visit(kb, vb, p0 + VISIT);
+        }
+      }
     }
     // the four row groups of a wave merge in registers, the sixteen waves in LDS
     merge_lanes(m, l, acc, 16);
