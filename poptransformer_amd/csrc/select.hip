@@ -15,7 +15,30 @@ __global__ __launch_bounds__(AM_THREADS) void argmax_kernel(const f16* __restric
   const f16* xr = x + (size_t)blockIdx.x * n;
   float best = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < n; i += AM_THREADS) {
+  // 16-byte vectors where the row allows them (a thread's loads of a row are independent: four at a time travel
+  // together), single elements for a row that does not start on a 16-byte boundary and for the tail
+  const int nvec = (reinterpret_cast<uintptr_t>(xr) & 15) == 0 ? n >> 3 : 0;
+  for (int c = threadIdx.x; c < nvec; c += 4 * AM_THREADS) {
+    f16x8 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int cu = c + u * AM_THREADS;
+      v[u] = *reinterpret_cast<const f16x8*>(xr + (size_t)(cu < nvec ? cu : c) * 8);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int cu = c + u * AM_THREADS;
+      if (cu < nvec) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float f = (float)v[u][e];
+          const int i = cu * 8 + e;
+          if (f > best || (f == best && i < bi)) { best = f; bi = i; }
+        }
+      }
+    }
+  }
+  for (int i = nvec * 8 + threadIdx.x; i < n; i += AM_THREADS) {
     const float v = (float)xr[i];
     if (v > best || (v == best && i < bi)) { best = v; bi = i; }
   }
