@@ -79,7 +79,7 @@ int pta_w4_tile(const int8_t* packed, void* tiled, int N, int K, pta_stream_t st
  * models/llama2/model.py:38-46); Y = Y * post_scale when post_scale != 0 (the halving of
  * models/rwkv/model.py:115-116).
  * workspace (optional): scratch of pta_linear_workspace_bytes(M, N) bytes, 16-byte aligned.  With it, a
- * single-weight launch of more than 32 rows whose channel count alone cannot fill the machine also
+ * single-weight launch of more than 16 rows whose channel count alone cannot fill the machine also
  * splits K across workgroups (fp32 partial sums in the workspace, summed by a second kernel that
  * applies the epilogue).  Calls sharing one workspace must not overlap.
  * Last of all, with out_fp8_scale: Y = pta_half_to_fp8_grid(Y) - the cast of the next FP8 Linear

@@ -1855,15 +1855,15 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
       const int cus = device_compute_units();
       const int wgs4 = total_nb / (PAIR ? 2 : 4), wgs8 = total_nb / (PAIR ? 1 : 2);
       int rc = 1;
-      // one matrix, more than 32 rows, too few channel blocks to fill the machine, scratch at hand: split K too
+      // one matrix, too few channel blocks to fill the machine, scratch at hand: split K too
       int nsl = wgs4 > 0 ? cus / wgs4 : 1;
       nsl = nsl > GEMM_MAX_KSPLIT ? GEMM_MAX_KSPLIT : nsl;
       while (nsl > 1 && a.KT < nsl * 8) --nsl;
-      if (!PAIR && a.count == 1 && a.M > 32 && a.part && nsl > 1 && tile_fits(a, 4, 4, false) &&
+      if (!PAIR && a.count == 1 && a.part && nsl > 1 && tile_fits(a, 4, 4, false) &&
           a.part_bytes >= (size_t)nsl * a.M * a.mat[0].N * sizeof(float)) {
         GemmArgs b = a;
         b.ksplit = nsl;
-        rc = launch_gemm_tile<Fmt, 4, 4, PAIR>(b, total_nb, s, name);
+        rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(b, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(b, total_nb, s, name);
       } else if (tile_fits(a, PAIR ? 2 : 4, 4, PAIR) && 2 * wgs4 >= cus) {
         rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(a, total_nb, s, name);
       } else if (a.M <= 32 && tile_fits(a, PAIR ? 1 : 2, 8, PAIR) && 2 * wgs8 >= cus) {

@@ -139,7 +139,8 @@ class LayerOps:
         self._fp8_buf = {k: buf(rows, k) for k in {d, ffn}}
         self._gate, self._up = buf(rows, ffn), buf(rows, ffn)
         self._on_grid = {}      # buffer address -> the FP8 grid (format, exponent) its values are on
-        self._lin_ws = None     # scratch that lets a many-row Linear with few output channels split K
+        # scratch that lets a Linear of more than 16 rows with few output channels (attention output, MLP down) split K
+        self._lin_ws = K.linear_workspace(rows, d, device) if rows > 16 else None
 
     def _norm(self, x, gb, out):
         if self.spec.norm == "rms":

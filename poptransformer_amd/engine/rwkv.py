@@ -98,6 +98,9 @@ class RWKVDecoder:
         self.st_max = [buf(B, d, dtype=f32) for _ in range(s.n_layer)]
         self.graph = None
         self._stream = torch.cuda.Stream()
+        # more than 16 rows: scratch that lets the two single-weight Linears of a layer (4096 channels: too few
+        # channel blocks to fill the machine) split K across workgroups
+        self._lin_ws = K.linear_workspace(B, d, device) if B > 16 else None
 
     @staticmethod
     def _group(xs, lws, outs, acts):
@@ -121,13 +124,14 @@ class RWKVDecoder:
                         [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
             K.rwkv_wkv(self.k, self.v, self.r, blk.time_decay, blk.time_first, self.st_num[i], self.st_den[i],
                        self.st_max[i], self.y)
-            K.linear(self.y, [blk.att_output.w], [x], residual=x)
+            K.linear(self.y, [blk.att_output.w], [x], residual=x, workspace=self._lin_ws)
             K.layer_norm_ce(x, blk.ln2[0], blk.ln2[1], s.eps, self.h)
             K.rwkv_mix(self.h, self.st_ffn[i], blk.ffn_mix, self.mix[:2])
             self._group(self.mix[:2], [blk.ffn_key, blk.ffn_receptance], [self.fk, self.fr],
                         [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
             halve = s.rescale_every > 0 and (i + 1) % s.rescale_every == 0
-            K.linear(self.fk, [blk.ffn_value.w], [x], mul=self.fr, residual=x, post_scale=0.5 if halve else 0.0)
+            K.linear(self.fk, [blk.ffn_value.w], [x], mul=self.fr, residual=x, post_scale=0.5 if halve else 0.0,
+                     workspace=self._lin_ws)
         K.layer_norm_ce(x, w.ln_out[0], w.ln_out[1], s.eps, self.h)
         K.linear(self.h, [w.head.w], [self.logits])
         self.select(self.logits, self.next_ids)

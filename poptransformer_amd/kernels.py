@@ -65,7 +65,7 @@ def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, po
 
 
 def linear_workspace(M, N, device):
-    """Scratch that lets a single-weight `linear` of more than 32 rows split K across workgroups."""
+    """Scratch that lets a single-weight `linear` of more than 16 rows split K across workgroups."""
     return torch.empty(_lib.load().pta_linear_workspace_bytes(M, N), dtype=torch.uint8, device=device)
 
 

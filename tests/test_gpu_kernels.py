@@ -114,10 +114,10 @@ def test_w4a16_gemm_many_rows_wide_outputs(K, M, Kdim, N):
     assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
 
 
-@pytest.mark.parametrize("M", [33, 64])
+@pytest.mark.parametrize("M", [17, 32, 33, 64])
 @pytest.mark.parametrize("Kdim,N", [(4096, 1024), (11008, 4096), (2872, 2048)])
 def test_w4a16_gemm_many_rows_few_outputs_split_k(K, M, Kdim, N):
-    """More than 32 rows and too few output channels to fill the machine: with a workspace the launch also
+    """More than 16 rows and too few output channels to fill the machine: with a workspace the launch also
     splits the features across workgroups (2872 features = 23 tiles, the last ragged: slices of unequal length)
     and a second kernel adds the slices and applies bias and residual.  Against the oracle, and against the
     launch without workspace (same sums in another order)."""
@@ -137,6 +137,15 @@ def test_w4a16_gemm_many_rows_few_outputs_split_k(K, M, Kdim, N):
     assert rel_err(got, plain) <= 2e-3
     small = torch.empty(64, dtype=torch.uint8, device="cuda")                      # too small: the one-kernel form runs
     assert rel_err(host(K.w4a16_gemm(dev(x), w, bias=dev(bias), residual=dev(res), workspace=small)), ref) <= 1e-2
+    # the gate and the halving of the RWKV channel mix (models/rwkv/ffn.py:58, model.py:115-116) behind the split
+    gate = rng.uniform(0, 1, (M, N)).astype(np.float16)
+    outs = []
+    for wsp in (ws, None):
+        y = dev(res.copy())
+        K.linear(dev(x), [w], [y], mul=dev(gate), residual=y, post_scale=0.5, workspace=wsp)
+        outs.append(host(y))
+    want = (((O.w4a16_matmul(x, packed, scale) * gate).astype(np.float16) + res).astype(np.float16) * np.float16(0.5)).astype(np.float16)
+    assert rel_err(outs[0], want) <= 1e-2 and rel_err(outs[0], outs[1]) <= 2e-3
 
 
 def test_w4a16_gemm_many_rows_exact_integers(K):
