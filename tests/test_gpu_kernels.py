@@ -872,6 +872,8 @@ def test_argmax(K, rows, n):
     rng = np.random.default_rng(rows + n)
     x = rng.standard_normal((rows, n)).astype(np.float16)
     x[0, [n // 3, n // 2]] = 9.0                       # a tie: the lower index wins
+    x[rows // 2, [n - 1, min(7, n - 1), min(8, n - 1)]] = 11.0      # ... across 16-byte vectors and threads, up to the last element
+    x[rows - 1, :] = 1.0                               # all equal: index 0 (a later row does not start on a 16-byte boundary when n is odd)
     got = host(K.argmax(dev(x)))
     _, ref = O.topk1(x, -1)
     assert np.array_equal(got, ref[:, 0])
