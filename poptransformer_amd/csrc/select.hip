@@ -81,36 +81,80 @@ __global__ __launch_bounds__(AM_THREADS) void topk_kernel(const f16* __restrict_
   __shared__ int pi;
   const f16* xr = x + (size_t)blockIdx.x * n;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float last_v = INFINITY;
-  int last_i = -1;
-  for (int j = 0; j < k; ++j) {
-    float best = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += AM_THREADS) {
-      const float v = (float)xr[i];
-      const bool after = v < last_v || (v == last_v && i > last_i);      // NaN compares false: never picked
-      if (after && (v > best || (v == best && i < bi))) { best = v; bi = i; }
+  // A row of up to 65536 elements that starts on a 16-byte boundary is read once: thread t keeps the 16-byte vectors
+  // t, t + 1024, ... in registers (NaN - never picked - past the end) and the k passes run over those.
+  constexpr int TK_VEC = 8;
+  const bool kept = (reinterpret_cast<uintptr_t>(xr) & 15) == 0 && (n & 7) == 0 && n <= TK_VEC * 8 * AM_THREADS;
+  f16x8 keep[TK_VEC];
+  if (kept) {
+    const f16 nan = bitcast<f16>((uint16_t)0x7E00u);
+#pragma unroll
+    for (int u = 0; u < TK_VEC; ++u) {
+      const int c = threadIdx.x + u * AM_THREADS;
+      keep[u] = f16x8{nan, nan, nan, nan, nan, nan, nan, nan};
+      if (c * 8 < n) keep[u] = *reinterpret_cast<const f16x8*>(xr + (size_t)c * 8);
     }
+  }
+  // A thread's best remaining element stays its best until that element is picked (it lost to every pick so far, so
+  // it comes after them in the order): only the thread whose element was picked looks through its elements again.
+  float last_v = INFINITY, best = -INFINITY;
+  int last_i = -1, bi = 0x7fffffff;
+  bool stale = true;
+  for (int j = 0; j < k; ++j) {
+    if (stale) {
+      best = -INFINITY;
+      bi = 0x7fffffff;
+      if (kept) {
+#pragma unroll
+        for (int u = 0; u < TK_VEC; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float v = (float)keep[u][e];
+            const int i = (threadIdx.x + u * AM_THREADS) * 8 + e;
+            const bool after = v < last_v || (v == last_v && i > last_i);      // NaN compares false: never picked
+            if (after && (v > best || (v == best && i < bi))) { best = v; bi = i; }
+          }
+      } else {
+        for (int i = threadIdx.x; i < n; i += AM_THREADS) {
+          const float v = (float)xr[i];
+          const bool after = v < last_v || (v == last_v && i > last_i);
+          if (after && (v > best || (v == best && i < bi))) { best = v; bi = i; }
+        }
+      }
+      stale = false;
+    }
+    float wb = best;
+    int wi = bi;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+      const float ov = __shfl_xor(wb, o, 64);
+      const int oi = __shfl_xor(wi, o, 64);
+      if (ov > wb || (ov == wb && oi < wi)) { wb = ov; wi = oi; }
     }
-    if (lane == 0) { sv[wave] = best; si[wave] = bi; }
+    if (lane == 0) { sv[wave] = wb; si[wave] = wi; }
     __syncthreads();
-    if (threadIdx.x == 0) {
-      for (int w = 1; w < AM_THREADS / 64; ++w)
-        if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
-      // fewer than k comparable values (NaN rows, or -inf repeated): index 0 with value -inf
-      idx[(size_t)blockIdx.x * k + j] = bi == 0x7fffffff ? 0 : bi;
-      if (val) val[(size_t)blockIdx.x * k + j] = (f16)best;
-      pv = best;
-      pi = bi;
+    if (wave == 0) {      // the sixteen waves' candidates meet in the first wave's lanes
+      static_assert(AM_THREADS / 64 == 16, "one lane per wave, four exchange steps");
+      wb = sv[lane & 15];
+      wi = si[lane & 15];
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(wb, o, 64);
+        const int oi = __shfl_xor(wi, o, 64);
+        if (ov > wb || (ov == wb && oi < wi)) { wb = ov; wi = oi; }
+      }
+      if (lane == 0) {
+        // fewer than k comparable values (NaN rows, or -inf repeated): index 0 with value -inf
+        idx[(size_t)blockIdx.x * k + j] = wi == 0x7fffffff ? 0 : wi;
+        if (val) val[(size_t)blockIdx.x * k + j] = (f16)wb;
+        pv = wb;
+        pi = wi;
+      }
     }
     __syncthreads();
     last_v = pv;
     last_i = pi;
+    stale = bi == last_i;          // the picked element was this thread's (or nothing is left to pick: every thread looks again, and finds nothing)
     __syncthreads();
   }
 }
