@@ -463,6 +463,28 @@ def test_fp8_gemm_many_rows_wide_outputs(K):
     assert rel_err(got, O.fp8_matmul(x, w8, [-1], [-1], "F143", "F143")) <= 1e-2
 
 
+@pytest.mark.parametrize("M", [24, 64])
+def test_fp8_gemm_few_outputs_split_k(K, M):
+    """FP8 weights, more than 16 rows and 4096 output channels (the attention output / MLP down of the FP8 models at
+    17..64 rows): with a workspace the features are split across workgroups; against the oracle and against the
+    launch without the split (the same sums in another order), bias and a residual that aliases the output."""
+    rng = np.random.default_rng(23 + M)
+    Kdim, N = 4096, 4096
+    x = rng.standard_normal((M, Kdim)).astype(np.float16)
+    w8 = O.f8_encode((rng.standard_normal((Kdim, N)) * 0.02).astype(np.float32), "F143", -1)
+    fw = K.F8Weight(dev(w8), dev(np.array([-1], np.int32)), "F143", kn=True)
+    bias = rng.standard_normal(N).astype(np.float16)
+    res = rng.standard_normal((M, N)).astype(np.float16)
+    ws = K.linear_workspace(M, N, "cuda")
+    ws.fill_(0xFF)
+    y = dev(res.copy())
+    K.linear(dev(x), [fw], [y], bias=dev(bias), residual=y, workspace=ws)
+    plain = dev(res.copy())
+    K.linear(dev(x), [fw], [plain], bias=dev(bias), residual=plain)
+    ref = ((O.fp8_matmul(x, w8, [-1], [-1], "F143", "F143") + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(host(y), ref) <= 1e-2 and rel_err(host(y), host(plain)) <= 2e-3
+
+
 def test_fp8_gemm_exact_on_representable_values(K):
     """Small integers and powers of two are exact in F143, in fp16 and in the fp32 sums."""
     rng = np.random.default_rng(32)
