@@ -429,8 +429,9 @@ def main():
         torch.cuda.synchronize()
         kernel_s = e0.elapsed_time(e1) * 1e-3 / reps
         kernel_bytes = float(np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(t_first, t_first + reps)]))
-        kernel_name = ("decode_step_kernel<2, 6, 3, %d>" % (1 if B == 1 else 4) if B <= 4 else
-                       "decode_step_wide_kernel<2, 6, 3>") + " (whole decode step)"
+        kv8 = "true" if args.fp8_cache else "false"      # the kernels' last template argument: FP8 KV rings
+        kernel_name = ("decode_step_kernel<2, 6, 3, %d, %s>" % (1 if B == 1 else 4, kv8) if B <= 4 else
+                       "decode_step_wide_kernel<2, 6, 3, %s>" % kv8) + " (whole decode step)"
     else:
         # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
         # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
