@@ -889,8 +889,11 @@ void gemv_stream_kernel(GemmArgs a, int total_nb) {
 // the shapes the streaming kernel takes
 static inline bool stream_fits(const GemmArgs& a) {
   if (a.M > 16 || a.KT < 8 || a.KT > STREAM_WAVES * STREAM_TILES || a.epi.norm != PTA_NORM_NONE) return false;
-  for (int i = 0; i < a.count; ++i)
+  for (int i = 0; i < a.count; ++i) {
     if (a.mat[i].X) return false;
+    // a matrix's tiles sit behind one buffer descriptor (32-bit range and offsets; four vectors per tile at most)
+    if ((size_t)((a.mat[i].N + 15) / 16) * (size_t)a.KT * 4096 > 0x7fffffffu) return false;
+  }
   return true;
 }
 
