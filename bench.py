@@ -279,7 +279,7 @@ def prompt_workload(args):
     passes = max(1, min(args.steps, (MAX_LEN - 2) // R))
     n = passes * R
     weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
-    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2), weights)
+    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
     rng = np.random.Generator(np.random.PCG64(1234))
     ids = np.zeros((B, MAX_LEN), np.int32)
     ids[:, :n + 1] = rng.integers(3, cfg["vocab_size"], size=(B, n + 1))
@@ -296,7 +296,8 @@ def prompt_workload(args):
     d, f, nl = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
     per_layer = (4 * d * d + 3 * d * f) // 2 + 2 * (4 * d + 2 * f + d) + 2 * 2 * d
     # per pass: every block's weights once, the pass's K/V rows written, the cache read once per sequence
-    kv = float(np.mean([B * nl * 2 * d * 2 * (p * R + R) + B * nl * 2 * d * 2 * R for p in range(passes)]))
+    kvb = 1 if args.fp8_cache else 2          # bytes per cache element
+    kv = float(np.mean([B * nl * 2 * d * kvb * (p * R + R) + B * nl * 2 * d * kvb * R for p in range(passes)]))
     pass_bytes = nl * per_layer + kv + 2 * B * R * d
     flops = 2.0 * B * R * nl * (4 * d * d + 3 * d * f)
     print(json.dumps({
@@ -304,7 +305,7 @@ def prompt_workload(args):
         "ms_per_step": dt / passes * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"Llama2-7B-shape INT4 prompt of {n} positions per sequence in {passes} passes of {R} positions, "
-                               f"batch {B}, KV cache length {MAX_LEN}", "batch": B, "rows_per_pass": B * R,
+                               f"batch {B}, {'F143' if args.fp8_cache else 'fp16'} KV cache of {MAX_LEN}", "batch": B, "rows_per_pass": B * R,
                    "executor": "operators"},
         "step_algorithmic_bytes": pass_bytes,
         "step_roofline_frac": pass_bytes / (dt / passes) / (HBM_PEAK_GBS * 1e9),

@@ -493,9 +493,13 @@ __device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + 
 // PA_RG: row groups of 16 per wave (a workgroup takes 4 * PA_RG * 16 rows of the pass).  Two where that still gives every
 // compute unit two workgroups or more (a wave's dependent chains - MFMA, maximum, exponentials, MFMA - need company
 // on their SIMD), else one.
-template <int PA_RG>
+// KV8: the rings hold F143 bytes of value * 2^-kv_scale (as in attn_partial_kernel): a thread loads eight bytes where
+// it loads eight halves of an fp16 ring, decodes them on their way into LDS, and the power of two goes to the fp32
+// scores before they are rounded and to the result.
+template <int PA_RG, bool KV8 = false>
 __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnArgs a) {
   constexpr int D = 128;
+  const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
   constexpr int PA_ROWS = 4 * PA_RG * 16;
   __shared__ __align__(16) f16 ks[32 * PA_KSTRIDE];
   __shared__ __align__(16) f16 vt[D * PA_VSTRIDE];
@@ -523,6 +527,8 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   const int wg_valid = valid_of(last_of_wg);
   const f16* kbase = a.kring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
   const f16* vbase = a.vring + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
+  const uint8_t* kbase8 = reinterpret_cast<const uint8_t*>(a.kring) + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
+  const uint8_t* vbase8 = reinterpret_cast<const uint8_t*>(a.vring) + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
 
   float run_m[PA_RG], run_l[PA_RG];
   f32x4 o[PA_RG][8];
@@ -536,15 +542,22 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   // cache rows p .. p + 31: 512 vectors of 16 bytes each of K and V, two per thread; they are requested one step
   // ahead, so that their way from memory runs beside the step's arithmetic
   f16x8 kv[2], vv[2];
+  u32x2 kq[2], vq[2];       // KV8: the bytes as stored
   auto request = [&](int p) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int c = (int)threadIdx.x + i * PA_THREADS;
       const int row = c >> 4, col = (c & 15) * 8;
       kv[i] = f16x8{}; vv[i] = f16x8{};
+      kq[i] = u32x2{0, 0}; vq[i] = u32x2{0, 0};      // (the byte 0 is the value 0)
       if (p + row < wg_valid) {
-        kv[i] = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p + row) * D + col);
-        vv[i] = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p + row) * D + col);
+        if constexpr (KV8) {
+          kq[i] = *reinterpret_cast<const u32x2*>(kbase8 + (size_t)(p + row) * D + col);
+          vq[i] = *reinterpret_cast<const u32x2*>(vbase8 + (size_t)(p + row) * D + col);
+        } else {
+          kv[i] = *reinterpret_cast<const f16x8*>(kbase + (size_t)(p + row) * D + col);
+          vv[i] = *reinterpret_cast<const f16x8*>(vbase + (size_t)(p + row) * D + col);
+        }
       }
     }
   };
@@ -555,6 +568,10 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
     for (int i = 0; i < 2; ++i) {
       const int c = (int)threadIdx.x + i * PA_THREADS;
       const int row = c >> 4, col = (c & 15) * 8;
+      if constexpr (KV8) {
+        kv[i] = f143_decode8(kq[i][0], kq[i][1]);
+        vv[i] = f143_decode8(vq[i][0], vq[i][1]);
+      }
       *reinterpret_cast<f16x8*>(ks + row * PA_KSTRIDE + col) = kv[i];
 #pragma unroll
       for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[i][e];
@@ -583,7 +600,7 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
       for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          f16 s16 = (f16)sc[g][hh][r];                // fp16 output of the q.K^T MatMul
+          f16 s16 = (f16)(KV8 ? sc[g][hh][r] * kv_mul : sc[g][hh][r]);      // fp16 output of the q.K^T MatMul
           if (a.use_scale) s16 = s16 * a.scale;       // fp16 multiply by fp16(1/sqrt(D))
           const int pos = p0 + hh * 16 + (lane >> 4) * 4 + r;
           x[hh * 4 + r] = pos < my_valid[g] ? (float)s16 : -INFINITY;
@@ -636,7 +653,8 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
       if (row >= a.rows) continue;
 #pragma unroll
       for (int jd = 0; jd < 8; ++jd)
-        a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] = attn_result(a, (f16)(o[g][jd][r] / lr[r]));
+        a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] =
+            attn_result(a, (f16)((KV8 ? o[g][jd][r] * kv_mul : o[g][jd][r]) / lr[r]));
     }
   }
 }
@@ -670,7 +688,7 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
   PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
   PTA_REQUIRE(rows > 0 && rows <= max_len, "%s: rows = %d must lie in [1, max_len = %d]", name, rows, max_len);
-  PTA_REQUIRE((rows >= 16 && D == 128 && !kv8) || (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
+  PTA_REQUIRE((rows >= 16 && D == 128) || (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
   PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "%s: q and kv_ring must be 16-byte aligned", name);
   PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
   const size_t ring_elems = (size_t)B * Hkv * max_len * D;
@@ -681,13 +699,18 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B * rows, Hq, max_len); a.rows = rows;
   a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
-  if (rows >= 16 && D == 128 && !kv8) {        // many rows: on the matrix unit, no splits, no workspace
+  if (rows >= 16 && D == 128) {        // many rows: on the matrix unit, no splits, no workspace
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-    if ((long)((rows + 127) / 128) * Hq * B >= 2L * cus)
-      hipLaunchKernelGGL(prompt_attention_mfma_kernel<2>, dim3((rows + 127) / 128, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
-    else
-      hipLaunchKernelGGL(prompt_attention_mfma_kernel<1>, dim3((rows + 63) / 64, Hq, B), dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    const bool two = (long)((rows + 127) / 128) * Hq * B >= 2L * cus;
+    const dim3 grid(two ? (rows + 127) / 128 : (rows + 63) / 64, Hq, B);
+    if (kv8) {
+      if (two) hipLaunchKernelGGL((prompt_attention_mfma_kernel<2, true>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+      else hipLaunchKernelGGL((prompt_attention_mfma_kernel<1, true>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    } else {
+      if (two) hipLaunchKernelGGL((prompt_attention_mfma_kernel<2, false>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+      else hipLaunchKernelGGL((prompt_attention_mfma_kernel<1, false>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    }
     PTA_CHECK_LAUNCH(name);
     return PTA_OK;
   }

@@ -815,6 +815,20 @@ def test_fp8_kv_cache_attention(K, family, B, Hq, Hkv, D, max_len, steps):
     got = host(out_rows).reshape(B, rows, Hq * D)
     for r in range(rows):
         assert rel_err(got[:, r], refs[r]) <= 1e-2, f"row {r}"
+    more = min(40, steps - rows)
+    if max_len >= rows + more and more >= 16:
+        # and the next `more` (head size 128: on the matrix unit, the cache rows staged 32 at a time, the last step ragged)
+        stack2 = lambda xs: dev(np.stack(xs[rows:rows + more], axis=1).reshape(B * more, -1))
+        q2 = torch.empty((B * more, Hq, D), dtype=torch.float16, device="cuda")
+        out2 = torch.empty((B * more, Hq * D), dtype=torch.float16, device="cuda")
+        ws2 = K.decode_attention_workspace(B * more, Hq, D, max_len, "cuda")
+        step.fill_(rows)
+        K.prompt_rope_append(stack2(qs), stack2(ks), stack2(vs), q2, rings[2], step, inv, B, more, Hq, Hkv, D, max_len, rope, kv_scale=1)
+        K.prompt_attention(q2, rings[2], step, ws2, out2, B, more, Hq, Hkv, D, max_len, family != "gpt2", kv_scale=1)
+        got2 = host(out2).reshape(B, more, Hq * D)
+        for r in range(more):
+            assert rel_err(got2[:, r], refs[rows + r]) <= 1e-2, f"row {rows + r}"
+        assert torch.equal(rings[2][:, :rows + more], rings[0][:, :rows + more]) or steps > max_len      # the loop's ring has wrapped by then
     with pytest.raises(ValueError):
         K.prompt_attention(q_rows, rings[2].view(torch.float16), step, ws_rows, out_rows, B, rows, Hq, Hkv, D, max_len, True, kv_scale=1)
 
