@@ -465,24 +465,23 @@ static int attn_splits(int B, int Hq, int max_len) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Attention of many rows at once (the prompt passes) on the matrix unit, head size 128, fp16 cache.
+// Attention of many rows at once (the prompt passes) on the matrix unit, head size D = 64 or 128, fp16 or F143 cache.
 // One workgroup of four waves per (sequence, query head, 64 or 128 rows of the pass); wave w owns one or two
 // groups of 16 rows.  The cache rows go through LDS 32 at a time, K as it lies, V transposed; per step a wave computes,
 // for each of its row groups,
-//   S^T = K Q^T     (two 16 x 16 tiles, 4 MFMAs each: lane l then holds the scores of query row l % 16 for
+//   S^T = K Q^T     (two 16 x 16 tiles, D / 32 MFMAs each: lane l then holds the scores of query row l % 16 for
 //                    cache rows (l / 16) * 4 + 0..3 of each tile - which IS the layout of an A operand whose
 //                    k index runs over those eight cache rows),
 //   the roundings of the reference on the scores (fp16 MatMul output, fp16 multiply by 1/sqrt(D)), the online
 //   softmax in fp32 per query row (partners: lanes l ^ 16, l ^ 32), probabilities rounded to fp16 (the
 //   reference's softmax output is fp16),
-//   O += P V        (eight 16 x 16 tiles over the head size, B operands from the transposed V rows);
+//   O += P V        (D / 16 tiles of 16 x 16 over the head size, B operands from the transposed V rows);
 // every K and V operand read from LDS serves all row groups of the wave.
 // Row r of the pass sits at position step + r and attends to cache rows [0, min(step + r + 1, max_len)), as in
 // attn_partial_kernel.  Outputs differ from that kernel in the last bits (another summation order, fp16
 // probabilities); both are held to 1e-2 against the oracle.
 // ------------------------------------------------------------------------------------------
 constexpr int PA_THREADS = 256;
-constexpr int PA_KSTRIDE = 128 + 8;      // halves per staged K row
 constexpr int PA_VSTRIDE = 32 + 8;       // halves per staged row of V^T
 
 // V^T in LDS: feature d, cache row p (of the 32 staged) at d * PA_VSTRIDE + (((p / 2) ^ (2 * (d / 16))) * 2 + p % 2.
@@ -496,9 +495,11 @@ __device__ __forceinline__ int pa_vt_at(int d, int p) { return d * PA_VSTRIDE + 
 // KV8: the rings hold F143 bytes of value * 2^-kv_scale (as in attn_partial_kernel): a thread loads eight bytes where
 // it loads eight halves of an fp16 ring, decodes them on their way into LDS, and the power of two goes to the fp32
 // scores before they are rounded and to the result.
-template <int PA_RG, bool KV8 = false>
+template <int D, int PA_RG, bool KV8 = false>
 __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnArgs a) {
-  constexpr int D = 128;
+  static_assert(D == 64 || D == 128, "head size");
+  constexpr int PA_KSTRIDE = D + 8;        // halves per staged K row
+  constexpr int NV = D / 64;               // 16-byte vectors of K (and of V) per thread and step: 32 rows of D / 8
   const float kv_mul = KV8 ? ldexpf(1.0f, a.kv_scale) : 1.0f;
   constexpr int PA_ROWS = 4 * PA_RG * 16;
   __shared__ __align__(16) f16 ks[32 * PA_KSTRIDE];
@@ -509,14 +510,14 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   const int step0 = *a.step;
   const int r0 = (int)blockIdx.x * PA_ROWS + wave * (PA_RG * 16);          // first row of this wave within the pass
   auto valid_of = [&](int row) { const int v = step0 + row + 1; return row < a.rows ? (v < a.max_len ? v : a.max_len) : 0; };
-  f16x8 qf[PA_RG][4];
+  f16x8 qf[PA_RG][D / 32];
   int my_valid[PA_RG];
 #pragma unroll
   for (int g = 0; g < PA_RG; ++g) {
     const int qrow = r0 + g * 16 + (lane & 15);
     my_valid[g] = valid_of(qrow);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
+    for (int m = 0; m < D / 32; ++m) {
       qf[g][m] = f16x8{};
       if (qrow < a.rows) qf[g][m] = *reinterpret_cast<const f16x8*>(a.q + (((size_t)b * a.rows + qrow) * a.Hq + h) * D + m * 32 + (lane >> 4) * 8);
     }
@@ -531,23 +532,23 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   const uint8_t* vbase8 = reinterpret_cast<const uint8_t*>(a.vring) + ((size_t)b * a.Hkv + kvh) * a.max_len * D;
 
   float run_m[PA_RG], run_l[PA_RG];
-  f32x4 o[PA_RG][8];
+  f32x4 o[PA_RG][D / 16];
 #pragma unroll
   for (int g = 0; g < PA_RG; ++g) {
     run_m[g] = -INFINITY; run_l[g] = 0.f;
 #pragma unroll
-    for (int jd = 0; jd < 8; ++jd) o[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int jd = 0; jd < D / 16; ++jd) o[g][jd] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // cache rows p .. p + 31: 512 vectors of 16 bytes each of K and V, two per thread; they are requested one step
+  // cache rows p .. p + 31: 32 * D / 8 vectors of 16 bytes each of K and V, NV per thread; they are requested one step
   // ahead, so that their way from memory runs beside the step's arithmetic
-  f16x8 kv[2], vv[2];
-  u32x2 kq[2], vq[2];       // KV8: the bytes as stored
+  f16x8 kv[NV], vv[NV];
+  u32x2 kq[NV], vq[NV];       // KV8: the bytes as stored
   auto request = [&](int p) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NV; ++i) {
       const int c = (int)threadIdx.x + i * PA_THREADS;
-      const int row = c >> 4, col = (c & 15) * 8;
+      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
       kv[i] = f16x8{}; vv[i] = f16x8{};
       kq[i] = u32x2{0, 0}; vq[i] = u32x2{0, 0};      // (the byte 0 is the value 0)
       if (p + row < wg_valid) {
@@ -565,9 +566,9 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   for (int p0 = 0; p0 < wg_valid; p0 += 32) {
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NV; ++i) {
       const int c = (int)threadIdx.x + i * PA_THREADS;
-      const int row = c >> 4, col = (c & 15) * 8;
+      const int row = c / (D / 8), col = (c % (D / 8)) * 8;
       if constexpr (KV8) {
         kv[i] = f143_decode8(kq[i][0], kq[i][1]);
         vv[i] = f143_decode8(vq[i][0], vq[i][1]);
@@ -585,7 +586,7 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
 #pragma unroll
       for (int g = 0; g < PA_RG; ++g) sc[g][hh] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
+      for (int m = 0; m < D / 32; ++m) {
         const f16x8 kf = *reinterpret_cast<const f16x8*>(ks + (hh * 16 + (lane & 15)) * PA_KSTRIDE + m * 32 + (lane >> 4) * 8);
 #pragma unroll
         for (int g = 0; g < PA_RG; ++g) sc[g][hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[g][m], sc[g][hh], 0, 0, 0);
@@ -628,7 +629,7 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
       for (int r = 0; r < 4; ++r) cr[g][r] = __shfl(corr, (lane >> 4) * 4 + r, 64);
     }
 #pragma unroll
-    for (int jd = 0; jd < 8; ++jd) {
+    for (int jd = 0; jd < D / 16; ++jd) {
       // cache rows (lane / 16) * 4 + 0..3 and 16 + the same of feature jd * 16 + lane % 16
       const int d = jd * 16 + (lane & 15);
       const f16x4 v0 = *reinterpret_cast<const f16x4*>(vt + pa_vt_at(d, (lane >> 4) * 4));
@@ -652,7 +653,7 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
       const int row = r0 + g * 16 + (lane >> 4) * 4 + r;
       if (row >= a.rows) continue;
 #pragma unroll
-      for (int jd = 0; jd < 8; ++jd)
+      for (int jd = 0; jd < D / 16; ++jd)
         a.out[(((size_t)b * a.rows + row) * a.Hq + h) * D + jd * 16 + (lane & 15)] =
             attn_result(a, (f16)((KV8 ? o[g][jd][r] * kv_mul : o[g][jd][r]) / lr[r]));
     }
@@ -688,7 +689,7 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   PTA_REQUIRE(D == 64 || D == 128, "%s: head size must be 64 or 128, got %d", name, D);
   PTA_REQUIRE(max_len > 0, "%s: max_len = %d", name, max_len);
   PTA_REQUIRE(rows > 0 && rows <= max_len, "%s: rows = %d must lie in [1, max_len = %d]", name, rows, max_len);
-  PTA_REQUIRE((rows >= 16 && D == 128) || (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
+  PTA_REQUIRE(rows >= 16 || (long)B * rows * Hq <= 65535, "%s: rows = %d (B*rows*Hq must stay below 65536)", name, rows);
   PTA_REQUIRE(pta_aligned(q, 16) && pta_aligned(kv_ring, 16), "%s: q and kv_ring must be 16-byte aligned", name);
   PTA_REQUIRE(!kv8 || (kv_scale >= -16 && kv_scale <= 16), "%s: kv_scale %d outside [-16, 16]", name, kv_scale);
   const size_t ring_elems = (size_t)B * Hkv * max_len * D;
@@ -699,17 +700,18 @@ static int attention_rows(const char* name, const pta_half* q, const void* kv_ri
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.max_len = max_len; a.nsplit = attn_splits(B * rows, Hq, max_len); a.rows = rows;
   a.kv_scale = kv_scale;
   a.use_scale = use_scale; a.scale = (f16)(1.0 / sqrt((double)D));
-  if (rows >= 16 && D == 128) {        // many rows: on the matrix unit, no splits, no workspace
+  if (rows >= 16) {        // many rows: on the matrix unit, no splits, no workspace
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
     const bool two = (long)((rows + 127) / 128) * Hq * B >= 2L * cus;
     const dim3 grid(two ? (rows + 127) / 128 : (rows + 63) / 64, Hq, B);
-    if (kv8) {
-      if (two) hipLaunchKernelGGL((prompt_attention_mfma_kernel<2, true>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
-      else hipLaunchKernelGGL((prompt_attention_mfma_kernel<1, true>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a); };
+    if (D == 128) {
+      if (kv8) { if (two) go(prompt_attention_mfma_kernel<128, 2, true>); else go(prompt_attention_mfma_kernel<128, 1, true>); }
+      else { if (two) go(prompt_attention_mfma_kernel<128, 2, false>); else go(prompt_attention_mfma_kernel<128, 1, false>); }
     } else {
-      if (two) hipLaunchKernelGGL((prompt_attention_mfma_kernel<2, false>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
-      else hipLaunchKernelGGL((prompt_attention_mfma_kernel<1, false>), grid, dim3(PA_THREADS), 0, (hipStream_t)stream, a);
+      if (kv8) { if (two) go(prompt_attention_mfma_kernel<64, 2, true>); else go(prompt_attention_mfma_kernel<64, 1, true>); }
+      else { if (two) go(prompt_attention_mfma_kernel<64, 2, false>); else go(prompt_attention_mfma_kernel<64, 1, false>); }
     }
     PTA_CHECK_LAUNCH(name);
     return PTA_OK;

@@ -705,7 +705,8 @@ def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, H
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,first,rows", [("llama", 2, 4, 4, 128, 160, 0, 32), ("llama", 1, 4, 4, 128, 160, 70, 64),
                                                                   ("gpt2", 3, 4, 4, 64, 64, 5, 21), ("glm2", 2, 8, 2, 128, 200, 64, 17),
                                                                   ("llama", 1, 4, 4, 128, 300, 3, 200), ("glm2", 2, 8, 2, 128, 256, 30, 130),
-                                                                  ("llama", 2, 2, 2, 128, 64, 0, 15), ("llama", 1, 2, 2, 128, 64, 0, 16)])
+                                                                  ("llama", 2, 2, 2, 128, 64, 0, 15), ("llama", 1, 2, 2, 128, 64, 0, 16),
+                                                                  ("glm2", 2, 8, 2, 64, 96, 10, 40), ("gpt2", 1, 6, 6, 64, 200, 20, 150)])
 def test_prompt_rows_equal_the_loop(K, family, B, Hq, Hkv, D, max_len, first, rows):
     """pta_prompt_rope_append + pta_prompt_attention over `rows` positions at once against the oracle's
     position-by-position attention (1e-2) and against the per-position calls: the ring is bit-identical, the
@@ -817,7 +818,7 @@ def test_fp8_kv_cache_attention(K, family, B, Hq, Hkv, D, max_len, steps):
         assert rel_err(got[:, r], refs[r]) <= 1e-2, f"row {r}"
     more = min(40, steps - rows)
     if max_len >= rows + more and more >= 16:
-        # and the next `more` (head size 128: on the matrix unit, the cache rows staged 32 at a time, the last step ragged)
+        # and the next `more` (on the matrix unit, the cache rows staged 32 at a time, the last step ragged)
         stack2 = lambda xs: dev(np.stack(xs[rows:rows + more], axis=1).reshape(B * more, -1))
         q2 = torch.empty((B * more, Hq, D), dtype=torch.float16, device="cuda")
         out2 = torch.empty((B * more, Hq * D), dtype=torch.float16, device="cuda")

@@ -213,6 +213,24 @@ def test_llama2_int4_decode_more_than_16_sequences():
     assert int(dec.step.item()) == ref_step
 
 
+def _equal_up_to_a_near_tie(got, ref, trace, tol=2e-3):
+    """Token ids per sequence equal the oracle's up to the first difference, which must sit where the oracle's two
+    best logits lie within `tol` (four fp16 steps below 1.0; exact ties occur in these tiny random models) and be
+    one of those two.  Returns whether any sequence parted there."""
+    parted = False
+    for b in range(ref.shape[0]):
+        diff = np.nonzero(got[b] != ref[b])[0]
+        if diff.size == 0:
+            continue
+        p_ = int(diff[0])                                  # chosen by loop iteration p_ - 1
+        lg = trace[p_ - 1][1].reshape(ref.shape[0], -1)[b].astype(np.float32)
+        best = np.argsort(lg)[-2:]
+        assert lg[best[1]] - lg[best[0]] <= tol, f"sequence {b}, position {p_}: tokens differ without a near tie"
+        assert got[b, p_] in best, f"sequence {b}, position {p_}: token {got[b, p_]} is not one of the two best"
+        parted = True
+    return parted
+
+
 def _prompt_then_loop(dec, ids, steps, rows_per_pass=None):
     dec.reset(ids)
     n = dec.consume_prompt(rows_per_pass=rows_per_pass)
@@ -226,8 +244,8 @@ def _prompt_then_loop(dec, ids, steps, rows_per_pass=None):
                                                           ("chatglm2_fp8", 2, 29, None)])
 def test_prompt_in_passes_equals_the_loop(family, B, plen, rows_per_pass):
     """The prompt taken several positions per pass (consume_prompt), then the loop: the container, the step and
-    the tokens are those of the oracle's position-by-position loop, and the KV rings hold what the loop leaves
-    there to fp16 rounding.  Prompts of different lengths: the passes stop at the shortest."""
+    the tokens are those of the oracle's position-by-position loop (up to a tie of the oracle's own two best logits),
+    and the KV rings hold what the loop leaves there to fp16 rounding.  Prompts of different lengths: the passes stop at the shortest."""
     from poptransformer_amd.engine import fused, loader
     L, steps, pad, eos = 64, 56, 0, 2
     if family == "llama2":
@@ -252,7 +270,8 @@ def test_prompt_in_passes_equals_the_loop(family, B, plen, rows_per_pass):
     ids = _prompt(np.random.default_rng(21), B, L, plen, vocab, pad)
     if B > 1:
         ids[B - 1, plen - 4:] = pad                                  # one shorter prompt
-    ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos)
+    trace = []
+    ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos, trace=trace)
     loop = make()
     c_loop, s_loop = loop.run(ids, steps)
     dec = make()
@@ -269,14 +288,20 @@ def test_prompt_in_passes_equals_the_loop(family, B, plen, rows_per_pass):
             assert ((a - b).abs().max() / b.abs().max()).item() <= 1e-1
         return
     assert np.array_equal(c_loop, ref_container)
-    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+    # the passes round the context vectors in another order than the loop: where the oracle's two best logits tie
+    # (ChatGLM2 here: exactly, at one late position), either token may come out; the rings are compared up to there
+    first_c = dec.container.cpu().numpy()
+    parted = _equal_up_to_a_near_tie(first_c, ref_container, trace)
+    upto = n if parted else L
     for a, b in zip(dec.rings, loop.rings):
-        err = (a.float() - b.float()).abs().max().item() / b.float().abs().max().item()
+        a, b = a[:, :upto].float(), b[:, :upto].float()
+        err = (a - b).abs().max().item() / b.abs().max().item()
         assert err <= 1e-2, f"KV ring differs from the loop's by {err}"
     # a second generation on the same decoder, graph-captured loop after the passes
     dec.capture()
     _prompt_then_loop(dec, ids, steps, rows_per_pass)
-    assert np.array_equal(dec.container.cpu().numpy(), ref_container)
+    assert np.array_equal(dec.container.cpu().numpy(), first_c)
+    _equal_up_to_a_near_tie(dec.container.cpu().numpy(), ref_container, trace)
 
 
 def test_prompt_passes_stop_before_an_end_token_and_check_their_arguments():
