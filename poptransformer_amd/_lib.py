@@ -10,7 +10,8 @@ import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libpoptransformer_hip.so")
+# POPTRANSFORMER_HIP_LIB names another build of the library (e.g. one compiled with -DDS_TRACE)
+LIB_PATH = os.environ.get("POPTRANSFORMER_HIP_LIB") or os.path.join(HERE, "libpoptransformer_hip.so")
 
 PTA_OK, PTA_EINVAL, PTA_EUNSUPPORTED, PTA_EHIP = 0, -1, -2, -3
 ACT_NONE, ACT_GELU_TANH, ACT_RELU_SQUARE, ACT_SIGMOID = 0, 1, 2, 3

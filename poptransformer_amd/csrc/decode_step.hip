@@ -36,6 +36,7 @@
 // and phase at the 7B shape) instead of being issued where registers first become free.  Every
 // tile has a fixed place in one register array for the whole layer loop, so that no requested tile
 // is ever moved between registers (a move waits for the load and for the burst around it).
+#include <cstdlib>
 #include <mutex>
 
 #include "common.h"
@@ -89,14 +90,21 @@ struct DsArgs {
   int nsplit;
   int kv_scale;          // KV8 kernels: the rings hold F143 bytes of value * 2^-kv_scale (custom_ops/kv_cache.cpp:43-74)
   int region0;           // bytes of the activation / attention area at the start of LDS
+  int xcd_groups;        // workgroups take their work by die: see logical_workgroup
   unsigned long long* trace;
 };
 
 #ifdef DS_TRACE
-#define TRACE(i) do { if (li == 1 && thread_id() == 0) a.trace[g.wg * 32 + (i)] = wall_clock64(); } while (0)
-#define TRACE_STEP(i) do { if (thread_id() == 0) a.trace[g.wg * 32 + (i)] = wall_clock64(); } while (0)
+constexpr int DS_TRACE_WORDS = 128;      // per workgroup: 32 of the first thread, then 6 per wave
+#define TRACE(i) do { if (li == 1 && thread_id() == 0) a.trace[g.wg * DS_TRACE_WORDS + (i)] = wall_clock64(); } while (0)
+#define TRACE_AT(i) (li == 1 ? a.trace + g.wg * DS_TRACE_WORDS + (i) : nullptr)
+#define TRACE_STEP(i) do { if (thread_id() == 0) a.trace[g.wg * DS_TRACE_WORDS + (i)] = wall_clock64(); } while (0)
+#define WTRACE(k) do { if (li == 1 && lane_id() == 0) a.trace[g.wg * DS_TRACE_WORDS + 32 + wave_id() * 6 + (k)] = wall_clock64(); } while (0)
 #else
+constexpr int DS_TRACE_WORDS = 32;
+#define WTRACE(k) do {} while (0)
 #define TRACE(i) do {} while (0)
+#define TRACE_AT(i) nullptr
 #define TRACE_STEP(i) do {} while (0)
 #endif
 
@@ -242,6 +250,16 @@ __device__ __forceinline__ void grid_barrier(unsigned* sync, unsigned epoch, int
     }
   }
   wg_sync();
+}
+
+// Which share of the work the workgroup with hardware index `block` takes.  The device hands workgroups to its eight
+// dies (each with an L2 of its own) in turn: block b runs on die b % 8.  A head's q | k | v channels, the splits of
+// its attention and the merge of their partials all belong to eight consecutive logical indices, so giving the 32
+// blocks of a die 32 consecutive logical indices keeps those hand-overs inside one L2 - a store followed by a load
+// that hits there - where a hand-over between dies goes through memory.  Any permutation is correct; this one is
+// only faster.
+__device__ __forceinline__ int logical_workgroup(int block, int G, int xcd_groups) {
+  return xcd_groups && G % 8 == 0 ? (block % 8) * (G / 8) + block / 8 : block;
 }
 
 // The 17 pointers of one layer as scalars: lane l reads descriptor word l from LDS (one read for
@@ -484,10 +502,18 @@ __device__ __forceinline__ void slots_product(const u32x4 (&S)[NSLOT], f32x4 (&s
 template <int NRB, int TPW, int EPI, int MAXB, int BASE, int SCBASE, int NSLOT, int NSC>
 __device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (&SC)[NSC], f16* const (&out)[NRB],
                                           int ostride, f16 res, int u, int n_units, int N, int KT, int M, const f16* xs,
-                                          int xstride, float* red, int& red_buf, const float* xsum) {
+                                          int xstride, float* red, int& red_buf, const float* xsum,
+                                          unsigned long long* trace = nullptr, unsigned long long* wtrace = nullptr) {
   if (u >= n_units) return res;
   f32x4 sum[NRB];
   slots_product<NRB, TPW, BASE>(S, sum, u, n_units, KT, M, xs, xstride);
+#ifdef DS_TRACE
+  if (trace) { asm volatile("" :: "v"(sum[0][0])); if (thread_id() == 0) *trace = wall_clock64(); }
+  if (wtrace && lane_id() == 0) { asm volatile("" :: "v"(sum[0][0])); wtrace[wave_id() * 6 + 1] = wall_clock64(); }
+  const f16 y = finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+  if (wtrace && lane_id() == 0) wtrace[wave_id() * 6 + 2] = wall_clock64();
+  return y;
+#endif
   return finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
 }
 
@@ -742,6 +768,9 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
                                                const f16* cs, Waiter& w) {
   constexpr int D = DS_D, LPP = D / 8, PPW = 64 / LPP, HALF = D / 2;
   const int wave = wave_id(), lane = lane_id();
+#ifdef DS_TRACE
+  struct { int wg; } g{logical_workgroup(blockIdx.x, gridDim.x, a.xcd_groups)};
+#endif
   const int bh = unit / a.nsplit, split = unit % a.nsplit;
   const int b = bh / a.H, h = bh % a.H;
   const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
@@ -782,6 +811,7 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
       q_s[which * D + d_] = y;
     }
   }
+  TRACE(10);
   wg_sync();
   {
     const int grp = lane / LPP, sub = lane % LPP, d0 = sub * 8;
@@ -854,6 +884,7 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
       for (int e = 0; e < 8; ++e) sm_acc[wave * D + d0 + e] = acc[e];
     }
   }
+  TRACE(11);
   wg_sync();
   float Mx = -INFINITY, Ls = 0.f, As = 0.f;
   float* part = a.part + (((size_t)li * a.B * a.H + bh) * a.nsplit) * DS_PART;
@@ -888,6 +919,7 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
       if (lane == 1) sm_l[wave] = ml;
     }
     wg_sync();
+    TRACE(12);
     if (thread_id() < D) {
       const int d_ = thread_id();
       for (int s = 1; s < nact; ++s) {
@@ -1169,7 +1201,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   const int M = a.B;
   const int step = *a.step;
   const int nb_d = (a.d + 15) / 16, nb_f = (a.ffn + 15) / 16, nb_v = (a.vocab + 15) / 16;
-  const int G = gridDim.x, wg = blockIdx.x;
+  const int G = gridDim.x, wg = logical_workgroup(blockIdx.x, G, a.xcd_groups);
   struct { int wg; } g{wg};       // for TRACE
   (void)g;
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
@@ -1256,25 +1288,36 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     TRACE(0);
     alive = stage<NS_D, MAXB>(x_in, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
     if (!alive) break;
+    TRACE(21);
     {
       const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
       load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
       load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
+    WTRACE(0);
     {
       f16* q = a.qkv + (size_t)li * M * 3 * a.d;
       f16* const o3[3] = {q, q + a.d, q + 2 * a.d};
       gemv_slots<3, T, EPI_STORE, MAXB, S_QKV, C_QKV>(S, SC, o3, 3 * a.d, (f16)0.0f, wg, nb_d, a.d, KT_D, M, xs, xstride,
-                                                      red, red_buf, scratch + DS_XSUM);
+                                                      red, red_buf, scratch + DS_XSUM, TRACE_AT(13), TRACE_AT(32));
     }
+    TRACE(14);
     load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     TRACE(2);
     // ---- rotary + KV append + attention.  Requests the second gate/up unit when it is done.
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
-      for (int u = wg; u < units; u += G) attention_unit<false, KV8>(a, li, kring, u, step, att_lds, cs, w);
+      // With as many units as workgroups, the M * nsplit units of head h go to the workgroups that produce the
+      // head's q | k | v (unit index: (sequence * H + head) * nsplit + split).
+      const int per = M * a.nsplit;
+      const bool by_head = per * a.H == G;
+      for (int u0 = wg; u0 < units; u0 += G) {
+        const int r = wg % per;
+        const int u = by_head ? ((r / a.nsplit) * a.H + wg / per) * a.nsplit + r % a.nsplit : u0;
+        attention_unit<false, KV8>(a, li, kring, u, step, att_lds, cs, w);
+      }
       if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
@@ -1282,13 +1325,15 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     //      down tiles (o_proj's place), the next layer's v and the RMSNorm weights of the MLP.
     alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
+    TRACE(20);
     if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     TRACE(4);
     {
       f16* const o1[1] = {x_mid};
       res = gemv_slots<1, T, EPI_RESIDUAL, MAXB, S_O, C_O>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_D, M, xs, xstride, red,
-                                                           red_buf, scratch + DS_XSUM);
+                                                           red_buf, scratch + DS_XSUM, TRACE_AT(15));
     }
+    TRACE(16);
     load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
     load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
@@ -1316,19 +1361,22 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       sg[0] = (float)SC[C_GU0][0]; su[0] = (float)SC[C_GU0 + 1][0];
       if constexpr (U_F > 1) { sg[1] = (float)SC[C_GU1][0]; su[1] = (float)SC[C_GU1 + 1][0]; }
       if constexpr (U_F > 2) { sg[2] = (float)SC[C_GU2][0]; su[2] = (float)SC[C_GU2 + 1][0]; }
+      TRACE(17);
       finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
+    TRACE(18);
     load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
     // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
     alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
+    TRACE(22);
     load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
       f16* const o1[1] = {x_out};
       res = gemv_slots<1, TPW_F, EPI_RESIDUAL, MAXB, S_D, C_D>(S, SC, o1, a.d, res, wg, nb_d, a.d, KT_F, M, xs, xstride,
-                                                               red, red_buf, scratch + DS_XSUM);
+                                                               red, red_buf, scratch + DS_XSUM, TRACE_AT(19));
     }
     normw_fetch(more ? Ln.get<const f16>(P_N1) : a.final_norm, normw, a.d);
     TRACE(9);
@@ -1651,7 +1699,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
   const int M = a.B;
   const int step = *a.step;
   const int nb_d = (a.d + 15) / 16, nb_f = (a.ffn + 15) / 16, nb_v = (a.vocab + 15) / 16;
-  const int G = gridDim.x, wg = blockIdx.x;
+  const int G = gridDim.x, wg = logical_workgroup(blockIdx.x, G, a.xcd_groups);
   struct { int wg; } g{wg};       // for TRACE
   (void)g;
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
@@ -1774,7 +1822,11 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
     {
       f16* kring = L.get<f16>(P_KV);
       const int units = M * a.H * a.nsplit;
-      if (a.nsplit == 1) {
+      if (a.nsplit == 1 && a.H * 8 == G) {
+        // sequences wg % 8 and wg % 8 + 8 of head wg / 8: the workgroups that produce the head's q | k | v
+        const int b0 = wg % 8, h = wg / 8;
+        if (b0 < M) attention_two<KV8>(a, li, kring, b0 * a.H + h, b0 + 8 < M ? (b0 + 8) * a.H + h : -1, step, att_lds, cs, w);
+      } else if (a.nsplit == 1) {
         for (int u = wg; u < units; u += 2 * G) attention_two<KV8>(a, li, kring, u, u + G < units ? u + G : -1, step, att_lds, cs, w);
       } else {
         for (int u = wg; u < units; u += G) attention_unit<true, KV8>(a, li, kring, u, step, att_lds, cs, w);
@@ -2051,7 +2103,7 @@ Layout layout_for(const pta_decode_model* m, int cus) {
   // arrival words and per-workgroup best logits: decode_step_wide_kernel only
   l.best = l.flags + (B > DS_MAXB ? align256((4 * L + 1) * DS_REPLICAS * flag_words_for(cus) * 4) : 0);
   l.trace = l.best + (B > DS_MAXB ? align256((size_t)cus * 16 * 2 * 4) : 0);
-  l.total = l.trace + (size_t)cus * 256;
+  l.total = l.trace + (size_t)cus * DS_TRACE_WORDS * 8;
   return l;
 }
 
@@ -2123,6 +2175,10 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.best = (uint32_t*)(ws + lay.best);
   a.nsplit = splits_for(cus, B, H);
   a.kv_scale = kv_scale;
+  {
+    static const int by_die = [] { const char* v = getenv("PTA_DS_XCD_GROUPS"); return v && v[0] == '0' ? 0 : 1; }();
+    a.xcd_groups = by_die;
+  }
   const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
   const int xstride = (KT_D > KT_F ? KT_D : KT_F) * 128 + 8;
   size_t region0 = wide ? 0 : (size_t)B * xstride * 2;
