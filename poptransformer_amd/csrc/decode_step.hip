@@ -44,6 +44,12 @@
 
 namespace {
 
+#ifndef DS_HOT
+#define DS_HOT 0     // experiments: every workgroup requests the same few tiles (they stay in L2): the chain without the stream
+#endif
+#ifndef DS_KO
+#define DS_KO 0      // experiments: bit k set = the k-th request site of the layer loop issues nothing (results are then wrong)
+#endif
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
@@ -395,6 +401,74 @@ __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (
   return y;
 }
 
+// Sum over the sixteen lanes of a row (lanes 16 k .. 16 k + 15), left in every lane of the row: data-parallel moves
+// inside the row, no LDS.
+__device__ __forceinline__ float row_sum16(float v) {
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1, 0, 3, 2]
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2, 3, 0, 1]
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return v;
+}
+
+// finish_unit with the sixteen waves' partial sums of an output met by the sixteen lanes of a row: lane w of the row
+// reads wave w's sum, the row adds up in registers, and the lane whose index in the row is the output's channel
+// finishes it (so the scale it holds, SC of lane % 16, is the channel's).  Output o of a pass is row o of the
+// workgroup's threads: o = (r * M + m) * 16 + ch; more than 64 outputs take several passes.  The residual element of
+// (row m, channel ch) therefore lives in thread (m * 16 + ch) * 16 + ch (see residual_thread).
+template <int NRB, int EPI, bool SCALED = false, class Scales = NoScales, int MB = DS_MAXB, int RED = DS_RED>
+__device__ __forceinline__ f16 finish_unit_rows(const f32x4 (&acc)[NRB], f16* const (&out)[NRB], int ostride, f16 res, int u,
+                                                int N, int M, float* red, int& red_buf, const float* xsum = nullptr,
+                                                const Scales& SC = Scales{}, int scbase = 0) {
+  static_assert(EPI != EPI_SWIGLU, "the gate / up pairs finish in finish_gate_up");
+  const int wave = wave_id(), lane = lane_id();
+  float* rb = red + red_buf * RED;
+  if ((lane & 15) < M) {
+#pragma unroll
+    for (int r = 0; r < NRB; ++r)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        rb[((wave * NRB + r) * 16 + (lane >> 4) * 4 + q) * MB + (lane & 15)] = acc[r][q];
+  }
+  wg_sync();
+  f16 y = res;
+  const int total = NRB * 16 * M * 16;      // sixteen lanes per output
+  for (int base = 0; base < total; base += DS_THREADS) {
+    const int idx = base + thread_id();
+    if (idx < total) {                       // whole rows: total is a multiple of 16
+      const int o = idx >> 4, w = idx & 15;
+      const int q = o >> 4, ch = o & 15;
+      const int r = (q >= M ? 1 : 0) + (q >= 2 * M ? 1 : 0);
+      const int m_ = q - r * M;
+      float s = row_sum16(rb[((w * NRB + r) * 16 + ch) * MB + m_]);
+      float off = 0.f;
+      if constexpr (SCALED) off = 8.0f * row_sum16(xsum[w * DS_MAXB + m_]);
+      const int n = u * 16 + ch;
+      if (w == ch && n < N) {
+        if constexpr (SCALED) {
+          float sc = (float)SC[scbase][0];
+#pragma unroll
+          for (int i = 1; i < NRB; ++i) sc = r == i ? (float)SC[scbase + i][0] : sc;
+          s = (s - off) * sc;
+        }
+        y = (f16)s;
+        if (EPI == EPI_RESIDUAL) y = y + res;
+        put(out[r] + (size_t)m_ * ostride + n, y);
+      }
+    }
+  }
+  red_buf ^= 1;
+  return y;
+}
+// the thread that finishes (row m, channel ch) of a one-matrix unit in finish_unit_rows, as (m, ch, whether this thread is one)
+__device__ __forceinline__ bool residual_thread(int& m_, int& ch) {
+  const int tid = thread_id();
+  const int o = tid >> 4;
+  m_ = o >> 4;
+  ch = o & 15;
+  return (tid & 15) == ch;
+}
+
 // out[r][m, n] = sum_k xs[m, k] * W_r[n, k] for unit u, whose tiles are in t.  `res` is the residual
 // element of this thread (EPI_RESIDUAL); the value the thread stored is returned (it is the
 // residual of the same thread in the next residual phase).
@@ -423,7 +497,7 @@ __device__ __forceinline__ f16 gemv_unit(const Unit<Fmt, NRB, TPW>& t, f16* cons
       }
     }
   }
-  return finish_unit<NRB, EPI>(acc, out, ostride, res, u, N, M, red, red_buf);
+  return finish_unit_rows<NRB, EPI>(acc, out, ostride, res, u, N, M, red, red_buf);
 }
 
 // The INT4 tiles of the layer phases live in ONE register array with a fixed place for every unit
@@ -440,6 +514,7 @@ __device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], 
   static_assert(FIRST >= 0 && COUNT >= 0 && FIRST + COUNT <= NRB * TPW, "tiles outside the unit");
   const int wave = wave_id(), lane = lane_id();
   u = u < n_units ? u : n_units - 1;
+  if (DS_HOT) u = 0;
 #pragma unroll
   for (int t = FIRST; t < FIRST + COUNT; ++t) {
     const int r = t / TPW, i = t % TPW;
@@ -510,11 +585,11 @@ __device__ __forceinline__ f16 gemv_slots(const u32x4 (&S)[NSLOT], const f16x2 (
 #ifdef DS_TRACE
   if (trace) { asm volatile("" :: "v"(sum[0][0])); if (thread_id() == 0) *trace = wall_clock64(); }
   if (wtrace && lane_id() == 0) { asm volatile("" :: "v"(sum[0][0])); wtrace[wave_id() * 6 + 1] = wall_clock64(); }
-  const f16 y = finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+  const f16 y = finish_unit_rows<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
   if (wtrace && lane_id() == 0) wtrace[wave_id() * 6 + 2] = wall_clock64();
   return y;
 #endif
-  return finish_unit<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
+  return finish_unit_rows<NRB, EPI, true>(sum, out, ostride, res, u, N, M, red, red_buf, xsum, SC, SCBASE);
 }
 
 // The gate/up units of a workgroup (units wg, wg + G, ...) finish together: one meeting of the partial
@@ -538,30 +613,27 @@ __device__ __forceinline__ void finish_gate_up(const float (&sg)[U_F], const flo
                                                int nb_f, int M, float* red, int& red_buf, const float* xsum) {
   float* rb = red + red_buf * DS_RED;
   wg_sync();
-  // thread (k * M + m_) * 16 + ch finishes channel ch of row m_ of unit k
-  const int tid = thread_id();
-  const int per = 16 * M;
-  if (tid < U_F * per) {
-    const int k = (tid >= per ? 1 : 0) + (tid >= 2 * per ? 1 : 0);
-    const int m_ = (tid - k * per) >> 4, ch = tid & 15;
-    const int u = wg + k * G, n = u * 16 + ch;
-    if (u < nb_f && n < ffn) {
-      float off = 0.f;
-#pragma unroll 8
-      for (int w = 0; w < DS_WAVES; ++w) off += xsum[w * DS_MAXB + m_];
-      off *= 8.0f;
-      float g = 0.f, v = 0.f;
-#pragma unroll 4
-      for (int w = 0; w < DS_WAVES; ++w) {
-        g += rb[((w * (2 * U_F) + 2 * k) * 16 + ch) * DS_MAXB + m_];
-        v += rb[((w * (2 * U_F) + 2 * k + 1) * 16 + ch) * DS_MAXB + m_];
-      }
-      float cg = sg[0], cu = su[0];
+  // as finish_unit_rows: output o = (k * M + m) * 16 + ch of a pass is row o of the threads, lane w of the row brings
+  // wave w's gate and up sums, the lane with index ch in the row finishes the output (it holds the channel's scales)
+  const int per = 16 * M, total = U_F * per * 16;
+  for (int base = 0; base < total; base += DS_THREADS) {
+    const int idx = base + thread_id();
+    if (idx < total) {
+      const int o = idx >> 4, w = idx & 15;
+      const int k = (o >= per ? 1 : 0) + (o >= 2 * per ? 1 : 0);
+      const int m_ = (o - k * per) >> 4, ch = o & 15;
+      float g = row_sum16(rb[((w * (2 * U_F) + 2 * k) * 16 + ch) * DS_MAXB + m_]);
+      float v = row_sum16(rb[((w * (2 * U_F) + 2 * k + 1) * 16 + ch) * DS_MAXB + m_]);
+      const float off = 8.0f * row_sum16(xsum[w * DS_MAXB + m_]);
+      const int u = wg + k * G, n = u * 16 + ch;
+      if (w == ch && u < nb_f && n < ffn) {
+        float cg = sg[0], cu = su[0];
 #pragma unroll
-      for (int i = 1; i < U_F; ++i) { cg = k == i ? sg[i] : cg; cu = k == i ? su[i] : cu; }
-      g = (g - off) * cg;
-      v = (v - off) * cu;
-      put(act + (size_t)m_ * ffn + n, (f16)v * swish_f16((f16)g));
+        for (int i = 1; i < U_F; ++i) { cg = k == i ? sg[i] : cg; cu = k == i ? su[i] : cu; }
+        g = (g - off) * cg;
+        v = (v - off) * cu;
+        put(act + (size_t)m_ * ffn + n, (f16)v * swish_f16((f16)g));
+      }
     }
   }
   red_buf ^= 1;
@@ -1267,18 +1339,20 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   // the residual element of this thread's output channel (epilogue mapping of gemv_unit, N = d)
   f16 res = (f16)0.0f;
   if (alive) {
-    const int tid = thread_id();
-    const int m_ = tid >> 4, n = wg * 16 + (tid & 15);
-    const bool on = m_ < M && n < a.d;
+    int m_, ch;
+    const bool mine = residual_thread(m_, ch);
+    const int n = wg * 16 + ch;
+    const bool on = mine && m_ < M && n < a.d;
     res = wait_value(a.xres + (on ? (size_t)m_ * a.d + n : 0), on, w);
   }
 
   for (int li = 0; li < a.n_layer && alive; ++li) {
     const LayerPtrs L = layer_ptrs(lds_layers, li);
     const bool more = li + 1 < a.n_layer;
-    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
-    const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
-    const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
+    const LayerPtrs Ln = layer_ptrs(lds_layers, DS_HOT ? 0 : more ? li + 1 : li);   // the last layer's own tiles again: never used
+    const LayerPtrs LW = DS_HOT ? layer_ptrs(lds_layers, 0) : L;
+    const Mat mgu[2] = {layer_mat(LW, P_WG, P_SG), layer_mat(LW, P_WU, P_SU)};
+    const Mat md[1] = {layer_mat(LW, P_WD, P_SD)};
     const Mat m3n[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
     f16* const x_in = a.xres + (size_t)(2 * li) * xslot;        // residual stream entering the layer
     f16* const x_mid = x_in + xslot;                             // after attention
@@ -1290,9 +1364,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     if (!alive) break;
     TRACE(21);
     {
-      const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
-      load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
-      load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+      const Mat mo[1] = {layer_mat(LW, P_WO, P_SO)};
+      if (!(DS_KO & 1)) load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
+      if (!(DS_KO & 2)) load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
     WTRACE(0);
@@ -1303,7 +1377,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                       red, red_buf, scratch + DS_XSUM, TRACE_AT(13), TRACE_AT(32));
     }
     TRACE(14);
-    load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+    if (!(DS_KO & 4)) load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     TRACE(2);
     // ---- rotary + KV append + attention.  Requests the second gate/up unit when it is done.
     {
@@ -1318,7 +1392,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
         const int u = by_head ? ((r / a.nsplit) * a.H + wg / per) * a.nsplit + r % a.nsplit : u0;
         attention_unit<false, KV8>(a, li, kring, u, step, att_lds, cs, w);
       }
-      if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
+      if constexpr (U_F > 1) if (!(DS_KO & 8)) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
     // ---- o_proj + residual.  Requests the third gate/up unit before the product; after it the first
@@ -1326,7 +1400,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
     TRACE(20);
-    if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
+    if constexpr (U_F > 2) if (!(DS_KO & 16)) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     TRACE(4);
     {
       f16* const o1[1] = {x_mid};
@@ -1334,8 +1408,8 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                            red_buf, scratch + DS_XSUM, TRACE_AT(15));
     }
     TRACE(16);
-    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    if (!(DS_KO & 32)) load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+    if (!(DS_KO & 64)) load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
     // ---- RMSNorm + gate/up + SwiGLU.  Requests the remaining down tiles once the first unit has been
@@ -1348,7 +1422,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       f32x4 gsum[2];
       slots_product<2, T, S_GU0>(S, gsum, wg, nb_f, KT_D, M, xs, xstride);
       stash_gate_up<U_F>(gsum, 0, M, red, red_buf);
-      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+      if (!(DS_KO & 128)) load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
       if constexpr (U_F > 1) {
         slots_product<2, T, S_GU1>(S, gsum, wg + G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 1, M, red, red_buf);
@@ -1365,13 +1439,13 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
     TRACE(18);
-    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    if (!(DS_KO & 256)) load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
     // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
     alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
     TRACE(22);
-    load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    if (!(DS_KO & 512)) load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
       f16* const o1[1] = {x_out};
@@ -2176,7 +2250,7 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   a.nsplit = splits_for(cus, B, H);
   a.kv_scale = kv_scale;
   {
-    static const int by_die = [] { const char* v = getenv("PTA_DS_XCD_GROUPS"); return v && v[0] == '0' ? 0 : 1; }();
+    static const int by_die = [] { const char* v = getenv("PTA_DS_XCD_GROUPS"); return v && v[0] == '1' ? 1 : 0; }();
     a.xcd_groups = by_die;
   }
   const bool wide = B > DS_MAXB;                 // nothing is staged: the head of LDS is the attention area only
