@@ -6,7 +6,7 @@ transformer blocks (RMSNorm, INT4 q/k/v/o and SwiGLU projections, rotary embeddi
 attention over the cache, residuals), final norm, fp16 lm_head, greedy selection and the loop
 bookkeeping.  The default run follows the headline configuration: batch 1, a 128-token prompt, then
 256 timed new tokens (contexts 128..383), KV cache length 2048.  The prompt's 128 loop iterations are
-always run untimed first (in passes of up to 64 rows; ``--prompt-loop``: one iteration per position, as
+always run untimed first (in passes of up to 1024 rows; ``--prompt-loop``: one iteration per position, as
 the reference's loop does), then ``--warmup`` further untimed iterations, then ``--steps`` timed ones: the
 timed iterations generate new tokens whatever the flags are.
 
@@ -14,7 +14,9 @@ By default the iteration runs as one persistent launch (pta_llama_decode_step, b
 ``--executor operators`` runs it as one launch per operator instead.
 
 The default run also measures batch 16 (same model, step counts and executor) and reports it under "batch16"
-beside the batch-1 headline.
+beside the batch-1 headline, and - bounded to a few seconds each - the other benchmark configurations under
+"single_operator" (the INT4 operator at M = 1, 4, 16, 64), "chatglm2_fp8_b8", "rwkv_b1", "rwkv_b32" and
+"gpt2_small" (``--no-extras`` skips them).  Progress lines go to stderr; the JSON line is the only stdout output.
 
 Prints ONE JSON line with tokens/s, the HBM roofline of the dominant kernel measured with events
 on the stream it runs on (the persistent decode-step kernel: one launch moves the whole step's
@@ -24,7 +26,7 @@ bytes; or, with the per-operator executor, the fused INT4 gate/up projection), a
 Other workloads (``--workload``), each printing one line of the same form: ``gemm`` = the single INT4
 weight-only operator X[M, 4096] by W[4096, 11008] at M = ``--batch``; ``chatglm2`` = ChatGLM2-6B-shape FP8
 decode; ``rwkv`` = RWKV-4-7B-shape INT4 recurrent decode; ``prompt`` = the prompt of the headline model taken in
-passes of up to 64 rows (a step is one pass) instead of one position per loop iteration.  ``--copy-calibration`` and ``--summarize-pmc``
+passes of ``--rows-per-pass`` rows (a step is one pass) instead of one position per loop iteration.  ``--copy-calibration`` and ``--summarize-pmc``
 serve the hardware-counter measurement of the HBM traffic (see their help).
 """
 import argparse
@@ -40,6 +42,33 @@ LLAMA2_7B = dict(vocab_size=32000, hidden_size=4096, rms_norm_eps=1e-5, num_atte
 MAX_LEN = 2048
 PROMPT = 128            # prompt positions of the headline configuration; always consumed untimed
 HBM_PEAK_GBS = 8000.0
+_T0 = time.perf_counter()
+
+
+def note(msg):
+    """Progress line on stderr (stdout carries the one JSON line): a run that is slow - under a profiler, say -
+    can be told from one that hangs."""
+    print("[bench %7.1fs] %s" % (time.perf_counter() - _T0, msg), file=sys.stderr, flush=True)
+
+
+def run_steps_noted(dec, n, what, chunk=64):
+    """dec.run_steps(n) in chunks, each followed by a synchronisation and a progress line.  Untimed phases only."""
+    import torch
+    done = 0
+    while done < n:
+        k = min(chunk, n - done)
+        dec.run_steps(k)
+        torch.cuda.synchronize()
+        done += k
+        note(f"{what}: {done}/{n} iterations")
+
+
+def check_persistent(dec, what):
+    """Exit at once, with the reason, when the persistent decode step has reported a failure."""
+    if getattr(dec, "persistent", None) is not None and dec.persistent.failed():
+        print(f"{what}: the persistent decode step reported a failure (a workgroup gave up waiting: the kernel needs every "
+              "compute unit of the device for itself while it runs)", file=sys.stderr, flush=True)
+        sys.exit(1)
 
 
 def algorithmic_step_bytes(cfg, B, t, kv_bytes=2):
@@ -144,21 +173,24 @@ def recorded_traffic(B):
     return None
 
 
-def gemm_workload(args):
+def gemm_measure(M, steps, warmup, weights=None):
     """Single-operator INT4 weight-only GEMV/GEMM: X[M, 4096] fp16 by W[4096, 11008] packed INT4 with
     per-output-channel fp16 scales -> fp16 [M, 11008].  A step is one launch; 48 copies of the weight
-    (1 GiB in all) are used in turn so that no launch finds its weight in a cache."""
+    (1 GiB in all) are used in turn so that no launch finds its weight in a cache.  Returns the result dict and
+    the weight copies (so that several M share them)."""
     import torch
     from poptransformer_amd import kernels as K
-    M, Kd, N, copies = args.batch, 4096, 11008, 48
+    Kd, N, copies = 4096, 11008, 48
     gen = torch.Generator(device="cuda").manual_seed(7)
     x = torch.randn(M, Kd, device="cuda", dtype=torch.float16, generator=gen)
-    ws = []
-    for _ in range(copies):
-        packed = torch.randint(0, 256, (N, Kd // 2), device="cuda", dtype=torch.uint8, generator=gen).view(torch.int8)
-        scale = (torch.rand(N, device="cuda", generator=gen) * 0.015 + 0.005).to(torch.float16)
-        ws.append(K.W4Weight(packed, scale))
-        del packed
+    ws = weights
+    if ws is None:
+        ws = []
+        for _ in range(copies):
+            packed = torch.randint(0, 256, (N, Kd // 2), device="cuda", dtype=torch.uint8, generator=gen).view(torch.int8)
+            scale = (torch.rand(N, device="cuda", generator=gen) * 0.015 + 0.005).to(torch.float16)
+            ws.append(K.W4Weight(packed, scale))
+            del packed
     out = torch.empty(M, N, device="cuda", dtype=torch.float16)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -169,8 +201,8 @@ def gemm_workload(args):
         with torch.cuda.graph(g, stream=stream):
             for w in ws:
                 K.w4a16_gemm(x, w, out=out)
-        rounds_w = max(1, args.warmup // copies)
-        rounds = max(1, args.steps // copies)
+        rounds_w = max(1, warmup // copies)
+        rounds = max(1, steps // copies)
         for _ in range(rounds_w):
             g.replay()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -179,19 +211,26 @@ def gemm_workload(args):
             g.replay()
         e1.record(stream)
     torch.cuda.synchronize()
-    steps = rounds * copies
-    sec = e0.elapsed_time(e1) * 1e-3 / steps
+    n = rounds * copies
+    sec = e0.elapsed_time(e1) * 1e-3 / n
     nbytes = Kd * N // 2 + 2 * N + 2 * M * Kd + 2 * M * N
     achieved = nbytes / sec / 1e9
-    print(json.dumps({
-        "metric": "INT4 weight-only GEMV/GEMM launches/s", "value": 1.0 / sec, "unit": "launches/s", "n_gpus": 1,
-        "steps": steps, "warmup": rounds_w * copies, "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
+    return {"M": M, "launches": n, "warmup": rounds_w * copies, "us_per_launch": sec * 1e6, "bytes_per_launch": nbytes,
+            "achieved_gbs": achieved, "frac": achieved / HBM_PEAK_GBS, "tflops": 2.0 * M * Kd * N / sec / 1e12}, ws
+
+
+def gemm_workload(args):
+    M = args.batch
+    r, _ = gemm_measure(M, args.steps, args.warmup)
+    return {
+        "metric": "INT4 weight-only GEMV/GEMM launches/s", "value": 1e6 / r["us_per_launch"], "unit": "launches/s", "n_gpus": 1,
+        "steps": r["launches"], "warmup": r["warmup"], "ms_per_step": r["us_per_launch"] * 1e-3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
         "config": {"workload": f"single-operator W4A16: X[{M},4096] fp16 by W[4096,11008] packed INT4, fp16 scales", "M": M},
-        "roofline": {"bound": "hbm", "kernel": "pta_w4a16_gemm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": nbytes, "avg_launch_us": sec * 1e6,
-                     "tflops": 2.0 * M * Kd * N / sec / 1e12},
-    }))
+        "roofline": {"bound": "hbm", "kernel": "pta_w4a16_gemm", "achieved": r["achieved_gbs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": r["frac"], "traffic": None, "bytes_per_launch": r["bytes_per_launch"],
+                     "avg_launch_us": r["us_per_launch"], "tflops": r["tflops"]},
+    }
 
 
 
@@ -201,18 +240,18 @@ RWKV4_7B = dict(num_hidden_layers=32, hidden_size=4096, attention_hidden_size=40
                 vocab_size=65536, layer_norm_epsilon=1e-5, rescale_every=6)
 
 
-def other_model_workload(args):
+def other_model_workload(workload, B, steps, warmup, prompt_loop=False):
     """ChatGLM2-6B-shape FP8 decode (F143 weights and activations, fp16 KV cache of length 4096) or
     RWKV-4-7B-shape INT4 recurrent decode, one launch per operator replayed from a HIP graph.  The prompt of
-    the configuration (512 / 64 positions) is consumed untimed, then --warmup further untimed iterations.
+    the configuration (512 / 64 positions) is consumed untimed, then `warmup` further untimed iterations.
     Reported like the headline, without a kernel leg."""
     import torch
     from poptransformer_amd.engine import fused, loader, rwkv, synthetic
-    B = args.batch
     rng = np.random.Generator(np.random.PCG64(1234))
-    prompt = 512 if args.workload == "chatglm2" else 64          # of the respective benchmark configuration
-    first = prompt + args.warmup                                  # first timed loop iteration
-    if args.workload == "chatglm2":
+    prompt = 512 if workload == "chatglm2" else 64          # of the respective benchmark configuration
+    first = prompt + warmup                                  # first timed loop iteration
+    note(f"{workload} batch {B}: generating weights")
+    if workload == "chatglm2":
         cfg, max_len = CHATGLM2_6B, 4096
         weights = synthetic.chatglm2_synthetic_weights(cfg, "fp8", seed=0)
         dec = fused.FusedDecoder(loader.chatglm2_spec(cfg, max_len, B, pad_id=0, eos_id=2), weights)
@@ -225,7 +264,7 @@ def other_model_workload(args):
         def step_bytes(t):
             return wbytes + per_pos * (t + 1) + B * cfg["hidden_size"] * 2
     else:
-        cfg, max_len = RWKV4_7B, first + args.steps + 2
+        cfg, max_len = RWKV4_7B, first + steps + 2
         weights = synthetic.rwkv_synthetic_weights(cfg, seed=0)
         dec = rwkv.RWKVDecoder(loader.rwkv_spec(cfg, max_len, B, pad_id=0, eos_id=-1), weights)
         wbytes, vocab = weights.nbytes(), cfg["vocab_size"]
@@ -235,32 +274,90 @@ def other_model_workload(args):
 
         def step_bytes(t):
             return wbytes + state + B * cfg["hidden_size"] * 2
-    if first + args.steps + 1 > max_len:
+    if first + steps + 1 > max_len:
         print(f"prompt ({prompt}) + warmup + steps must stay below the sequence length {max_len}", file=sys.stderr)
         sys.exit(2)
     dec.capture()
     ids = np.zeros((B, max_len), np.int32)
     ids[:, :prompt] = rng.integers(3, vocab, size=(B, prompt))
     dec.reset(ids)
-    done = dec.consume_prompt(dec.prompt_positions()) if hasattr(dec, "consume_prompt") and not args.prompt_loop else 0
-    dec.run_steps(first - done)
+    done = dec.consume_prompt(dec.prompt_positions()) if hasattr(dec, "consume_prompt") and not prompt_loop else 0
+    note(f"{workload} batch {B}: prompt ({done} positions in passes), {first - done} untimed iterations")
+    run_steps_noted(dec, first - done, f"{workload} batch {B} untimed")
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    dec.run_steps(args.steps)
+    dec.run_steps(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    mean_bytes = float(np.mean([step_bytes(t) for t in range(first, first + args.steps)]))
-    print(json.dumps({
-        "metric": "decode tokens/s + % of HBM roofline", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+    note(f"{workload} batch {B}: {steps} timed iterations, {dt / steps * 1e3:.3f} ms each")
+    mean_bytes = float(np.mean([step_bytes(t) for t in range(first, first + steps)]))
+    return {
+        "metric": "decode tokens/s + % of HBM roofline", "value": B * steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": dt / steps * 1e3, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": f"{name}, batch {B}, prompt {prompt} consumed "
-                               f"{'in passes of up to 64 rows' if done else 'token by token'} (untimed), timed context "
-                               f"{first}..{first + args.steps - 1}", "batch": B, "executor": "operators"},
+                               f"{'in passes of up to 1024 rows' if done else 'token by token'} (untimed), timed context "
+                               f"{first}..{first + steps - 1}", "batch": B, "executor": "operators"},
         "step_algorithmic_bytes": mean_bytes,
-        "step_roofline_frac": mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9),
-    }))
+        "step_roofline_frac": mean_bytes / (dt / steps) / (HBM_PEAK_GBS * 1e9),
+    }
 
+
+def brief(r):
+    """The figures of a full result line that go under a key of the headline's line."""
+    return {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
+            "workload": r["config"]["workload"], "step_algorithmic_bytes": r["step_algorithmic_bytes"],
+            "step_roofline_frac": r["step_roofline_frac"]}
+
+
+GPT2_SMALL = dict(vocab_size=50257, n_embd=768, n_head=12, n_layer=12, n_positions=1024, layer_norm_epsilon=1e-5)
+
+
+def gpt2_small_workload(cpu=True):
+    """GPT-2 small fp16 greedy decode, batch 1, prompt 16, 32 new tokens, KV length 128 (the plumbing configuration):
+    the decode loop on the GPU (one launch per operator, HIP graph) and - the configuration's CPU reference path -
+    the numpy oracle of the same graph on the host cores, with the generated tokens compared."""
+    import torch
+    from poptransformer_amd.engine import fused, loader, synthetic
+    cfg, L, B, prompt, new = GPT2_SMALL, 128, 1, 16, 32
+    pad, eos = 50257 - 1, 50257 - 2          # ids the random prompt avoids
+    note("gpt2 small: generating weights")
+    sd = synthetic.gpt2_synthetic_state_dict(cfg, seed=0)
+    dec = fused.FusedDecoder(loader.gpt2_spec(cfg, L, B, pad, eos), loader.gpt2_weights(sd, cfg))
+    dec.capture()
+    rng = np.random.Generator(np.random.PCG64(1234))
+    ids = np.full((B, L), pad, np.int32)
+    ids[:, :prompt] = rng.integers(0, eos, size=(B, prompt))
+    dec.reset(ids)
+    dec.run_steps(prompt)                     # the prompt's iterations, one position each, untimed
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.run_steps(new)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    got = dec.container.cpu().numpy()
+    wbytes = sum(int(np.prod(v.shape)) * 2 for k, v in sd.items() if "wpe" not in k)
+    out = {"value": B * new / dt, "unit": "tokens/s", "ms_per_step": dt / new * 1e3, "steps": new,
+           "workload": f"GPT-2 small fp16 greedy decode, batch 1, prompt {prompt} (untimed, token by token), {new} new tokens, "
+                       f"KV cache of {L}", "executor": "operators",
+           "step_algorithmic_bytes": float(wbytes), "step_roofline_frac": wbytes / (dt / new) / (HBM_PEAK_GBS * 1e9)}
+    note(f"gpt2 small: {dt / new * 1e3:.3f} ms per token on the GPU")
+    if cpu:
+        from oracle import models as OM
+        try:
+            from threadpoolctl import threadpool_info
+            threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+        except Exception:
+            threads = os.cpu_count() or 1
+        model = OM.GPT2Oracle(sd, cfg, L, B)
+        t0 = time.perf_counter()
+        ref, _ = OM.run_decode_loop(model, ids, L, prompt + new, pad, eos)
+        cdt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": B * (prompt + new) / cdt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
+                               "sample": f"numpy oracle of the same graph, all 12 layers, {prompt + new} loop iterations at batch 1"}
+        out["tokens_equal_cpu"] = bool(np.array_equal(np.asarray(ref)[:, :prompt + new + 1], got[:, :prompt + new + 1]))
+        note(f"gpt2 small: {cdt / (prompt + new) * 1e3:.1f} ms per token on the host, tokens equal: {out['tokens_equal_cpu']}")
+    return out
 
 
 def prompt_workload(args):
@@ -300,7 +397,7 @@ def prompt_workload(args):
     kv = float(np.mean([B * nl * 2 * d * kvb * (p * R + R) + B * nl * 2 * d * kvb * R for p in range(passes)]))
     pass_bytes = nl * per_layer + kv + 2 * B * R * d
     flops = 2.0 * B * R * nl * (4 * d * d + 3 * d * f)
-    print(json.dumps({
+    return {
         "metric": "prompt tokens/s", "value": B * n / dt, "unit": "tokens/s", "n_gpus": 1, "steps": passes, "warmup": passes,
         "ms_per_step": dt / passes * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights, f16 activations, f32 accumulation", "data": "synthetic",
@@ -310,7 +407,7 @@ def prompt_workload(args):
         "step_algorithmic_bytes": pass_bytes,
         "step_roofline_frac": pass_bytes / (dt / passes) / (HBM_PEAK_GBS * 1e9),
         "projection_tflops": flops / (dt / passes) / 1e12,
-    }))
+    }
 
 
 def main():
@@ -327,7 +424,7 @@ def main():
                     help="decode: the Llama2-7B-shape INT4 decode loop (the headline); gemm: the single INT4 "
                          "weight-only operator at M = --batch rows; chatglm2: ChatGLM2-6B-shape FP8 decode; "
                          "rwkv: RWKV-4-7B-shape INT4 recurrent decode; prompt: the headline model's prompt in passes "
-                         "of up to 64 rows (--steps passes)")
+                         "of --rows-per-pass rows (--steps passes)")
     ap.add_argument("--rows-per-pass", type=int, default=64,
                     help="prompt workload: rows (batch x positions) per pass, up to 2048")
     ap.add_argument("--fp8-cache", action="store_true",
@@ -339,6 +436,9 @@ def main():
                          "loop does, instead of in passes of up to 1024 rows (FusedDecoder.consume_prompt)")
     ap.add_argument("--no-batch16", action="store_true",
                     help="default run only: skip the second, batch-16 measurement that is reported beside the headline")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default run only: skip the other benchmark configurations (single operator, ChatGLM2, RWKV, GPT-2 small) "
+                         "that are reported under keys of their own")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain elementwise kernel over 1 GiB three times (reads 1 GiB, writes 1 GiB): a kernel "
@@ -365,78 +465,87 @@ def main():
         print("no GPU visible", file=sys.stderr)
         sys.exit(1)
     if args.workload == "gemm":
-        gemm_workload(args)
+        print(json.dumps(gemm_workload(args)))
         return
     if args.workload in ("chatglm2", "rwkv"):
-        other_model_workload(args)
+        print(json.dumps(other_model_workload(args.workload, args.batch, args.steps, args.warmup, args.prompt_loop)))
         return
     if args.workload == "prompt":
-        prompt_workload(args)
+        print(json.dumps(prompt_workload(args)))
         return
     B, cfg = args.batch, LLAMA2_7B
-    weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
-    dec = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
     executor = args.executor or ("persistent" if B <= 16 else "operators")
-    if args.fuse_norm is not None:
-        dec.fuse_norm = args.fuse_norm == "on"
-    if executor == "persistent":
-        dec.enable_persistent()
-    dec.capture()
-
+    kvb = 1 if args.fp8_cache else 2          # bytes per KV cache element
+    note("generating the Llama2-7B-shape INT4 weights on the device")
+    weights = synthetic.llama2_synthetic_weights(cfg, seed=0)
     rng = np.random.Generator(np.random.PCG64(1234))
     prompt = PROMPT
-    ids = np.zeros((B, MAX_LEN), np.int32)                       # pad id 0 after the prompt
-    ids[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B, prompt))
+    t_first = prompt + args.warmup
 
-    def to_first_timed_context(d, ids):
-        """Untimed: the prompt's 128 loop iterations (contexts 0..127; in passes of up to 64 rows unless
-        --prompt-loop), then --warmup further iterations.  Whatever --warmup is, the timed iterations start at
-        context 128 + warmup: they are iterations that generate new tokens."""
+    def decoder(batch):
+        d = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, batch, pad_id=0, eos_id=2, fp8_cache=args.fp8_cache), weights)
+        if args.fuse_norm is not None:
+            d.fuse_norm = args.fuse_norm == "on"
+        if executor == "persistent":
+            d.enable_persistent()
+        d.capture()                       # one eager iteration, then the recording of one
+        torch.cuda.synchronize()
+        check_persistent(d, f"batch {batch}, first launches")
+        note(f"batch {batch}: decoder ready ({executor}), first launches completed")
+        return d
+
+    def timed_decode(d, batch):
+        """The prompt's 128 loop iterations untimed (contexts 0..127; in passes of up to 1024 rows unless
+        --prompt-loop), then --warmup further iterations, then --steps timed ones: whatever --warmup is, the timed
+        iterations start at context 128 + warmup and generate new tokens.  Wall clock around the timed iterations,
+        and events around the same launches on the stream they are launched on."""
+        ids = np.zeros((batch, MAX_LEN), np.int32)                       # pad id 0 after the prompt
+        ids[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(batch, prompt))
         d.reset(ids)
         done = 0 if args.prompt_loop else d.consume_prompt(d.prompt_positions())
-        d.run_steps(prompt - done + args.warmup)
+        note(f"batch {batch}: prompt consumed ({'in one pass' if done else 'token by token'})")
+        run_steps_noted(d, prompt - done + args.warmup, f"batch {batch} untimed")
+        check_persistent(d, f"batch {batch}, untimed iterations")
+        cur = torch.cuda.current_stream()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        return done
+        t0 = time.perf_counter()
+        e0.record(cur)
+        d.run_steps(args.steps)
+        e1.record(cur)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        check_persistent(d, f"batch {batch}, timed iterations")
+        note(f"batch {batch}: {args.steps} timed iterations, {dt / args.steps * 1e3:.4f} ms each")
+        mean_bytes = float(np.mean([algorithmic_step_bytes(cfg, batch, t, kvb) for t in range(t_first, t_first + args.steps)]))
+        return dt, e0.elapsed_time(e1) * 1e-3, mean_bytes, done
 
-    in_passes = to_first_timed_context(dec, ids)
-    t_first = prompt + args.warmup
-    t0 = time.perf_counter()
-    dec.run_steps(args.steps)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    def step_kernel_name(batch):
+        kv8 = "true" if args.fp8_cache else "false"      # the kernels' last template argument: FP8 KV rings
+        return ("decode_step_kernel<2, 6, 3, %d, %s>" % (1 if batch == 1 else 4, kv8) if batch <= 4 else
+                "decode_step_wide_kernel<2, 6, 3, %s>" % kv8) + " (whole decode step)"
+
+    def traffic_fields(batch):
+        t = recorded_traffic(batch) if executor == "persistent" and not args.fp8_cache else None
+        return {"traffic": t,
+                "traffic_source": ("recorded, not measured in this run: hardware counters of an earlier profiled run, "
+                                   "profiles/" + os.path.basename(pmc_summary_path(batch))) if t is not None else None}
+
+    dec = decoder(B)
+    dt, ev_s, mean_bytes, in_passes = timed_decode(dec, B)
     ms_per_step = dt / args.steps * 1e3
     tokens_per_s = B * args.steps / dt
-    kvb = 1 if args.fp8_cache else 2
-    mean_bytes = np.mean([algorithmic_step_bytes(cfg, B, t, kvb) for t in range(t_first, t_first + args.steps)])
     step_frac = mean_bytes / (dt / args.steps) / (HBM_PEAK_GBS * 1e9)
 
-    stream = torch.cuda.Stream()
     if executor == "persistent":
-        if dec.persistent.failed():
-            print("the persistent decode step reported a failure", file=sys.stderr)
-            sys.exit(1)
-        # Dominant kernel: the decode-step kernel itself, one launch per step.  Timed with events on the
-        # stream it is launched on, over the SAME contexts as the timed region above: the loop's step counter is
-        # set back (the container keeps the tokens generated above, so the iterations repeat exactly).
-        reps = args.steps
-        dec.step.fill_(t_first)
-        with torch.cuda.stream(stream):
-            stream.wait_stream(torch.cuda.current_stream())
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
-                dec.persistent.launch()
-            e1.record(stream)
-        torch.cuda.synchronize()
-        kernel_s = e0.elapsed_time(e1) * 1e-3 / reps
-        kernel_bytes = float(np.mean([algorithmic_step_bytes(cfg, B, t) for t in range(t_first, t_first + reps)]))
-        kv8 = "true" if args.fp8_cache else "false"      # the kernels' last template argument: FP8 KV rings
-        kernel_name = ("decode_step_kernel<2, 6, 3, %d, %s>" % (1 if B == 1 else 4, kv8) if B <= 4 else
-                       "decode_step_wide_kernel<2, 6, 3, %s>" % kv8) + " (whole decode step)"
+        # Dominant kernel: the decode-step kernel itself, one launch per step: the events around the timed
+        # iterations time exactly those launches (gaps between launches included).
+        kernel_s, kernel_bytes, kernel_name = ev_s / args.steps, mean_bytes, step_kernel_name(B)
     else:
         # Dominant kernel: the fused INT4 gate/up (SwiGLU) projection, 2 x [11008, 4096] nibbles per
         # launch.  Timed with events on the stream it runs on, over every layer's weights in turn
         # (1.4 GB in total, so no launch finds its weights in a cache).
+        stream = torch.cuda.Stream()
         d, f = cfg["hidden_size"], cfg["intermediate_size"]
         reps = 10
         with torch.cuda.stream(stream):
@@ -475,44 +584,64 @@ def main():
         "step_algorithmic_bytes": float(mean_bytes), "step_roofline_frac": step_frac,
         "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": recorded_traffic(B) if executor == "persistent" else None,
-                     "traffic_source": ("recorded, not measured in this run: hardware counters of an earlier profiled "
-                                        "run, profiles/" + os.path.basename(pmc_summary_path(B)))
-                     if executor == "persistent" and recorded_traffic(B) is not None else None,
-                     "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
+                     **traffic_fields(B), "bytes_per_launch": kernel_bytes, "avg_launch_us": kernel_s * 1e6},
     }
-    if B == 1 and not args.no_batch16 and not args.copy_calibration:
+    default_run = B == 1 and not args.copy_calibration
+    if default_run and not args.no_batch16:
         # the metric names batch 1 and batch 16: the same model, prompt, step counts and executor at batch 16,
         # reported beside the headline; `value` stays the batch-1 figure
         del dec
         torch.cuda.empty_cache()
         B16 = 16
-        dec16 = fused.FusedDecoder(loader.llama2_spec(cfg, MAX_LEN, B16, pad_id=0, eos_id=2), weights)
-        if executor == "persistent":
-            dec16.enable_persistent()
-        dec16.capture()
-        ids16 = np.zeros((B16, MAX_LEN), np.int32)
-        ids16[:, :prompt] = rng.integers(3, cfg["vocab_size"], size=(B16, prompt))
-        to_first_timed_context(dec16, ids16)
-        t0 = time.perf_counter()
-        dec16.run_steps(args.steps)
-        torch.cuda.synchronize()
-        dt16 = time.perf_counter() - t0
-        if executor == "persistent" and dec16.persistent.failed():
-            print("the persistent decode step reported a failure at batch 16", file=sys.stderr)
-            sys.exit(1)
-        bytes16 = float(np.mean([algorithmic_step_bytes(cfg, B16, t) for t in range(t_first, t_first + args.steps)]))
+        dec16 = decoder(B16)
+        dt16, ev16, bytes16, _ = timed_decode(dec16, B16)
         out["batch16"] = {"value": B16 * args.steps / dt16, "unit": "tokens/s", "ms_per_step": dt16 / args.steps * 1e3,
                           "executor": executor, "timed_context": [t_first, t_first + args.steps - 1],
                           "step_algorithmic_bytes": bytes16,
                           "step_roofline_frac": bytes16 / (dt16 / args.steps) / (HBM_PEAK_GBS * 1e9)}
+        if executor == "persistent":
+            out["batch16"]["roofline"] = {"bound": "hbm", "kernel": step_kernel_name(B16),
+                                          "achieved": bytes16 / (ev16 / args.steps) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                          "frac": bytes16 / (ev16 / args.steps) / 1e9 / HBM_PEAK_GBS, **traffic_fields(B16),
+                                          "bytes_per_launch": bytes16, "avg_launch_us": ev16 / args.steps * 1e6}
+        del dec16
     if args.copy_calibration:
         src = torch.empty(1 << 29, dtype=torch.float16, device="cuda").normal_()
         dst = torch.empty_like(src)
         for _ in range(3):
             torch.neg(src, out=dst)
         torch.cuda.synchronize()
+        del src, dst
+    if default_run and not args.no_extras:
+        # the other benchmark configurations, each bounded to a few seconds, under keys of their own
+        dec = None
+        del weights
+        torch.cuda.empty_cache()
+
+        def extra(key, fn):
+            try:
+                out[key] = fn()
+            except Exception as e:          # the headline line is printed whatever happens here
+                out[key] = {"error": f"{type(e).__name__}: {e}"}
+                note(f"{key}: failed: {e}")
+            torch.cuda.empty_cache()
+
+        def single_operator():
+            rows, ws = [], None
+            for M in (1, 4, 16, 64):
+                r, ws = gemm_measure(M, 192, 48, ws)
+                rows.append(r)
+                note(f"single operator M = {M}: {r['us_per_launch']:.2f} us")
+            return {"workload": "X[M,4096] fp16 by W[4096,11008] packed INT4 with fp16 scales, 48 weight copies in turn",
+                    "rows": rows}
+
+        extra("single_operator", single_operator)
+        extra("chatglm2_fp8_b8", lambda: brief(other_model_workload("chatglm2", 8, args.steps, args.warmup)))
+        extra("rwkv_b1", lambda: brief(other_model_workload("rwkv", 1, args.steps, args.warmup)))
+        extra("rwkv_b32", lambda: brief(other_model_workload("rwkv", 32, args.steps, args.warmup)))
+        extra("gpt2_small", lambda: gpt2_small_workload(cpu=not args.no_cpu_baseline))
     if not args.no_cpu_baseline:
+        note("CPU baseline: the numpy oracle of the headline graph on the host cores")
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 

@@ -44,15 +44,10 @@
 
 namespace {
 
-#ifndef DS_HOT
-#define DS_HOT 0     // experiments: every workgroup requests the same few tiles (they stay in L2): the chain without the stream
-#endif
-#ifndef DS_KO
-#define DS_KO 0      // experiments: bit k set = the k-th request site of the layer loop issues nothing (results are then wrong)
-#endif
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
+constexpr unsigned long long DS_LAUNCH_TICKS = 20000000ull;   // a launch gives up 200 ms after it started (constant 100 MHz clock)
 constexpr int DS_REPLICAS = 16;                             // copies of a row of arrival words, see grid_barrier
 constexpr int DS_MAXB = 4;
 constexpr int DS_D = 128;                                   // head size
@@ -170,18 +165,22 @@ __device__ __forceinline__ bool has_empty16(u32x4 v) {
   return e;
 }
 
-// Bounded waiting of one wave.  `give_up` turns true when the wave has polled DS_SPIN_LIMIT times
-// or another workgroup has reported a failure; the wave then sets the error word and the
+// Bounded waiting of one wave.  `give_up` turns true when the wave has polled DS_SPIN_LIMIT times,
+// when the launch has run for DS_LAUNCH_TICKS (a launch whose workgroups cannot all be resident ends
+// within a quarter of a second instead of spinning through every wait), or when another workgroup has
+// reported a failure; the wave then sets the error word and the
 // workgroup-wide flag in LDS and stops waiting.
 struct Waiter {
   unsigned* err;     // sync[1]
   int* lds_dead;
   unsigned spins;
+  unsigned long long deadline;     // of the launch, on the constant-rate clock
   __device__ __forceinline__ bool give_up() {
     ++spins;
     bool stop = spins > DS_SPIN_LIMIT;
     if ((spins & 63u) == 0)
-      stop = stop || __hip_atomic_load((DS_GLOBAL unsigned*)err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
+      stop = stop || wall_clock64() > deadline ||
+             __hip_atomic_load((DS_GLOBAL unsigned*)err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0;
     if (stop) {
       __hip_atomic_store((DS_GLOBAL unsigned*)err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       *lds_dead = 1;
@@ -514,7 +513,6 @@ __device__ __forceinline__ void load_slots(u32x4 (&S)[NSLOT], f16x2 (&SC)[NSC], 
   static_assert(FIRST >= 0 && COUNT >= 0 && FIRST + COUNT <= NRB * TPW, "tiles outside the unit");
   const int wave = wave_id(), lane = lane_id();
   u = u < n_units ? u : n_units - 1;
-  if (DS_HOT) u = 0;
 #pragma unroll
   for (int t = FIRST; t < FIRST + COUNT; ++t) {
     const int r = t / TPW, i = t % TPW;
@@ -648,7 +646,7 @@ __device__ __forceinline__ int row_of(int i, int per) { return (i >= per ? 1 : 0
 // (layers/rms_layer_norm.py:26-36).  Returns false when the wait was given up.
 template <int NS, int MAXB>
 __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* xs, int xstride, const f16* norm_w,
-                                      float eps, float* scratch, Waiter& w) {
+                                      float eps, float* scratch, Waiter& w, unsigned long long* trace = nullptr) {
   const int vec_per_row = KT * 16, total = M * vec_per_row;
   const int lane = lane_id(), wave = wave_id();
   u32x4 v[NS];
@@ -676,8 +674,14 @@ __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* x
         else need[k] = false;
       }
     }
+#ifdef DS_TRACE
+    if (trace && thread_id() == 0) { trace[2] = trace[2] + 1; if (trace[2] == 1) trace[0] = wall_clock64(); }
+#endif
     if (!__any(pending) || w.give_up()) break;
   }
+#ifdef DS_TRACE
+  if (trace && thread_id() == 0) trace[1] = wall_clock64();
+#endif
   float pq[MAXB];
 #pragma unroll
   for (int mm = 0; mm < MAXB; ++mm) pq[mm] = 0.f;
@@ -1277,7 +1281,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   struct { int wg; } g{wg};       // for TRACE
   (void)g;
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-  Waiter w{a.sync + 1, lds_dead, 0};
+  Waiter w{a.sync + 1, lds_dead, 0, wall_clock64() + DS_LAUNCH_TICKS};
   int red_buf = 0;
   const size_t xslot = (size_t)M * a.d;      // halves of one residual-stream slot
 
@@ -1349,10 +1353,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
   for (int li = 0; li < a.n_layer && alive; ++li) {
     const LayerPtrs L = layer_ptrs(lds_layers, li);
     const bool more = li + 1 < a.n_layer;
-    const LayerPtrs Ln = layer_ptrs(lds_layers, DS_HOT ? 0 : more ? li + 1 : li);   // the last layer's own tiles again: never used
-    const LayerPtrs LW = DS_HOT ? layer_ptrs(lds_layers, 0) : L;
-    const Mat mgu[2] = {layer_mat(LW, P_WG, P_SG), layer_mat(LW, P_WU, P_SU)};
-    const Mat md[1] = {layer_mat(LW, P_WD, P_SD)};
+    const LayerPtrs Ln = layer_ptrs(lds_layers, more ? li + 1 : li);   // the last layer's own tiles again: never used
+    const Mat mgu[2] = {layer_mat(L, P_WG, P_SG), layer_mat(L, P_WU, P_SU)};
+    const Mat md[1] = {layer_mat(L, P_WD, P_SD)};
     const Mat m3n[3] = {layer_mat(Ln, P_WQ, P_SQ), layer_mat(Ln, P_WK, P_SK), layer_mat(Ln, P_WV, P_SV)};
     f16* const x_in = a.xres + (size_t)(2 * li) * xslot;        // residual stream entering the layer
     f16* const x_mid = x_in + xslot;                             // after attention
@@ -1364,9 +1367,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     if (!alive) break;
     TRACE(21);
     {
-      const Mat mo[1] = {layer_mat(LW, P_WO, P_SO)};
-      if (!(DS_KO & 1)) load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
-      if (!(DS_KO & 2)) load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+      const Mat mo[1] = {layer_mat(L, P_WO, P_SO)};
+      load_slots<1, T, S_O, C_O>(S, SC, mo, wg, nb_d, a.d, KT_D);
+      load_slots<2, T, S_GU0, C_GU0, 0, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     }
     TRACE(1);
     WTRACE(0);
@@ -1377,7 +1380,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                       red, red_buf, scratch + DS_XSUM, TRACE_AT(13), TRACE_AT(32));
     }
     TRACE(14);
-    if (!(DS_KO & 4)) load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
+    load_slots<2, T, S_GU0, C_GU0, T, T>(S, SC, mgu, wg, nb_f, a.ffn, KT_D);
     TRACE(2);
     // ---- rotary + KV append + attention.  Requests the second gate/up unit when it is done.
     {
@@ -1392,7 +1395,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
         const int u = by_head ? ((r / a.nsplit) * a.H + wg / per) * a.nsplit + r % a.nsplit : u0;
         attention_unit<false, KV8>(a, li, kring, u, step, att_lds, cs, w);
       }
-      if constexpr (U_F > 1) if (!(DS_KO & 8)) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
+      if constexpr (U_F > 1) load_slots<2, T, S_GU1, C_GU1>(S, SC, mgu, wg + G, nb_f, a.ffn, KT_D);
     }
     TRACE(3);
     // ---- o_proj + residual.  Requests the third gate/up unit before the product; after it the first
@@ -1400,7 +1403,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_D, MAXB>(a.ctx + (size_t)li * xslot, M, a.d, KT_D, xs, xstride, nullptr, 0.f, scratch, w);
     if (!alive) break;
     TRACE(20);
-    if constexpr (U_F > 2) if (!(DS_KO & 16)) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
+    if constexpr (U_F > 2) load_slots<2, T, S_GU2, C_GU2>(S, SC, mgu, wg + 2 * G, nb_f, a.ffn, KT_D);
     TRACE(4);
     {
       f16* const o1[1] = {x_mid};
@@ -1408,13 +1411,16 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                            red_buf, scratch + DS_XSUM, TRACE_AT(15));
     }
     TRACE(16);
-    if (!(DS_KO & 32)) load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-    if (!(DS_KO & 64)) load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
     // ---- RMSNorm + gate/up + SwiGLU.  Requests the remaining down tiles once the first unit has been
     //      multiplied (they take its place), and the next layer's q after the last unit.
-    alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w);
+#ifdef DS_TRACE
+    if (li == 1 && thread_id() == 0) a.trace[g.wg * DS_TRACE_WORDS + 25] = 0;
+#endif
+    alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w, TRACE_AT(23));
     if (!alive) break;
     TRACE(6);
     {
@@ -1422,7 +1428,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       f32x4 gsum[2];
       slots_product<2, T, S_GU0>(S, gsum, wg, nb_f, KT_D, M, xs, xstride);
       stash_gate_up<U_F>(gsum, 0, M, red, red_buf);
-      if (!(DS_KO & 128)) load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
       if constexpr (U_F > 1) {
         slots_product<2, T, S_GU1>(S, gsum, wg + G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 1, M, red, red_buf);
@@ -1439,13 +1445,16 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
     TRACE(18);
-    if (!(DS_KO & 256)) load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(7);
     // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
-    alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w);
+#ifdef DS_TRACE
+    if (li == 1 && thread_id() == 0) a.trace[g.wg * DS_TRACE_WORDS + 28] = 0;
+#endif
+    alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w, TRACE_AT(26));
     if (!alive) break;
     TRACE(22);
-    if (!(DS_KO & 512)) load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+    load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
       f16* const o1[1] = {x_out};
@@ -1777,7 +1786,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
   struct { int wg; } g{wg};       // for TRACE
   (void)g;
   const unsigned epoch = __hip_atomic_load((DS_GLOBAL unsigned*)a.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-  Waiter w{a.sync + 1, lds_dead, 0};
+  Waiter w{a.sync + 1, lds_dead, 0, wall_clock64() + DS_LAUNCH_TICKS};
   int red_buf = 0;
   const size_t xslot = (size_t)DW_MAXB * a.d;      // halves of one residual-stream slot: always sixteen rows
 

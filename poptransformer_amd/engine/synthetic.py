@@ -128,3 +128,36 @@ def rwkv_synthetic_weights(cfg, seed=0, device="cuda"):
     head = LinearWeights(K.F16Weight((torch.randn((v, d), generator=gen, device=device, dtype=torch.float32) * 0.02).half()))
     torch.cuda.synchronize()
     return RWKVWeights(embed=embed, blocks=blocks, ln_out=ln(d), head=head)
+
+
+def gpt2_synthetic_state_dict(cfg, seed=0):
+    """Random-init GPT-2-shaped checkpoint (numpy, on the host) as the reference holds it after
+    GPT2DecModel.process_hf_model_state_dict (poptransformer/models/gpt2/model.py:154-166): Linear weights in
+    [out, in] orientation, the query third of c_attn pre-multiplied by 1 / sqrt(head size); N(0, 0.02) weights,
+    zero biases, LayerNorm gamma 1 / beta 0.  What `loader.gpt2_weights` reads."""
+    rng = np.random.Generator(np.random.PCG64(seed))
+    d, v, npos = cfg["n_embd"], cfg["vocab_size"], cfg["n_positions"]
+    hd = d // cfg["n_head"]
+
+    def normal(*shape):
+        return (rng.standard_normal(shape, dtype=np.float32) * 0.02).astype(np.float16)
+
+    sd = {"transformer.wte.weight": normal(v, d), "transformer.wpe.weight": normal(npos, d)}
+    for i in range(cfg["n_layer"]):
+        p = f"transformer.h.{i}."
+        for ln in ("ln_1", "ln_2"):
+            sd[p + ln + ".weight"] = np.ones(d, np.float16)
+            sd[p + ln + ".bias"] = np.zeros(d, np.float16)
+        w = rng.standard_normal((3 * d, d), dtype=np.float32) * 0.02
+        w[:d] *= np.float32(1 / hd ** 0.5)
+        sd[p + "attn.c_attn.weight"] = w.astype(np.float16)
+        sd[p + "attn.c_attn.bias"] = np.zeros(3 * d, np.float16)
+        sd[p + "attn.c_proj.weight"] = normal(d, d)
+        sd[p + "attn.c_proj.bias"] = np.zeros(d, np.float16)
+        sd[p + "mlp.c_fc.weight"] = normal(4 * d, d)
+        sd[p + "mlp.c_fc.bias"] = np.zeros(4 * d, np.float16)
+        sd[p + "mlp.c_proj.weight"] = normal(d, 4 * d)
+        sd[p + "mlp.c_proj.bias"] = np.zeros(d, np.float16)
+    sd["transformer.ln_f.weight"] = np.ones(d, np.float16)
+    sd["transformer.ln_f.bias"] = np.zeros(d, np.float16)
+    return sd
