@@ -350,9 +350,11 @@ class ChatGLM2Oracle:
     def _attention(self, lay, x, step, mask4):
         """MultiQueryAttention.forward_qkv / forward_attention / forward_output
         (poptransformer/models/chatglm2/attention.py:166-302)."""
+        return self._attention_from_projections(lay, lay["query"](x), lay["key_value"](x), step, mask4)
+
+    def _attention_from_projections(self, lay, q, mixed, step, mask4):
+        """The same from the outputs of the query and key_value Linears on."""
         B, H, G, D = self.B, self.H, self.G, self.D
-        q = lay["query"](x)
-        mixed = lay["key_value"](x)
         k, v = mixed[..., : G * D], mixed[..., G * D:]
         q = q.reshape(B, 1, H, D)
         k = k.reshape(B, 1, G, D)
@@ -368,18 +370,25 @@ class ChatGLM2Oracle:
         a = a.transpose(0, 2, 1, 3).reshape(B, 1, H * D)
         return lay["dense"](a)
 
+    def mlp_half(self, lay, x):
+        """The second half of a GLMBlock: x + MLP(RMSNorm(x)) (models/chatglm2/model.py:110-117, mlp.py:51-59)."""
+        t = O.rms_norm(x, lay["ln2"], self.eps).reshape(-1, self.d)
+        g = O.swish(lay["gate"](t))
+        u = (lay["up"](t) * g).astype(f16)
+        return (x + lay["down"](u).reshape(self.B, -1, self.d)).astype(f16)
+
+    def block(self, lay, x, step, mask4):
+        """One GLMBlock (poptransformer/models/chatglm2/model.py:95-117) on the residual stream x [B, 1, d]."""
+        t = O.rms_norm(x, lay["ln1"], self.eps)
+        t = self._attention(lay, t, step, mask4)
+        return self.mlp_half(lay, (x + t).astype(f16))
+
     def step(self, ids, step, mask):
         B = self.B
         x = self.embed[ids.reshape(B, 1)]
         mask4 = mask[:, None, None, :]
         for lay in self.layers:
-            t = O.rms_norm(x, lay["ln1"], self.eps)
-            t = self._attention(lay, t, step, mask4)
-            x = (x + t).astype(f16)
-            t = O.rms_norm(x, lay["ln2"], self.eps).reshape(-1, self.d)      # BaseMLP (models/chatglm2/mlp.py:51-59)
-            g = O.swish(lay["gate"](t))
-            u = (lay["up"](t) * g).astype(f16)
-            x = (x + lay["down"](u).reshape(B, -1, self.d)).astype(f16)
+            x = self.block(lay, x, step, mask4)
         x = O.rms_norm(x, self.norm, self.eps)
         logits = self.head(x)
         _, idx = O.topk1(logits, axis=2)

@@ -290,6 +290,7 @@ class FusedDecoder(LayerOps):
         self.graph = None
         self._stream = torch.cuda.Stream()
         self.persistent = None
+        self.probe = None                # callable(name, block index, tensor or tensors): looks into eager iterations of the per-operator path
 
     def enable_persistent(self):
         """Run each loop iteration as one persistent launch (pta_llama_decode_step) instead of one
@@ -331,8 +332,13 @@ class FusedDecoder(LayerOps):
         for li, blk in enumerate(w.blocks):
             if not hasattr(self, "_qkv_views"):
                 self._prepare_qkv_views(blk)
+            probe = self.probe                           # diagnostics of eager iterations: callable(name, block, tensor(s))
+            if probe is not None:
+                probe("block_in", li, self.x)
             h, nrm = self._normed(self.x, blk.norm1, blk.qkv)
             self._linear_group(h, blk.qkv, self._qkv_bufs, nrm)
+            if probe is not None:
+                probe("projections", li, self._qkv_bufs)
             qp, kp, vp, qs, ks, vs = self._qkv_views
             # the output projection's cast of its input to FP8 is done by the attention where it stores the context
             grid = self._common_grid([blk.out]) if self.kv_scale is None else None
@@ -343,12 +349,16 @@ class FusedDecoder(LayerOps):
             if grid is not None:
                 self._on_grid[self.ctx.data_ptr()] = self._grid_id(blk.out)
             self._linear(self.ctx, blk.out, self.x, residual=self.x)
+            if probe is not None:
+                probe("after_attention", li, self.x)
             h, nrm = self._normed(self.x, blk.norm2, blk.mlp_in)
             if len(blk.mlp_in) == 2:
                 self._linear_group(h, blk.mlp_in, [self.act, self.act], nrm, swiglu=True, consumer=blk.mlp_out)
             else:
                 self._linear(h, blk.mlp_in[0], self.act, act=_lib.ACT_GELU_TANH, norm=nrm)
             self._linear(self.act, blk.mlp_out, self.x, residual=self.x)
+        if self.probe is not None:                       # ... and the stream leaving the last block
+            self.probe("block_in", len(w.blocks), self.x)
         h, nrm = self._normed(self.x, w.final_norm, [w.head])
         self._linear(h, w.head, self.logits, norm=nrm)
         self.select(self.logits, self.next_ids)

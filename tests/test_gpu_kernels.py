@@ -754,6 +754,125 @@ def test_prompt_rows_equal_the_loop(K, family, B, Hq, Hkv, D, max_len, first, ro
         K.prompt_attention(q_rows, rings[1], step, ws, out_rows, B, rows, Hq, Hkv, D, max_len, True)   # workspace of one row
 
 
+def _prefix_reference(family, qs, ks, vs, D, rows, fp8_cache=False):
+    """The oracle's attention chain for the positions in `rows`, each over the cache rows 0..r it sees (newest first,
+    as the KVCache op holds them) instead of over a cache that is stepped through every position: a masked row's
+    probability is exactly zero in both chains, so the two differ only in the order of sums
+    (test_prefix_reference_is_the_stepped_reference).  Returns {r: context [B, Hq * D]}."""
+    B, Hq, Hkv = qs[0].shape[0], qs[0].shape[1], ks[0].shape[1]
+
+    def rotated(x, pos):
+        x4 = x.reshape(B, -1, 1, D)
+        if family == "llama":
+            sin, cos = O.llama_sincos(pos, D)
+            return O.llama_rope(x4, sin, cos)
+        if family == "glm2":
+            cos, sin = O.glm2_sincos(pos, D)
+            return np.swapaxes(O.glm2_rope(np.swapaxes(x4, 1, 2), cos, sin), 1, 2)
+        return x4
+
+    def stored(x4):
+        return O.f8_decode(O.f8_encode(x4, "F143", O.KVCache.FP8_SCALE), "F143", O.KVCache.FP8_SCALE, np.float16) if fp8_cache else x4
+
+    last = max(rows)
+    kc = [stored(rotated(ks[p], p)) for p in range(last + 1)]
+    vc = [stored(vs[p].reshape(B, Hkv, 1, D)) for p in range(last + 1)]
+    scale = None if family == "gpt2" else 1 / np.sqrt(D)
+    sdt = np.float32 if family == "llama" else np.float16
+    out = {}
+    for r in rows:
+        kk = np.concatenate(kc[r::-1], axis=2)
+        vv = np.concatenate(vc[r::-1], axis=2)
+        if Hkv != Hq:
+            kk, vv = np.repeat(kk, Hq // Hkv, axis=1), np.repeat(vv, Hq // Hkv, axis=1)
+        ctx = O.attention_scores_to_context(rotated(qs[r], r), np.swapaxes(kk, 2, 3), vv, np.zeros((B, 1, 1, r + 1), np.float16), scale, sdt)
+        out[r] = np.swapaxes(ctx, 1, 2).reshape(B, Hq * D)
+    return out
+
+
+@pytest.mark.parametrize("family,fp8", [("llama", False), ("glm2", False), ("gpt2", False), ("llama", True)])
+def test_prefix_reference_is_the_stepped_reference(family, fp8):
+    """CPU only: _prefix_reference against _attention_reference (the oracle stepped through every position)."""
+    rng = np.random.default_rng(5)
+    B, Hq, Hkv, D, n = 2, 4, 2 if family == "glm2" else 4, 64, 40
+    qs = [(rng.standard_normal((B, Hq, D)) * (0.3 if family == "gpt2" else 1.0)).astype(np.float16) for _ in range(n)]
+    ks = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(n)]
+    vs = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(n)]
+    stepped = _attention_reference(family, qs, ks, vs, 48, D, fp8_cache=fp8)
+    for r, ctx in _prefix_reference(family, qs, ks, vs, D, [0, 1, 17, 39], fp8_cache=fp8).items():
+        assert rel_err(ctx, stepped[r]) <= 2e-3, f"position {r}"
+
+
+@pytest.mark.parametrize("D,kv8", [(64, False), (128, False), (64, True), (128, True)])
+def test_prompt_attention_two_row_groups(K, D, kv8):
+    """A pass with enough (sequence, head, 128 rows) tiles to fill every compute unit twice takes the workgroups of
+    128 rows whose waves hold two row groups each: 4 sequences x 32 heads x 512 rows, fp16 and F143 rings, head sizes
+    64 and 128, against the oracle's chain at rows spread over the pass (first and last rows of row groups, of
+    128-row tiles and of the 32-row stages of cache rows)."""
+    from poptransformer_amd import _lib
+    B, Hq, Hkv, rows, max_len = 4, 32, 32, 512, 520
+    print(f"case: prompt attention, two row groups per wave, head size {D}, {'F143' if kv8 else 'fp16'} ring", flush=True)
+    rng = np.random.default_rng(D + kv8)
+    qs = [rng.standard_normal((B, Hq, D)).astype(np.float16) for _ in range(rows)]
+    ks = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(rows)]
+    vs = [(rng.standard_normal((B, Hkv, D)) * (40.0 if kv8 else 1.0)).astype(np.float16) for _ in range(rows)]
+    check = [0, 1, 15, 16, 31, 32, 33, 63, 64, 127, 128, 129, 200, 255, 256, 300, 383, 384, 447, 480, 510, 511]
+    refs = _prefix_reference("llama", qs, ks, vs, D, check, fp8_cache=kv8)
+    inv = dev(np.array([1.0 / (10000 ** (i / D)) for i in range(0, D, 2)]).astype(np.float16))
+    ring = torch.zeros((2 * B * Hkv, max_len, D), dtype=torch.uint8 if kv8 else torch.float16, device="cuda")
+    stack = lambda xs: dev(np.stack(xs, axis=1).reshape(B * rows, -1))
+    q_rows = torch.empty((B * rows, Hq, D), dtype=torch.float16, device="cuda")
+    out_rows = torch.empty((B * rows, Hq * D), dtype=torch.float16, device="cuda")
+    ws_rows = K.decode_attention_workspace(B * rows, Hq, D, max_len, "cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    kw = dict(kv_scale=1) if kv8 else {}
+    K.prompt_rope_append(stack(qs), stack(ks), stack(vs), q_rows, ring, step, inv, B, rows, Hq, Hkv, D, max_len, _lib.ROPE_LLAMA, **kw)
+    K.prompt_attention(q_rows, ring, step, ws_rows, out_rows, B, rows, Hq, Hkv, D, max_len, True, **kw)
+    got = host(out_rows).reshape(B, rows, Hq * D)
+    assert np.isfinite(got).all()
+    for r in check:
+        assert rel_err(got[:, r], refs[r]) <= 1e-2, f"row {r}"
+
+
+def test_decode_attention_beyond_1024_rows_grouped_heads(K):
+    """The ChatGLM2 benchmark's attention shape: 8 sequences, 32 query heads on 2 KV heads of 128, a ring of 4096,
+    contexts 1100..1103 (the splits of a (sequence, head) all hold rows).  The ring is filled by passes of 256
+    positions, the next positions run one per call through the pass that prepares its own operands and through the two
+    separate calls."""
+    from poptransformer_amd import _lib
+    B, Hq, Hkv, D, max_len, n0, more = 8, 32, 2, 128, 4096, 1100, 4
+    print("case: decode attention at context 1100, 32 query / 2 KV heads, ring of 4096", flush=True)
+    rng = np.random.default_rng(11)
+    n = n0 + more
+    qs = [rng.standard_normal((B, Hq, D)).astype(np.float16) for _ in range(n)]
+    ks = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(n)]
+    vs = [rng.standard_normal((B, Hkv, D)).astype(np.float16) for _ in range(n)]
+    refs = _prefix_reference("glm2", qs, ks, vs, D, list(range(n0, n)))
+    inv = dev(np.array([1.0 / (10000 ** (i / (D // 2))) for i in range(0, D // 2, 2)]).astype(np.float32))
+    rings = [torch.zeros((2 * B * Hkv, max_len, D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    R = 256
+    for p0 in range(0, n0, R):
+        rc = min(R, n0 - p0)
+        stack = lambda xs: dev(np.stack(xs[p0:p0 + rc], axis=1).reshape(B * rc, -1))
+        q_rows = torch.empty((B * rc, Hq, D), dtype=torch.float16, device="cuda")
+        step.fill_(p0)
+        for ring in rings:
+            K.prompt_rope_append(stack(qs), stack(ks), stack(vs), q_rows, ring, step, inv, B, rc, Hq, Hkv, D, max_len, _lib.ROPE_GLM2)
+    ws = K.decode_attention_workspace(B, Hq, D, max_len, "cuda")
+    q_rot = torch.empty((B, Hq, D), dtype=torch.float16, device="cuda")
+    outs = [torch.empty((B, Hq * D), dtype=torch.float16, device="cuda") for _ in range(2)]
+    for it in range(n0, n):
+        step.fill_(it)
+        q, k, v = dev(qs[it]), dev(ks[it]), dev(vs[it])
+        K.qkv_rope_append(q, k, v, q_rot, rings[0], step, inv, B, Hq, Hkv, D, max_len, _lib.ROPE_GLM2)
+        K.decode_attention(q_rot, rings[0], step, ws, outs[0], B, Hq, Hkv, D, max_len, True)
+        K.decode_attention_qkv(q, k, v, rings[1], step, inv, ws, outs[1], B, Hq, Hkv, D, max_len, _lib.ROPE_GLM2, True)
+        assert rel_err(host(outs[0]), refs[it]) <= 1e-2, f"context {it}"
+        assert torch.equal(outs[0], outs[1]), f"context {it}: the pass that prepares its operands differs"
+    assert torch.equal(rings[0], rings[1])
+
+
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 130), ("glm2", 2, 8, 2, 128, 96, 70),
                                                              ("gpt2", 1, 4, 4, 64, 48, 50)])
 def test_fp8_kv_cache_attention(K, family, B, Hq, Hkv, D, max_len, steps):
