@@ -2204,20 +2204,21 @@ extern "C" size_t pta_decode_step_workspace_bytes(const pta_decode_model* model)
   return layout_for(model, cus).total;
 }
 
-static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace, pta_stream_t stream,
-                              bool kv8 = false, int kv_scale = 0) {
-  PTA_REQUIRE(mdl && st && workspace, "pta_llama_decode_step: null pointer");
+// `who`: the entry point's name, for its messages
+static int decode_step_launch(const char* who, const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
+                              pta_stream_t stream, bool kv8 = false, int kv_scale = 0) {
+  PTA_REQUIRE(mdl && st && workspace, "%s: null pointer", who);
   PTA_REQUIRE(mdl->layers && mdl->n_layer > 0 && mdl->embed && mdl->final_norm && mdl->head && mdl->inv_freq,
-              "pta_llama_decode_step: incomplete model");
+              "%s: incomplete model", who);
   PTA_REQUIRE(st->container && st->mask && st->stop_mask && st->step && st->keep_going && st->next_ids && st->logits,
-              "pta_llama_decode_step: incomplete state");
+              "%s: incomplete state", who);
   PTA_REQUIRE(pta_aligned(workspace, 256) && pta_aligned(st->logits, 16),
-              "pta_llama_decode_step: the workspace must be 256-byte aligned and the logits 16-byte aligned");
+              "%s: the workspace must be 256-byte aligned and the logits 16-byte aligned", who);
   const int B = mdl->batch, d = mdl->hidden, H = mdl->n_head, ffn = mdl->ffn;
   PTA_REQUIRE(B >= 1 && d > 0 && H > 0 && ffn > 0 && mdl->vocab > 0 && mdl->max_len > 0,
-              "pta_llama_decode_step: empty shape");
+              "%s: empty shape", who);
   int cus = 0;
-  PTA_REQUIRE(device_cus(&cus) == 0, "pta_llama_decode_step: cannot read the compute-unit count of the current device");
+  PTA_REQUIRE(device_cus(&cus) == 0, "%s: cannot read the compute-unit count of the current device", who);
   const int KT_D = (d + 127) / 128, KT_F = (ffn + 127) / 128;
   const int tpw_d = (KT_D + DS_WAVES - 1) / DS_WAVES, tpw_f = (KT_F + DS_WAVES - 1) / DS_WAVES;
   const int nb_d = (d + 15) / 16, nb_f = (ffn + 15) / 16;
@@ -2226,9 +2227,9 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
   for (Variant& v : g_variants)
     if (v.tpw_d == tpw_d && v.tpw_f == tpw_f && u_f <= v.u_f && B >= v.minb && B <= v.maxb && v.kv8 == kv8 && !var) var = &v;
   if (!shape_ok(mdl) || nb_d > cus || !var) {
-    pta_set_error("pta_llama_decode_step: supports batch <= %d, head size %d, hidden = heads * head size <= %d, ffn "
+    pta_set_error("%s: supports batch <= %d, head size %d, hidden = heads * head size <= %d, ffn "
                   "and vocabulary sizes that are multiples of 8, and the (hidden, ffn) of the 7B model or small test "
-                  "shapes (got batch %d, head size %d, hidden %d, heads %d, ffn %d, vocabulary %d)",
+                  "shapes (got batch %d, head size %d, hidden %d, heads %d, ffn %d, vocabulary %d)", who,
                   DW_MAXB, DS_D, 16 * cus, B, mdl->head_dim, d, H, ffn, mdl->vocab);
     return PTA_EUNSUPPORTED;
   }
@@ -2272,33 +2273,33 @@ static int decode_step_launch(const pta_decode_model* mdl, const pta_decode_stat
                                 (size_t)mdl->n_layer * sizeof(pta_decode_layer)
                           : region0 + (size_t)(2 * DS_RED + DS_TAIL_FLOATS) * 4 + (size_t)((d + 511) & ~511) * 2 + DS_D * 2 +
                                 (size_t)mdl->n_layer * sizeof(pta_decode_layer);
-  PTA_REQUIRE(lds <= 160 * 1024, "pta_llama_decode_step: %zu bytes of LDS exceed a compute unit's 160 KiB", lds);
+  PTA_REQUIRE(lds <= 160 * 1024, "%s: %zu bytes of LDS exceed a compute unit's 160 KiB", who, lds);
 
   if (!var->ready) {
     PTA_REQUIRE(hipFuncSetAttribute((const void*)var->kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) ==
                     hipSuccess,
-                "pta_llama_decode_step: cannot reserve dynamic LDS");
+                "%s: cannot reserve dynamic LDS", who);
     // every workgroup must be resident at once: one per compute unit, so the kernel must fit one
     int per_cu = 0;
     PTA_REQUIRE(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)var->kern, DS_THREADS, lds) ==
                         hipSuccess && per_cu >= 1,
-                "pta_llama_decode_step: the kernel does not fit a compute unit");
+                "%s: the kernel does not fit a compute unit", who);
     var->ready = true;
   }
   hipLaunchKernelGGL(var->kern, dim3(cus), dim3(DS_THREADS), lds, (hipStream_t)stream, a);
-  PTA_CHECK_LAUNCH("pta_llama_decode_step");
+  PTA_CHECK_LAUNCH(who);
   return PTA_OK;
 }
 
 extern "C" int pta_llama_decode_step(const pta_decode_model* mdl, const pta_decode_state* st, void* workspace,
                                      pta_stream_t stream) {
-  return decode_step_launch(mdl, st, workspace, stream);
+  return decode_step_launch("pta_llama_decode_step", mdl, st, workspace, stream);
 }
 
 extern "C" int pta_llama_decode_step_f8(const pta_decode_model* mdl, const pta_decode_state* st, int kv_scale, void* workspace,
                                         pta_stream_t stream) {
   PTA_REQUIRE(kv_scale >= -16 && kv_scale <= 16, "pta_llama_decode_step_f8: kv_scale %d outside [-16, 16]", kv_scale);
-  return decode_step_launch(mdl, st, workspace, stream, true, kv_scale);
+  return decode_step_launch("pta_llama_decode_step_f8", mdl, st, workspace, stream, true, kv_scale);
 }
 
 // ------------------------------------------------------------------------------------------ the same step without a workspace argument
@@ -2358,7 +2359,7 @@ extern "C" int pta_llama_decode_step_static(const pta_decode_model* mdl, const p
     hipLaunchKernelGGL(clear_failure_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned*)ws);
     PTA_CHECK_LAUNCH("pta_llama_decode_step_static");
   }
-  return decode_step_launch(mdl, st, ws, stream);
+  return decode_step_launch("pta_llama_decode_step_static", mdl, st, ws, stream);
 }
 
 extern "C" int pta_decode_step_failed(const void* workspace, int* failed, pta_stream_t stream) {

@@ -76,12 +76,13 @@ def _prompt(rng, B, L, n, vocab, pad):
     return ids
 
 
-def _follow(dec, oracle, ids, L, steps, pad, eos, tol=1e-2):
+def _follow(dec, oracle, ids, L, steps, pad, eos, tol=1e-2, within_tol=False):
     """Runs `steps` loop iterations on both sides.  Every iteration: fp16 logits within `tol` (max relative
     error), the selected ids equal wherever the oracle's two best logits are further apart than 0.3 % of the
     largest logit.  At a nearer tie either candidate is a correct greedy choice; when the decoder took the other
-    one its container entry is set to the oracle's, so that the two generations stay comparable.  Returns the
-    number of such ties."""
+    one its container entry is set to the oracle's, so that the two generations stay comparable.  within_tol (FP8
+    rings, whose logits are held to a looser `tol`): a token counts as tied when the oracle scores it within 2 * tol of
+    its best.  Returns the number of such ties."""
     trace = []
     ref_container, ref_step = OM.run_decode_loop(oracle, ids, L, steps, pad, eos, trace=trace)
     dec.reset(ids)
@@ -95,12 +96,14 @@ def _follow(dec, oracle, ids, L, steps, pad, eos, tol=1e-2):
         worst = max(worst, np.abs(got - ref).max() / np.abs(ref).max())
         got_ids = dec.next_ids.cpu().numpy()
         top2 = np.sort(ref, axis=1)[:, -2:]
-        clear = (top2[:, 1] - top2[:, 0]) > 3e-3 * np.abs(ref).max()
+        clear = (top2[:, 1] - top2[:, 0]) > (2 * tol if within_tol else 3e-3) * np.abs(ref).max()
         assert np.array_equal(got_ids[clear], ref_ids[clear]), f"token ids differ at step {it} without a near tie"
         for b in np.nonzero(got_ids != ref_ids)[0]:
             ties += 1
-            order = np.argsort(ref[b])
-            assert got_ids[b] in order[-2:], f"step {it}: the decoder's token is not one of the two tied candidates"
+            if within_tol:
+                assert ref[b, got_ids[b]] >= ref[b].max() - 2 * tol * np.abs(ref).max(), f"step {it}: the decoder's token is no near-best candidate"
+            else:
+                assert got_ids[b] in np.argsort(ref[b])[-2:], f"step {it}: the decoder's token is not one of the two tied candidates"
             if it + 1 < L and ids[b, it + 1] == pad:
                 dec.container[b, it + 1] = int(ref_ids[b])
     assert worst <= tol, f"logits max rel err {worst}"
@@ -161,6 +164,30 @@ def test_persistent_step_at_7b_width_batch_16_matches_oracle(wide):
     ties = _follow(dec, oracle, ids, L, steps, pad, eos)
     assert not dec.persistent.failed()
     assert ties <= 40
+
+
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("B,plen,L", [(1, 136, 176), (4, 72, 112), (16, 72, 112)])
+def test_persistent_step_with_fp8_rings_at_7b_width_matches_oracle(wide, B, plen, L):
+    """decode_step_kernel<2,6,3,1,true>, <2,6,3,4,true> and decode_step_wide_kernel<2,6,3,true>: the persistent step
+    over F143 KV rings (pta_llama_decode_step_f8) at the 7B width against the oracle with KVCache(fp8 = true).  Logits
+    to 3e-2, as at the small shapes (5e-2 at batch 16, where the worst of 16 x 103 rows of logits was 3.1e-2): where
+    one of this kernel's k or v elements, equal to the oracle's up to the last fp16 bit, lies at an FP8 rounding
+    boundary, its byte comes out one step of three mantissa bits away."""
+    from poptransformer_amd.engine import fused, loader
+    pad, eos = 0, 2
+    steps = plen - 1 + 32
+    print(f"case: persistent step over FP8 rings at the 7B width, batch {B}, {steps} iterations", flush=True)
+    sd, template = wide
+    oracle = _oracle(template, L, B)
+    oracle.layers = [dict(lay, cache=O.KVCache(L, 3, 1, fp8=True)) for lay in template.layers]
+    dec = fused.FusedDecoder(loader.llama2_spec(LLAMA_7B_WIDTH, L, B, pad, eos, fp8_cache=True),
+                             loader.llama2_weights(sd, LLAMA_7B_WIDTH))
+    dec.enable_persistent()
+    ids = _prompt(np.random.default_rng(131 + B), B, L, plen, LLAMA_7B_WIDTH["vocab_size"], pad)
+    ties = _follow(dec, oracle, ids, L, steps, pad, eos, tol=3e-2 if B <= 4 else 5e-2, within_tol=True)
+    assert not dec.persistent.failed()
+    assert ties <= 4 * B + 12
 
 
 # ---------------------------------------------------------------- the single INT4 operator at its own shape

@@ -67,6 +67,21 @@ def test_decode_step_without_a_workspace_argument():
         assert int(builtin.persistent.workspace.view(torch.int32)[0].item()) == 0
 
 
+def test_static_decode_step_of_many_sequences_after_a_larger_model():
+    """Batch 8 and 16 (decode_step_wide_kernel: its arrival words and per-workgroup best logits sit behind the
+    model-dependent slots of the shared array) after a launch of a different model with more layers through the same
+    array, bit for bit against the entry point with a workspace of its own."""
+    rng = np.random.default_rng(5)
+    for cfg, B, L, steps, seed in [(FIRST, 3, 48, 8, 5), (SECOND, 16, 40, 24, 7), (FIRST, 8, 48, 24, 8)]:
+        print(f"case: static decode step, hidden {cfg['hidden_size']}, batch {B}", flush=True)
+        ids = np.zeros((B, L), np.int32)
+        ids[:, :6] = rng.integers(3, cfg["vocab_size"], size=(B, 6))
+        own = _decoder(cfg, B, L, seed)
+        ref = _generate(own, ids, steps, static=False)
+        assert not own.persistent.failed() and ref[4] == steps
+        _same(_generate(_decoder(cfg, B, L, seed), ids, steps, static=True), ref)
+
+
 def test_static_decode_step_refuses_what_the_built_in_array_cannot_hold():
     """A model whose workspace exceeds the 16 MiB array is refused before anything is launched (only sizes are
     read on the host: the pointers of this descriptor are never followed)."""
