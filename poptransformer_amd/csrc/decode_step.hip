@@ -44,6 +44,9 @@
 
 namespace {
 
+#ifndef DS_X2
+#define DS_X2 0
+#endif
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
@@ -267,6 +270,25 @@ __device__ __forceinline__ int logical_workgroup(int block, int G, int xcd_group
   return xcd_groups && G % 8 == 0 ? (block % 8) * (G / 8) + block / 8 : block;
 }
 
+// Sum over the sixteen lanes of a row (lanes 16 k .. 16 k + 15), left in every lane of the row: data-parallel moves
+// inside the row, no LDS.
+__device__ __forceinline__ float row_sum16(float v) {
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1, 0, 3, 2]
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2, 3, 0, 1]
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  return v;
+}
+
+// Sum over all 64 lanes, the same in every lane: the rows' sums by data-parallel moves, then the four rows' totals
+// through scalar registers (a shuffle through the LDS crossbar per step takes several times as long).
+__device__ __forceinline__ float wave_total(float v) {
+  v = row_sum16(v);
+  const int b = bitcast<int>(v);
+  return bitcast<float>(__builtin_amdgcn_readlane(b, 0)) + bitcast<float>(__builtin_amdgcn_readlane(b, 16)) +
+         (bitcast<float>(__builtin_amdgcn_readlane(b, 32)) + bitcast<float>(__builtin_amdgcn_readlane(b, 48)));
+}
+
 // The 17 pointers of one layer as scalars: lane l reads descriptor word l from LDS (one read for
 // the whole descriptor), and each pointer is two lane reads.
 struct LayerPtrs {
@@ -398,16 +420,6 @@ __device__ __forceinline__ f16 finish_unit(const f32x4 (&acc)[NRB], f16* const (
   }
   red_buf ^= 1;
   return y;
-}
-
-// Sum over the sixteen lanes of a row (lanes 16 k .. 16 k + 15), left in every lane of the row: data-parallel moves
-// inside the row, no LDS.
-__device__ __forceinline__ float row_sum16(float v) {
-  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1, 0, 3, 2]
-  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2, 3, 0, 1]
-  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
-  v += bitcast<float>(__builtin_amdgcn_update_dpp(0, bitcast<int>(v), 0x140, 0xF, 0xF, true));   // row_mirror
-  return v;
 }
 
 // finish_unit with the sixteen waves' partial sums of an output met by the sixteen lanes of a row: lane w of the row
@@ -700,7 +712,7 @@ __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* x
       }
     }
 #pragma unroll
-    for (int mm = 0; mm < MAXB; ++mm) pq[mm] = wave_sum(pq[mm]);
+    for (int mm = 0; mm < MAXB; ++mm) pq[mm] = wave_total(pq[mm]);
     if (lane == 0) {
 #pragma unroll
       for (int mm = 0; mm < MAXB; ++mm) scratch[wave * DS_MAXB + mm] = pq[mm];
@@ -736,7 +748,7 @@ __device__ __forceinline__ bool stage(const f16* X, int M, int K, int KT, f16* x
   }
   // The INT4 products below multiply by the stored codes q + 8 and take 8 * sum(x) off at the end.
 #pragma unroll
-  for (int mm = 0; mm < MAXB; ++mm) ps[mm] = wave_sum(ps[mm]);
+  for (int mm = 0; mm < MAXB; ++mm) ps[mm] = wave_total(ps[mm]);
   if (lane == 0) {
 #pragma unroll
     for (int mm = 0; mm < MAXB; ++mm) scratch[DS_XSUM + wave * DS_MAXB + mm] = ps[mm];
@@ -1411,8 +1423,10 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                            red_buf, scratch + DS_XSUM, TRACE_AT(15));
     }
     TRACE(16);
+#if !(DS_X2 & 3)
     load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
     load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+#endif
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
     // ---- RMSNorm + gate/up + SwiGLU.  Requests the remaining down tiles once the first unit has been
@@ -1423,16 +1437,29 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w, TRACE_AT(23));
     if (!alive) break;
     TRACE(6);
+#if (DS_X2 & 1)
+    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+#elif (DS_X2 & 2)
+    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+#endif
     {
       f16* act = a.act + (size_t)li * M * a.ffn;
       f32x4 gsum[2];
       slots_product<2, T, S_GU0>(S, gsum, wg, nb_f, KT_D, M, xs, xstride);
       stash_gate_up<U_F>(gsum, 0, M, red, red_buf);
+#if (DS_X2 & 2)
+      load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+#else
       load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+#endif
       if constexpr (U_F > 1) {
         slots_product<2, T, S_GU1>(S, gsum, wg + G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 1, M, red, red_buf);
       }
+#if (DS_X2 & 2)
+      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
+#endif
       if constexpr (U_F > 2) {
         slots_product<2, T, S_GU2>(S, gsum, wg + 2 * G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 2, M, red, red_buf);
@@ -1445,7 +1472,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
     TRACE(18);
+#if !(DS_X2 & 4)
     load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+#endif
     TRACE(7);
     // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
 #ifdef DS_TRACE
@@ -1454,6 +1483,9 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w, TRACE_AT(26));
     if (!alive) break;
     TRACE(22);
+#if (DS_X2 & 4)
+    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
+#endif
     load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
