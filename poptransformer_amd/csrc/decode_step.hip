@@ -44,9 +44,6 @@
 
 namespace {
 
-#ifndef DS_X2
-#define DS_X2 0
-#endif
 constexpr int DS_WAVES = 16;
 constexpr int DS_THREADS = DS_WAVES * 64;
 constexpr unsigned DS_SPIN_LIMIT = 1u << 20;
@@ -778,15 +775,19 @@ __device__ __forceinline__ void normw_fetch(const f16* w, f16* lds_w, int d) {
 // delivers at twice the rate of sixteen 64-byte pieces of sixteen rows.
 __device__ __forceinline__ size_t grouped_at(int m, int n) { return (size_t)(n >> 3) * 128 + m * 8 + (n & 7); }
 
-// merges the online-softmax state of the lane `o` lanes away into this lane's
-__device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8], int o) {
-  const float mo = __shfl_xor(m, o, 64), lo = __shfl_xor(l, o, 64);
+// merges the online-softmax state of the lane O (16 or 32) lanes away into this lane's
+template <int O>
+__device__ __forceinline__ void merge_lanes(float& m, float& l, float (&acc)[8]) {
+  static_assert(O == 16 || O == 32, "row or half of the wave");
+  // (the row / half swaps of gfx950 in place of these shuffles were measured: 2 % slower per step at batch 1)
+  auto other = [](float v) { return __shfl_xor(v, O, 64); };
+  const float mo = other(m), lo = other(l);
   const float mn = fmaxf(m, mo);
   const float ca = m == -INFINITY ? 0.f : __expf(m - mn);
   const float cb = mo == -INFINITY ? 0.f : __expf(mo - mn);
   l = l * ca + lo * cb;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = acc[e] * ca + __shfl_xor(acc[e], o, 64) * cb;
+  for (int e = 0; e < 8; ++e) acc[e] = acc[e] * ca + other(acc[e]) * cb;
   m = mn;
 }
 
@@ -964,8 +965,8 @@ __device__ __forceinline__ void attention_unit(const DsArgs& a, int li, f16* kri
       }
     }
     // the four row groups of a wave merge in registers, the sixteen waves in LDS
-    merge_lanes(m, l, acc, 16);
-    merge_lanes(m, l, acc, 32);
+    merge_lanes<16>(m, l, acc);
+    merge_lanes<32>(m, l, acc);
     if (lane == 0) { sm_m[wave] = m; sm_l[wave] = l; }
     if (lane < LPP) {
 #pragma unroll
@@ -1134,8 +1135,8 @@ __device__ __forceinline__ void attention_two(const DsArgs& a, int li, f16* krin
         request(kp[it], vp[it], r0 + it + NPRE);
       }
     }
-    merge_lanes(m, l, acc, 16);
-    merge_lanes(m, l, acc, 32);
+    merge_lanes<16>(m, l, acc);
+    merge_lanes<32>(m, l, acc);
     if (lane == 0) { sm_m[wave] = m; sm_l[wave] = l; }
     if (lane < LPP) {
 #pragma unroll
@@ -1423,10 +1424,8 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
                                                            red_buf, scratch + DS_XSUM, TRACE_AT(15));
     }
     TRACE(16);
-#if !(DS_X2 & 3)
     load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
     load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-#endif
     normw_fetch(L.get<const f16>(P_N2), normw, a.d);
     TRACE(5);
     // ---- RMSNorm + gate/up + SwiGLU.  Requests the remaining down tiles once the first unit has been
@@ -1437,29 +1436,16 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_D, MAXB>(x_mid, M, a.d, KT_D, xs, xstride, normw, a.eps, scratch, w, TRACE_AT(23));
     if (!alive) break;
     TRACE(6);
-#if (DS_X2 & 1)
-    load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-#elif (DS_X2 & 2)
-    load_slots<3, T, S_QKV, C_QKV, 2 * T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-#endif
     {
       f16* act = a.act + (size_t)li * M * a.ffn;
       f32x4 gsum[2];
       slots_product<2, T, S_GU0>(S, gsum, wg, nb_f, KT_D, M, xs, xstride);
       stash_gate_up<U_F>(gsum, 0, M, red, red_buf);
-#if (DS_X2 & 2)
-      load_slots<1, TPW_F, S_D, C_D, 0, D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-#else
       load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-#endif
       if constexpr (U_F > 1) {
         slots_product<2, T, S_GU1>(S, gsum, wg + G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 1, M, red, red_buf);
       }
-#if (DS_X2 & 2)
-      load_slots<1, TPW_F, S_D, C_D, D_EARLY, TPW_F - D_EARLY>(S, SC, md, wg, nb_d, a.d, KT_F);
-#endif
       if constexpr (U_F > 2) {
         slots_product<2, T, S_GU2>(S, gsum, wg + 2 * G, nb_f, KT_D, M, xs, xstride);
         stash_gate_up<U_F>(gsum, 2, M, red, red_buf);
@@ -1472,9 +1458,7 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
       finish_gate_up<U_F, MAXB>(sg, su, act, a.ffn, wg, G, nb_f, M, red, red_buf, scratch + DS_XSUM);
     }
     TRACE(18);
-#if !(DS_X2 & 4)
     load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-#endif
     TRACE(7);
     // ---- down + residual.  Requests the next layer's k and the next RMSNorm weights.
 #ifdef DS_TRACE
@@ -1483,9 +1467,6 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_kernel(DsArgs a) {
     alive = stage<NS_F, MAXB>(a.act + (size_t)li * M * a.ffn, M, a.ffn, KT_F, xs, xstride, nullptr, 0.f, scratch, w, TRACE_AT(26));
     if (!alive) break;
     TRACE(22);
-#if (DS_X2 & 4)
-    load_slots<3, T, S_QKV, C_QKV, 0, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
-#endif
     load_slots<3, T, S_QKV, C_QKV, T, T>(S, SC, m3n, wg, nb_d, a.d, KT_D);
     TRACE(8);
     {
