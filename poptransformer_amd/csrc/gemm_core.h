@@ -1365,6 +1365,114 @@ static int launch_gemm_rows(const GemmArgs& a, int total_nb, hipStream_t s, cons
   return PTA_OK;
 }
 
+// The sums of a wave's tile (RG row groups x NST channel blocks; lane l holds channels st * 16 + (l / 16) * 4 + r of
+// row l % 16 of each row group) go out: unit cw of the workgroup, first block blk0 of matrix mi, rows from row0.
+template <class Fmt, int NST, int RG, bool PAIR>
+__device__ __forceinline__ void panel_store(const GemmArgs& a, f32x4 (&acc)[RG][NST], unsigned char* smem, int cw, int mi, int blk0,
+                                            int row0, int nsl, typename Fmt::Scale s0, typename Fmt::Scale s1) {
+  constexpr int SW = NST * 16 + 4;                // floats per row of a wave's epilogue strip
+  const int lane = threadIdx.x & 63;
+  const int M = a.M;
+  // Lane l holds channels st * 16 + (l / 16) * 4 + r of row l % 16 of each row group.  Row group by row group the
+  // sums pass through a strip of LDS of the wave's own (the row buffers are free after the last barrier) and come
+  // back with eight consecutive channels of one row per lane: one 16-byte store per lane, whole 128-byte stretches
+  // of a row per wave.  (A wave's LDS accesses complete in order.)
+  float* strip = reinterpret_cast<float*>(smem) + (size_t)cw * (16 * SW);
+  const GemmMat& mat = a.mat[PAIR ? 0 : mi];
+  const int N = mat.N;
+  const bool direct = !mat.bias && mat.act == PTA_ACT_NONE && !a.epi.bias && a.epi.act == PTA_ACT_NONE && !a.epi.mul &&
+                      a.epi.post_scale == 0.0f && !a.epi.out_fp8_scale;
+  auto put = [&](const f32x4 (&sums)[NST]) {
+#pragma unroll
+    for (int st = 0; st < NST; ++st)
+      *reinterpret_cast<f32x4*>(strip + (lane & 15) * SW + st * 16 + (lane >> 4) * 4) = sums[st];
+  };
+  // (one copy of the epilogue code: unrolled over the row groups it is too large to unroll, and an accumulator
+  // array indexed by a loop counter lives in scratch memory for the whole kernel - hence the chain of comparisons)
+#pragma unroll 1
+  for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+    for (int r = 0; r < RG; ++r)
+      if (r == rg) put(acc[r]);
+    if constexpr (PAIR) {
+      constexpr int LPR = NST / 2 * 16 / 8;                      // lanes per row: eight output channels each
+      constexpr int RPP = 64 / LPR;                              // rows per pass
+#pragma unroll 1
+      for (int it = 0; it < 16 / RPP; ++it) {
+        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
+        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
+        if (rr >= 16) continue;
+        const f32x4 g0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), g1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
+        const f32x4 u0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0), u1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0 + 4);
+        if (m >= M) continue;
+        f16x8 y;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          y[j] = swiglu_out(a.epi, (f16)Fmt::finish(j < 4 ? g0[j & 3] : g1[j & 3], s0), (f16)Fmt::finish(j < 4 ? u0[j & 3] : u1[j & 3], s1));
+        if (n + 8 <= N && (N & 7) == 0) {
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
+        }
+      }
+    } else {
+      constexpr int LPR = NST * 16 / 8;
+      constexpr int RPP = 64 / LPR;
+#pragma unroll 1
+      for (int it = 0; it < (16 + RPP - 1) / RPP; ++it) {
+        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
+        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
+        if (rr >= 16) continue;
+        const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), v1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
+        if (m >= M) continue;
+        if (nsl > 1) {
+          float* p = a.part + ((size_t)blockIdx.y * M + m) * N + n;
+          if (n + 8 <= N && (N & 3) == 0) {
+            *reinterpret_cast<f32x4*>(p) = v0;
+            *reinterpret_cast<f32x4*>(p + 4) = v1;
+          } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              if (n + j < N) p[j] = j < 4 ? v0[j & 3] : v1[j & 3];
+          }
+          continue;
+        }
+        f16x8 y;
+        if (direct && n + 8 <= N && (N & 7) == 0) {                // nothing but the residual stream to add: whole vectors
+          f16x8 res;
+          if (a.epi.residual) res = *reinterpret_cast<const f16x8*>(a.epi.residual + (size_t)m * N + n);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            y[j] = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
+            if (a.epi.residual) y[j] = y[j] + res[j];
+          }
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+          continue;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          f16 y0 = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
+          if (n + j < N) {
+            if (mat.bias) y0 = y0 + mat.bias[n + j];
+            y0 = apply_act(mat.act, y0);
+            y0 = apply_epilogue(a.epi, y0, m, n + j, N);
+          }
+          y[j] = y0;
+        }
+        if (n + 8 <= N && (N & 7) == 0) {
+          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j)
+            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
+        }
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // Variant for hundreds of rows: the roles turned round.  The tiled weight format IS the A operand order, so a
 // wave fetches the tiles of its own NST channel blocks straight into registers (1 KiB per instruction, no LDS)
@@ -1568,106 +1676,9 @@ __global__ __launch_bounds__(PANEL_WAVES * 64) __attribute__((amdgpu_waves_per_e
   }
   if (!active) return;
 
-  // Lane l holds channels st * 16 + (l / 16) * 4 + r of row l % 16 of each row group.  Row group by row group the
-  // sums pass through a strip of LDS of the wave's own (the row buffers are free after the last barrier) and come
-  // back with eight consecutive channels of one row per lane: one 16-byte store per lane, whole 128-byte stretches
-  // of a row per wave.  (A wave's LDS accesses complete in order.)
-  float* strip = reinterpret_cast<float*>(smem) + (size_t)cw * (16 * SW);
-  const GemmMat& mat = a.mat[PAIR ? 0 : mi];
-  const int N = mat.N;
-  const bool direct = !mat.bias && mat.act == PTA_ACT_NONE && !a.epi.bias && a.epi.act == PTA_ACT_NONE && !a.epi.mul &&
-                      a.epi.post_scale == 0.0f && !a.epi.out_fp8_scale;
   const typename Fmt::Scale s0 = Fmt::load_scale(a.mat[PAIR ? 0 : mi].scale, a.x_scale, 0, 1);   // no format's finish uses the per-channel part
   const typename Fmt::Scale s1 = Fmt::load_scale(a.mat[PAIR ? 1 : mi].scale, a.x_scale, 0, 1);
-  auto put = [&](const f32x4 (&sums)[NST]) {
-#pragma unroll
-    for (int st = 0; st < NST; ++st)
-      *reinterpret_cast<f32x4*>(strip + (lane & 15) * SW + st * 16 + (lane >> 4) * 4) = sums[st];
-  };
-  // (one copy of the epilogue code: unrolled over the row groups it is too large to unroll, and an accumulator
-  // array indexed by a loop counter lives in scratch memory for the whole kernel - hence the chain of comparisons)
-#pragma unroll 1
-  for (int rg = 0; rg < RG; ++rg) {
-#pragma unroll
-    for (int r = 0; r < RG; ++r)
-      if (r == rg) put(acc[r]);
-    if constexpr (PAIR) {
-      constexpr int LPR = NST / 2 * 16 / 8;                      // lanes per row: eight output channels each
-      constexpr int RPP = 64 / LPR;                              // rows per pass
-#pragma unroll 1
-      for (int it = 0; it < 16 / RPP; ++it) {
-        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
-        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
-        if (rr >= 16) continue;
-        const f32x4 g0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), g1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
-        const f32x4 u0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0), u1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + NST / 2 * 16 + c0 + 4);
-        if (m >= M) continue;
-        f16x8 y;
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          y[j] = swiglu_out(a.epi, (f16)Fmt::finish(j < 4 ? g0[j & 3] : g1[j & 3], s0), (f16)Fmt::finish(j < 4 ? u0[j & 3] : u1[j & 3], s1));
-        if (n + 8 <= N && (N & 7) == 0) {
-          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
-        }
-      }
-    } else {
-      constexpr int LPR = NST * 16 / 8;
-      constexpr int RPP = 64 / LPR;
-#pragma unroll 1
-      for (int it = 0; it < (16 + RPP - 1) / RPP; ++it) {
-        const int rr = it * RPP + lane / LPR, c0 = (lane % LPR) * 8;
-        const int m = row0 + rg * 16 + rr, n = blk0 * 16 + c0;
-        if (rr >= 16) continue;
-        const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0), v1 = *reinterpret_cast<const f32x4*>(strip + rr * SW + c0 + 4);
-        if (m >= M) continue;
-        if (nsl > 1) {
-          float* p = a.part + ((size_t)blockIdx.y * M + m) * N + n;
-          if (n + 8 <= N && (N & 3) == 0) {
-            *reinterpret_cast<f32x4*>(p) = v0;
-            *reinterpret_cast<f32x4*>(p + 4) = v1;
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-              if (n + j < N) p[j] = j < 4 ? v0[j & 3] : v1[j & 3];
-          }
-          continue;
-        }
-        f16x8 y;
-        if (direct && n + 8 <= N && (N & 7) == 0) {                // nothing but the residual stream to add: whole vectors
-          f16x8 res;
-          if (a.epi.residual) res = *reinterpret_cast<const f16x8*>(a.epi.residual + (size_t)m * N + n);
-#pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            y[j] = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
-            if (a.epi.residual) y[j] = y[j] + res[j];
-          }
-          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
-          continue;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          f16 y0 = (f16)Fmt::finish(j < 4 ? v0[j & 3] : v1[j & 3], s0);
-          if (n + j < N) {
-            if (mat.bias) y0 = y0 + mat.bias[n + j];
-            y0 = apply_act(mat.act, y0);
-            y0 = apply_epilogue(a.epi, y0, m, n + j, N);
-          }
-          y[j] = y0;
-        }
-        if (n + 8 <= N && (N & 7) == 0) {
-          *reinterpret_cast<f16x8*>(mat.Y + (size_t)m * N + n) = y;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            if (n + j < N) mat.Y[(size_t)m * N + n + j] = y[j];
-        }
-      }
-    }
-  }
+  panel_store<Fmt, NST, RG, PAIR>(a, acc, smem, cw, mi, blk0, row0, nsl, s0, s1);
 }
 
 // whether every matrix of the launch is a whole number of wave tiles of `nst` channel blocks and all share one input

@@ -26,7 +26,20 @@ static bool fp8_native_enabled() {
   return on;
 }
 
-// x_bytes: X holds F143 bytes [M, K] instead of fp16 values (FP8 weights of format F143 only)
+// The FP8 instruction's many-row kernel takes launches of more rows than this.  Up to 64 rows a launch is bound by
+// the weights' way from memory and the fp16 instruction's kernels for few rows are as fast or faster (measured at
+// 32 and 64 rows: 13 and 23 against 27 and 38 us for q | kv of the ChatGLM2-6B shape, 28 and 46 against 33 and 44
+// for the gate / up pair).  PTA_FP8_PANEL_MIN_ROWS in the environment overrides it (for comparisons); read once.
+static int f8n_panel_min_rows() {
+  static const int rows = [] {
+    const char* v = getenv("PTA_FP8_PANEL_MIN_ROWS");
+    return v ? atoi(v) : 64;
+  }();
+  return rows;
+}
+
+// x_bytes: 1 - X holds F143 bytes [M, K] instead of fp16 values (FP8 weights of format F143 only); 2 - fp16 values with
+// an exponent (x_scale) that are not known to lie on the F143 grid (they keep to the fp16 instruction)
 static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int count, const pta_weight* host_w,
                        const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
                        const pta_fusion* fuse, pta_stream_t stream) {
@@ -80,12 +93,15 @@ static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int c
   // So fp16 grid values come here for a SwiGLU pair outside that kernel's shapes only; an uint8 left-hand side always.
   const bool several = swiglu != 0;
   const bool stream_pair = several && !x_bytes && stream_fits(a) && nb >= device_compute_units();
-  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes || (fp8_native_enabled() && several && !stream_pair))) {
+  if (kind == PTA_W_F143 && f8n_fits(a) && (x_bytes == 1 || (x_bytes == 0 && fp8_native_enabled() && several && !stream_pair))) {
     if (x_bytes) return swiglu ? dispatch_gemv_f8n<true, true>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, true>(a, nb, s, "pta_linear");
     return swiglu ? dispatch_gemv_f8n<true, false>(a, nb, s, "pta_linear") : dispatch_gemv_f8n<false, false>(a, nb, s, "pta_linear");
   }
   a.prefer_stream = stream_pair && (kind == PTA_W_F143 || kind == PTA_W_F152);
-  PTA_REQUIRE(!x_bytes, "pta_linear: an uint8 left-hand side needs F143 weights, M <= 16 and K >= 1024");
+  PTA_REQUIRE(x_bytes != 1, "pta_linear: an uint8 left-hand side needs F143 weights, M <= 16 and K >= 1024");
+  // more than 16 rows of F143-grid values by F143 weights (a prompt pass): the 16x16x128 FP8 instruction
+  if (kind == PTA_W_F143 && x_bytes == 0 && fp8_native_enabled() && f8n_panel_fits(a, swiglu != 0) && M > f8n_panel_min_rows())
+    return swiglu ? dispatch_f8n_panel<true>(a, nb, s, "pta_linear") : dispatch_f8n_panel<false>(a, nb, s, "pta_linear");
   switch (kind) {
     case PTA_W_INT4: return run_linear<FmtW4>(a, nb, swiglu, s, "pta_linear");
     case PTA_W_F16: return run_linear<FmtF16>(a, nb, swiglu, s, "pta_linear");
@@ -167,5 +183,6 @@ extern "C" int pta_fp8_gemm(const void* lhs, int lhs_is_fp8, const void* tiled_r
     xs = scale_lhs;
   }
   pta_weight w{format_rhs == PTA_F143 ? PTA_W_F143 : PTA_W_F152, tiled_rhs, scale_rhs, N, K, nullptr, PTA_ACT_NONE};
-  return pta_linear((const pta_half*)X, xs, 1, &w, nullptr, &Y, M, 0, fuse, stream);
+  // a decoded left-hand side lies on its own format's grid; an fp16 one is multiplied as it is (no x_scale)
+  return linear_impl(X, xs, lhs_is_fp8 && format_lhs != PTA_F143 ? 2 : 0, 1, &w, nullptr, &Y, M, 0, fuse, stream);
 }

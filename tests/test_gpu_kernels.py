@@ -1227,6 +1227,70 @@ def test_fp8_products_pair_multi_and_nan(K):
     assert np.abs(got[ok].astype(np.float64) - ref[ok].astype(np.float64)).max() <= 2.0 ** -10 * np.abs(ref[ok].astype(np.float64)).max()
 
 
+@pytest.mark.parametrize("M,Kdim,N", [(M, Kdim, N) for M in (48, 65, 200, 256, 1024)
+                                      for Kdim, N in ((4096, 4096), (1160, 8192), (2048, 512), (1024, 100))] + [(2048, 1024, 8192)])
+@pytest.mark.parametrize("specials", [False, True])
+def test_fp8_products_of_many_rows_on_the_fp8_matrix_instruction(K, M, Kdim, N, specials):
+    """Both operands F143, more than 64 rows (a prompt pass): the 16x16x128 FP8 instruction with the activations turned
+    into bytes on their way to LDS.  The shapes reach all five forms of the kernel - row blocks of 128 rows (2048 x
+    1024 x 8192), of 64 (1024 x 1160 x 8192; with K in halves 1024 x 4096 x 4096) and of 32 (200 x 1160 x 8192; in
+    halves 200 x 4096 x 4096) -, ragged last row blocks (65, 200) and feature tiles (1160), a channel count outside
+    the kernel's tiles (100) and a row count below it (48), which take the fp16 instruction's paths; +-240, stretches
+    of them, and the smallest subnormals in both operands.  Left-hand side as fp16 values on the grid and as bytes;
+    within one fp16 rounding of the largest output of the oracle's product."""
+    rng = np.random.default_rng(M + Kdim + N)
+    scale = -1
+    x8, w8 = _f143_case(rng, M, Kdim, N, scale, specials)
+    if specials:
+        x8[M // 2, :64] = 0x7F                 # a stretch of saturated activations, and rows of them in other row groups
+        x8[M - 1, Kdim - 40:] = 0xFF
+        x8[16, 129] = 0xFF
+    sd = dev(np.array([scale], np.int32))
+    fw = K.F8Weight(dev(w8), sd, "F143", kn=True)
+    ref = O.fp8_matmul(x8, w8, [scale], [scale], "F143", "F143")
+    tol = 2.0 ** -10 * np.abs(ref.astype(np.float64)).max()
+    xg = dev(O.f8_decode(x8, "F143", 0, np.float16))
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    K.linear(xg, [fw], [out], x_scale=sd)
+    assert np.abs(host(out).astype(np.float64) - ref.astype(np.float64)).max() <= tol
+    got = host(K.fp8_gemm(dev(x8), fw, K.fp8_gemm_workspace(M, Kdim, "cuda"), x_scale=sd, x_format="F143"))
+    assert np.abs(got.astype(np.float64) - ref.astype(np.float64)).max() <= tol
+
+
+@pytest.mark.parametrize("M", [100, 200])
+def test_fp8_products_of_many_rows_pair_multi_and_nan(K, M):
+    rng = np.random.default_rng(79 + M)
+    Kdim, N, scale = 2048, 1408, -2
+    sd = dev(np.array([scale], np.int32))
+    x8, wg8 = _f143_case(rng, M, Kdim, N, scale, True)
+    _, wu8 = _f143_case(rng, M, Kdim, N, scale, True)
+    xg = dev(O.f8_decode(x8, "F143", 0, np.float16))
+    g, u = K.F8Weight(dev(wg8), sd, "F143", kn=True), K.F8Weight(dev(wu8), sd, "F143", kn=True)
+    out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    K.linear(xg, [g, u], [out, out], x_scale=sd, swiglu=True)
+    rg, ru = (O.fp8_matmul(x8, w, [scale], [scale]) for w in (wg8, wu8))
+    ref = (ru * O.swish(rg)).astype(np.float16)
+    assert rel_err(host(out), ref) <= 1e-2
+    # two matrices of different widths in one launch, each with a bias; a residual on a single one
+    _, w2 = _f143_case(rng, M, Kdim, 512, scale, True)
+    b1, b2 = rng.standard_normal(N).astype(np.float16), rng.standard_normal(512).astype(np.float16)
+    o1, o2 = torch.empty((M, N), dtype=torch.float16, device="cuda"), torch.empty((M, 512), dtype=torch.float16, device="cuda")
+    K.linear(xg, [g, K.F8Weight(dev(w2), sd, "F143", kn=True)], [o1, o2], biases=[dev(b1), dev(b2)], x_scale=sd)
+    assert rel_err(host(o1), (rg + b1).astype(np.float16)) <= 1e-2
+    assert rel_err(host(o2), (O.fp8_matmul(x8, w2, [scale], [scale]) + b2).astype(np.float16)) <= 1e-2
+    # the NaN code: as a weight it poisons its output channel, as an activation its row - and nothing else
+    wn, xn = wg8.copy(), x8.copy()
+    wn[900, 33] = 0x80
+    xn[M - 2, 1000] = 0x80
+    got = host(K.fp8_gemm(dev(xn), K.F8Weight(dev(wn), sd, "F143", kn=True), K.fp8_gemm_workspace(M, Kdim, "cuda"),
+                          x_scale=sd, x_format="F143"))
+    with np.errstate(invalid="ignore"):
+        ref = O.fp8_matmul(xn, wn, [scale], [scale])
+    assert np.array_equal(np.isnan(got), np.isnan(ref)) and np.isnan(ref[M - 2]).all() and np.isnan(ref[:, 33]).all()
+    ok = ~np.isnan(ref)
+    assert np.abs(got[ok].astype(np.float64) - ref[ok].astype(np.float64)).max() <= 2.0 ** -10 * np.abs(ref[ok].astype(np.float64)).max()
+
+
 # ---------------------------------------------------------------- more than 64 rows
 @pytest.mark.parametrize("M", [65, 128, 200, 256, 600, 1024])
 @pytest.mark.parametrize("Kdim,N", [(4096, 4096), (1160, 8192), (11008, 4096), (512, 100)])
