@@ -388,7 +388,8 @@ typedef struct pta_weight {
 
 /* Y_i[M, N_i] = fp16(X' @ W_i) + bias_i for `count` (1..4) weights of one kind and one K in one
  * launch; with swiglu != 0 (count == 2: gate, up) Y_0 = fp16(up * swish(gate)).  x_scale (FP8
- * weights only, may be NULL): X holds unscaled FP8-grid values whose device int32 exponent it is.
+ * weights only, may be NULL): X holds unscaled values on the weights' FP8 grid, whose device int32 exponent it is
+ * (from 65 rows on, F143 weights and such an X are multiplied as bytes on the FP8 matrix instruction).
  * host_bias may be NULL.  With count == 1 all of `fuse` applies, otherwise its norm fields. */
 int pta_linear(const pta_half* X, const int32_t* x_scale, int count, const pta_weight* host_w,
                const pta_half* const* host_bias, pta_half* const* host_Y, int M, int swiglu,
