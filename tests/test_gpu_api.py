@@ -189,6 +189,44 @@ def test_rwkv_through_the_operator_api(int4):
            lambda: OM.RWKVOracle(sd, RWKV, L, B), ids, extra={"state_dict_is_processed": True})
 
 
+@pytest.mark.parametrize("family", ["llama2-int4", "chatglm2-fp8"])
+def test_a_vocabulary_of_32k_reaches_the_fused_executors(family):
+    """With tens of thousands of logits (and, for `fp8`, activations on a 3-bit grid) two of them come within a last-bit
+    difference of each other after a few tokens, so a check on tokens alone would keep such a graph on the
+    interpreter.  The compiler checks the executors' logits against the graph's instead: a strict session compiles -
+    INT4 Llama 2 to the one-launch iteration -, and its tokens equal the interpreter's up to the oracle's first near
+    tie."""
+    B, L, steps, pad, eos = 2, 32, 16, 0, 2
+    if family == "llama2-int4":
+        from poptransformer_amd.models.llama2 import LLAMA2DecModel as model_cls
+        cfg = dict(LLAMA, vocab_size=32000)
+        sd = OM.make_llama2_state_dict(cfg, seed=25, int4=True)
+        oracle, precision, kind, vocab, extra = OM.Llama2Oracle(sd, cfg, L, B), "int4", "fused:llama2:persistent", 32000, {}
+    else:
+        from poptransformer_amd.models.chatglm2 import ChatGLM2DecModel as model_cls
+        cfg = dict(GLM2, padded_vocab_size=32000)
+        sd = OM.make_chatglm2_state_dict(cfg, seed=26)
+        oracle, precision, kind, vocab, extra = OM.ChatGLM2Oracle(sd, cfg, L, B, "fp8"), "fp8", "fused:chatglm2", 32000, {}
+    ids = _ids(np.random.default_rng(500), B, L, 5, vocab, pad)
+    trace = []
+    OM.run_decode_loop(oracle, ids, L, steps, pad, eos, trace=trace)
+    cols = L
+    for t, (_, logits) in enumerate(trace):
+        top2 = np.sort(logits.astype(np.float32), axis=1)[:, -2:]
+        if (top2[:, 1] - top2[:, 0] < (0.05 if precision == "fp8" else 0.005) * np.abs(logits).max()).any():
+            cols = t + 1
+            break
+    outs = []
+    for allow_fused in (False, True):
+        kw = dict(hf_config=cfg, state_dict=sd, pad_token_id=pad, eos_token_id=eos, max_length=L, max_loop=steps, **extra)
+        session, model = _session(model_cls, precision, B, kw, allow_fused, **({"strict": True} if allow_fused else {}))
+        assert session.executor_kind == (kind if allow_fused else "interpreter"), getattr(session.session.executor, "persistent_reason", None)
+        session.run(model.build_input_dict(input_ids=[list(r[r != pad]) for r in ids]))
+        out = model.build_output_dict(session.anchor_arrays)
+        outs.append(np.stack([out["output"][str(i)] for i in range(B)]))
+    assert np.array_equal(outs[0][:, :cols], outs[1][:, :cols])
+
+
 def test_early_stop_and_unknown_graphs_stay_on_the_interpreter():
     from poptransformer_amd.models.llama2 import LLAMA2DecModel
     B, L, pad = 2, 24, 0
