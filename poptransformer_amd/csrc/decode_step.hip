@@ -1576,6 +1576,33 @@ __device__ __forceinline__ void load_xtile(const f16* X, int M, int K, int kt, X
   }
 }
 
+// The same fragments requested into a wave's 4 KiB of LDS instead of registers (no register is held while they are
+// on their way), and read back from there: vector j of lane l lies at j KiB + 16 l.
+__device__ __forceinline__ void load_xtile_lds(const f16* X, int M, int K, int kt, float* slot) {
+  const int lane = lane_id();
+  const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16*>(X), 0, ((K + 127) / 128) * (16 * 128 * 2), 0x00020000);
+  int no_row = (lane & 15) < M ? 0 : -1;
+  asm volatile("" : "+v"(no_row));
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int no_k = kt * 128 + j * 32 + (lane >> 4) * 8 < K ? 0 : -1;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (__attribute__((address_space(3))) void*)(slot + j * 256), 16,
+                                             ((kt * 4 + j) * 64 + lane) * 16 | no_row | no_k, 0, 0, 0);
+  }
+}
+__device__ __forceinline__ void read_xtile_lds(const float* slot, XTile& t) {
+  const int lane = lane_id();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) t.v[j] = *reinterpret_cast<const f16x8*>(slot + j * 256 + lane * 4);
+}
+// waits until at most n of this wave's vector memory loads are in flight (n: 0, 4 or 8 - a constant wherever the
+// caller's loop is unrolled)
+__device__ __forceinline__ void wait_loads_but(int n) {
+  if (n >= 8) __builtin_amdgcn_s_waitcnt(0x0f70 | 8);
+  else if (n >= 4) __builtin_amdgcn_s_waitcnt(0x0f70 | 4);
+  else __builtin_amdgcn_s_waitcnt(0x0f70);
+}
+
 // sums over the lane groups that share a row: afterwards lanes 0..15 (and their images) hold the row's total of the wave
 __device__ __forceinline__ float rows_of_wave(float v) {
   v += __shfl_xor(v, 16, 64);
@@ -2003,15 +2030,38 @@ __global__ __launch_bounds__(DS_THREADS) void decode_step_wide_kernel(DsArgs a) 
       f16 sv[1] = {};
       if (wave == 0) { const Mat mm[1] = MD; request_scales<1>(mm, wg, nb_d, a.d, sv); }
       await_row(phase_rows(4 * li + 3), a.flag_words, G, wg, w);
+      // Two tiles' fragments are on their way at any time: the even tiles into registers, the odd ones into 4 KiB
+      // of LDS per wave - the reduction buffer the last gate/up unit used and the part of the current one beyond
+      // this phase's single matrix, both idle here.  (One tile ahead, in registers alone, left the phase waiting a
+      // round trip per tile.)  A wave's loads return in order, so a wait names how many younger loads may still
+      // be out: the next even tile's four and, at the third tile, the next layer's four weight tiles as well.
       XTile ahead;
+      float* const slot = wave < 12 ? red + (red_buf ^ 1) * DW_RED + wave * 1024 : red + red_buf * DW_RED + 4096 + (wave - 12) * 1024;
       load_xtile(actx, M, a.ffn, wave, ahead);
+      if constexpr (TPW_F > 1) load_xtile_lds(actx, M, a.ffn, wave + DS_WAVES, slot);
       if (wave == 0) keep_scales<1>(sv, scl + DW_SCL);      // requested before the arrival row: here by now
-      { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 2 * T, T>(S, mm, wg, nb_d, KT_D); }      // the next layer's v and q
-      { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 0, T>(S, mm, wg, nb_d, KT_D); }
+      if constexpr (TPW_F == 1) {
+        { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 2 * T, T>(S, mm, wg, nb_d, KT_D); }      // the next layer's v and q
+        { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 0, T>(S, mm, wg, nb_d, KT_D); }
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TPW_F; ++i) {
-        const XTile x1 = ahead;
-        if (i + 1 < TPW_F) load_xtile(actx, M, a.ffn, wave + (i + 1) * DS_WAVES, ahead);      // (a tile beyond the last: zeros)
+        XTile x1;
+        if (i % 2 == 0) {
+          x1 = ahead;
+          if (i + 2 < TPW_F) load_xtile(actx, M, a.ffn, wave + (i + 2) * DS_WAVES, ahead);      // (a tile beyond the last: zeros)
+        } else {
+          wait_loads_but((i + 1 < TPW_F ? 4 : 0) + (i == 3 ? 2 * T : 0));
+          read_xtile_lds(slot, x1);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // read before the slot is requested again
+          if (i + 2 < TPW_F) load_xtile_lds(actx, M, a.ffn, wave + (i + 2) * DS_WAVES, slot);
+          if (i == 1) {
+            { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 2 * T, T>(S, mm, wg, nb_d, KT_D); }      // the next layer's v and q
+            { const Mat mm[3] = M3N; load_tiles<3, T, S_QKV, 0, T>(S, mm, wg, nb_d, KT_D); }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (wave + i * DS_WAVES < KT_F) {
           const XTile one[1] = {x1};
           s1 += xtiles_rowsum<1>(one);
