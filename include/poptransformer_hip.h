@@ -99,6 +99,13 @@ typedef struct pta_fusion {
   const int32_t* out_fp8_scale;/* NULL, or: leave the result on the FP8 grid of this device exponent, as the
                                   half_to_uint8 of the Linear that consumes it would (pta_half_to_fp8_grid)   */
   int out_fp8_format;          /* PTA_F143 / PTA_F152                           */
+  pta_half* mix_state;         /* NULL, or [2][M, K]: the (normalised) rows of the previous token, two copies used in
+                                  turn - the token shift of models/rwkv/attention.py:59-72 and ffn.py:47-51 done
+                                  inside the Linears that consume it: weight i with a `mix` vector w_i is fed
+                                  x * w_i + (1 - w_i) * prev (fp16 operations in that order, as pta_rwkv_mix), x being
+                                  X after the fused norm and prev copy (*mix_step & 1); the launch leaves x in the
+                                  other copy, which the next token's launch reads.  Up to 4 rows with M * K <= 20480 */
+  const int32_t* mix_step;     /* device int32: the loop's step counter (with mix_state)                              */
 } pta_fusion;
 
 size_t pta_linear_workspace_bytes(int M, int N);
@@ -384,6 +391,7 @@ typedef struct pta_weight {
   const pta_half* x;   /* NULL, or this weight's own input [M, K] instead of X (the three token-shift
                           mixes of models/rwkv/attention.py:69-71 feed three Linears)          */
   int act;             /* PTA_ACT_* applied to this weight's output in a multi-weight launch  */
+  const pta_half* mix; /* NULL, or this weight's token-shift mixing vector [K] (see pta_fusion.mix_state) */
 } pta_weight;
 
 /* Y_i[M, N_i] = fp16(X' @ W_i) + bias_i for `count` (1..4) weights of one kind and one K in one

@@ -26,7 +26,7 @@ NORM_NONE, NORM_RMS, NORM_LAYER = 0, 1, 2
 
 class Weight(ctypes.Structure):
     _fields_ = [("kind", c_int), ("tiled", c_void_p), ("scale", c_void_p), ("N", c_int), ("K", c_int),
-                ("x", c_void_p), ("act", c_int)]
+                ("x", c_void_p), ("act", c_int), ("mix", c_void_p)]
 
 
 W_INT4, W_F16, W_F143, W_F152 = 0, 1, 2, 3
@@ -54,7 +54,8 @@ class Fusion(ctypes.Structure):
                 ("norm", c_int),
                 ("norm_weight", c_void_p), ("norm_bias", c_void_p), ("norm_eps", c_float),
                 ("workspace", c_void_p), ("workspace_bytes", c_size_t),
-                ("out_fp8_scale", c_void_p), ("out_fp8_format", c_int)]
+                ("out_fp8_scale", c_void_p), ("out_fp8_format", c_int),
+                ("mix_state", c_void_p), ("mix_step", c_void_p)]
 
 
 # name -> (restype, argtypes); the order follows include/poptransformer_hip.h

@@ -20,6 +20,8 @@ struct GemmEpilogue {
   float norm_eps;
   const int32_t* out_fp8_scale;   // when set: the result is left on the FP8 grid of this exponent (unscaled)
   int out_fp8_format;
+  f16* mix_state;                 // [2][M, K] or null: the previous token's rows for the token-shift mixes (gemv_lds_kernel)
+  const int32_t* mix_step;
 };
 
 __device__ __forceinline__ f16 sigmoid_f16(f16 x) {
@@ -66,7 +68,7 @@ __device__ __forceinline__ f16 swiglu_out(const GemmEpilogue& e, f16 gate, f16 u
 }
 
 static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const char* name) {
-  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, nullptr, 0.f, PTA_NORM_NONE, nullptr, nullptr, 0.f, nullptr, PTA_F143};
+  *out = GemmEpilogue{nullptr, nullptr, PTA_ACT_NONE, nullptr, 0.f, PTA_NORM_NONE, nullptr, nullptr, 0.f, nullptr, PTA_F143, nullptr, nullptr};
   if (!in) return PTA_OK;
   PTA_REQUIRE(in->act >= PTA_ACT_NONE && in->act <= PTA_ACT_SIGMOID, "%s: unknown activation %d", name, in->act);
   PTA_REQUIRE(in->norm >= PTA_NORM_NONE && in->norm <= PTA_NORM_LAYER, "%s: unknown norm %d", name, in->norm);
@@ -79,6 +81,8 @@ static inline int make_epilogue(const pta_fusion* in, GemmEpilogue* out, const c
   PTA_REQUIRE(!in->out_fp8_scale || in->out_fp8_format == PTA_F143 || in->out_fp8_format == PTA_F152,
               "%s: unsupported fp8 format %d, it must be F143 or F152", name, in->out_fp8_format);
   out->out_fp8_scale = in->out_fp8_scale; out->out_fp8_format = in->out_fp8_format;
+  PTA_REQUIRE(!in->mix_state == !in->mix_step, "%s: mix_state and mix_step come together", name);
+  out->mix_state = (f16*)in->mix_state; out->mix_step = in->mix_step;
   return PTA_OK;
 }
 
@@ -98,6 +102,7 @@ struct GemmMat {
   const void* scale;   // fp16 [N] (INT4), device int32 exponent (FP8), unused (FP16)
   const f16* bias;     // [N] or null; used when the launch holds several matrices
   const f16* X;        // this matrix's own input, or null for the shared one
+  const f16* mix;      // this matrix's token-shift mixing vector [K], or null (with GemmEpilogue::mix_state)
   int act;             // activation of this matrix's output when the launch holds several
   f16* Y;
   int N;
@@ -279,6 +284,28 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
   {
     const int vec_per_row = KT * 16;               // 8-half vectors per padded row
     float ps[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
+    // What the norm and the token shift apply to this thread's FIRST vector (with one row of up to 8192 features its
+    // only one) is requested together with the rows: one round trip to memory instead of one per pass.
+    const int i0 = threadIdx.x;
+    const bool first = i0 < M * vec_per_row && (i0 % vec_per_row) * 8 < K;
+    const f16* mix_prev = nullptr;
+    f16* mix_next = nullptr;
+    const f16* mix_w = a.epi.mix_state ? a.mat[mi].mix : nullptr;
+    if (a.epi.mix_state) {
+      const int parity = a.epi.mix_step[0] & 1;
+      mix_prev = a.epi.mix_state + (size_t)parity * M * K;
+      mix_next = a.epi.mix_state + (size_t)(parity ^ 1) * M * K;
+    }
+    f16x8 gm0 = {0, 0, 0, 0, 0, 0, 0, 0}, bt0 = gm0, pv0 = gm0, wv0 = gm0;
+    if (first) {
+      const int m = i0 / vec_per_row, c = i0 % vec_per_row;
+      if (a.epi.norm != PTA_NORM_NONE) gm0 = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
+      if (a.epi.norm == PTA_NORM_LAYER) bt0 = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
+      if (mix_w) {
+        pv0 = *reinterpret_cast<const f16x8*>(mix_prev + (size_t)m * K + c * 8);
+        wv0 = *reinterpret_cast<const f16x8*>(mix_w + c * 8);
+      }
+    }
     for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
       const int m = i / vec_per_row, c = i % vec_per_row;
       f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -293,9 +320,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
       }
     }
     if (a.epi.norm != PTA_NORM_NONE) {
-      // per-row sums over the workgroup: wave shuffle, then LDS (the reduction buffer is free here)
+      // per-row sums over the workgroup: over the wave by data-parallel moves (a chain of six LDS-crossbar shuffles
+      // per sum took longer than the norm launch this replaces), then LDS (the reduction buffer is free here)
 #pragma unroll
-      for (int mm = 0; mm < 4; ++mm) { ps[mm] = wave_sum(ps[mm]); pq[mm] = wave_sum(pq[mm]); }
+      for (int mm = 0; mm < 4; ++mm)
+        if (mm < M) { ps[mm] = wave_total_dpp(ps[mm]); pq[mm] = wave_total_dpp(pq[mm]); }
       if (lane == 0) {
 #pragma unroll
         for (int mm = 0; mm < 4; ++mm) { red[(wave * 4 + mm) * 2] = ps[mm]; red[(wave * 4 + mm) * 2 + 1] = pq[mm]; }
@@ -309,13 +338,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 #pragma unroll
         for (int w = 0; w < NW; ++w) { sum += red[(w * 4 + m) * 2]; sq += red[(w * 4 + m) * 2 + 1]; }
         f16x8 v = *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8);
-        const f16x8 gm = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
+        const f16x8 gm = i == i0 ? gm0 : *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
         if (a.epi.norm == PTA_NORM_RMS) {
           const f16 r16 = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = (v[e] * r16) * gm[e];
         } else {
-          const f16x8 bt = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
+          const f16x8 bt = i == i0 ? bt0 : *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
           const float mean = sum * inv_n;
           const f16 mean16 = (f16)mean;
           float var;
@@ -326,6 +355,29 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
           for (int e = 0; e < 8; ++e) v[e] = ((v[e] - mean16) * r16) * gm[e] + bt[e];
         }
         *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+      }
+    }
+    if (a.epi.mix_state) {
+      // token shift: this matrix's input is x * w + (1 - w) * prev, each step an fp16 operation as in pta_rwkv_mix;
+      // prev is the copy of the state that the previous token's launch wrote, x goes to the other one (first
+      // workgroup) - no workgroup of this launch reads the copy that is written
+      // (a thread mixes the vectors it staged and normalised itself: no barrier in between)
+      const f16* prev = mix_prev;
+      f16* next = mix_next;
+      const f16* mw = mix_w;
+      const f16 one = (f16)1.0f;
+      for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
+        const int m = i / vec_per_row, c = i % vec_per_row;
+        if (c * 8 >= K) continue;
+        f16x8 v = *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8);
+        if (blockIdx.x == 0) *reinterpret_cast<f16x8*>(next + (size_t)m * K + c * 8) = v;
+        if (mw) {
+          const f16x8 pv = i == i0 ? pv0 : *reinterpret_cast<const f16x8*>(prev + (size_t)m * K + c * 8);
+          const f16x8 wv = i == i0 ? wv0 : *reinterpret_cast<const f16x8*>(mw + c * 8);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = v[e] * wv[e] + (one - wv[e]) * pv[e];
+          *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
+        }
       }
     }
   }

@@ -65,7 +65,7 @@ static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int c
     PTA_REQUIRE(w.act >= PTA_ACT_NONE && w.act <= PTA_ACT_SIGMOID, "pta_linear: unknown activation %d in entry %d", w.act, i);
     PTA_REQUIRE(!swiglu || (!w.x && w.act == PTA_ACT_NONE), "pta_linear: the SwiGLU pair shares X and takes no activation");
     PTA_REQUIRE(!w.x || pta_aligned(w.x, 16), "pta_linear: x[%d] must be 16-byte aligned", i);
-    a.mat[i] = GemmMat{w.tiled, w.scale, host_bias ? (const f16*)host_bias[i] : nullptr, (const f16*)w.x, w.act,
+    a.mat[i] = GemmMat{w.tiled, w.scale, host_bias ? (const f16*)host_bias[i] : nullptr, (const f16*)w.x, (const f16*)w.mix, w.act,
                        (f16*)host_Y[i], w.N, swiglu ? 0 : nb};
     nb += (w.N + 15) / 16;
   }
@@ -75,6 +75,18 @@ static int linear_impl(const void* X, const int32_t* x_scale, int x_bytes, int c
   }
   rc = make_epilogue(fuse, &a.epi, "pta_linear");
   if (rc) return rc;
+  {
+    bool any_mix = false;
+    for (int i = 0; i < count; ++i) any_mix = any_mix || host_w[i].mix;
+    PTA_REQUIRE(!any_mix || a.epi.mix_state, "pta_linear: a mixing vector needs pta_fusion.mix_state and mix_step");
+    if (a.epi.mix_state) {
+      // the token shift runs where the rows are staged in LDS: gemv_lds_kernel's shapes, one shared input
+      PTA_REQUIRE(X && M <= 4 && (size_t)M * (a.KT * 128 + 8) * 2 <= 40 * 1024 && K % 8 == 0 && !swiglu && !x_bytes && !x_scale,
+                  "pta_linear: mix_state needs one shared fp16 X of up to 4 rows with M * K <= 20480 (got M=%d K=%d)", M, K);
+      for (int i = 0; i < count; ++i) PTA_REQUIRE(!host_w[i].x, "pta_linear: mix_state and a weight's own input exclude each other");
+      PTA_REQUIRE(pta_aligned(a.epi.mix_state, 16), "pta_linear: mix_state must be 16-byte aligned");
+    }
+  }
   if (fuse && fuse->workspace) {
     PTA_REQUIRE(pta_aligned(fuse->workspace, 16), "pta_linear: the workspace must be 16-byte aligned");
     a.part = (float*)fuse->workspace;

@@ -130,11 +130,12 @@ class LayerOps:
         self.q_rot = buf(rows, s.n_head, s.head_dim)
         self.act = buf(rows, ffn)
         self.attn_ws = K.decode_attention_workspace(rows, s.n_head, s.head_dim, s.max_len, device)
-        # Measured on MI355X at d = 4096: the norm inside the GEMM costs every workgroup a pass over X and two
-        # barriers: +5 us per launch at batch <= 4 (the stand-alone norm kernel takes 2.4 us) and +4 us per
-        # launch at batch 16 as well (stand-alone 4.4 us, but two of the three GEMMs that follow a norm each
-        # pay for it), so it stays separate.  The kernels support it (rows <= 16); tests cover it.
-        self.fuse_norm = False
+        # The norm inside the GEMM: every workgroup normalises the rows it stages.  Up to 4 rows that is cheaper than
+        # a launch of its own since the rows' sums over a wave are made by data-parallel moves (Llama 2 at the 7B
+        # width, batch 1, one launch per operator: 1.687 -> 1.593 ms per step; with shuffles it cost 5 us per
+        # launch and lost).  At batch 16 it costs 4 us per launch against a 4.4 us kernel, and two of the three
+        # GEMMs that follow a norm each pay for it: separate there.  The kernels support up to 16 rows.
+        self.fuse_norm = rows <= 4 and K.norm_fusable(rows, d)
         # fp16 staging of activations rounded to the FP8 grid, one buffer per input width
         self._fp8_buf = {k: buf(rows, k) for k in {d, ffn}}
         self._gate, self._up = buf(rows, ffn), buf(rows, ffn)

@@ -91,8 +91,10 @@ class RWKVDecoder:
         self.keep_going = torch.ones((), dtype=i32, device=device)
         # states per block: token-shift rows for the FFN and the attention (fp16), numerator,
         # denominator and running maximum of the WKV recurrence (fp32)
-        self.st_ffn = [buf(B, d) for _ in range(s.n_layer)]
-        self.st_att = [buf(B, d) for _ in range(s.n_layer)]
+        # (two copies of the token-shift rows, used in turn, where the shift runs inside the Linears: see step_fn)
+        self.fuse_shift = K.norm_fusable(B, d)
+        self.st_ffn = [buf(2, B, d) if self.fuse_shift else buf(B, d) for _ in range(s.n_layer)]
+        self.st_att = [buf(2, B, d) if self.fuse_shift else buf(B, d) for _ in range(s.n_layer)]
         self.st_num = [buf(B, d, dtype=f32) for _ in range(s.n_layer)]
         self.st_den = [buf(B, d, dtype=f32) for _ in range(s.n_layer)]
         self.st_max = [buf(B, d, dtype=f32) for _ in range(s.n_layer)]
@@ -110,6 +112,16 @@ class RWKVDecoder:
             for x, lw, o, a in zip(xs, lws, outs, acts):
                 K.linear(x, [lw.w], [o], act=a)
 
+    def _shifted(self, x, ln, lws, mixes, state, outs, acts):
+        """outs[i] = act_i(Linear_i(shift_i(LayerNorm(x)))) with the norm and the shifts inside the launch(es); every
+        launch reads the state's copy of this step's parity and leaves the normalised rows in the other."""
+        norm = K.Norm(ln[0], ln[1], self.spec.eps)
+        if len({lw.group_key() for lw in lws}) == 1 and not lws[0].is_fp8:
+            K.linear(x, [lw.w for lw in lws], outs, acts=acts, norm=norm, mixes=mixes, mix=(state, self.step))
+        else:
+            for lw, m_, o, a in zip(lws, mixes, outs, acts):
+                K.linear(x, [lw.w], [o], act=a, norm=norm, mixes=[m_], mix=(state, self.step))
+
     def step_fn(self):
         s, w = self.spec, self.w
         K.embedding(w.embed, self.container, self.x, ids_index=self.step)
@@ -118,17 +130,27 @@ class RWKVDecoder:
             if blk.pre_ln is not None:
                 K.layer_norm_ce(x, blk.pre_ln[0], blk.pre_ln[1], s.eps, spare)
                 x, spare = spare, x
-            K.layer_norm_ce(x, blk.ln1[0], blk.ln1[1], s.eps, self.h)
-            K.rwkv_mix(self.h, self.st_att[i], blk.att_mix, self.mix)
-            self._group(self.mix, [blk.att_key, blk.att_value, blk.att_receptance], [self.k, self.v, self.r],
-                        [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
+            if self.fuse_shift:
+                # up to 4 rows: LayerNorm and the token shift run where the Linears stage their input (two launches
+                # fewer); the shift's rows of the previous token live in two copies that the steps use in turn
+                self._shifted(x, blk.ln1, [blk.att_key, blk.att_value, blk.att_receptance], blk.att_mix, self.st_att[i],
+                              [self.k, self.v, self.r], [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
+            else:
+                K.layer_norm_ce(x, blk.ln1[0], blk.ln1[1], s.eps, self.h)
+                K.rwkv_mix(self.h, self.st_att[i], blk.att_mix, self.mix)
+                self._group(self.mix, [blk.att_key, blk.att_value, blk.att_receptance], [self.k, self.v, self.r],
+                            [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
             K.rwkv_wkv(self.k, self.v, self.r, blk.time_decay, blk.time_first, self.st_num[i], self.st_den[i],
                        self.st_max[i], self.y)
             K.linear(self.y, [blk.att_output.w], [x], residual=x, workspace=self._lin_ws)
-            K.layer_norm_ce(x, blk.ln2[0], blk.ln2[1], s.eps, self.h)
-            K.rwkv_mix(self.h, self.st_ffn[i], blk.ffn_mix, self.mix[:2])
-            self._group(self.mix[:2], [blk.ffn_key, blk.ffn_receptance], [self.fk, self.fr],
-                        [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
+            if self.fuse_shift:
+                self._shifted(x, blk.ln2, [blk.ffn_key, blk.ffn_receptance], blk.ffn_mix, self.st_ffn[i], [self.fk, self.fr],
+                              [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
+            else:
+                K.layer_norm_ce(x, blk.ln2[0], blk.ln2[1], s.eps, self.h)
+                K.rwkv_mix(self.h, self.st_ffn[i], blk.ffn_mix, self.mix[:2])
+                self._group(self.mix[:2], [blk.ffn_key, blk.ffn_receptance], [self.fk, self.fr],
+                            [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
             halve = s.rescale_every > 0 and (i + 1) % s.rescale_every == 0
             K.linear(self.fk, [blk.ffn_value.w], [x], mul=self.fr, residual=x, post_scale=0.5 if halve else 0.0,
                      workspace=self._lin_ws)

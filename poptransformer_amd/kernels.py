@@ -50,17 +50,22 @@ def norm_fusable(M, K):
 
 
 def _fusion(bias=None, residual=None, act=_lib.ACT_NONE, norm=None, mul=None, post_scale=0.0, workspace=None,
-            out_grid=None):
-    """out_grid: (device int32 exponent, 'F143' | 'F152') - leave the result on that FP8 grid (half_to_fp8_grid)."""
+            out_grid=None, mix=None):
+    """out_grid: (device int32 exponent, 'F143' | 'F152') - leave the result on that FP8 grid (half_to_fp8_grid).
+    mix: (state [2, M, K] fp16, device int32 step) - the token shift done inside the Linears (pta_fusion.mix_state)."""
     if (bias is None and residual is None and act == _lib.ACT_NONE and norm is None and mul is None and not post_scale
-            and workspace is None and out_grid is None):
+            and workspace is None and out_grid is None and mix is None):
         return None
+    if mix is not None:
+        _need(mix[0], torch.float16, "mix state", 3)
+        _need(mix[1], _i32, "step")
     if out_grid is not None:
         _need(out_grid[0], _i32, "fp8_scale")
     e = Fusion(_p(bias), _p(residual), act, _p(mul), float(post_scale), norm.kind if norm else _lib.NORM_NONE,
                _p(norm.weight) if norm else None, _p(norm.bias) if norm else None, norm.eps if norm else 0.0,
                _p(workspace), workspace.numel() * workspace.element_size() if workspace is not None else 0,
-               _p(out_grid[0]) if out_grid is not None else None, _fmt(out_grid[1]) if out_grid is not None else 0)
+               _p(out_grid[0]) if out_grid is not None else None, _fmt(out_grid[1]) if out_grid is not None else 0,
+               _p(mix[0]) if mix is not None else None, _p(mix[1]) if mix is not None else None)
     return ctypes.byref(e)
 
 
@@ -256,29 +261,36 @@ def half_to_fp8_grid(x, scale, fp8_format="F143", out=None):
 
 
 # ------------------------------------------------------------------ general Linear -------
-def _desc(w, x=None, act=_lib.ACT_NONE):
+def _desc(w, x=None, act=_lib.ACT_NONE, mix=None):
     xp = x.data_ptr() if x is not None else None
+    mp = mix.data_ptr() if mix is not None else None
     if isinstance(w, W4Weight):
-        return _lib.Weight(_lib.W_INT4, w.tiled.data_ptr(), w.scale.data_ptr(), w.N, w.K, xp, act)
+        return _lib.Weight(_lib.W_INT4, w.tiled.data_ptr(), w.scale.data_ptr(), w.N, w.K, xp, act, mp)
     if isinstance(w, F16Weight):
-        return _lib.Weight(_lib.W_F16, w.tiled.data_ptr(), None, w.N, w.K, xp, act)
+        return _lib.Weight(_lib.W_F16, w.tiled.data_ptr(), None, w.N, w.K, xp, act, mp)
     if isinstance(w, F8Weight):
         return _lib.Weight(_lib.W_F143 if w.format == _lib.F143 else _lib.W_F152, w.tiled.data_ptr(), w.scale.data_ptr(),
-                           w.N, w.K, xp, act)
+                           w.N, w.K, xp, act, mp)
     raise TypeError(f"not a tiled weight: {type(w)}")
 
 
 def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None, residual=None, act=_lib.ACT_NONE,
-           norm=None, mul=None, post_scale=0.0, xs=None, acts=None, workspace=None, out_grid=None):
+           norm=None, mul=None, post_scale=0.0, xs=None, acts=None, workspace=None, out_grid=None, mixes=None, mix=None):
     """pta_linear: up to four weights of one kind.  They share x, or each takes its own input from
     `xs`.  `biases` / `acts` are per-weight lists (or None); bias / residual / act / mul / post_scale
-    apply to the single-weight form only."""
+    apply to the single-weight form only.  mixes (per-weight mixing vectors) with mix = (state [2, M, K], step):
+    the RWKV token shift inside the launch - weight i is fed norm(x) * mixes[i] + (1 - mixes[i]) * previous rows."""
     if xs is not None:
         x = xs[0]
     _need(x, torch.float16, "x", 2)
     M = x.shape[0]
     n = len(weights)
-    descs = (_lib.Weight * n)(*[_desc(w, xs[i] if xs is not None else None, acts[i] if acts is not None else _lib.ACT_NONE)
+    if mixes is not None:
+        for m_ in mixes:
+            if m_ is not None:
+                _need(m_, torch.float16, "mixing vector", 1)
+    descs = (_lib.Weight * n)(*[_desc(w, xs[i] if xs is not None else None, acts[i] if acts is not None else _lib.ACT_NONE,
+                                      mixes[i] if mixes is not None else None)
                                 for i, w in enumerate(weights)])
     VP = ctypes.c_void_p * n
     ys = VP(*[o.data_ptr() for o in outs])
@@ -289,7 +301,7 @@ def linear(x, weights, outs, biases=None, x_scale=None, swiglu=False, bias=None,
         if w.K != x.shape[1]:
             raise ValueError(f"matmul: contracting dimensions differ ({x.shape[1]} vs {w.K})")
     check(_lib.load().pta_linear(_p(x), _p(x_scale), n, descs, bs, ys, M, 1 if swiglu else 0,
-                                 _fusion(bias, residual, act, norm, mul, post_scale, workspace, out_grid), _stream()))
+                                 _fusion(bias, residual, act, norm, mul, post_scale, workspace, out_grid, mix), _stream()))
     return outs
 
 

@@ -979,6 +979,49 @@ def test_rope_bit_exact(K):
 
 
 # ---------------------------------------------------------------- RWKV pieces
+def _lib_act(name):
+    from poptransformer_amd import _lib
+    return {"none": _lib.ACT_NONE, "sigmoid": _lib.ACT_SIGMOID, "relu_square": _lib.ACT_RELU_SQUARE}[name]
+
+
+@pytest.mark.parametrize("B,d,N", [(1, 4096, 4096), (3, 256, 512), (4, 1024, 2048)])
+@pytest.mark.parametrize("with_norm", [True, False])
+def test_token_shift_inside_the_linears(K, B, d, N, with_norm):
+    """LayerNorm and the RWKV token shift done where the Linears stage their rows (pta_fusion.mix_state): three
+    Linears with a mixing vector each, over three consecutive steps of the step counter - against the separate
+    launches (layer_norm_ce, rwkv_mix, linear).  The state's two copies take turns: each step reads the rows the
+    previous step left and leaves its own; a Linear without a mixing vector in the same launch gets the rows
+    unshifted."""
+    rng = np.random.default_rng(B + d)
+    packed = [rng.integers(-128, 128, size=(N, d // 2), dtype=np.int8) for _ in range(3)]
+    scales = [rng.uniform(0.005, 0.02, N).astype(np.float16) for _ in range(3)]
+    ws = [K.W4Weight(dev(p_), dev(s_)) for p_, s_ in zip(packed, scales)]
+    mixes = [dev(rng.uniform(0, 1, d).astype(np.float16)) for _ in range(2)] + [None]
+    g, b = dev(rng.uniform(0.5, 1.5, d).astype(np.float16)), dev((rng.standard_normal(d) * 0.1).astype(np.float16))
+    state = torch.zeros((2, B, d), dtype=torch.float16, device="cuda")
+    prev = torch.zeros((B, d), dtype=torch.float16, device="cuda")
+    step = torch.zeros((), dtype=torch.int32, device="cuda")
+    for t in range(3):
+        x = dev(rng.standard_normal((B, d)).astype(np.float16))
+        outs = [torch.empty((B, N), dtype=torch.float16, device="cuda") for _ in range(3)]
+        K.linear(x, ws, outs, norm=K.Norm(g, b, 1e-5) if with_norm else None, mixes=mixes, mix=(state, step),
+                 acts=[_lib_act("none"), _lib_act("sigmoid"), _lib_act("none")])
+        xn = K.layer_norm_ce(x, g, b, 1e-5) if with_norm else x.clone()
+        shifted = [torch.empty_like(xn) for _ in range(2)]
+        K.rwkv_mix(xn, prev, mixes[:2], shifted)                      # (overwrites prev with xn)
+        ref = [torch.empty((B, N), dtype=torch.float16, device="cuda") for _ in range(3)]
+        K.linear(None, ws, ref, xs=shifted + [xn], acts=[_lib_act("none"), _lib_act("sigmoid"), _lib_act("none")])
+        for o, r_ in zip(outs, ref):
+            assert rel_err(host(o), host(r_)) <= (2e-3 if with_norm else 0.0)
+        # the rows this step left for the next: the other copy
+        left = state[(t + 1) & 1]
+        assert rel_err(host(left), host(xn)) <= (2e-3 if with_norm else 0.0)
+        step += 1
+    with pytest.raises(Exception, match="mix_state"):
+        K.linear(dev(np.zeros((8, d), np.float16)), ws, [torch.empty((8, N), dtype=torch.float16, device="cuda") for _ in range(3)],
+                 mixes=mixes, mix=(torch.zeros((2, 8, d), dtype=torch.float16, device="cuda"), step))
+
+
 def test_rwkv_mix_bit_exact_and_wkv(K):
     rng = np.random.default_rng(41)
     B, d = 3, 256
