@@ -12,7 +12,7 @@ constexpr int NORM_THREADS = 256;
 constexpr int NORM_MAX_VEC = 4;  // 8-element vectors per thread: rows up to 8192 columns
 
 __device__ __forceinline__ float block_sum(float v, float* sh) {
-  v = wave_sum(v);
+  v = wave_total_dpp(v);      // (every thread of the workgroup calls this)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   __syncthreads();
   if (lane == 0) sh[wave] = v;
@@ -32,13 +32,22 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restric
   __shared__ float sh[NORM_THREADS / 64];
   const size_t base = (size_t)blockIdx.x * cols;
   const int nvec = cols >> 3;
-  f16x8 v[NORM_MAX_VEC];
+  f16x8 v[NORM_MAX_VEC], gv[NORM_MAX_VEC], bv[NORM_MAX_VEC];
   float s = 0.f, sq = 0.f;
+  // (the weights are requested with the row: one round trip to memory before the sums instead of one on either side)
 #pragma unroll
   for (int i = 0; i < NORM_MAX_VEC; ++i) {
     const int c = threadIdx.x + i * NORM_THREADS;
     if (c < nvec) {
       v[i] = *reinterpret_cast<const f16x8*>(x + base + (size_t)c * 8);
+      gv[i] = *reinterpret_cast<const f16x8*>(gamma + (size_t)c * 8);
+      if (MODE != 0) bv[i] = *reinterpret_cast<const f16x8*>(beta + (size_t)c * 8);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NORM_MAX_VEC; ++i) {
+    const int c = threadIdx.x + i * NORM_THREADS;
+    if (c < nvec) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float f = (float)v[i][e];
@@ -70,13 +79,13 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restric
   for (int i = 0; i < NORM_MAX_VEC; ++i) {
     const int c = threadIdx.x + i * NORM_THREADS;
     if (c < nvec) {
-      const f16x8 g = *reinterpret_cast<const f16x8*>(gamma + (size_t)c * 8);
+      const f16x8 g = gv[i];
       f16x8 o;
       if (MODE == 0) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = (v[i][e] * r16) * g[e];
       } else {
-        const f16x8 b = *reinterpret_cast<const f16x8*>(beta + (size_t)c * 8);
+        const f16x8 b = bv[i];
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = ((v[i][e] - mean16) * r16) * g[e] + b[e];
       }
