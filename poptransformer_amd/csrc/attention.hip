@@ -370,8 +370,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_partial_kernel(AttnArgs a) {
       float s = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) s = __builtin_fmaf(qf[e], (float)k8[u][e], s);
-#pragma unroll
-      for (int o = LPP / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      s = lane_group_sum<LPP>(s);
       if (KV8) s *= kv_mul;
       f16 s16 = (f16)s;                       // fp16 output of the q.K^T MatMul
       if (a.use_scale) s16 = s16 * a.scale;   // fp16 multiply by fp16(1/sqrt(D))
