@@ -284,28 +284,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
   {
     const int vec_per_row = KT * 16;               // 8-half vectors per padded row
     float ps[4] = {0.f, 0.f, 0.f, 0.f}, pq[4] = {0.f, 0.f, 0.f, 0.f};
-    // What the norm and the token shift apply to this thread's FIRST vector (with one row of up to 8192 features its
-    // only one) is requested together with the rows: one round trip to memory instead of one per pass.
-    const int i0 = threadIdx.x;
-    const bool first = i0 < M * vec_per_row && (i0 % vec_per_row) * 8 < K;
-    const f16* mix_prev = nullptr;
-    f16* mix_next = nullptr;
-    const f16* mix_w = a.epi.mix_state ? a.mat[mi].mix : nullptr;
-    if (a.epi.mix_state) {
-      const int parity = a.epi.mix_step[0] & 1;
-      mix_prev = a.epi.mix_state + (size_t)parity * M * K;
-      mix_next = a.epi.mix_state + (size_t)(parity ^ 1) * M * K;
-    }
-    f16x8 gm0 = {0, 0, 0, 0, 0, 0, 0, 0}, bt0 = gm0, pv0 = gm0, wv0 = gm0;
-    if (first) {
-      const int m = i0 / vec_per_row, c = i0 % vec_per_row;
-      if (a.epi.norm != PTA_NORM_NONE) gm0 = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
-      if (a.epi.norm == PTA_NORM_LAYER) bt0 = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
-      if (mix_w) {
-        pv0 = *reinterpret_cast<const f16x8*>(mix_prev + (size_t)m * K + c * 8);
-        wv0 = *reinterpret_cast<const f16x8*>(mix_w + c * 8);
-      }
-    }
     for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
       const int m = i / vec_per_row, c = i % vec_per_row;
       f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -338,13 +316,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
 #pragma unroll
         for (int w = 0; w < NW; ++w) { sum += red[(w * 4 + m) * 2]; sq += red[(w * 4 + m) * 2 + 1]; }
         f16x8 v = *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8);
-        const f16x8 gm = i == i0 ? gm0 : *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
+        const f16x8 gm = *reinterpret_cast<const f16x8*>(a.epi.norm_weight + c * 8);
         if (a.epi.norm == PTA_NORM_RMS) {
           const f16 r16 = (f16)(1.0f / sqrtf(sq * inv_n + a.epi.norm_eps));
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = (v[e] * r16) * gm[e];
         } else {
-          const f16x8 bt = i == i0 ? bt0 : *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
+          const f16x8 bt = *reinterpret_cast<const f16x8*>(a.epi.norm_bias + c * 8);
           const float mean = sum * inv_n;
           const f16 mean16 = (f16)mean;
           float var;
@@ -362,9 +340,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
       // prev is the copy of the state that the previous token's launch wrote, x goes to the other one (first
       // workgroup) - no workgroup of this launch reads the copy that is written
       // (a thread mixes the vectors it staged and normalised itself: no barrier in between)
-      const f16* prev = mix_prev;
-      f16* next = mix_next;
-      const f16* mw = mix_w;
+      const int parity = a.epi.mix_step[0] & 1;
+      const f16* prev = a.epi.mix_state + (size_t)parity * M * K;
+      f16* next = a.epi.mix_state + (size_t)(parity ^ 1) * M * K;
+      const f16* mw = a.mat[mi].mix;
       const f16 one = (f16)1.0f;
       for (int i = threadIdx.x; i < M * vec_per_row; i += NW * 64) {
         const int m = i / vec_per_row, c = i % vec_per_row;
@@ -372,8 +351,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_lds_kernel(GemmArgs a) {
         f16x8 v = *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8);
         if (blockIdx.x == 0) *reinterpret_cast<f16x8*>(next + (size_t)m * K + c * 8) = v;
         if (mw) {
-          const f16x8 pv = i == i0 ? pv0 : *reinterpret_cast<const f16x8*>(prev + (size_t)m * K + c * 8);
-          const f16x8 wv = i == i0 ? wv0 : *reinterpret_cast<const f16x8*>(mw + c * 8);
+          const f16x8 pv = *reinterpret_cast<const f16x8*>(prev + (size_t)m * K + c * 8);
+          const f16x8 wv = *reinterpret_cast<const f16x8*>(mw + c * 8);
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = v[e] * wv[e] + (one - wv[e]) * pv[e];
           *reinterpret_cast<f16x8*>(xs + (size_t)m * xstride + c * 8) = v;
