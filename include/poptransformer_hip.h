@@ -416,6 +416,13 @@ int pta_swiglu(const pta_half* gate, const pta_half* up, pta_half* out, size_t n
 int pta_rwkv_mix(const pta_half* x, pta_half* prev, const pta_half* w0, const pta_half* w1, const pta_half* w2,
                  pta_half* o0, pta_half* o1, pta_half* o2, int rows, int cols, pta_stream_t stream);
 
+/* pta_layer_norm_ce followed by pta_rwkv_mix in one launch (the LayerNorm before each token shift:
+ * models/rwkv/attention.py:66-72, models/rwkv/ffn.py:44-51): h = LayerNorm(x); o_i = h*w_i + (1 - w_i)*prev;
+ * prev <- h.  Bit-identical to the two calls.  y receives h, or may be NULL. */
+int pta_layer_norm_ce_mix(const pta_half* x, const pta_half* gamma, const pta_half* beta, pta_half* y, pta_half* prev,
+                          const pta_half* w0, const pta_half* w1, const pta_half* w2, pta_half* o0, pta_half* o1,
+                          pta_half* o2, int rows, int cols, float eps, pta_stream_t stream);
+
 /* The WKV recurrence in fp32 (attention.py:78-100) followed by y = r * fp16(out) (:101-103).
  * k, v, r, y fp16 [rows, cols]; time_decay, time_first fp16 [cols]; num, den, max_state fp32
  * [rows, cols], updated in place (initial values 0, 0, -1e30: models/rwkv/model.py:157-187). */

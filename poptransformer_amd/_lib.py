@@ -122,6 +122,7 @@ SIGNATURES = {
                            POINTER(Fusion), c_void_p]),
     "pta_swiglu": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "pta_rwkv_mix": (c_int, [c_void_p] * 8 + [c_int, c_int, c_void_p]),
+    "pta_layer_norm_ce_mix": (c_int, [c_void_p] * 11 + [c_int, c_int, c_float, c_void_p]),
     "pta_rwkv_wkv": (c_int, [c_void_p] * 9 + [c_int, c_int, c_void_p]),
     "pta_step_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                 c_int, c_int, c_int, c_void_p]),

@@ -23,16 +23,24 @@ __device__ __forceinline__ float block_sum(float v, float* sh) {
   return t;
 }
 
+// The RWKV token shift behind a LayerNorm (models/rwkv/attention.py:59-72, models/rwkv/ffn.py:44-51): the
+// normalised row h feeds out[i] = h * w[i] + (1 - w[i]) * prev for up to three mixing vectors, then prev <- h.
+struct NormMix {
+  f16* prev;          // [rows, cols], or null: no shift
+  const f16* w[3];    // [cols] each; null entries are skipped
+  f16* out[3];
+};
+
 // mode 0: RMSNorm.  mode 1: NormCE with one row.  mode 2: NormCE with several rows.
-template <int MODE>
+template <int MODE, bool MIX = false>
 __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restrict__ x, const f16* __restrict__ gamma,
                                                             const f16* __restrict__ beta, f16* __restrict__ y,
                                                             int cols, float eps, const int32_t* __restrict__ grid_scale,
-                                                            int grid_format) {
+                                                            int grid_format, NormMix mix = NormMix{}) {
   __shared__ float sh[NORM_THREADS / 64];
   const size_t base = (size_t)blockIdx.x * cols;
   const int nvec = cols >> 3;
-  f16x8 v[NORM_MAX_VEC], gv[NORM_MAX_VEC], bv[NORM_MAX_VEC];
+  f16x8 v[NORM_MAX_VEC], gv[NORM_MAX_VEC], bv[NORM_MAX_VEC], pv[MIX ? NORM_MAX_VEC : 1];
   float s = 0.f, sq = 0.f;
   // (the weights are requested with the row: one round trip to memory before the sums instead of one on either side)
 #pragma unroll
@@ -42,6 +50,7 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restric
       v[i] = *reinterpret_cast<const f16x8*>(x + base + (size_t)c * 8);
       gv[i] = *reinterpret_cast<const f16x8*>(gamma + (size_t)c * 8);
       if (MODE != 0) bv[i] = *reinterpret_cast<const f16x8*>(beta + (size_t)c * 8);
+      if (MIX) pv[i] = *reinterpret_cast<const f16x8*>(mix.prev + base + (size_t)c * 8);
     }
   }
 #pragma unroll
@@ -94,7 +103,21 @@ __global__ __launch_bounds__(NORM_THREADS) void norm_kernel(const f16* __restric
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = f8_grid_value(o[e], gs, grid_format);
       }
-      *reinterpret_cast<f16x8*>(y + base + (size_t)c * 8) = o;
+      if (!MIX || y) *reinterpret_cast<f16x8*>(y + base + (size_t)c * 8) = o;
+      if (MIX) {
+        // each step an fp16 operation, in the order of the separate kernel: h * w + (1 - w) * prev
+        const f16 one = (f16)1.0f;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+          if (!mix.w[j]) continue;
+          const f16x8 wv = *reinterpret_cast<const f16x8*>(mix.w[j] + (size_t)c * 8);
+          f16x8 m;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) m[e] = o[e] * wv[e] + (one - wv[e]) * pv[i][e];
+          *reinterpret_cast<f16x8*>(mix.out[j] + base + (size_t)c * 8) = m;
+        }
+        *reinterpret_cast<f16x8*>(mix.prev + base + (size_t)c * 8) = o;
+      }
     }
   }
 }
@@ -146,5 +169,28 @@ extern "C" int pta_layer_norm_ce(const pta_half* x, const pta_half* gamma, const
     hipLaunchKernelGGL(norm_kernel<2>, dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
                        (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps, (const int32_t*)nullptr, 0);
   PTA_CHECK_LAUNCH("pta_layer_norm_ce");
+  return PTA_OK;
+}
+
+extern "C" int pta_layer_norm_ce_mix(const pta_half* x, const pta_half* gamma, const pta_half* beta, pta_half* y,
+                                     pta_half* prev, const pta_half* w0, const pta_half* w1, const pta_half* w2,
+                                     pta_half* o0, pta_half* o1, pta_half* o2, int rows, int cols, float eps,
+                                     pta_stream_t stream) {
+  int rc = check_norm("pta_layer_norm_ce_mix", x, gamma, prev, rows, cols);
+  if (rc) return rc;
+  PTA_REQUIRE(beta && pta_aligned(beta, 16), "pta_layer_norm_ce_mix: beta must be a 16-byte aligned pointer");
+  PTA_REQUIRE(cols < 8192, "pta_layer_norm_ce_mix: the normalised size must be below 8192, got %d", cols);
+  PTA_REQUIRE(w0 && o0, "pta_layer_norm_ce_mix: null pointer");
+  PTA_REQUIRE((!w1 || o1) && (!w2 || o2), "pta_layer_norm_ce_mix: a mixing vector needs its output");
+  const void* ptrs[7] = {y, w0, w1, w2, o0, o1, o2};
+  for (const void* q : ptrs) PTA_REQUIRE(!q || pta_aligned(q, 16), "pta_layer_norm_ce_mix: pointers must be 16-byte aligned");
+  const NormMix mix{(f16*)prev, {(const f16*)w0, (const f16*)w1, (const f16*)w2}, {(f16*)o0, (f16*)o1, (f16*)o2}};
+  if (rows == 1)
+    hipLaunchKernelGGL((norm_kernel<1, true>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps, (const int32_t*)nullptr, 0, mix);
+  else
+    hipLaunchKernelGGL((norm_kernel<2, true>), dim3(rows), dim3(NORM_THREADS), 0, (hipStream_t)stream, (const f16*)x,
+                       (const f16*)gamma, (const f16*)beta, (f16*)y, cols, eps, (const int32_t*)nullptr, 0, mix);
+  PTA_CHECK_LAUNCH("pta_layer_norm_ce_mix");
   return PTA_OK;
 }

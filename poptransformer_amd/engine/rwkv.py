@@ -136,8 +136,7 @@ class RWKVDecoder:
                 self._shifted(x, blk.ln1, [blk.att_key, blk.att_value, blk.att_receptance], blk.att_mix, self.st_att[i],
                               [self.k, self.v, self.r], [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
             else:
-                K.layer_norm_ce(x, blk.ln1[0], blk.ln1[1], s.eps, self.h)
-                K.rwkv_mix(self.h, self.st_att[i], blk.att_mix, self.mix)
+                K.layer_norm_ce_mix(x, blk.ln1[0], blk.ln1[1], s.eps, self.st_att[i], blk.att_mix, self.mix)
                 self._group(self.mix, [blk.att_key, blk.att_value, blk.att_receptance], [self.k, self.v, self.r],
                             [_lib.ACT_NONE, _lib.ACT_NONE, _lib.ACT_SIGMOID])
             K.rwkv_wkv(self.k, self.v, self.r, blk.time_decay, blk.time_first, self.st_num[i], self.st_den[i],
@@ -147,8 +146,7 @@ class RWKVDecoder:
                 self._shifted(x, blk.ln2, [blk.ffn_key, blk.ffn_receptance], blk.ffn_mix, self.st_ffn[i], [self.fk, self.fr],
                               [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
             else:
-                K.layer_norm_ce(x, blk.ln2[0], blk.ln2[1], s.eps, self.h)
-                K.rwkv_mix(self.h, self.st_ffn[i], blk.ffn_mix, self.mix[:2])
+                K.layer_norm_ce_mix(x, blk.ln2[0], blk.ln2[1], s.eps, self.st_ffn[i], blk.ffn_mix, self.mix[:2])
                 self._group(self.mix[:2], [blk.ffn_key, blk.ffn_receptance], [self.fk, self.fr],
                             [_lib.ACT_RELU_SQUARE, _lib.ACT_SIGMOID])
             halve = s.rescale_every > 0 and (i + 1) % s.rescale_every == 0

@@ -588,6 +588,19 @@ def step_update(container, mask, stop_mask, step, next_ids, ids_out, keep_going,
 
 
 # ------------------------------------------------------------------ RWKV -----------------
+def layer_norm_ce_mix(x, gamma, beta, eps, prev, ws, outs, out=None):
+    """LayerNorm (NormCE) and the token-shift mixes of its result in one launch; prev is overwritten with the
+    normalised rows, which `out` also receives when given."""
+    _need(x, torch.float16, "x", 2)
+    _need(prev, torch.float16, "prev", 2)
+    rows, cols = x.shape
+    w = list(ws) + [None] * (3 - len(ws))
+    o = list(outs) + [None] * (3 - len(outs))
+    check(_lib.load().pta_layer_norm_ce_mix(_p(x), _p(gamma), _p(beta), _p(out), _p(prev), _p(w[0]), _p(w[1]), _p(w[2]),
+                                            _p(o[0]), _p(o[1]), _p(o[2]), rows, cols, float(eps), _stream()))
+    return outs
+
+
 def rwkv_mix(x, prev, ws, outs):
     """Token-shift mixes for 1..3 mixing vectors; prev is overwritten with x."""
     rows, cols = x.shape

@@ -1022,6 +1022,45 @@ def test_token_shift_inside_the_linears(K, B, d, N, with_norm):
                  mixes=mixes, mix=(torch.zeros((2, 8, d), dtype=torch.float16, device="cuda"), step))
 
 
+@pytest.mark.parametrize("rows,cols,nmix", [(1, 768, 3), (5, 4096, 3), (32, 4096, 2), (7, 1000, 1)])
+def test_layer_norm_and_token_shift_in_one_launch(K, rows, cols, nmix):
+    """pta_layer_norm_ce_mix against pta_layer_norm_ce followed by pta_rwkv_mix, bit for bit (outputs, the state it
+    leaves, the normalised rows), and against the oracle's gate of the oracle's LayerNorm."""
+    print(f"case: layer norm + token shift, rows {rows}, cols {cols}, {nmix} mixing vectors", flush=True)
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float16)
+    prev = rng.standard_normal((rows, cols)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, cols).astype(np.float16)
+    b = rng.uniform(-0.5, 0.5, cols).astype(np.float16)
+    ws = [rng.uniform(0, 1, cols).astype(np.float16) for _ in range(nmix)]
+    wd = [dev(w) for w in ws]
+    h = K.layer_norm_ce(dev(x), dev(g), dev(b), 1e-5)
+    p_two = dev(prev)
+    two = [torch.empty((rows, cols), dtype=torch.float16, device="cuda") for _ in range(nmix)]
+    K.rwkv_mix(h, p_two, wd, two)
+    p_one = dev(prev)
+    one = [torch.empty((rows, cols), dtype=torch.float16, device="cuda") for _ in range(nmix)]
+    h_one = torch.empty((rows, cols), dtype=torch.float16, device="cuda")
+    K.layer_norm_ce_mix(dev(x), dev(g), dev(b), 1e-5, p_one, wd, one, out=h_one)
+    torch.cuda.synchronize()
+    assert torch.equal(h_one, h) and torch.equal(p_one, p_two) and torch.equal(p_one, h)
+    for a_, b_ in zip(one, two):
+        assert torch.equal(a_, b_)
+    want_h = O.layer_norm_ce(x, g, b, 1e-5, rows, 1, cols)
+    assert np.abs(host(h_one).astype(np.float32) - want_h.astype(np.float32)).max() <= 4 * 2.0 ** -10 * np.abs(want_h).max()
+    for w, o in zip(ws, one):                   # the shift's fp16 steps, on the rows the launch normalised
+        assert np.array_equal(host(o).view(np.uint16), OM_gate(host(h_one), w, prev).view(np.uint16))
+    # without the copy of the normalised rows
+    p_none = dev(prev)
+    none = [torch.empty((rows, cols), dtype=torch.float16, device="cuda") for _ in range(nmix)]
+    K.layer_norm_ce_mix(dev(x), dev(g), dev(b), 1e-5, p_none, wd, none)
+    assert torch.equal(p_none, h) and all(torch.equal(a_, b_) for a_, b_ in zip(none, two))
+    with pytest.raises(Exception, match="mixing vector needs its output"):
+        lib = K._lib.load()
+        K.check(lib.pta_layer_norm_ce_mix(K._p(dev(x)), K._p(dev(g)), K._p(dev(b)), None, K._p(p_none), K._p(wd[0]), K._p(wd[0]), None,
+                                          K._p(none[0]), None, None, rows, cols, 1e-5, None))
+
+
 def test_rwkv_mix_bit_exact_and_wkv(K):
     rng = np.random.default_rng(41)
     B, d = 3, 256
