@@ -114,6 +114,33 @@ def test_w4a16_gemm_many_rows_wide_outputs(K, M, Kdim, N):
     assert np.abs(got.astype(np.float64) - ref64).max() <= 2.0 ** -10 * np.abs(ref64).max() + 1e-3
 
 
+@pytest.mark.parametrize("M", [20, 33, 64])
+def test_w4a16_gemm_many_rows_more_workgroups_than_compute_units(K, M):
+    """17..64 rows and more than 256 workgroups of 64 channels: beyond 32 rows the launch takes workgroups of 128
+    channels (four weight streams per wave).  The two weights of the RWKV channel mix (16384 and 4096 channels, models/rwkv/ffn.py:
+    47-56) with an input and an activation each, and one weight of 20480 channels with bias and residual; 1160
+    features = a ragged last tile."""
+    print(f"case: four streams per wave, {M} rows", flush=True)
+    rng = np.random.default_rng(M)
+    Kdim = 1160
+    xs = [rng.standard_normal((M, Kdim)).astype(np.float16) for _ in range(2)]
+    cases = [_w4_case(M + n, 1, Kdim, n)[1:] for n in (16384, 4096)]
+    ws = [K.W4Weight(dev(p_), dev(s_)) for p_, s_ in cases]
+    outs = [torch.empty((M, n), dtype=torch.float16, device="cuda") for n in (16384, 4096)]
+    K.linear(None, ws, outs, xs=[dev(x) for x in xs], acts=[K._lib.ACT_RELU_SQUARE, K._lib.ACT_SIGMOID])
+    ref0 = O.w4a16_matmul(xs[0], *cases[0]); ref0 = (np.maximum(ref0, np.float16(0)) ** 2).astype(np.float16)
+    ref1 = O.w4a16_matmul(xs[1], *cases[1]).astype(np.float32); ref1 = (1.0 / (1.0 + np.exp(-ref1))).astype(np.float16)
+    assert rel_err(host(outs[0]), ref0) <= 1e-2 and rel_err(host(outs[1]), ref1) <= 1e-2
+    x, packed, scale = _w4_case(M * 5, M, Kdim, 20480)
+    bias = rng.standard_normal(20480).astype(np.float16)
+    res = rng.standard_normal((M, 20480)).astype(np.float16)
+    got = host(K.w4a16_gemm(dev(x), K.W4Weight(dev(packed), dev(scale)), bias=dev(bias), residual=dev(res)))
+    ref = ((O.w4a16_matmul(x, packed, scale) + bias).astype(np.float16) + res).astype(np.float16)
+    assert rel_err(got, ref) <= 1e-2
+    ref64 = x.astype(np.float64) @ O.int4_to_half(packed, scale, 1).astype(np.float64) + bias.astype(np.float64) + res.astype(np.float64)
+    assert np.abs(got.astype(np.float64) - ref64).max() <= 3 * 2.0 ** -10 * np.abs(ref64).max() + 1e-3
+
+
 @pytest.mark.parametrize("M", [17, 32, 33, 64])
 @pytest.mark.parametrize("Kdim,N", [(4096, 1024), (11008, 4096), (2872, 2048)])
 def test_w4a16_gemm_many_rows_few_outputs_split_k(K, M, Kdim, N):
