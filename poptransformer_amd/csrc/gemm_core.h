@@ -952,18 +952,17 @@ static int launch_gemv_stream(const GemmArgs& a, int total_nb, int cus, hipStrea
 constexpr int TILE_WAVES = 8;
 constexpr int TILE_XSTRIDE = 128 + 8;      // halves per staged row: 16 consecutive rows hit 16 different bank groups
 
-template <class Fmt, int MT, int KQ, bool PAIR, int NS = 2>
-__global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) {
+template <class Fmt, int MT, int KQ, bool PAIR, int NWV = TILE_WAVES>
+__global__ __launch_bounds__(NWV * 64) void gemm_tile_kernel(GemmArgs a) {
   constexpr int KV = Fmt::kVec;
-  constexpr int WPG = TILE_WAVES / KQ;          // waves per K group
+  constexpr int WPG = NWV / KQ;          // waves per K group
   constexpr int ROWS = MT * 16;
   constexpr int XBUF = ROWS * TILE_XSTRIDE;     // halves of one staged tile
   constexpr int VPT = ROWS * 16 / (WPG * 64);   // 16-byte vectors of a tile per thread of its group
   static_assert(VPT >= 1 && ROWS * 16 % (WPG * 64) == 0, "staging must divide evenly");
-  static_assert(!PAIR || NS == 2, "a SwiGLU pair is two streams");
   extern __shared__ __align__(16) unsigned char smem[];
   f16* xs = reinterpret_cast<f16*>(smem);       // [KQ][2][ROWS][TILE_XSTRIDE]
-  float* red = reinterpret_cast<float*>(smem);  // after the product: [TILE_WAVES][NS][MT][256]
+  float* red = reinterpret_cast<float*>(smem);  // after the product: [NWV][2][MT][256]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int kq = wave / WPG, wg_ = wave % WPG;  // K group, wave within the group
   const int tig = wg_ * 64 + lane;              // thread index within the group
@@ -974,29 +973,29 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
   const int kt_first = (int)blockIdx.y * per_slice;
   const int KT = kt_first + per_slice < a.KT ? kt_first + per_slice : a.KT;     // end of the slice
 
-  // the NS weight streams of this wave
+  // the two weight streams of this wave
   int mi = 0;
-  const int first_blk = PAIR ? (int)blockIdx.x * WPG : (int)blockIdx.x * NS * WPG;
+  const int first_blk = PAIR ? (int)blockIdx.x * WPG : (int)blockIdx.x * 2 * WPG;
   if (!PAIR) {
 #pragma unroll
     for (int i = 1; i < 4; ++i)
       if (i < a.count && first_blk >= a.mat[i].nb_begin) mi = i;
   }
-  int nb[NS];
-  typename Fmt::Scale sc[NS];
-  const u32x4* wp[NS];
+  int nb[2];
+  typename Fmt::Scale sc[2];
+  const u32x4* wp[2];
 #pragma unroll
-  for (int st = 0; st < NS; ++st) {
+  for (int st = 0; st < 2; ++st) {
     const GemmMat& m = a.mat[PAIR ? st : mi];
-    nb[st] = PAIR ? first_blk + wg_ : first_blk - m.nb_begin + NS * wg_ + st;
+    nb[st] = PAIR ? first_blk + wg_ : first_blk - m.nb_begin + 2 * wg_ + st;
     sc[st] = Fmt::load_scale(m.scale, a.x_scale, nb[st] * 16 + (lane & 15), m.N);
     wp[st] = reinterpret_cast<const u32x4*>(m.tiled) + (size_t)nb[st] * a.KT * (64 * KV) + lane;
   }
   const f16* X = a.mat[mi].X ? a.mat[mi].X : a.X;
 
-  f32x4 acc[NS][MT];
+  f32x4 acc[2][MT];
 #pragma unroll
-  for (int st = 0; st < NS; ++st)
+  for (int st = 0; st < 2; ++st)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[st][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -1017,17 +1016,17 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
       *reinterpret_cast<u32x4*>(buf + (v >> 4) * TILE_XSTRIDE + (v & 15) * 8) = xv[i];
     }
   };
-  auto fetch_w = [&](int kt, u32x4 (&w)[NS][KV]) {
+  auto fetch_w = [&](int kt, u32x4 (&w)[2][KV]) {
     const int ktc = kt < KT ? kt : KT - 1;
 #pragma unroll
-    for (int st = 0; st < NS; ++st)
+    for (int st = 0; st < 2; ++st)
 #pragma unroll
       for (int v = 0; v < KV; ++v) w[st][v] = __builtin_nontemporal_load(wp[st] + ((size_t)ktc * KV + v) * 64);
   };
 
   f16* xbuf = xs + (size_t)kq * 2 * XBUF;
   const int steps = (KT - kt_first + KQ - 1) / KQ;
-  u32x4 w_cur[NS][KV], w_nxt[NS][KV], xv[VPT];
+  u32x4 w_cur[2][KV], w_nxt[2][KV], xv[VPT];
   fetch_w(kt_first + kq, w_cur);
   fetch_x(kt_first + kq, xv);
   store_x(xbuf, xv);
@@ -1045,7 +1044,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) xb[mt] = *reinterpret_cast<const f16x8*>(cur + mt * 16 * TILE_XSTRIDE + m * 32);
 #pragma unroll
-          for (int st = 0; st < NS; ++st) {
+          for (int st = 0; st < 2; ++st) {
             const f16x8 av = Fmt::a_operand(w_cur[st], m, sc[st]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) acc[st][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, xb[mt], acc[st][mt], 0, 0, 0);
@@ -1065,7 +1064,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     if (more) {
       store_x(xbuf + ((i + 1) & 1) * XBUF, xv);
 #pragma unroll
-      for (int st = 0; st < NS; ++st)
+      for (int st = 0; st < 2; ++st)
 #pragma unroll
         for (int v = 0; v < KV; ++v) w_cur[st][v] = w_nxt[st][v];
     }
@@ -1090,7 +1089,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
           mat.Y[(size_t)m * N + n] = swiglu_out(a.epi, gate, up);
         } else {
 #pragma unroll
-          for (int st = 0; st < NS; ++st) {
+          for (int st = 0; st < 2; ++st) {
             const int n = nb[st] * 16 + (lane >> 4) * 4 + r;
             if (n >= N) continue;
             if (nsl > 1) { a.part[((size_t)blockIdx.y * M + m) * N + n] = acc[st][mt][r]; continue; }
@@ -1106,24 +1105,24 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
   }
   // partial sums of the K groups meet in LDS (the staging area is free after the last barrier)
 #pragma unroll
-  for (int st = 0; st < NS; ++st)
+  for (int st = 0; st < 2; ++st)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[(((wave * NS + st) * MT + mt) * 4 + r) * 64 + lane] = acc[st][mt][r];
+      for (int r = 0; r < 4; ++r) red[(((wave * 2 + st) * MT + mt) * 4 + r) * 64 + lane] = acc[st][mt][r];
   __syncthreads();
-  // outputs of the workgroup: WPG wave slots x NS streams x MT row groups x 256; PAIR: one output per stream pair
-  constexpr int OUTS = WPG * (PAIR ? 1 : NS) * MT * 256;
-  for (int o = threadIdx.x; o < OUTS; o += TILE_WAVES * 64) {
+  // outputs of the workgroup: WPG wave slots x 2 streams x MT row groups x 256; PAIR: one output per stream pair
+  constexpr int OUTS = WPG * (PAIR ? 1 : 2) * MT * 256;
+  for (int o = threadIdx.x; o < OUTS; o += NWV * 64) {
     const int nn = o & 15, m16 = (o >> 4) & 15;
     int rest = o >> 8;
     const int mt = rest % MT; rest /= MT;
-    const int st = PAIR ? 0 : rest % NS;
-    const int wslot = PAIR ? rest : rest / NS;
+    const int st = PAIR ? 0 : rest & 1;
+    const int wslot = PAIR ? rest : rest >> 1;
     const int m = mt * 16 + m16;
     const GemmMat& mat = a.mat[PAIR ? 0 : mi];
     const int N = mat.N;
-    const int blk = PAIR ? first_blk + wslot : first_blk - mat.nb_begin + NS * wslot + st;
+    const int blk = PAIR ? first_blk + wslot : first_blk - mat.nb_begin + 2 * wslot + st;
     const int n = blk * 16 + nn;
     if (m >= M || n >= N) continue;
     const int r = nn & 3, ln = (nn >> 2) * 16 + m16;
@@ -1132,7 +1131,7 @@ __global__ __launch_bounds__(TILE_WAVES * 64) void gemm_tile_kernel(GemmArgs a) 
     for (int g = 0; g < (PAIR ? 2 : 1); ++g) {
       float t = 0.f;
 #pragma unroll
-      for (int q = 0; q < KQ; ++q) t += red[((((q * WPG + wslot) * NS + (PAIR ? g : st)) * MT + mt) * 4 + r) * 64 + ln];
+      for (int q = 0; q < KQ; ++q) t += red[((((q * WPG + wslot) * 2 + (PAIR ? g : st)) * MT + mt) * 4 + r) * 64 + ln];
       sum[g] = t;
     }
     if (!PAIR && nsl > 1) {                // a slice of a K split: the raw fp32 sum; the finishing kernel does the rest
@@ -1172,23 +1171,23 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs a) {
   mat.Y[i] = apply_epilogue(a.epi, y0, m, n, N);
 }
 
-template <class Fmt, int MT, int KQ, bool PAIR, int NS = 2>
+template <class Fmt, int MT, int KQ, bool PAIR, int NWV = TILE_WAVES>
 static int launch_gemm_tile(const GemmArgs& a, int total_nb, hipStream_t s, const char* name) {
   static bool ready = false;
-  constexpr int WPG = TILE_WAVES / KQ;
+  constexpr int WPG = NWV / KQ;
   const size_t stage = (size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2;
-  const size_t redb = KQ == 1 ? 0 : (size_t)TILE_WAVES * NS * MT * 256 * 4;     // one K group: no meeting in LDS
+  const size_t redb = KQ == 1 ? 0 : (size_t)NWV * 2 * MT * 256 * 4;      // one K group: no meeting in LDS
   const size_t smem = stage > redb ? stage : redb;
   static_assert((size_t)KQ * 2 * MT * 16 * TILE_XSTRIDE * 2 <= 160 * 1024, "staging beyond the LDS of a compute unit");
   if (!ready) {
-    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_tile_kernel<Fmt, MT, KQ, PAIR, NS>,
+    PTA_REQUIRE(hipFuncSetAttribute((const void*)gemm_tile_kernel<Fmt, MT, KQ, PAIR, NWV>,
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) == hipSuccess,
                 "%s: cannot reserve %zu bytes of LDS", name, smem);
     ready = true;
   }
-  const int per_wg = PAIR ? WPG : NS * WPG;
+  const int per_wg = PAIR ? WPG : 2 * WPG;
   const int nsl = a.ksplit > 1 ? a.ksplit : 1;
-  hipLaunchKernelGGL((gemm_tile_kernel<Fmt, MT, KQ, PAIR, NS>), dim3(total_nb / per_wg, nsl), dim3(TILE_WAVES * 64), smem, s, a);
+  hipLaunchKernelGGL((gemm_tile_kernel<Fmt, MT, KQ, PAIR, NWV>), dim3(total_nb / per_wg, nsl), dim3(NWV * 64), smem, s, a);
   if (nsl > 1) {
     const size_t total = (size_t)a.M * a.mat[0].N;
     hipLaunchKernelGGL(splitk_finish_kernel<Fmt>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
@@ -1912,23 +1911,20 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
         rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(b, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(b, total_nb, s, name);
       } else if (tile_fits(a, PAIR ? 2 : 4, 4, PAIR) && 2 * wgs4 >= cus) {
         // What bounds these launches is the bytes through the busiest compute unit: a workgroup reads all rows of X
-        // beside its weights.  More workgroups than compute units (20480 channels: 320 of 64) and more than 32
-        // rows: four streams per wave, workgroups of 128 channels, where their rounds come out shorter - 160 of
-        // 768 KiB against two rounds of 640 at 64 rows (4096 x 20480: 32.6 against 40.9 us, 31.2 against 38.2 at
-        // 48 rows).  Up to 32 rows two workgroups share a compute unit and hide each other's barriers; there the
-        // two forms take the same time (21.0 against 21.1 us) and the narrow one stays.
-        bool four = false;
+        // beside its weights.  More workgroups than compute units (20480 channels: 320 of 64 channels): workgroups
+        // of 16 waves and 128 channels where their rounds come out shorter - 160 of 768 KiB against two rounds of
+        // 640 at 64 rows.  Measured, 4096 x 20480: 26.0 against 40.7 us at 64 rows, 24.7 against 38.2 at 48, 18.8
+        // against 20.8 at 32; in a single round they lose (4096 x 11008 at 64 rows: 24.9 against 21.5 us).
+        bool wide = false;
         if constexpr (!PAIR && Fmt::kVec <= 2) {
-          if (a.M > 32 && tile_fits(a, 8, 4, false) && wgs4 > cus) {
+          if (tile_fits(a, 8, 4, false) && wgs4 > cus) {
             const double xb = (double)a.M * a.K * 2, wb = (double)a.KT * Fmt::kVec * 1024;
             const int wgs_wide = total_nb / 8;
-            four = ((wgs_wide + cus - 1) / cus) * (xb + 8 * wb) < ((wgs4 + cus - 1) / cus) * (xb + 4 * wb);
+            wide = ((wgs_wide + cus - 1) / cus) * (xb + 8 * wb) < ((wgs4 + cus - 1) / cus) * (xb + 4 * wb);
           }
+          if (wide) rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, false, 16>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, false, 16>(a, total_nb, s, name);
         }
-        if constexpr (!PAIR && Fmt::kVec <= 2) {
-          if (four) rc = launch_gemm_tile<Fmt, 4, 4, false, 4>(a, total_nb, s, name);
-        }
-        if (!four)
+        if (!wide)
         rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(a, total_nb, s, name);
       } else if (a.M <= 32 && tile_fits(a, PAIR ? 1 : 2, 8, PAIR) && 2 * wgs8 >= cus) {
         rc = launch_gemm_tile<Fmt, 2, 8, PAIR>(a, total_nb, s, name);

@@ -116,8 +116,8 @@ def test_w4a16_gemm_many_rows_wide_outputs(K, M, Kdim, N):
 
 @pytest.mark.parametrize("M", [20, 33, 64])
 def test_w4a16_gemm_many_rows_more_workgroups_than_compute_units(K, M):
-    """17..64 rows and more than 256 workgroups of 64 channels: beyond 32 rows the launch takes workgroups of 128
-    channels (four weight streams per wave).  The two weights of the RWKV channel mix (16384 and 4096 channels, models/rwkv/ffn.py:
+    """17..64 rows and more than 256 workgroups of 64 channels: the launch takes workgroups of 16 waves and 128
+    channels.  The two weights of the RWKV channel mix (16384 and 4096 channels, models/rwkv/ffn.py:
     47-56) with an input and an activation each, and one weight of 20480 channels with bias and residual; 1160
     features = a ragged last tile."""
     print(f"case: four streams per wave, {M} rows", flush=True)
