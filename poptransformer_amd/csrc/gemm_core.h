@@ -1917,12 +1917,16 @@ static int dispatch_gemv(const GemmArgs& a, int total_nb, hipStream_t s, const c
         // against 20.8 at 32; in a single round they lose (4096 x 11008 at 64 rows: 24.9 against 21.5 us).
         bool wide = false;
         if constexpr (!PAIR && Fmt::kVec <= 2) {
-          if (tile_fits(a, 8, 4, false) && wgs4 > cus) {
+          // (beyond 32 rows with INT4 weights only: with two vectors per tile the 16 waves' registers do not hold it)
+          if (tile_fits(a, 8, 4, false) && wgs4 > cus && (a.M <= 32 || Fmt::kVec == 1)) {
             const double xb = (double)a.M * a.K * 2, wb = (double)a.KT * Fmt::kVec * 1024;
             const int wgs_wide = total_nb / 8;
             wide = ((wgs_wide + cus - 1) / cus) * (xb + 8 * wb) < ((wgs4 + cus - 1) / cus) * (xb + 4 * wb);
           }
-          if (wide) rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, false, 16>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, false, 16>(a, total_nb, s, name);
+          if (wide) {
+            if (a.M <= 32) rc = launch_gemm_tile<Fmt, 2, 4, false, 16>(a, total_nb, s, name);
+            else if constexpr (Fmt::kVec == 1) rc = launch_gemm_tile<Fmt, 4, 4, false, 16>(a, total_nb, s, name);
+          }
         }
         if (!wide)
         rc = a.M <= 32 ? launch_gemm_tile<Fmt, 2, 4, PAIR>(a, total_nb, s, name) : launch_gemm_tile<Fmt, 4, 4, PAIR>(a, total_nb, s, name);

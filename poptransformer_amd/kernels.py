@@ -593,7 +593,13 @@ def layer_norm_ce_mix(x, gamma, beta, eps, prev, ws, outs, out=None):
     normalised rows, which `out` also receives when given."""
     _need(x, torch.float16, "x", 2)
     _need(prev, torch.float16, "prev", 2)
+    _need(gamma, torch.float16, "gamma", 1)
+    _need(beta, torch.float16, "beta", 1)
     rows, cols = x.shape
+    if tuple(prev.shape) != (rows, cols) or len(ws) != len(outs) or not 1 <= len(ws) <= 3:
+        raise ValueError("layer_norm_ce_mix: prev must have x's shape, and one to three mixing vectors an output each")
+    for t in list(ws) + list(outs):
+        _need(t, torch.float16, "mixing vector / output")
     w = list(ws) + [None] * (3 - len(ws))
     o = list(outs) + [None] * (3 - len(outs))
     check(_lib.load().pta_layer_norm_ce_mix(_p(x), _p(gamma), _p(beta), _p(out), _p(prev), _p(w[0]), _p(w[1]), _p(w[2]),

@@ -480,9 +480,11 @@ def test_casts_done_by_the_producer_are_bit_identical(K, fmt, scale):
         assert np.array_equal(host(out).view(np.uint16), ref.view(np.uint16)), f"values of group {g0}"
 
 
-def test_fp8_gemm_many_rows_wide_outputs(K):
-    rng = np.random.default_rng(22)
-    M, Kdim, N = 48, 1024, 8192
+@pytest.mark.parametrize("M,Kdim,N", [(48, 1024, 8192), (24, 1024, 20480), (48, 1024, 20480)])
+def test_fp8_gemm_many_rows_wide_outputs(K, M, Kdim, N):
+    """FP8 weights at 17..64 rows; 20480 channels: more 64-channel workgroups than compute units (up to 32 rows in
+    workgroups of 16 waves and 128 channels)."""
+    rng = np.random.default_rng(22 + N // 4096)
     x = rng.standard_normal((M, Kdim)).astype(np.float16)
     w8 = O.f8_encode((rng.standard_normal((Kdim, N)) * 0.02).astype(np.float32), "F143", -1)
     fw = K.F8Weight(dev(w8), dev(np.array([-1], np.int32)), "F143", kn=True)
