@@ -440,14 +440,32 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
   const int chunk = attn_chunk(valid, a.nsplit);
   const int nact = (valid + chunk - 1) / chunk;
   const float* p = a.part + (size_t)bh * a.nsplit * (D + 2);
+  // eight chunks at a time: their maxima, denominators and numerators are requested together (a chunk past the last
+  // reads the last one again and counts for nothing); the order of the sums is that of one chunk after the other
   float M = -INFINITY;
-  for (int s = 0; s < nact; ++s) M = fmaxf(M, p[(size_t)s * (D + 2)]);
+  for (int s0 = 0; s0 < nact; s0 += 8) {
+    float mv[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) mv[i] = p[(size_t)(s0 + i < nact ? s0 + i : nact - 1) * (D + 2)];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) M = fmaxf(M, mv[i]);
+  }
   float L = 0.f, A = 0.f;
-  for (int s = 0; s < nact; ++s) {
-    const float* ps = p + (size_t)s * (D + 2);
-    const float w = __expf(ps[0] - M);
-    L = __builtin_fmaf(ps[1], w, L);
-    A = __builtin_fmaf(ps[2 + d], w, A);
+  for (int s0 = 0; s0 < nact; s0 += 8) {
+    float mv[8], lv[8], av[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float* ps = p + (size_t)(s0 + i < nact ? s0 + i : nact - 1) * (D + 2);
+      mv[i] = ps[0]; lv[i] = ps[1]; av[i] = ps[2 + d];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (s0 + i < nact) {
+        const float w = __expf(mv[i] - M);
+        L = __builtin_fmaf(lv[i], w, L);
+        A = __builtin_fmaf(av[i], w, A);
+      }
+    }
   }
   a.out[(size_t)bh * D + d] = attn_result(a, (f16)(A / L));
 }
@@ -659,6 +677,255 @@ __global__ __launch_bounds__(PA_THREADS) void prompt_attention_mfma_kernel(AttnA
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Decode attention of grouped heads on the matrix unit: sixteen query heads share a KV head (ChatGLM2: 32 query
+// heads on 2, chatglm2/attention.py:166-302), so the sixteen heads of a group are the sixteen columns of one MFMA
+// tile and a workgroup reads the group's cache rows once for all of them - attn_partial_kernel reads them once per
+// query head, sixteen times through the compute units.  One workgroup of four waves per (sequence, KV head, chunk of
+// cache rows); wave w takes the chunk's rows 32 w .. 32 w + 31, then 128 further on.  Per step of 32 rows, as in
+// prompt_attention_mfma_kernel with the query heads where that kernel has query rows:
+//   S^T = K Q^T   (K rows straight from the ring as A operands: lane l holds row l % 16, features (l / 16) * 8 + 0..7
+//                  of each 32; Q, rotated, from LDS), the reference's roundings of the scores, the online softmax per
+//   head in fp32 (partners: lanes l ^ 16, l ^ 32), probabilities rounded to fp16,
+//   O += P V      (V transposed through 10 KiB of LDS that belong to the wave).
+// The waves' states meet in LDS; the chunk's (maximum, denominator, numerator) go to the workspace in
+// attn_partial_kernel's layout, for attn_combine_kernel.  FUSED as there: the workgroup rotates its sixteen query
+// heads itself, and the one whose chunk holds this step's position rotates the new key, uses it and the new value
+// from LDS, and writes both to the ring.
+// ------------------------------------------------------------------------------------------
+constexpr int GQA_HEADS = 16;
+
+template <int D, bool FUSED>
+__global__ __launch_bounds__(256) void attn_gqa_partial_kernel(AttnArgs a) {
+  static_assert(D == 64 || D == 128, "head size");
+  constexpr int QS = D + 8;                         // halves per staged query row
+  constexpr int VPR = D / 8;                        // 16-byte vectors per row
+  __shared__ f16 cs[2][64];
+  __shared__ __align__(16) f16 sm_q[GQA_HEADS * QS];
+  __shared__ __align__(16) f16 sm_kv[2 * D];
+  __shared__ __align__(16) f16 vt_all[4 * D * PA_VSTRIDE];       // per wave: V^T of its 32 rows; after the loop: the waves' numerators
+  __shared__ float sm_m[4][GQA_HEADS], sm_l[4][GQA_HEADS];
+  static_assert(4 * D * PA_VSTRIDE * 2 >= 4 * GQA_HEADS * D * 4, "the numerators fit the staging area");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int split = blockIdx.x, bg = blockIdx.y;
+  const int b = bg / a.Hkv, g = bg % a.Hkv;
+  const int step = *a.step;
+  const int valid = step + 1 < a.max_len ? step + 1 : a.max_len;
+  const int chunk = attn_chunk(valid, a.nsplit);
+  const int c0 = split * chunk;
+  if (c0 >= valid) return;
+  const int c1 = c0 + chunk < valid ? c0 + chunk : valid;
+  const int pos = step % a.max_len;
+  const bool owner = FUSED && pos >= c0 && pos < c1;
+  const size_t ring_at = ((size_t)b * a.Hkv + g) * a.max_len * D;
+  const f16* kbase = a.kring + ring_at;
+  const f16* vbase = a.vring + ring_at;
+
+  // a step's rows: K as the A operands of its two tiles (lane l: row l % 16, features (l / 16) * 8 + 0..7 of each 32),
+  // V for the transposition; rows past the chunk read its last row (finite values under a probability of zero).  The
+  // first step's rows are requested before the queries are prepared: they do not depend on them.
+  f16x8 kf[2][D / 32], vv[VPR / 2];
+  auto request = [&](int p0) {
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      const int row = p0 + hh * 16 + (lane & 15);
+      const int rc = row < c1 ? row : c1 - 1;
+#pragma unroll
+      for (int m = 0; m < D / 32; ++m)
+        kf[hh][m] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(kbase + (size_t)rc * D + m * 32 + (lane >> 4) * 8));
+    }
+#pragma unroll
+    for (int i = 0; i < VPR / 2; ++i) {
+      const int c = lane + i * 64;
+      const int row = c / VPR, col = (c % VPR) * 8;
+      const int rc = p0 + row < c1 ? p0 + row : c1 - 1;
+      vv[i] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(vbase + (size_t)rc * D + col));
+    }
+  };
+  if (c0 + wave * 32 < c1) request(c0 + wave * 32);
+
+  if constexpr (FUSED) {
+    // the angles of this position, once for all heads (the arithmetic of qkv_rope_append_rows_kernel: the same bits)
+    if (a.rope == PTA_ROPE_LLAMA && tid < (D >> 1)) {
+      const f16 ang = rope_llama_angle(step, ((const f16*)a.inv_freq)[tid]);
+      cs[0][tid] = (f16)cosf((float)ang); cs[1][tid] = (f16)sinf((float)ang);
+    } else if (a.rope == PTA_ROPE_GLM2 && tid < (D >> 2)) {
+      const f16 ang = (f16)((float)step * ((const float*)a.inv_freq)[tid]);
+      cs[0][tid] = (f16)cosf((float)ang); cs[1][tid] = (f16)sinf((float)ang);
+    }
+    __syncthreads();
+  }
+  {
+    const int nvec = GQA_HEADS * VPR + (owner ? 2 * VPR : 0);
+    for (int vi = tid; vi < nvec; vi += 256) {
+      const int sect = vi < GQA_HEADS * VPR ? 0 : 1 + (vi - GQA_HEADS * VPR) / VPR;
+      const int h = sect == 0 ? vi / VPR : 0, d0 = (vi % VPR) * 8;
+      const f16* x;
+      if constexpr (FUSED)
+        x = sect == 0 ? a.q_raw + (size_t)b * a.q_stride + (size_t)(g * GQA_HEADS + h) * D
+          : sect == 1 ? a.k_raw + (size_t)b * a.k_stride + (size_t)g * D : a.v_raw + (size_t)b * a.v_stride + (size_t)g * D;
+      else
+        x = a.q + ((size_t)b * a.Hq + g * GQA_HEADS + h) * D;
+      f16x8 y = *reinterpret_cast<const f16x8*>(x + d0);
+      if constexpr (FUSED) {
+        if (sect < 2 && a.rope == PTA_ROPE_LLAMA) {
+          const int half = D >> 1;
+          const bool low = d0 < half;
+          const f16x8 o = *reinterpret_cast<const f16x8*>(x + (low ? d0 + half : d0 - half));
+          const int i0 = low ? d0 : d0 - half;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) y[j] = rope_mix(y[j], low ? -o[j] : o[j], cs[0][i0 + j], cs[1][i0 + j]);
+        } else if (sect < 2 && a.rope == PTA_ROPE_GLM2 && d0 < (D >> 1)) {
+          const f16x8 xin = y;
+#pragma unroll
+          for (int j = 0; j < 8; ++j) y[j] = rope_mix(xin[j], (j & 1) ? xin[j - 1] : -xin[j + 1], cs[0][(d0 + j) >> 1], cs[1][(d0 + j) >> 1]);
+        }
+      }
+      if (sect == 0) {
+        *reinterpret_cast<f16x8*>(sm_q + h * QS + d0) = y;
+      } else {
+        *reinterpret_cast<f16x8*>(sm_kv + (sect - 1) * D + d0) = y;
+        *reinterpret_cast<f16x8*>((sect == 1 ? a.kring_w : a.vring_w) + ring_at + (size_t)pos * D + d0) = y;
+      }
+    }
+  }
+  __syncthreads();
+  f16x8 qf[D / 32];
+#pragma unroll
+  for (int m = 0; m < D / 32; ++m) qf[m] = *reinterpret_cast<const f16x8*>(sm_q + (lane & 15) * QS + m * 32 + (lane >> 4) * 8);
+
+  f16* vt = vt_all + wave * (D * PA_VSTRIDE);
+  float run_m = -INFINITY, run_l = 0.f;
+  f32x4 o[D / 16];
+#pragma unroll
+  for (int jd = 0; jd < D / 16; ++jd) o[jd] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int p0 = c0 + wave * 32; p0 < c1; p0 += 128) {
+    // this step's position comes from LDS (its ring copy is being written by this launch)
+    if (owner) {
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        const int row = p0 + hh * 16 + (lane & 15);
+        if ((row < c1 ? row : c1 - 1) == pos) {
+#pragma unroll
+          for (int m = 0; m < D / 32; ++m) kf[hh][m] = *reinterpret_cast<const f16x8*>(sm_kv + m * 32 + (lane >> 4) * 8);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < VPR / 2; ++i) {
+        const int c = lane + i * 64;
+        const int row = c / VPR, col = (c % VPR) * 8;
+        if ((p0 + row < c1 ? p0 + row : c1 - 1) == pos) vv[i] = *reinterpret_cast<const f16x8*>(sm_kv + D + col);
+      }
+    }
+    f32x4 sc[2];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      sc[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int m = 0; m < D / 32; ++m) sc[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[hh][m], qf[m], sc[hh], 0, 0, 0);
+    }
+    // (the wave's own staging area: its LDS accesses complete in the order of their issue)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int i = 0; i < VPR / 2; ++i) {
+      const int c = lane + i * 64;
+      const int row = c / VPR, col = (c % VPR) * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[pa_vt_at(col + e, row)] = vv[i][e];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if (p0 + 128 < c1) request(p0 + 128);           // the next step's rows travel during this step's softmax and products
+    float x[8];
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        f16 s16 = (f16)sc[hh][r];                   // fp16 output of the q.K^T MatMul
+        if (a.use_scale) s16 = s16 * a.scale;       // fp16 multiply by fp16(1/sqrt(D))
+        const int row = p0 + hh * 16 + (lane >> 4) * 4 + r;
+        x[hh * 4 + r] = row < c1 ? (float)s16 : -INFINITY;
+      }
+    float mx = x[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float new_m = fmaxf(run_m, mx);           // (finite: the step's first row lies inside the chunk)
+    const float corr = run_m == -INFINITY ? 0.f : __expf(run_m - new_m);
+    float psum = 0.f;
+    f16x8 pa;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pe = x[e] == -INFINITY ? 0.f : __expf(x[e] - new_m);
+      psum += pe;
+      pa[e] = (f16)pe;
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    run_l = run_l * corr + psum;
+    run_m = new_m;
+    // the accumulators' rows are heads (lane / 16) * 4 + r: their correction factors sit in the lanes of that index
+    float cr[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cr[r] = __shfl(corr, (lane >> 4) * 4 + r, 64);
+#pragma unroll
+    for (int jd = 0; jd < D / 16; ++jd) {
+      const int d = jd * 16 + (lane & 15);
+      const f16x4 v0 = *reinterpret_cast<const f16x4*>(vt + pa_vt_at(d, (lane >> 4) * 4));
+      const f16x4 v1 = *reinterpret_cast<const f16x4*>(vt + pa_vt_at(d, 16 + (lane >> 4) * 4));
+      const f16x8 vb = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[jd][r] *= cr[r];
+      o[jd] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[jd], 0, 0, 0);
+    }
+  }
+
+  // the waves' states meet in LDS (the staging areas are done with)
+  __syncthreads();
+  float* sm_o = reinterpret_cast<float*>(vt_all);        // [4][GQA_HEADS][D]
+  if (lane < GQA_HEADS) { sm_m[wave][lane] = run_m; sm_l[wave][lane] = run_l; }
+#pragma unroll
+  for (int jd = 0; jd < D / 16; ++jd)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sm_o[((size_t)wave * GQA_HEADS + (lane >> 4) * 4 + r) * D + jd * 16 + (lane & 15)] = o[jd][r];
+  __syncthreads();
+  for (int idx = tid; idx < GQA_HEADS * D; idx += 256) {
+    const int h = idx / D, d = idx % D;
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) M = fmaxf(M, sm_m[i][h]);
+    float L = 0.f, A = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float w = sm_m[i][h] == -INFINITY ? 0.f : __expf(sm_m[i][h] - M);
+      L = __builtin_fmaf(sm_l[i][h], w, L);
+      A = __builtin_fmaf(sm_o[((size_t)i * GQA_HEADS + h) * D + d], w, A);
+    }
+    const size_t bh = (size_t)b * a.Hq + g * GQA_HEADS + h;
+    if (a.nsplit == 1) {                     // the only chunk: the context vector itself
+      a.out[bh * D + d] = attn_result(a, (f16)(A / L));
+      continue;
+    }
+    float* out = a.part + (bh * a.nsplit + split) * (D + 2);
+    out[2 + d] = A;
+    if (d == 0) { out[0] = M; out[1] = L; }
+  }
+}
+
+// chunks per (sequence, KV head) for attn_gqa_partial_kernel: about 128 workgroups in all (ChatGLM2-6B, 8 sequences,
+// contexts 512..1023: 2.27 ms per step with 128, 2.29 with 256, 2.33 with 512, 2.34 with 64), never more than one per
+// 64 cache rows
+static int attn_gqa_splits(int B, int Hkv, int max_len) {
+  const int cap = (max_len + 63) / 64;
+  int n = (128 + B * Hkv - 1) / (B * Hkv);
+  n = n < 1 ? 1 : n;
+  return n > cap ? cap : n;
+}
+
 extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int max_len) {
   if (B <= 0 || Hq <= 0 || D <= 0 || max_len <= 0) return 0;
   const int chunk = 64;
@@ -666,8 +933,32 @@ extern "C" size_t pta_decode_attention_workspace_bytes(int B, int Hq, int D, int
   return (size_t)B * Hq * nsplit * (D + 2) * sizeof(float);
 }
 
+// whether a decode-attention launch goes to attn_gqa_partial_kernel: one row per sequence, sixteen query heads per KV
+// head, an fp16 ring, and 16-byte vectors wherever that kernel reads its operands
+static bool attn_gqa_fits(const AttnArgs& a, bool kv8, bool fused) {
+  if (kv8 || a.rows != 1 || a.Hq != GQA_HEADS * a.Hkv) return false;
+  if (fused)
+    return a.q_stride % 8 == 0 && a.k_stride % 8 == 0 && a.v_stride % 8 == 0 &&
+           (((uintptr_t)a.q_raw | (uintptr_t)a.k_raw | (uintptr_t)a.v_raw) & 15) == 0;
+  return true;
+}
+
 template <bool FUSED>
-static void launch_attention(const AttnArgs& a, int D, bool kv8, int heads_rows, hipStream_t s) {
+static void launch_attention(const AttnArgs& a_in, int D, bool kv8, int heads_rows, hipStream_t s) {
+  if (attn_gqa_fits(a_in, kv8, FUSED)) {
+    AttnArgs a = a_in;
+    a.nsplit = attn_gqa_splits(a.B, a.Hkv, a.max_len);
+    const dim3 grid(a.nsplit, a.B * a.Hkv);
+    if (D == 128) {
+      hipLaunchKernelGGL((attn_gqa_partial_kernel<128, FUSED>), grid, dim3(256), 0, s, a);
+      if (a.nsplit > 1) hipLaunchKernelGGL(attn_combine_kernel<128>, dim3(heads_rows), dim3(128), 0, s, a);
+    } else {
+      hipLaunchKernelGGL((attn_gqa_partial_kernel<64, FUSED>), grid, dim3(256), 0, s, a);
+      if (a.nsplit > 1) hipLaunchKernelGGL(attn_combine_kernel<64>, dim3(heads_rows), dim3(64), 0, s, a);
+    }
+    return;
+  }
+  const AttnArgs& a = a_in;
   dim3 grid(a.nsplit, heads_rows);
   if (D == 128) {
     if (kv8) hipLaunchKernelGGL((attn_partial_kernel<128, FUSED, true>), grid, dim3(ATT_THREADS), 0, s, a);
