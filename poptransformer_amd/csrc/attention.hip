@@ -744,6 +744,32 @@ __global__ __launch_bounds__(256) void attn_gqa_partial_kernel(AttnArgs a) {
   };
   if (c0 + wave * 32 < c1) request(c0 + wave * 32);
 
+  // the queries of the sixteen heads (and, in the chunk that holds this step's position, the new key and value): one
+  // vector of eight per thread, a second one for 2 * D / 8 threads of that chunk; requested before the angles are
+  // worked out
+  const int nvec = GQA_HEADS * VPR + (owner ? 2 * VPR : 0);
+  int p_sect[2], p_h[2], p_d0[2];
+  bool p_on[2];
+  f16x8 p_y[2], p_o[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int vi = tid + u * 256;
+    p_on[u] = vi < nvec;
+    p_sect[u] = vi < GQA_HEADS * VPR ? 0 : 1 + (vi - GQA_HEADS * VPR) / VPR;
+    p_h[u] = p_sect[u] == 0 ? vi / VPR : 0;
+    p_d0[u] = (vi % VPR) * 8;
+    p_y[u] = f16x8{}; p_o[u] = f16x8{};
+    if (!p_on[u]) continue;
+    const f16* x;
+    if constexpr (FUSED)
+      x = p_sect[u] == 0 ? a.q_raw + (size_t)b * a.q_stride + (size_t)(g * GQA_HEADS + p_h[u]) * D
+        : p_sect[u] == 1 ? a.k_raw + (size_t)b * a.k_stride + (size_t)g * D : a.v_raw + (size_t)b * a.v_stride + (size_t)g * D;
+    else
+      x = a.q + ((size_t)b * a.Hq + g * GQA_HEADS + p_h[u]) * D;
+    p_y[u] = *reinterpret_cast<const f16x8*>(x + p_d0[u]);
+    if (FUSED && p_sect[u] < 2 && a.rope == PTA_ROPE_LLAMA)
+      p_o[u] = *reinterpret_cast<const f16x8*>(x + (p_d0[u] < (D >> 1) ? p_d0[u] + (D >> 1) : p_d0[u] - (D >> 1)));
+  }
   if constexpr (FUSED) {
     // the angles of this position, once for all heads (the arithmetic of qkv_rope_append_rows_kernel: the same bits)
     if (a.rope == PTA_ROPE_LLAMA && tid < (D >> 1)) {
@@ -755,38 +781,28 @@ __global__ __launch_bounds__(256) void attn_gqa_partial_kernel(AttnArgs a) {
     }
     __syncthreads();
   }
-  {
-    const int nvec = GQA_HEADS * VPR + (owner ? 2 * VPR : 0);
-    for (int vi = tid; vi < nvec; vi += 256) {
-      const int sect = vi < GQA_HEADS * VPR ? 0 : 1 + (vi - GQA_HEADS * VPR) / VPR;
-      const int h = sect == 0 ? vi / VPR : 0, d0 = (vi % VPR) * 8;
-      const f16* x;
-      if constexpr (FUSED)
-        x = sect == 0 ? a.q_raw + (size_t)b * a.q_stride + (size_t)(g * GQA_HEADS + h) * D
-          : sect == 1 ? a.k_raw + (size_t)b * a.k_stride + (size_t)g * D : a.v_raw + (size_t)b * a.v_stride + (size_t)g * D;
-      else
-        x = a.q + ((size_t)b * a.Hq + g * GQA_HEADS + h) * D;
-      f16x8 y = *reinterpret_cast<const f16x8*>(x + d0);
-      if constexpr (FUSED) {
-        if (sect < 2 && a.rope == PTA_ROPE_LLAMA) {
-          const int half = D >> 1;
-          const bool low = d0 < half;
-          const f16x8 o = *reinterpret_cast<const f16x8*>(x + (low ? d0 + half : d0 - half));
-          const int i0 = low ? d0 : d0 - half;
 #pragma unroll
-          for (int j = 0; j < 8; ++j) y[j] = rope_mix(y[j], low ? -o[j] : o[j], cs[0][i0 + j], cs[1][i0 + j]);
-        } else if (sect < 2 && a.rope == PTA_ROPE_GLM2 && d0 < (D >> 1)) {
-          const f16x8 xin = y;
+  for (int u = 0; u < 2; ++u) {
+    if (!p_on[u]) continue;
+    const int sect = p_sect[u], d0 = p_d0[u];
+    f16x8 y = p_y[u];
+    if constexpr (FUSED) {
+      if (sect < 2 && a.rope == PTA_ROPE_LLAMA) {
+        const bool low = d0 < (D >> 1);
+        const int i0 = low ? d0 : d0 - (D >> 1);
 #pragma unroll
-          for (int j = 0; j < 8; ++j) y[j] = rope_mix(xin[j], (j & 1) ? xin[j - 1] : -xin[j + 1], cs[0][(d0 + j) >> 1], cs[1][(d0 + j) >> 1]);
-        }
+        for (int j = 0; j < 8; ++j) y[j] = rope_mix(y[j], low ? -p_o[u][j] : p_o[u][j], cs[0][i0 + j], cs[1][i0 + j]);
+      } else if (sect < 2 && a.rope == PTA_ROPE_GLM2 && d0 < (D >> 1)) {
+        const f16x8 xin = y;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = rope_mix(xin[j], (j & 1) ? xin[j - 1] : -xin[j + 1], cs[0][(d0 + j) >> 1], cs[1][(d0 + j) >> 1]);
       }
-      if (sect == 0) {
-        *reinterpret_cast<f16x8*>(sm_q + h * QS + d0) = y;
-      } else {
-        *reinterpret_cast<f16x8*>(sm_kv + (sect - 1) * D + d0) = y;
-        *reinterpret_cast<f16x8*>((sect == 1 ? a.kring_w : a.vring_w) + ring_at + (size_t)pos * D + d0) = y;
-      }
+    }
+    if (sect == 0) {
+      *reinterpret_cast<f16x8*>(sm_q + p_h[u] * QS + d0) = y;
+    } else {
+      *reinterpret_cast<f16x8*>(sm_kv + (sect - 1) * D + d0) = y;
+      *reinterpret_cast<f16x8*>((sect == 1 ? a.kring_w : a.vring_w) + ring_at + (size_t)pos * D + d0) = y;
     }
   }
   __syncthreads();
