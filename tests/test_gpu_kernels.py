@@ -666,7 +666,9 @@ def _attention_reference(family, qs, ks, vs, max_len, D, fp8_cache=False):
                                                              # sixteen query heads per KV head: the grouped kernel on the
                                                              # matrix unit (one chunk and several, a ring that wraps)
                                                              ("glm2", 2, 32, 2, 128, 150, 170), ("llama", 1, 16, 1, 64, 40, 50),
-                                                             ("glm2", 2, 16, 1, 64, 300, 200)])
+                                                             ("glm2", 2, 16, 1, 64, 300, 200),
+                                                             # 128 (sequence, KV head) pairs: one chunk each, several steps per wave
+                                                             ("glm2", 64, 32, 2, 64, 200, 170)])
 def test_rope_append_attention(K, family, B, Hq, Hkv, D, max_len, steps):
     from poptransformer_amd import _lib
     rng = np.random.default_rng(B + Hq + D)
@@ -696,7 +698,8 @@ def test_rope_append_attention(K, family, B, Hq, Hkv, D, max_len, steps):
 
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 130), ("gpt2", 1, 12, 12, 64, 40, 45),
                                                              ("glm2", 3, 8, 2, 128, 150, 90),
-                                                             ("glm2", 2, 32, 2, 128, 150, 170), ("llama", 1, 16, 1, 64, 70, 90)])
+                                                             ("glm2", 2, 32, 2, 128, 150, 170), ("llama", 1, 16, 1, 64, 70, 90),
+                                                             ("glm2", 64, 32, 2, 64, 200, 170)])
 def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, Hkv, D, max_len, steps):
     """pta_decode_attention_qkv (rotary + append inside the attention pass) against the two separate calls: the
     same context vectors and the same ring, bit for bit, at every step including those after the ring has
