@@ -476,6 +476,9 @@ __global__ __launch_bounds__(D) void attn_combine_kernel(AttnArgs a) {
 static int attn_splits(int B, int Hq, int max_len) {
   const int cap = (max_len + 63) / 64;
   if (B * Hq >= 512) return 1;
+  // a ring of up to 256 rows: one workgroup walks it in four rounds of loads, which costs less than the merging launch
+  // (GPT-2 small, 12 heads, ring of 128: 0.312 -> 0.285 ms per token)
+  if (max_len <= 256) return 1;
   int n = (1024 + B * Hq - 1) / (B * Hq);
   n = n < 1 ? 1 : n;
   return n > cap ? cap : n;
@@ -937,6 +940,7 @@ __global__ __launch_bounds__(256) void attn_gqa_partial_kernel(AttnArgs a) {
 // 64 cache rows
 static int attn_gqa_splits(int B, int Hkv, int max_len) {
   const int cap = (max_len + 63) / 64;
+  if (max_len <= 256) return 1;
   int n = (128 + B * Hkv - 1) / (B * Hkv);
   n = n < 1 ? 1 : n;
   return n > cap ? cap : n;

@@ -663,6 +663,8 @@ def _attention_reference(family, qs, ks, vs, max_len, D, fp8_cache=False):
 
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 70), ("gpt2", 1, 12, 12, 64, 40, 40),
                                                              ("glm2", 2, 8, 2, 128, 150, 80), ("llama", 1, 2, 2, 128, 16, 20),
+                                                             # rings of more than 256 rows: several chunks per head and the merging launch
+                                                             ("llama", 2, 4, 4, 128, 300, 330), ("gpt2", 1, 12, 12, 64, 320, 100),
                                                              # sixteen query heads per KV head: the grouped kernel on the
                                                              # matrix unit (one chunk and several, a ring that wraps)
                                                              ("glm2", 2, 32, 2, 128, 150, 170), ("llama", 1, 16, 1, 64, 40, 50),
@@ -697,7 +699,7 @@ def test_rope_append_attention(K, family, B, Hq, Hkv, D, max_len, steps):
 
 
 @pytest.mark.parametrize("family,B,Hq,Hkv,D,max_len,steps", [("llama", 2, 4, 4, 128, 100, 130), ("gpt2", 1, 12, 12, 64, 40, 45),
-                                                             ("glm2", 3, 8, 2, 128, 150, 90),
+                                                             ("glm2", 3, 8, 2, 128, 150, 90), ("glm2", 3, 8, 2, 128, 320, 350),
                                                              ("glm2", 2, 32, 2, 128, 150, 170), ("llama", 1, 16, 1, 64, 70, 90),
                                                              ("glm2", 64, 32, 2, 64, 200, 170)])
 def test_attention_with_its_own_preparation_is_bit_identical(K, family, B, Hq, Hkv, D, max_len, steps):
